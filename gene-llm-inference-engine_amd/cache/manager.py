@@ -1,0 +1,251 @@
+"""The cache manager: pages of keys and values with a page table per request, and slots of
+fixed-size state.
+
+Layers of the run order whose cache needs are equal (same key/value geometry, same window) form
+a group.  A group owns a pool of pages, storage [layer][page][K|V][kv_head][place][head_dim]
+and one page table per request slot: table[slot][i] is the page that holds positions
+i*page_size .. (i+1)*page_size-1 of that request in every layer of the group, or -1.  A group
+with a window gives pages back as soon as no later position can see them; a request that ends
+gives back everything.  Requests also hold a slot in every fixed-size state tensor
+[slot][...], zeroed when the request opens.
+
+The reference's pool is one group over all layers with per-sequence tables kept on the host
+(src/model/kv_cache.h:4-13, 73-118); groups, windows and state slots have no counterpart there.
+"""
+from __future__ import annotations
+
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from .needs import PagedKvNeed, StateNeed
+from .pages import OutOfPages, PagePool
+
+
+class CacheError(RuntimeError):
+    pass
+
+
+class PageGroup:
+    def __init__(self, need: PagedKvNeed, entries: List[int], n_pages: int, page_size: int, max_requests: int,
+                 max_positions: int, dtype, device, allocate_storage: bool):
+        self.need = need
+        self.entries = list(entries)                 # run-order entries, in run order
+        self.page_size = page_size
+        self.pool = PagePool(n_pages)
+        self.table_width = -(-max_positions // page_size)
+        self.table_host = np.full((max_requests, self.table_width), -1, dtype=np.int32)
+        self.first_live = np.zeros(max_requests, dtype=np.int64)     # pages below this index were given back (windows)
+        self.n_held = np.zeros(max_requests, dtype=np.int64)         # table entries in use, counted from 0
+        self.dirty: set = set()
+        self.storage = None
+        self.table_dev = None
+        if allocate_storage:
+            self.storage = torch.zeros((len(entries), n_pages, 2, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
+            self.table_dev = torch.full((max_requests, self.table_width), -1, dtype=torch.int32, device=device)
+
+    def pages_for(self, slot: int, new_length: int) -> int:
+        """Pages to allocate so that positions below new_length have one."""
+        return max(0, -(-new_length // self.page_size) - int(self.n_held[slot]))
+
+    def grow(self, slot: int, new_length: int) -> None:
+        for _ in range(self.pages_for(slot, new_length)):
+            i = int(self.n_held[slot])
+            self.table_host[slot, i] = self.pool.allocate()
+            self.n_held[slot] = i + 1
+        self.dirty.add(slot)
+
+    def drop_behind_window(self, slot: int, length: int) -> None:
+        """After `length` positions the next row is at position `length`; it sees keys from
+        length - window + 1 on, so pages that end at or before that are given back."""
+        if self.need.window is None:
+            return
+        keep_from = (length - self.need.window + 1) // self.page_size       # first page still visible
+        i = int(self.first_live[slot])
+        while i < min(keep_from, int(self.n_held[slot])):
+            self.pool.release(int(self.table_host[slot, i]))
+            self.table_host[slot, i] = -1
+            i += 1
+            self.dirty.add(slot)
+        self.first_live[slot] = max(int(self.first_live[slot]), i)
+
+    def release_all(self, slot: int) -> None:
+        for i in range(int(self.first_live[slot]), int(self.n_held[slot])):
+            self.pool.release(int(self.table_host[slot, i]))
+        self.table_host[slot, :] = -1
+        self.first_live[slot] = 0
+        self.n_held[slot] = 0
+        self.dirty.add(slot)
+
+    def held_pages(self, slot: int) -> List[int]:
+        return [int(p) for p in self.table_host[slot, int(self.first_live[slot]):int(self.n_held[slot])]]
+
+    def sync(self) -> None:
+        if self.table_dev is None or not self.dirty:
+            self.dirty.clear()
+            return
+        rows = sorted(self.dirty)
+        self.dirty.clear()
+        idx = torch.tensor(rows, dtype=torch.int64)
+        data = torch.from_numpy(self.table_host[rows])
+        self.table_dev.index_copy_(0, idx.to(self.table_dev.device), data.to(self.table_dev.device))
+
+
+class CacheManager:
+    """`needs[i]` is the need of run-order entry i (PagedKvNeed, StateNeed or None); `reads_from[i]`
+    is the entry whose pages entry i reads instead of keeping its own (or None)."""
+
+    def __init__(self, needs: Sequence, reads_from: Sequence[Optional[int]], *, page_size: int, n_pages: int, max_requests: int,
+                 max_positions: int, dtype=torch.float32, device="cpu", allocate_storage: bool = True):
+        if page_size < 1 or n_pages < 1 or max_requests < 1 or max_positions < 1:
+            raise ValueError("page_size, n_pages, max_requests and max_positions must be positive")
+        self.page_size, self.max_requests, self.max_positions = int(page_size), int(max_requests), int(max_positions)
+        self.groups: List[PageGroup] = []
+        self._entry_group: Dict[int, Tuple[int, int]] = {}          # entry -> (group index, layer index in group)
+        self.states: Dict[int, torch.Tensor] = {}
+        by_need: Dict[PagedKvNeed, List[int]] = {}
+        for i, (need, src) in enumerate(zip(needs, reads_from)):
+            if src is not None:
+                if needs[src] != need or not isinstance(need, PagedKvNeed):
+                    raise CacheError(f"run-order entry {i} reads the cache of entry {src}, whose need differs: {needs[src]} against {need}")
+                continue
+            if isinstance(need, PagedKvNeed):
+                by_need.setdefault(need, []).append(i)
+            elif isinstance(need, StateNeed):
+                if allocate_storage:
+                    self.states[i] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
+            elif need is not None:
+                raise CacheError(f"run-order entry {i} has an unknown cache need {need!r}")
+        for need, entries in by_need.items():
+            g = PageGroup(need, entries, n_pages, page_size, max_requests, max_positions, dtype, device, allocate_storage)
+            for li, e in enumerate(entries):
+                self._entry_group[e] = (len(self.groups), li)
+            self.groups.append(g)
+        for i, src in enumerate(reads_from):
+            if src is not None:
+                self._entry_group[i] = self._entry_group[src]
+        self._free_slots = list(range(max_requests - 1, -1, -1))
+        self._slot: Dict[Hashable, int] = {}
+        self._length: Dict[Hashable, int] = {}
+
+    # ------------------------------------------------------------------------------ requests
+    def open(self, request: Hashable) -> int:
+        if request in self._slot:
+            raise CacheError(f"request {request!r} is already open")
+        if not self._free_slots:
+            raise CacheError(f"all {self.max_requests} request slots are in use")
+        slot = self._free_slots.pop()
+        self._slot[request] = slot
+        self._length[request] = 0
+        for s in self.states.values():
+            s[slot].zero_()
+        return slot
+
+    def close(self, request: Hashable) -> None:
+        slot = self.slot(request)
+        for g in self.groups:
+            g.release_all(slot)
+        del self._slot[request], self._length[request]
+        self._free_slots.append(slot)
+
+    def is_open(self, request: Hashable) -> bool:
+        return request in self._slot
+
+    def slot(self, request: Hashable) -> int:
+        try:
+            return self._slot[request]
+        except KeyError:
+            raise CacheError(f"request {request!r} is not open") from None
+
+    def length(self, request: Hashable) -> int:
+        self.slot(request)
+        return self._length[request]
+
+    def open_requests(self):
+        return list(self._slot)
+
+    @property
+    def free_slots(self) -> int:
+        return len(self._free_slots)
+
+    # --------------------------------------------------------------------------------- pages
+    def pages_needed(self, request: Hashable, n_new: int) -> List[int]:
+        """New pages per group for n_new more positions of the request."""
+        slot, length = self.slot(request), self._length[request]
+        return [g.pages_for(slot, length + n_new) for g in self.groups]
+
+    def free_pages(self) -> List[int]:
+        return [g.pool.free_count for g in self.groups]
+
+    def fits(self, additions: Sequence[Tuple[Hashable, int]]) -> bool:
+        need = [0] * len(self.groups)
+        for request, n_new in additions:
+            for gi, n in enumerate(self.pages_needed(request, n_new)):
+                need[gi] += n
+        return all(n <= g.pool.free_count for n, g in zip(need, self.groups))
+
+    def reserve(self, additions: Sequence[Tuple[Hashable, int]]) -> None:
+        """Pages for n_new more positions of every named request, or `OutOfPages` with nothing changed."""
+        seen = set()
+        for request, n_new in additions:
+            if request in seen:
+                raise CacheError(f"request {request!r} is named twice in one reservation")
+            seen.add(request)
+            if n_new < 1:
+                raise CacheError("a reservation must add at least one position")
+            if self.length(request) + n_new > self.max_positions:
+                raise CacheError(f"request {request!r} would reach position {self._length[request] + n_new}, beyond the limit {self.max_positions}")
+        if not self.fits(additions):
+            raise OutOfPages(f"not enough free pages (free per group: {self.free_pages()})")
+        for request, n_new in additions:
+            slot, length = self._slot[request], self._length[request]
+            for g in self.groups:
+                g.grow(slot, length + n_new)
+
+    def advance(self, request: Hashable, n_new: int) -> None:
+        """The reserved positions have been written: the request is n_new longer; pages behind a
+        window are given back."""
+        slot = self.slot(request)
+        self._length[request] += n_new
+        for g in self.groups:
+            if self._length[request] > int(g.n_held[slot]) * g.page_size:
+                raise CacheError(f"request {request!r} advanced beyond its reserved pages")
+            g.drop_behind_window(slot, self._length[request])
+
+    def sync(self) -> None:
+        """Brings the device copies of changed page tables up to date."""
+        for g in self.groups:
+            g.sync()
+
+    # --------------------------------------------------------------------------------- views
+    def kv(self, entry: int):
+        """(cache of the entry's layer [page, 2, kv_head, place, hd], device page table, window)."""
+        gi, li = self._entry_group[entry]
+        g = self.groups[gi]
+        return g.storage[li], g.table_dev, g.need.window
+
+    def state(self, entry: int) -> torch.Tensor:
+        return self.states[entry]
+
+    def check_consistency(self) -> None:
+        """Every page is either free or held by exactly one open request (no sharing is used)."""
+        for gi, g in enumerate(self.groups):
+            held: Dict[int, Hashable] = {}
+            for request, slot in self._slot.items():
+                for p in g.held_pages(slot):
+                    if p < 0:
+                        raise CacheError(f"group {gi}: request {request!r} holds no page at a live place")
+                    if p in held:
+                        raise CacheError(f"group {gi}: page {p} is held by {held[p]!r} and {request!r}")
+                    held[p] = request
+            free = set(g.pool._free)
+            if len(free) != len(g.pool._free):
+                raise CacheError(f"group {gi}: a page is twice in the free stack")
+            if free & set(held):
+                raise CacheError(f"group {gi}: pages {sorted(free & set(held))} are free and held")
+            if len(free) + len(held) != g.pool.n_pages:
+                raise CacheError(f"group {gi}: {g.pool.n_pages - len(free) - len(held)} pages are lost")
+            for p in range(g.pool.n_pages):
+                if g.pool.ref_count(p) != (1 if p in held else 0):
+                    raise CacheError(f"group {gi}: page {p} has reference count {g.pool.ref_count(p)}")

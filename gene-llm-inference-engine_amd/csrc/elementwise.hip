@@ -1,0 +1,203 @@
+// Row-wise kernels around the matrix products: token embedding, RMS norm, rotary angles,
+// rotation + cache write, SiLU gating, row gather.  All arithmetic is 32-bit (angles 64-bit);
+// only what is loaded or stored may be bfloat16.
+#include "common.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+static thread_local char g_error[512] = "";
+
+int gi_fail(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return -1;
+}
+
+GI_API const char* gi_last_error() { return g_error; }
+
+GI_API int gi_device_arch(char* out, int cap) {
+    hipDeviceProp_t p;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&p, dev) != hipSuccess) return gi_fail("no HIP device");
+    snprintf(out, cap, "%s", p.gcnArchName);
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------- embedding
+// x[t, :] = table[tokens[t], :], widened to 32-bit.  Reference: src/gpu/device_kernels.inc:37-51.
+template <typename TT>
+__global__ void embed_kernel(const TT* __restrict__ table, const int* __restrict__ tokens, float* __restrict__ x, int dim) {
+    const int t = blockIdx.x;
+    const TT* row = table + (size_t)tokens[t] * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) x[(size_t)t * dim + d] = load_f32(row, d);
+}
+
+GI_API int gi_embed(const void* table, int table_dtype, const int* tokens, float* x, int n_rows, int dim, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && dim > 0, "embed: n_rows %d and dim %d must be positive", n_rows, dim);
+    if (table_dtype == GI_F32)
+        embed_kernel<float><<<n_rows, 256, 0, stream>>>((const float*)table, tokens, x, dim);
+    else if (table_dtype == GI_BF16)
+        embed_kernel<bf16_t><<<n_rows, 256, 0, stream>>>((const bf16_t*)table, tokens, x, dim);
+    else
+        return gi_fail("embed: unknown table dtype %d", table_dtype);
+    GI_CHECK_LAUNCH("embed");
+    return 0;
+}
+
+// -------------------------------------------------------------------------------------- RMS norm
+// out = w * (x * rsqrt(mean(x^2) + eps)), one workgroup per row; the sum of squares is taken in
+// 32-bit in an order that depends on the row's length only.  Reference: src/kernels/kernels.cpp:72-83.
+template <typename TW, typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ w, TO* __restrict__ out, int dim, float eps,
+                               size_t x_stride, size_t out_stride) {
+    __shared__ float red[4];
+    const float* xr = x + (size_t)blockIdx.x * x_stride;
+    TO* orow = out + (size_t)blockIdx.x * out_stride;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 256) ss = fmaf(xr[d], xr[d], ss);
+    ss = block_sum<256>(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)dim + eps);
+    for (int d = threadIdx.x; d < dim; d += 256) store_f32(orow, d, load_f32(w, d) * (scale * xr[d]));
+}
+
+GI_API int gi_rmsnorm(const float* x, const void* w, int w_dtype, void* out, int out_dtype, int n_rows, int dim, float eps,
+                      long x_stride, long out_stride, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && dim > 0, "rmsnorm: n_rows %d and dim %d must be positive", n_rows, dim);
+    GI_REQUIRE(x_stride >= dim && out_stride >= dim, "rmsnorm: row strides must be at least dim");
+#define LAUNCH(TW, TO) rmsnorm_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(x, (const TW*)w, (TO*)out, dim, eps, (size_t)x_stride, (size_t)out_stride)
+    if (w_dtype == GI_F32 && out_dtype == GI_F32) LAUNCH(float, float);
+    else if (w_dtype == GI_F32 && out_dtype == GI_BF16) LAUNCH(float, bf16_t);
+    else if (w_dtype == GI_BF16 && out_dtype == GI_F32) LAUNCH(bf16_t, float);
+    else if (w_dtype == GI_BF16 && out_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t);
+    else return gi_fail("rmsnorm: unknown dtypes %d, %d", w_dtype, out_dtype);
+#undef LAUNCH
+    GI_CHECK_LAUNCH("rmsnorm");
+    return 0;
+}
+
+// -------------------------------------------------------------------------------- rotary angles
+// cos and sin of pos * f_k for every row, the angle taken in 64-bit: a 32-bit angle loses digits
+// at large positions (reference: src/kernels/kernels.cpp:145-161).
+__global__ void rope_cos_sin_kernel(const int* __restrict__ pos, const double* __restrict__ inv_freq, float* __restrict__ cos_out,
+                                    float* __restrict__ sin_out, int n_rows, int half) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_rows * half) return;
+    const double a = (double)pos[i / half] * inv_freq[i % half];
+    cos_out[i] = (float)cos(a);
+    sin_out[i] = (float)sin(a);
+}
+
+GI_API int gi_rope_cos_sin(const int* pos, const double* inv_freq, float* cos_out, float* sin_out, int n_rows, int half,
+                           hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && half > 0, "rope_cos_sin: n_rows %d and half %d must be positive", n_rows, half);
+    const int n = n_rows * half;
+    rope_cos_sin_kernel<<<(n + 255) / 256, 256, 0, stream>>>(pos, inv_freq, cos_out, sin_out, n_rows, half);
+    GI_CHECK_LAUNCH("rope_cos_sin");
+    return 0;
+}
+
+// ---------------------------------------------------------------- rotation and cache write, fused
+// For row t at position pos[t] of the request in slot[t]:
+//   q heads are rotated and written to q_out [n_rows, n_heads*hd];
+//   k heads are rotated and, with the v heads as they are, written into the page
+//   table[slot[t]][pos / page_size] at place pos % page_size.
+// Pairs are (k, k + hd/2): a' = a*cos - b*sin, b' = a*sin + b*cos (src/kernels/kernels.cpp:165-180).
+// Cache of one layer: [page][K|V][kv_head][place][hd].  cos == nullptr means no rotation.
+// k == nullptr means the layer reads another layer's cache and writes none.
+template <typename TQ, typename TC>
+__global__ void rope_store_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, long ldq, long ldk,
+                                  long ldv, const float* __restrict__ cos_t, const float* __restrict__ sin_t, const int* __restrict__ pos,
+                                  const int* __restrict__ slot, const int* __restrict__ table, int table_stride, TQ* __restrict__ q_out,
+                                  TC* __restrict__ cache, long page_stride, int page_size, int n_heads, int n_kv, int hd) {
+    const int t = blockIdx.x, half = hd / 2;
+    const float* c = cos_t ? cos_t + (size_t)t * half : nullptr;
+    const float* s = sin_t ? sin_t + (size_t)t * half : nullptr;
+    const int n_q_items = n_heads * half;
+    for (int i = threadIdx.x; i < n_q_items; i += blockDim.x) {
+        const int h = i / half, kk = i % half;
+        const float a = q[(size_t)t * ldq + h * hd + kk], b = q[(size_t)t * ldq + h * hd + kk + half];
+        const float cc = c ? c[kk] : 1.f, ss = s ? s[kk] : 0.f;
+        store_f32(q_out, (size_t)t * n_heads * hd + h * hd + kk, a * cc - b * ss);
+        store_f32(q_out, (size_t)t * n_heads * hd + h * hd + kk + half, a * ss + b * cc);
+    }
+    if (k == nullptr) return;
+    const int p = pos[t];
+    const long page = table[(size_t)slot[t] * table_stride + p / page_size];
+    const int place = p % page_size;
+    TC* kbase = cache + page * page_stride;
+    TC* vbase = kbase + (size_t)n_kv * page_size * hd;
+    const int n_k_items = n_kv * half;
+    for (int i = threadIdx.x; i < n_k_items; i += blockDim.x) {
+        const int g = i / half, kk = i % half;
+        const float a = k[(size_t)t * ldk + g * hd + kk], b = k[(size_t)t * ldk + g * hd + kk + half];
+        const float cc = c ? c[kk] : 1.f, ss = s ? s[kk] : 0.f;
+        const size_t o = ((size_t)g * page_size + place) * hd;
+        store_f32(kbase, o + kk, a * cc - b * ss);
+        store_f32(kbase, o + kk + half, a * ss + b * cc);
+        store_f32(vbase, o + kk, v[(size_t)t * ldv + g * hd + kk]);
+        store_f32(vbase, o + kk + half, v[(size_t)t * ldv + g * hd + kk + half]);
+    }
+}
+
+GI_API int gi_rope_store(const float* q, const float* k, const float* v, long ldq, long ldk, long ldv, const float* cos_t,
+                         const float* sin_t, const int* pos, const int* slot, const int* table, int table_stride, void* q_out,
+                         int q_dtype, void* cache, int cache_dtype, long page_stride, int page_size, int n_rows, int n_heads,
+                         int n_kv, int hd, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && hd > 0 && hd % 2 == 0, "rope_store: bad sizes (rows %d heads %d kv %d hd %d)",
+               n_rows, n_heads, n_kv, hd);
+    GI_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "rope_store: cos and sin must both be given or both be absent");
+    GI_REQUIRE(k == nullptr || (v != nullptr && cache != nullptr && table != nullptr && page_size > 0 &&
+                                page_stride >= 2L * n_kv * page_size * hd),
+               "rope_store: cache write needs v, a cache, a table and a page stride of at least 2*n_kv*page_size*hd");
+#define LAUNCH(TQ, TC)                                                                                                       \
+    rope_store_kernel<TQ, TC><<<n_rows, 256, 0, stream>>>(q, k, v, ldq, ldk, ldv, cos_t, sin_t, pos, slot, table, table_stride, \
+                                                          (TQ*)q_out, (TC*)cache, page_stride, page_size, n_heads, n_kv, hd)
+    if (q_dtype == GI_F32 && cache_dtype == GI_F32) LAUNCH(float, float);
+    else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t);
+    else if (q_dtype == GI_F32 && cache_dtype == GI_BF16) LAUNCH(float, bf16_t);
+    else if (q_dtype == GI_BF16 && cache_dtype == GI_F32) LAUNCH(bf16_t, float);
+    else return gi_fail("rope_store: unknown dtypes %d, %d", q_dtype, cache_dtype);
+#undef LAUNCH
+    GI_CHECK_LAUNCH("rope_store");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------ SiLU gate
+// h[t, i] = silu(gu[t, i]) * gu[t, inter + i], silu(g) = g * (1 / (1 + exp(-g)))
+// (src/gpu/device_kernels.inc:460-469).  gu is the product with the stacked [gate; up] matrix.
+template <typename TO>
+__global__ void silu_mul_kernel(const float* __restrict__ gu, TO* __restrict__ h, int inter, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t t = i / inter, c = i % inter;
+    const float g = gu[t * 2 * inter + c], u = gu[t * 2 * inter + inter + c];
+    store_f32(h, i, (g * (1.0f / (1.0f + expf(-g)))) * u);
+}
+
+GI_API int gi_silu_mul(const float* gate_up, void* h, int h_dtype, int n_rows, int inter, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && inter > 0, "silu_mul: n_rows %d and inter %d must be positive", n_rows, inter);
+    const size_t n = (size_t)n_rows * inter;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (h_dtype == GI_F32) silu_mul_kernel<float><<<blocks, 256, 0, stream>>>(gate_up, (float*)h, inter, n);
+    else if (h_dtype == GI_BF16) silu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>(gate_up, (bf16_t*)h, inter, n);
+    else return gi_fail("silu_mul: unknown dtype %d", h_dtype);
+    GI_CHECK_LAUNCH("silu_mul");
+    return 0;
+}
+
+// ----------------------------------------------------------------------------------- row gather
+// out[i, :] = x[rows[i], :] (the rows whose logits are wanted; src/gpu/gpu_transformer.cpp:441).
+__global__ void gather_rows_kernel(const float* __restrict__ x, const int* __restrict__ rows, float* __restrict__ out, int dim) {
+    const float* src = x + (size_t)rows[blockIdx.x] * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) out[(size_t)blockIdx.x * dim + d] = src[d];
+}
+
+GI_API int gi_gather_rows(const float* x, const int* rows, float* out, int n_out, int dim, hipStream_t stream) {
+    GI_REQUIRE(n_out > 0 && dim > 0, "gather_rows: n_out %d and dim %d must be positive", n_out, dim);
+    gather_rows_kernel<<<n_out, 256, 0, stream>>>(x, rows, out, dim);
+    GI_CHECK_LAUNCH("gather_rows");
+    return 0;
+}

@@ -1,0 +1,3 @@
+"""Model assembly, the step function, the scheduler and the single-request loop."""
+from .model import DecoderModel, compute_dtype, load_model, random_model
+from .runner import Runner, StepEntry, StepError

@@ -1,0 +1,92 @@
+"""A decoder assembled from a `ModelSpec`: token table, the layers in their run order, final
+norm, output head.  It knows parts and the order they run in, not an architecture."""
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Dict, List, Optional
+
+import torch
+
+from ..config import ModelSpec, read_config
+from ..kernels import ops
+from ..parts import LayerCache, StepContext, block_class, linear, model_tensor_needs, norm_class
+from ..parts.linear import activation_dtype_for
+from ..weights import load_tensors, random_tensors
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           torch.bfloat16: torch.bfloat16, torch.float32: torch.float32}
+
+
+def compute_dtype(name) -> torch.dtype:
+    try:
+        return _DTYPES[name]
+    except KeyError:
+        raise ValueError(f"unknown dtype {name!r}: bfloat16 or float32") from None
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device):
+        self.spec, self.dtype, self.device = spec, dtype, torch.device(device)
+        self.embedding = tensors[spec.embedding]
+        self.lm_head = tensors[spec.lm_head]
+        self.layers = [block_class(l.block)(l, tensors, dtype, device) for l in spec.layers]
+        self.final_norm = norm_class(spec.final_norm)(spec.final_norm, tensors, dtype, device)
+        self.head_in_dtype = activation_dtype_for(self.lm_head, dtype)
+        self.run_order = spec.run_order
+
+    # ----------------------------------------------------------------------------- what it needs
+    def cache_needs(self):
+        """Per run-order entry: its cache need, and the entry whose cache it reads (or None)."""
+        needs = [block_class(self.spec.layers[e.layer].block).cache_need(self.spec.layers[e.layer]) for e in self.run_order]
+        return needs, [e.cache_of for e in self.run_order]
+
+    def weight_bytes_read_per_step(self) -> int:
+        """Bytes of weights one step reads when it uses every matrix once (the token table is read by row)."""
+        seen, total = set(), 0
+        for block, entry in ((self.layers[e.layer], e) for e in self.run_order):
+            for part in (block.mixer, block.feed_forward, block.mixer_norm, block.feed_forward_norm):
+                for t in vars(part).values():
+                    if isinstance(t, torch.Tensor) and t.dtype in (torch.bfloat16, torch.float32):
+                        total += t.numel() * t.element_size()
+        total += self.lm_head.numel() * self.lm_head.element_size() + self.final_norm.weight.numel() * self.final_norm.weight.element_size()
+        return total
+
+    # ------------------------------------------------------------------------------- the pass
+    def forward(self, ctx: StepContext, cache, logit_rows: Optional[torch.Tensor], n_logit_rows: int):
+        """Runs the step's rows through every layer of the run order; returns float32 logits
+        [n_logit_rows, vocab] of the rows listed in `logit_rows`, or None if there are none."""
+        x = torch.empty((ctx.n_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device)
+        ops.embed(self.embedding, ctx.tokens, x)
+        for i, entry in enumerate(self.run_order):
+            self.layers[entry.layer].forward(x, ctx, cache.layer_cache(i))
+        if n_logit_rows == 0:
+            return None
+        picked = torch.empty((n_logit_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device)
+        ops.gather_rows(x, logit_rows, picked)
+        normed = self.final_norm(picked, self.head_in_dtype)
+        logits = torch.empty((n_logit_rows, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        linear(normed, self.lm_head, logits)
+        return logits
+
+
+def load_model(folder, dtype="bfloat16", device="cuda:0") -> DecoderModel:
+    """The model a folder (config.json, model.safetensors) describes; the class of its
+    configuration is chosen by config.json."""
+    dtype = compute_dtype(dtype)
+    config = read_config(folder)
+    spec = config.model_spec()
+    tensors = load_tensors(folder, model_tensor_needs(spec), dtype, device, spec.ignorable_tensors)
+    model = DecoderModel(spec, tensors, dtype, device)
+    model.config = config
+    return model
+
+
+def random_model(config, seed: int, dtype="bfloat16", device="cuda:0", std: float = 0.02) -> DecoderModel:
+    """A model of `config` with seeded random weights, without a folder in between."""
+    dtype = compute_dtype(dtype)
+    spec = config.model_spec()
+    host = random_tensors(model_tensor_needs(spec), seed, dtype, std)
+    tensors = {k: v.to(device) for k, v in host.items()}
+    model = DecoderModel(spec, tensors, dtype, device)
+    model.config = config
+    return model

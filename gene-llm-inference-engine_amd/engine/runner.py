@@ -1,0 +1,140 @@
+"""The step function: one batch of (request, its next tokens) through the model, from the cache.
+
+A step holds, for each of its requests, the request's next tokens: a portion of a prompt, cut
+anywhere, or a single decoded token.  All rows run as one batch; positions are never passed in,
+a step always appends to what the cache holds of the request.  Logits come back only for the
+rows asked for.  Everything is checked before anything changes, and a step that cannot get its
+pages raises `OutOfPages` and leaves every request as it was (the reference's `forward_rows`
+keeps the same promises, src/model/model.h:63-76, src/model/transformer.cpp:483-518).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager
+from ..parts import LayerCache, StepContext
+from .model import DecoderModel
+
+
+class StepError(ValueError):
+    """The batch is not valid; nothing was changed."""
+
+
+@dataclass
+class StepEntry:
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=tuple)      # places among `tokens` whose logits are asked for
+
+
+class _CacheView:
+    def __init__(self, manager: CacheManager, needs, reads_from):
+        self._layer = []
+        for i, (need, src) in enumerate(zip(needs, reads_from)):
+            from ..cache import PagedKvNeed, StateNeed
+            if isinstance(need, PagedKvNeed):
+                kv, table, _ = manager.kv(i)
+                self._layer.append(LayerCache(kv=kv, table=table, writes=src is None))
+            elif isinstance(need, StateNeed):
+                self._layer.append(LayerCache(state=manager.state(i)))
+            else:
+                self._layer.append(LayerCache())
+
+    def layer_cache(self, entry: int) -> LayerCache:
+        return self._layer[entry]
+
+
+class Runner:
+    """Model + cache + the step function.
+
+    page_size    positions per page
+    max_tokens   positions the page pool holds (per layer group)
+    max_requests live requests (request slots)
+    max_rows     most rows one step may hold
+    max_positions longest request; defaults to the model's limit
+    """
+
+    def __init__(self, model: DecoderModel, *, page_size: int = 16, max_tokens: int = 4096, max_requests: int = 8,
+                 max_rows: int = 4096, max_positions: Optional[int] = None):
+        self.model = model
+        self.page_size = int(page_size)
+        self.max_rows = int(max_rows)
+        self.max_positions = int(max_positions or model.spec.max_positions)
+        needs, reads_from = model.cache_needs()
+        n_pages = max(1, -(-int(max_tokens) // self.page_size))
+        self.cache = CacheManager(needs, reads_from, page_size=self.page_size, n_pages=n_pages, max_requests=max_requests,
+                                  max_positions=self.max_positions, dtype=model.dtype, device=model.device)
+        self._view = _CacheView(self.cache, needs, reads_from)
+        self.steps_run = 0
+
+    # -------------------------------------------------------------------------------- requests
+    def open(self, request: Hashable) -> None:
+        self.cache.open(request)
+
+    def close(self, request: Hashable) -> None:
+        self.cache.close(request)
+
+    def is_open(self, request: Hashable) -> bool:
+        return self.cache.is_open(request)
+
+    def length(self, request: Hashable) -> int:
+        return self.cache.length(request)
+
+    # ------------------------------------------------------------------------------------ step
+    def _validate(self, entries: Sequence[StepEntry]):
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        seen, n_rows, vocab = set(), 0, self.model.spec.vocab_size
+        for e in entries:
+            if e.request in seen:
+                raise StepError(f"request {e.request!r} appears twice in one step")
+            seen.add(e.request)
+            if not self.cache.is_open(e.request):
+                raise StepError(f"request {e.request!r} is not open")
+            if len(e.tokens) == 0:
+                raise StepError(f"request {e.request!r} brings no tokens")
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    raise StepError(f"token {t} of request {e.request!r} is outside the vocabulary [0, {vocab})")
+            for w in e.want:
+                if not 0 <= int(w) < len(e.tokens):
+                    raise StepError(f"request {e.request!r} wants logits at place {w} of {len(e.tokens)} tokens")
+            if self.cache.length(e.request) + len(e.tokens) > self.max_positions:
+                raise StepError(f"request {e.request!r} would pass the position limit {self.max_positions}")
+            n_rows += len(e.tokens)
+        if n_rows > self.max_rows:
+            raise StepError(f"the step holds {n_rows} rows, more than max_rows = {self.max_rows}")
+        return n_rows
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Runs the batch; returns float32 logits [wanted, vocab] on the device in the order of the
+        entries and of each entry's `want`, or None if nothing was wanted."""
+        n_rows = self._validate(entries)
+        self.cache.reserve([(e.request, len(e.tokens)) for e in entries])       # OutOfPages: nothing changed
+        self.cache.sync()
+
+        dev = self.model.device
+        meta = np.empty((3, n_rows), dtype=np.int32)                            # tokens, positions, slots
+        seg_slot, seg_start, seg_len, seg_pos0, logit_rows = [], [], [], [], []
+        row = 0
+        for e in entries:
+            n, slot, pos0 = len(e.tokens), self.cache.slot(e.request), self.cache.length(e.request)
+            meta[0, row:row + n] = np.asarray(e.tokens, dtype=np.int32)
+            meta[1, row:row + n] = np.arange(pos0, pos0 + n, dtype=np.int32)
+            meta[2, row:row + n] = slot
+            seg_slot.append(slot); seg_start.append(row); seg_len.append(n); seg_pos0.append(pos0)
+            logit_rows += [row + int(w) for w in e.want]
+            row += n
+        meta_dev = torch.from_numpy(meta).to(dev)
+        rows_dev = torch.tensor(logit_rows, dtype=torch.int32).to(dev) if logit_rows else None
+        ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
+                          row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0)
+        logits = self.model.forward(ctx, self._view, rows_dev, len(logit_rows))
+        for e in entries:
+            self.cache.advance(e.request, len(e.tokens))
+        self.steps_run += 1
+        return logits

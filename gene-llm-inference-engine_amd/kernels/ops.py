@@ -1,0 +1,248 @@
+"""Python faces of the HIP kernels: each checks its operands on the host (device, dtype, shape,
+contiguity) and launches on torch's current stream.  Tensors are torch tensors used as plain
+device memory; no torch arithmetic happens here.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_long, c_void_p
+
+import torch
+
+from . import library
+
+F32, BF16 = 0, 1
+_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_SIGNATURES = {
+    "gi_embed": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "gi_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_long, c_long, c_void_p],
+    "gi_rope_cos_sin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "gi_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                      c_int, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "gi_silu_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "gi_gather_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "gi_gemm_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
+    "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
+                           c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "gi_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
+    "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
+}
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        l = library.load()
+        for name, sig in _SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.argtypes = sig
+            fn.restype = c_int
+        _lib = l
+    return _lib
+
+
+def _call(name, *args):
+    l = lib()
+    rc = getattr(l, name)(*args)
+    if rc != 0:
+        raise KernelError(l.gi_last_error().decode())
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    try:
+        return _CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"{what} has dtype {t.dtype}; float32 or bfloat16 is needed") from None
+
+
+def _need(cond, msg):
+    if not cond:
+        raise KernelError(msg)
+
+
+def _dev(*tensors):
+    for t in tensors:
+        if t is not None:
+            _need(t.is_cuda, "kernel operands must lie in device memory")
+
+
+def _i32(t, what, n=None):
+    _need(t.dtype == torch.int32 and t.is_contiguous(), f"{what} must be a contiguous int32 tensor")
+    if n is not None:
+        _need(t.numel() >= n, f"{what} holds {t.numel()} entries, {n} are needed")
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def device_arch() -> str:
+    buf = ctypes.create_string_buffer(64)
+    l = lib()
+    if l.gi_device_arch(buf, 64) != 0:
+        raise KernelError(l.gi_last_error().decode())
+    return buf.value.decode()
+
+
+# ------------------------------------------------------------------------------------------------
+def embed(table, tokens, out):
+    """out[t, :] = table[tokens[t], :] widened to float32."""
+    _dev(table, tokens, out)
+    n, dim = out.shape
+    _need(table.dim() == 2 and table.shape[1] == dim and table.is_contiguous(), "embed: table must be [vocab, dim], contiguous")
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "embed: out must be contiguous float32")
+    _i32(tokens, "embed: tokens", n)
+    _call("gi_embed", table.data_ptr(), _code(table, "embed: table"), tokens.data_ptr(), out.data_ptr(), n, dim, _stream())
+    return out
+
+
+def rmsnorm(x, weight, eps, out):
+    """out = weight * (x * rsqrt(mean(x^2) + eps)) per row; x float32 [n, dim]."""
+    _dev(x, weight, out)
+    n, dim = x.shape
+    _need(x.dtype == torch.float32 and x.stride(1) == 1, "rmsnorm: x must be float32 with unit inner stride")
+    _need(out.shape == x.shape and out.stride(1) == 1, "rmsnorm: out must have x's shape and unit inner stride")
+    _need(weight.shape == (dim,) and weight.is_contiguous(), "rmsnorm: weight must be [dim]")
+    _call("gi_rmsnorm", x.data_ptr(), weight.data_ptr(), _code(weight, "rmsnorm: weight"), out.data_ptr(), _code(out, "rmsnorm: out"),
+          n, dim, float(eps), x.stride(0), out.stride(0), _stream())
+    return out
+
+
+def rope_cos_sin(positions, inv_freq, cos_out, sin_out):
+    """cos/sin of positions[t] * inv_freq[k] with 64-bit angles; outputs float32 [n, half]."""
+    _dev(positions, inv_freq, cos_out, sin_out)
+    n, half = cos_out.shape
+    _i32(positions, "rope_cos_sin: positions", n)
+    _need(inv_freq.dtype == torch.float64 and inv_freq.shape == (half,) and inv_freq.is_contiguous(), "rope_cos_sin: inv_freq must be float64 [half]")
+    for t in (cos_out, sin_out):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.shape == (n, half), "rope_cos_sin: outputs must be float32 [n, half]")
+    _call("gi_rope_cos_sin", positions.data_ptr(), inv_freq.data_ptr(), cos_out.data_ptr(), sin_out.data_ptr(), n, half, _stream())
+
+
+def _check_cache(cache, table, page_size, n_kv, hd, what):
+    _need(cache.dim() == 5 and tuple(cache.shape[1:]) == (2, n_kv, page_size, hd) and cache.is_contiguous(),
+          f"{what}: the cache must be [pages, 2, {n_kv}, {page_size}, {hd}], contiguous; it is {tuple(cache.shape)}")
+    _need(table.dim() == 2 and table.dtype == torch.int32 and table.stride(1) == 1, f"{what}: the page table must be int32 [slots, pages]")
+
+
+def rope_store(q, k, v, cos, sin, positions, slots, table, q_out, cache, n_heads, n_kv, hd):
+    """Rotates q into q_out and, if k is given, rotates k and writes k and v into the cache pages.
+    q, k, v are float32 views [n, heads*hd] with unit inner stride (columns of one product are fine)."""
+    _dev(q, k, v, cos, sin, positions, slots, table, q_out, cache)
+    n = q.shape[0]
+    _need(q.dtype == torch.float32 and q.shape[1] == n_heads * hd and q.stride(1) == 1, "rope_store: q must be float32 [n, heads*hd]")
+    _need(q_out.shape == (n, n_heads * hd) and q_out.is_contiguous(), "rope_store: q_out must be [n, heads*hd], contiguous")
+    if cos is not None:
+        for t in (cos, sin):
+            _need(t.dtype == torch.float32 and t.shape == (n, hd // 2) and t.is_contiguous(), "rope_store: cos/sin must be float32 [n, hd/2]")
+    page_size = page_stride = 0
+    cache_code = _code(q_out, "rope_store: q_out")
+    if k is not None:
+        for t, name in ((k, "k"), (v, "v")):
+            _need(t.dtype == torch.float32 and t.shape == (n, n_kv * hd) and t.stride(1) == 1, f"rope_store: {name} must be float32 [n, kv_heads*hd]")
+        page_size = cache.shape[3]
+        _check_cache(cache, table, page_size, n_kv, hd, "rope_store")
+        page_stride = cache.stride(0)
+        cache_code = _code(cache, "rope_store: cache")
+        _i32(positions, "rope_store: positions", n)
+        _i32(slots, "rope_store: slots", n)
+    _call("gi_rope_store", q.data_ptr(), _ptr(k), _ptr(v), q.stride(0), k.stride(0) if k is not None else 0,
+          v.stride(0) if v is not None else 0, _ptr(cos), _ptr(sin), _ptr(positions), _ptr(slots),
+          _ptr(table) if k is not None else None, table.stride(0) if k is not None else 0, q_out.data_ptr(),
+          _code(q_out, "rope_store: q_out"), _ptr(cache) if k is not None else None, cache_code, page_stride, page_size,
+          n, n_heads, n_kv, hd, _stream())
+
+
+def silu_mul(gate_up, out):
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, inter + i]."""
+    _dev(gate_up, out)
+    n, inter = out.shape
+    _need(gate_up.dtype == torch.float32 and gate_up.shape == (n, 2 * inter) and gate_up.is_contiguous(), "silu_mul: gate_up must be float32 [n, 2*inter]")
+    _need(out.is_contiguous(), "silu_mul: out must be contiguous")
+    _call("gi_silu_mul", gate_up.data_ptr(), out.data_ptr(), _code(out, "silu_mul: out"), n, inter, _stream())
+    return out
+
+
+def gather_rows(x, rows, out):
+    _dev(x, rows, out)
+    k, dim = out.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.shape[1] == dim, "gather_rows: x must be contiguous float32 [n, dim]")
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "gather_rows: out must be contiguous float32")
+    _i32(rows, "gather_rows: rows", k)
+    _call("gi_gather_rows", x.data_ptr(), rows.data_ptr(), out.data_ptr(), k, dim, _stream())
+    return out
+
+
+def gemm_exact(a, w, out, accumulate=False):
+    """out (=|+=) a @ w.T in 32-bit arithmetic with one summation order for every batch size."""
+    _dev(a, w, out)
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape == (n, k), f"gemm: weight is {tuple(w.shape)}, activations are {tuple(a.shape)}")
+    _need(out.shape == (m, n), f"gemm: out is {tuple(out.shape)}, ({m}, {n}) is needed")
+    _need(a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, "gemm: operands need unit inner stride")
+    _call("gi_gemm_exact", a.data_ptr(), _code(a, "gemm: a"), w.data_ptr(), _code(w, "gemm: w"), out.data_ptr(), _code(out, "gemm: out"),
+          1 if accumulate else 0, m, n, k, a.stride(0), w.stride(0), out.stride(0), _stream())
+    return out
+
+
+def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None):
+    """Each row attends over its request's cached keys up to its own position."""
+    _dev(q, cache, out, positions, slots, table)
+    n = q.shape[0]
+    _need(q.shape == (n, n_heads * hd) and q.is_contiguous() and out.shape == q.shape and out.is_contiguous(),
+          "attention: q and out must be [n, heads*hd], contiguous")
+    page_size = cache.shape[3]
+    _check_cache(cache, table, page_size, n_kv, hd, "attention")
+    _i32(positions, "attention: positions", n)
+    _i32(slots, "attention: slots", n)
+    _call("gi_attention_exact", q.data_ptr(), _code(q, "attention: q"), cache.data_ptr(), _code(cache, "attention: cache"), out.data_ptr(),
+          _code(out, "attention: out"), positions.data_ptr(), slots.data_ptr(), table.data_ptr(), table.stride(0), cache.stride(0),
+          page_size, n, n_heads, n_kv, hd, int(window or 0), float(scale if scale is not None else hd ** -0.5), _stream())
+    return out
+
+
+def attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window=None):
+    """Attention of a step's rows; the kernel is chosen by the storage dtype and the batch's shape."""
+    return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window)
+
+
+def gemm_bf16_supports(a, w, out) -> bool:
+    return False
+
+
+def gemm_bf16(a, w, out, accumulate=False):
+    raise KernelError("no bfloat16 matrix-core kernel is built")
+
+
+def argmax(logits, out):
+    _dev(logits, out)
+    n, vocab = logits.shape
+    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "argmax: logits must be float32 with unit inner stride")
+    _i32(out, "argmax: out", n)
+    _call("gi_argmax", logits.data_ptr(), out.data_ptr(), n, vocab, logits.stride(0), _stream())
+    return out
+
+
+def sample_temperature(logits, temperature, uniform, out):
+    _dev(logits, temperature, uniform, out)
+    n, vocab = logits.shape
+    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "sample: logits must be float32 with unit inner stride")
+    for t, name in ((temperature, "temperature"), (uniform, "uniform")):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= n, f"sample: {name} must be float32 [n]")
+    _i32(out, "sample: out", n)
+    _call("gi_sample_temperature", logits.data_ptr(), temperature.data_ptr(), uniform.data_ptr(), out.data_ptr(), n, vocab,
+          logits.stride(0), _stream())
+    return out

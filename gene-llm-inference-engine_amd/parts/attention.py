@@ -1,0 +1,61 @@
+"""Causal attention with grouped key/value heads over the paged cache (optionally windowed).
+
+Order of operations as the reference's pass (src/gpu/gpu_transformer.cpp:390-409): q, k, v
+products; rotation of q and k; all new keys and values are written to their pages; then every
+row attends over its request's pages up to its own position; output product added onto the
+residual.  The three input products run as one with the stacked matrix [q; k; v]."""
+from __future__ import annotations
+
+import torch
+
+from ..cache.needs import PagedKvNeed
+from ..kernels import ops
+from ..weights.loader import TensorNeed
+from .base import Mixer, position_class, register_mixer
+from .linear import activation_dtype_for, linear
+
+
+class Attention(Mixer):
+    def __init__(self, spec, tensors, dtype, device):
+        super().__init__(spec, tensors, dtype, device)
+        s = spec
+        if s.n_heads % s.n_kv_heads:
+            raise ValueError("the number of heads must be a multiple of the number of key/value heads")
+        self.a_dim, self.kv_dim = s.n_heads * s.head_dim, s.n_kv_heads * s.head_dim
+        self.w_qkv = torch.cat([tensors[s.q_proj], tensors[s.k_proj], tensors[s.v_proj]], dim=0).contiguous()
+        self.w_o = tensors[s.o_proj]
+        self.position = None if s.position is None else position_class(s.position)(s.position, tensors, dtype, device)
+        self.in_dtype = activation_dtype_for(self.w_qkv, dtype)
+        self.att_dtype = activation_dtype_for(self.w_o, dtype)
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        a, kv, d = spec.n_heads * spec.head_dim, spec.n_kv_heads * spec.head_dim, spec.hidden_size
+        return [TensorNeed(spec.q_proj, (a, d)), TensorNeed(spec.k_proj, (kv, d)), TensorNeed(spec.v_proj, (kv, d)),
+                TensorNeed(spec.o_proj, (d, a))]
+
+    @classmethod
+    def cache_need(cls, spec):
+        return PagedKvNeed(spec.n_kv_heads, spec.head_dim, spec.window)
+
+    def forward(self, h, residual, ctx, cache):
+        s, T = self.spec, ctx.n_rows
+        cos, sin = self.position.prepare(ctx) if self.position is not None else (None, None)
+        q_rot = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
+        if cache.writes:
+            qkv = torch.empty((T, self.a_dim + 2 * self.kv_dim), dtype=torch.float32, device=ctx.device)
+            linear(h, self.w_qkv, qkv)
+            q, k, v = qkv[:, :self.a_dim], qkv[:, self.a_dim:self.a_dim + self.kv_dim], qkv[:, self.a_dim + self.kv_dim:]
+            ops.rope_store(q, k, v, cos, sin, ctx.row_pos, ctx.row_slot, cache.table, q_rot, cache.kv, s.n_heads, s.n_kv_heads, s.head_dim)
+        else:                       # the pages are another layer's: only the queries are made
+            q = torch.empty((T, self.a_dim), dtype=torch.float32, device=ctx.device)
+            linear(h, self.w_qkv[:self.a_dim], q)
+            ops.rope_store(q, None, None, cos, sin, ctx.row_pos, ctx.row_slot, cache.table, q_rot, cache.kv, s.n_heads, s.n_kv_heads, s.head_dim)
+        att = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
+        ops.attention(q_rot, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, s.window)
+        if att.dtype != self.att_dtype:
+            att = att.to(self.att_dtype)
+        linear(att, self.w_o, residual, accumulate=True)
+
+
+register_mixer("attention", Attention)

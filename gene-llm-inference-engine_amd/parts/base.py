@@ -1,0 +1,128 @@
+"""Interfaces of the parts a layer is put together from, and the registries that map a spec's
+`kind` to the class that implements it.
+
+A part is built from its spec (all sizes and constants), the weight tensors it named, the compute
+dtype and the device.  It never sees the model it is in.  During a step it gets a `StepContext`
+(what the batch looks like) and, if it keeps a cache, a `LayerCache` (its own view of the cache
+manager).
+
+Kinds of parts and what each must provide:
+
+* norm:              `tensor_needs(spec)`, `__call__(x_f32[T, size], out_dtype) -> [T, size]`
+* position encoding: `prepare(ctx) -> tables` (made once per step and kept in ctx.memo)
+* mixer:             `tensor_needs(spec)`, `cache_need(spec)`, `forward(h, residual, ctx, cache)`
+* feed-forward:      `tensor_needs(spec)`, `forward(h, residual, ctx)`
+* block:             `forward(x, ctx, cache)` wiring norms, mixer and feed-forward around the
+                     32-bit residual stream `x`
+
+Mixers and feed-forwards add their result onto `residual` (float32 [T, hidden]) in place.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional
+
+import torch
+
+from ..weights.loader import TensorNeed
+
+
+@dataclass
+class StepContext:
+    """One step's batch as the parts see it.  Rows are the tokens of the step in the order given;
+    the rows of one request are consecutive and in position order."""
+    n_rows: int
+    dtype: torch.dtype                       # compute dtype: what activations between parts are stored as
+    device: torch.device
+    tokens: torch.Tensor                     # int32 [T]
+    row_pos: torch.Tensor                    # int32 [T]  position of each row in its request
+    row_slot: torch.Tensor                   # int32 [T]  the request's slot (row of page tables and state tensors)
+    seg_slot: List[int]                      # per request of the step, on the host: slot,
+    seg_start: List[int]                     # first row,
+    seg_len: List[int]                       # number of rows,
+    seg_pos0: List[int]                      # position of the first row
+    memo: Dict[Any, Any] = field(default_factory=dict)     # per-step tables shared by layers (rotary cos/sin)
+
+    @property
+    def max_seg_len(self) -> int:
+        return max(self.seg_len)
+
+    @property
+    def max_context(self) -> int:
+        return max(p + n for p, n in zip(self.seg_pos0, self.seg_len))
+
+
+@dataclass
+class LayerCache:
+    """A run-order entry's view of the cache manager."""
+    kv: Optional[torch.Tensor] = None        # [page, 2, kv_head, place, head_dim] of this layer
+    table: Optional[torch.Tensor] = None     # int32 [slot, pages]
+    state: Optional[torch.Tensor] = None     # [slot, ...] fixed-size state
+    writes: bool = True                      # False: the pages belong to another entry, read only
+
+
+class Part:
+    """Common construction: `spec`, `tensors` (by name, on the device), compute dtype, device."""
+
+    def __init__(self, spec, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device):
+        self.spec, self.dtype, self.device = spec, dtype, device
+
+    @classmethod
+    def tensor_needs(cls, spec) -> List[TensorNeed]:
+        return []
+
+
+class Mixer(Part):
+    @classmethod
+    def cache_need(cls, spec):
+        """A `PagedKvNeed`, a `StateNeed` or None."""
+        return None
+
+    def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx: StepContext) -> None:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def prepare(self, ctx: StepContext):
+        raise NotImplementedError
+
+
+_REGISTRIES: Dict[str, Dict[str, type]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}}
+
+
+def _register(family: str, kind: str, cls: type) -> None:
+    table = _REGISTRIES[family]
+    if kind in table and table[kind] is not cls:
+        raise ValueError(f"{family} kind '{kind}' is already registered")
+    table[kind] = cls
+
+
+def _lookup(family: str, kind: str) -> type:
+    try:
+        return _REGISTRIES[family][kind]
+    except KeyError:
+        raise KeyError(f"no {family} of kind '{kind}' is registered; known: {', '.join(sorted(_REGISTRIES[family]))}") from None
+
+
+def register_mixer(kind, cls): _register("mixer", kind, cls)
+def register_feed_forward(kind, cls): _register("feed_forward", kind, cls)
+def register_norm(kind, cls): _register("norm", kind, cls)
+def register_position_encoding(kind, cls): _register("position", kind, cls)
+def register_block(kind, cls): _register("block", kind, cls)
+
+
+def mixer_class(spec): return _lookup("mixer", spec.kind)
+def feed_forward_class(spec): return _lookup("feed_forward", spec.kind)
+def norm_class(spec): return _lookup("norm", spec.kind)
+def position_class(spec): return _lookup("position", spec.kind)
+def block_class(kind: str): return _lookup("block", kind)

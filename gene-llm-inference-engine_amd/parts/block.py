@@ -1,0 +1,36 @@
+"""Arrangements of a layer's parts around the residual stream.
+
+"prenorm" (reference: src/model/transformer.cpp:385-450):
+    x += mixer(norm_1(x));  x += feed_forward(norm_2(x))
+The residual stream x is float32 [T, hidden] and is changed in place."""
+from __future__ import annotations
+
+from .base import feed_forward_class, mixer_class, norm_class, register_block
+
+
+class PreNormBlock:
+    def __init__(self, spec, tensors, dtype, device):
+        self.spec = spec
+        self.mixer_norm = norm_class(spec.mixer_norm)(spec.mixer_norm, tensors, dtype, device)
+        self.mixer = mixer_class(spec.mixer)(spec.mixer, tensors, dtype, device)
+        self.feed_forward_norm = norm_class(spec.feed_forward_norm)(spec.feed_forward_norm, tensors, dtype, device)
+        self.feed_forward = feed_forward_class(spec.feed_forward)(spec.feed_forward, tensors, dtype, device)
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        return (norm_class(spec.mixer_norm).tensor_needs(spec.mixer_norm) + mixer_class(spec.mixer).tensor_needs(spec.mixer) +
+                norm_class(spec.feed_forward_norm).tensor_needs(spec.feed_forward_norm) +
+                feed_forward_class(spec.feed_forward).tensor_needs(spec.feed_forward))
+
+    @classmethod
+    def cache_need(cls, spec):
+        return mixer_class(spec.mixer).cache_need(spec.mixer)
+
+    def forward(self, x, ctx, cache):
+        h = self.mixer_norm(x, getattr(self.mixer, "in_dtype", ctx.dtype))
+        self.mixer.forward(h, x, ctx, cache)
+        h = self.feed_forward_norm(x, getattr(self.feed_forward, "in_dtype", ctx.dtype))
+        self.feed_forward.forward(h, x, ctx)
+
+
+register_block("prenorm", PreNormBlock)

@@ -1,0 +1,36 @@
+"""SwiGLU feed-forward: residual += down( silu(gate(h)) * up(h) ), silu(g) = g / (1 + exp(-g))
+(reference: src/model/transformer.cpp:437-450).  gate and up run as one product with the stacked
+matrix [gate; up]."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.loader import TensorNeed
+from .base import FeedForward, register_feed_forward
+from .linear import activation_dtype_for, linear
+
+
+class SwiGlu(FeedForward):
+    def __init__(self, spec, tensors, dtype, device):
+        super().__init__(spec, tensors, dtype, device)
+        self.w_gate_up = torch.cat([tensors[spec.gate_proj], tensors[spec.up_proj]], dim=0).contiguous()
+        self.w_down = tensors[spec.down_proj]
+        self.in_dtype = activation_dtype_for(self.w_gate_up, dtype)
+        self.mid_dtype = activation_dtype_for(self.w_down, dtype)
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        i, d = spec.intermediate_size, spec.hidden_size
+        return [TensorNeed(spec.gate_proj, (i, d)), TensorNeed(spec.up_proj, (i, d)), TensorNeed(spec.down_proj, (d, i))]
+
+    def forward(self, h, residual, ctx):
+        T, inter = ctx.n_rows, self.spec.intermediate_size
+        gate_up = torch.empty((T, 2 * inter), dtype=torch.float32, device=ctx.device)
+        linear(h, self.w_gate_up, gate_up)
+        mid = torch.empty((T, inter), dtype=self.mid_dtype, device=ctx.device)
+        ops.silu_mul(gate_up, mid)
+        linear(mid, self.w_down, residual, accumulate=True)
+
+
+register_feed_forward("swiglu", SwiGlu)

@@ -1,0 +1,103 @@
+"""Tiny model folders for the tests, written without any of the engine's code: config.json and a
+safetensors file made by hand here, so that the engine's loader reads a file it did not write.
+
+Weights are drawn as the reference's test generator draws them (tools/make_dummy_hf.py:99-106):
+matrices 0.2 * N(0, 1) (large enough that logits are of order one and relative errors mean
+something), norm weights 1 + 0.1 * N(0, 1), stored in a shuffled order."""
+from __future__ import annotations
+
+import json
+import struct
+from pathlib import Path
+
+import numpy as np
+import torch
+
+# Two configurations that differ in every size and option, and a third with odd sizes.
+TINY_A = dict(hidden_size=64, intermediate_size=192, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+              vocab_size=256, rope_theta=10000.0, rope_scaling=None, rms_norm_eps=1e-5, tie_word_embeddings=True,
+              max_position_embeddings=512)
+TINY_B = dict(hidden_size=96, intermediate_size=160, num_hidden_layers=3, num_attention_heads=3, num_key_value_heads=1,
+              head_dim=32, vocab_size=384, rope_theta=500000.0,
+              rope_scaling=dict(rope_type="llama3", factor=4.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                original_max_position_embeddings=32),
+              rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=1024)
+TINY_C = dict(hidden_size=80, intermediate_size=112, num_hidden_layers=1, num_attention_heads=6, num_key_value_heads=3,
+              head_dim=48, vocab_size=301, rope_theta=25000.0, rope_scaling=None, rms_norm_eps=3e-5,
+              tie_word_embeddings=False, max_position_embeddings=256)
+PAGE_SIZE = {"A": 4, "B": 8, "C": 16}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+
+
+def full_config(sizes: dict) -> dict:
+    return {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_act": "silu", "attention_bias": False,
+            "mlp_bias": False, **sizes}
+
+
+def tensor_layout(cfg: dict):
+    """Names and shapes of a Llama folder (src/loader/hf_checkpoint.cpp:214-235)."""
+    d, i, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    heads = cfg["num_attention_heads"]
+    kvh = cfg.get("num_key_value_heads") or heads
+    hd = cfg.get("head_dim") or d // heads
+    out = [("model.embed_tokens.weight", (v, d))]
+    for l in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{l}."
+        out += [(p + "input_layernorm.weight", (d,)), (p + "self_attn.q_proj.weight", (heads * hd, d)),
+                (p + "self_attn.k_proj.weight", (kvh * hd, d)), (p + "self_attn.v_proj.weight", (kvh * hd, d)),
+                (p + "self_attn.o_proj.weight", (d, heads * hd)), (p + "post_attention_layernorm.weight", (d,)),
+                (p + "mlp.gate_proj.weight", (i, d)), (p + "mlp.up_proj.weight", (i, d)), (p + "mlp.down_proj.weight", (d, i))]
+    out.append(("model.norm.weight", (d,)))
+    if not cfg.get("tie_word_embeddings", False):
+        out.append(("lm_head.weight", (v, d)))
+    return out
+
+
+def random_weights(cfg: dict, seed: int, std: float = 0.2):
+    rng = np.random.default_rng(seed)
+    w = {}
+    for name, shape in tensor_layout(cfg):
+        if name.endswith("norm.weight"):
+            w[name] = torch.from_numpy((1.0 + 0.1 * rng.standard_normal(shape)).astype(np.float32))
+        else:
+            w[name] = torch.from_numpy((std * rng.standard_normal(shape)).astype(np.float32))
+    return w
+
+
+_NAMES = {torch.float32: "F32", torch.bfloat16: "BF16", torch.float16: "F16", torch.int32: "I32", torch.float64: "F64"}
+
+
+def write_safetensors_by_hand(path, tensors: dict, shuffle_seed=None, header_pad=0):
+    names = list(tensors)
+    if shuffle_seed is not None:
+        np.random.default_rng(shuffle_seed).shuffle(names)
+    header, blobs, off = {"__metadata__": {"format": "pt"}}, [], 0
+    for n in names:
+        t = tensors[n].contiguous()
+        raw = t.reshape(-1).view(torch.uint8).numpy().tobytes()
+        header[n] = {"dtype": _NAMES[t.dtype], "shape": list(t.shape), "data_offsets": [off, off + len(raw)]}
+        off += len(raw)
+        blobs.append(raw)
+    text = json.dumps(header).encode() + b" " * header_pad
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(text)) + text + b"".join(blobs))
+
+
+def write_model(folder, sizes: dict, seed: int = 0, dtype=torch.bfloat16, norm_dtype=None, std: float = 0.2, weights=None):
+    """Writes the folder; returns the float32 weights before rounding to the storage dtype."""
+    folder = Path(folder)
+    folder.mkdir(parents=True, exist_ok=True)
+    cfg = full_config(sizes)
+    (folder / "config.json").write_text(json.dumps(cfg, indent=2))
+    w = weights if weights is not None else random_weights(cfg, seed, std)
+    stored = {n: t.to(norm_dtype or dtype) if n.endswith("norm.weight") else t.to(dtype) for n, t in w.items()}
+    write_safetensors_by_hand(folder / "model.safetensors", stored, shuffle_seed=seed + 17)
+    return w
+
+
+def relative_error(got, want) -> float:
+    """max|got - want| / max|want|: stricter than the reference's measure, which floors the
+    denominator at 1 (tests/verify_forward.py:72-77)."""
+    got = torch.as_tensor(got).double().cpu()
+    want = torch.as_tensor(want).double().cpu()
+    return float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))

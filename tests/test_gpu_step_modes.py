@@ -1,0 +1,112 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16, under every way of
+cutting the work into steps.  In 32-bit the ways of cutting must also agree with each other bit
+for bit: the 32-bit kernels sum in an order that does not depend on the batch."""
+import random
+
+import pytest
+import torch
+
+import traces
+from model_folders import CONFIGS, PAGE_SIZE, relative_error, write_model
+from plain_llama import PlainLlama
+
+pytestmark = pytest.mark.gpu
+
+# float32 is compared with the plain model in 64-bit.  bfloat16 is compared with the plain model
+# rounding to bfloat16 at the same places as the engine (a tight bound: what is left is the order
+# of 32-bit sums and values that fall on the other side of a rounding edge), and with the exact
+# 64-bit model under a loose bound that only says the logits are the same function.
+TOLERANCE = {"float32": 2e-5, "bfloat16": 1.5e-2}
+LOOSE_BF16 = 0.12
+LENGTHS = {"A": [5, 11, 17, 70, 45], "B": [1, 9, 33, 40, 75, 51], "C": [3, 66, 37, 50]}
+
+
+def make_requests(name, seed=5):
+    rng = random.Random(seed)
+    vocab = CONFIGS[name]["vocab_size"]
+    return {f"r{i}": [rng.randrange(vocab) for _ in range(n)] for i, n in enumerate(LENGTHS[name])}
+
+
+@pytest.fixture(scope="module", params=["A", "B", "C"])
+def case(request, tmp_path_factory):
+    name = request.param
+    folder = tmp_path_factory.mktemp(f"tiny{name}")
+    write_model(folder, CONFIGS[name], seed=11 + ord(name))
+    requests = make_requests(name)
+    plain, rounded = PlainLlama(folder), PlainLlama(folder, storage=torch.bfloat16)
+    want = {"float32": {rid: plain.logits(toks) for rid, toks in requests.items()},
+            "bfloat16": {rid: rounded.logits(toks) for rid, toks in requests.items()}}
+    return name, folder, requests, want
+
+
+def replay(folder, dtype, steps, page_size, max_tokens):
+    from geneinfer_amd.engine import Runner, StepEntry, load_model
+    model = load_model(folder, dtype, "cuda:0")
+    runner = Runner(model, page_size=page_size, max_tokens=max_tokens, max_requests=4, max_rows=4096)
+    got = {}
+    where = traces.wanted_positions(steps)
+    for s in steps:
+        for e in s["entries"]:
+            if not runner.is_open(e["id"]):
+                runner.open(e["id"])
+        logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        if logits is not None:
+            assert logits.shape[0] == len(where[s["step"]])
+            for row, key in zip(logits.cpu(), where[s["step"]]):
+                got[key] = row
+        for rid in s["end"]:
+            runner.close(rid)
+    runner.cache.check_consistency()
+    assert all(f == g.pool.n_pages for f, g in zip(runner.cache.free_pages(), runner.cache.groups)), "pages were not all given back"
+    return got
+
+
+def check(got, want, dtype):
+    assert got, "the trace wanted no logits"
+    worst = 0.0
+    for (rid, pos), row in got.items():
+        worst = max(worst, relative_error(row, want[rid][pos]))
+    assert worst < TOLERANCE[dtype], f"worst relative error {worst:.3e}"
+    return worst
+
+
+_WHOLE = {}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", ["whole", "tail_singly", "portions", "mixed"])
+def test_step_modes(case, dtype, mode):
+    name, folder, requests, want = case
+    ps = PAGE_SIZE[name]
+    if mode == "whole":
+        steps = traces.whole(requests)
+    elif mode == "tail_singly":
+        steps = traces.tail_singly(requests, 32)
+    elif mode == "portions":
+        steps = traces.portions(requests)
+    else:
+        steps = traces.mixed(requests, seed=3)
+        assert max(len(s["entries"]) for s in steps) >= 3, "the mixed trace never held three requests in a step"
+    max_tokens = traces.peak_tokens(steps, round_to=ps)          # so few pages that they are used again
+    got = replay(folder, dtype, steps, ps, max_tokens)
+    assert len(got) == sum(len(t) for t in requests.values())
+    worst = check(got, want[dtype], dtype)
+    if dtype == "bfloat16":
+        loose = max(relative_error(row, want["float32"][rid][pos]) for (rid, pos), row in got.items())
+        assert loose < LOOSE_BF16, f"bfloat16 against the exact model: {loose:.3e}"
+        print(f"  against the exact model: {loose:.2e}")
+    print(f"{name} {dtype} {mode}: worst relative error {worst:.2e}, {len(steps)} steps, pool of {max_tokens} positions")
+    if dtype == "float32":
+        ref = _WHOLE.setdefault((name, "ref"), got if mode == "whole" else replay(folder, dtype, traces.whole(requests), ps, 4096))
+        for key, row in got.items():
+            assert torch.equal(row, ref[key]), f"{mode}: logits of {key} differ in bits from the whole-prompt run"
+
+
+def test_changing_first_token_changes_logits(case):
+    """The comparison is not vacuous: another first token gives other logits at the last position."""
+    name, folder, requests, want = case
+    rid = "r2"
+    toks = list(requests[rid])
+    toks[0] = (toks[0] + 1) % CONFIGS[name]["vocab_size"]
+    got = replay(folder, "float32", traces.whole({rid: toks}), PAGE_SIZE[name], 4096)
+    assert relative_error(got[(rid, len(toks) - 1)], want["float32"][rid][len(toks) - 1]) > 1e-3
