@@ -1,0 +1,144 @@
+"""Decode and prefill throughput of the engine at the Llama-3.2-1B shape, random weights, one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the whole batch (default batch 8, each request on a 2,048-token
+prompt in a 4,096-token context).  Prints ONE JSON line: decoded tokens a second as `value`, the
+2,048-token prefill, the decode step's HBM roofline fraction, and decode at batch 1 and 64.
+"""
+import argparse
+import json
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+# MI355X published peaks
+HBM_GBS = 8000.0
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+
+LLAMA_1B = dict(hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8,
+                head_dim=64, vocab_size=128256, max_position_embeddings=4096, rope_theta=500000.0, rms_norm_eps=1e-5,
+                tie_word_embeddings=True,
+                rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                  original_max_position_embeddings=8192))
+PROMPT, NEW_TOKENS, CONTEXT, PAGE = 2048, 256, 4096, 16
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0 = all); named in the record")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
+        return 2
+
+    import torch
+    from geneinfer_amd.config import LlamaConfig
+    from geneinfer_amd.engine import Runner, StepEntry, random_model
+    from geneinfer_amd.sampling import Sampler, SamplerConfig, sample_rows
+
+    sizes = dict(LLAMA_1B)
+    layers_full = sizes["num_hidden_layers"]
+    if args.layers:
+        sizes["num_hidden_layers"] = args.layers
+    config = LlamaConfig.from_dict(sizes)
+    dtype = "bfloat16" if args.dtype == "bf16" else "float32"
+    model = random_model(config, seed=0, dtype=dtype, device="cuda:0", draw_on_device=True)
+    vocab = config.vocab_size
+    gen = torch.Generator().manual_seed(1)
+
+    def make_runner(batch):
+        per_request = -(-(PROMPT + NEW_TOKENS + args.steps + args.warmup) // 64) * 64
+        return Runner(model, page_size=PAGE, max_tokens=batch * per_request, max_requests=batch, max_rows=max(PROMPT, batch),
+                      max_positions=CONTEXT)
+
+    def prefill(runner, rid):
+        toks = torch.randint(0, vocab, (PROMPT,), generator=gen).tolist()
+        runner.open(rid)
+        return runner.step([StepEntry(rid, toks, (PROMPT - 1,))])
+
+    def decode(batch, steps, warmup):
+        """Greedy decoding of `batch` requests after their prompts; returns (seconds for `steps` steps, context at the middle)."""
+        runner = make_runner(batch)
+        samplers = [Sampler(SamplerConfig(temperature=0.0), vocab) for _ in range(batch)]
+        tokens = [sample_rows(prefill(runner, r), [samplers[r]])[0] for r in range(batch)]
+
+        def one():
+            nonlocal tokens
+            logits = runner.step([StepEntry(r, [tokens[r]], (0,)) for r in range(batch)])
+            tokens = sample_rows(logits, samplers)
+
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        context = PROMPT + warmup + steps // 2
+        del runner
+        torch.cuda.empty_cache()
+        return dt, context
+
+    # ---- prefill of one 2,048-token prompt (median of 5 after one warm-up)
+    runner = make_runner(1)
+    times = []
+    for i in range(6):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = prefill(runner, i)
+        int(torch.argmax(logits[0]))           # the first token reaches the host
+        times.append(time.perf_counter() - t0)
+        runner.close(i)
+    prefill_s = sorted(times[1:])[len(times[1:]) // 2]
+    del runner
+    torch.cuda.empty_cache()
+    L, D, I, V = config.num_hidden_layers, config.hidden_size, config.intermediate_size, vocab
+    A, KV, hd, H = config.attn_dim, config.kv_dim, config.head_dim, config.num_attention_heads
+    layer_params = D * (A + 2 * KV) + A * D + 3 * I * D
+    prefill_flops = 2.0 * L * layer_params * PROMPT + L * 4.0 * H * hd * PROMPT * (PROMPT + 1) / 2 + 2.0 * V * D
+    prefill_rec = {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
+                   "frac": round(prefill_flops / prefill_s / (PEAK_TFLOPS[args.dtype] * 1e12), 4)}
+
+    # ---- decode
+    dt, context = decode(args.batch, args.steps, args.warmup)
+    elem = 2 if args.dtype == "bf16" else 4
+    weight_bytes = model.weight_bytes_read_per_step()
+    kv_bytes = args.batch * context * L * 2 * KV * elem
+    achieved = (weight_bytes + kv_bytes) / (dt / args.steps) / 1e9
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            s = max(8, args.steps // 4)
+            d, _ = decode(b, s, 4)
+            points[f"decode_b{b}"] = round(b * s / d, 1)
+
+    rec = {
+        "metric": "decode tok/s at batch 1/8/64 + prefill tok/s at 2,048 tokens, Llama-3.2-1B",
+        "value": round(args.batch * args.steps / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(dt / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "config": {"model": "Llama-3.2-1B shape", "layers": L, "layers_of_config": layers_full, "hidden": D, "heads": H,
+                   "kv_heads": config.num_key_value_heads, "head_dim": hd, "intermediate": I, "vocab": V, "global_batch": args.batch,
+                   "seq_len": CONTEXT, "prompt_len": PROMPT, "decode_context": context, "page_size": PAGE, "tied_embeddings": True,
+                   "rope": "llama3 theta 5e5 factor 32", "parallelism": "single_gpu"},
+        "prefill": prefill_rec,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s", "frac": round(achieved / HBM_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(rec))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

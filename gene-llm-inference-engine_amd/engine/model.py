@@ -81,12 +81,23 @@ def load_model(folder, dtype="bfloat16", device="cuda:0") -> DecoderModel:
     return model
 
 
-def random_model(config, seed: int, dtype="bfloat16", device="cuda:0", std: float = 0.02) -> DecoderModel:
-    """A model of `config` with seeded random weights, without a folder in between."""
+def random_model(config, seed: int, dtype="bfloat16", device="cuda:0", std: float = 0.02, draw_on_device: bool = False) -> DecoderModel:
+    """A model of `config` with seeded random weights, without a folder in between.  With
+    `draw_on_device` the numbers come from the device's generator (fast for large models; other
+    numbers than the host generator gives for the same seed)."""
     dtype = compute_dtype(dtype)
     spec = config.model_spec()
-    host = random_tensors(model_tensor_needs(spec), seed, dtype, std)
-    tensors = {k: v.to(device) for k, v in host.items()}
+    if draw_on_device:
+        from ..weights import merge_needs
+        gen = torch.Generator(device=device)
+        gen.manual_seed(int(seed))
+        tensors = {}
+        for name, need in merge_needs(model_tensor_needs(spec)).items():
+            t = torch.randn(need.shape, generator=gen, dtype=torch.float32, device=device)
+            tensors[name] = (1.0 + 0.1 * t if need.role == "norm" else std * t).to(dtype)
+    else:
+        host = random_tensors(model_tensor_needs(spec), seed, dtype, std)
+        tensors = {k: v.to(device) for k, v in host.items()}
     model = DecoderModel(spec, tensors, dtype, device)
     model.config = config
     return model

@@ -1,0 +1,221 @@
+"""The scheduler: continuous batching above the step function.
+
+Policy, as the reference's engine (src/runtime/engine.cpp:64-205):
+  * admission: first come first served while fewer than `max_running` requests run; admission
+    does not look at free memory.
+  * a step has a budget of `step_rows` rows.  First every request with exactly one pending token
+    (decoding, or at the last token of its prompt) gets one row, in admission order; then the
+    others get a portion of their prompt, oldest first, of at most `prefill_chunk` rows.  A
+    portion is shortened until its new pages fit in the free pages.
+  * when no row fits: a lone request is finished with the error "the KV pool is too small for
+    this request"; otherwise the youngest running request is preempted: its pages are freed,
+    it goes to the front of the waiting queue and is later fed again from its first token,
+    prompt and generated tokens alike, with its sampler's state kept, so that it continues as if
+    nothing had happened.
+  * only the row of a request's last known token returns logits; the request's own sampler draws
+    the next token from them.  A sampled end token finishes the request (it stays the last
+    generated token); so does reaching `max_positions` (prompt plus generated tokens).
+Each request gets the tokens it would get alone through `generate()` with the same seed.
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Callable, Deque, Iterable, List, Optional, Sequence
+
+from ..sampling import Sampler, SamplerConfig, sample_rows
+from .runner import Runner, StepEntry
+
+POOL_TOO_SMALL = "the KV pool is too small for this request"
+
+
+@dataclass
+class EngineConfig:
+    max_running: int = 8        # requests that hold cache memory and take part in steps at the same time
+    step_rows: int = 0          # rows per step; 0 = the runner's max_rows
+    prefill_chunk: int = 0      # most prompt tokens one request adds to a step; 0 = no limit besides step_rows
+
+
+@dataclass
+class EngineRequest:
+    prompt: Sequence[int]
+    max_positions: int = 0                                   # prompt + generated tokens at most; 0 or too large = the context length
+    sampler: SamplerConfig = field(default_factory=SamplerConfig)
+    on_token: Optional[Callable[[int], None]] = None         # every generated token that is not an end token
+
+
+@dataclass
+class EngineResult:
+    id: int = -1
+    prompt_tokens: List[int] = field(default_factory=list)
+    generated_tokens: List[int] = field(default_factory=list)
+    finished: bool = False
+    stopped_by_end_token: bool = False
+    error: str = ""
+    preemptions: int = 0
+    first_pass: int = -1
+    first_token_pass: int = -1
+    last_pass: int = -1
+
+
+@dataclass
+class EngineStats:
+    passes: int = 0
+    rows: int = 0
+    logits_rows: int = 0
+    preemptions: int = 0
+    max_rows_in_pass: int = 0
+    max_chunk: int = 0
+    max_running_seen: int = 0
+
+
+class _Job:
+    def __init__(self, jid: int, request: EngineRequest, sampler: Sampler, steps: int):
+        self.id, self.request, self.sampler, self.steps = jid, request, sampler, steps
+        self.tokens: List[int] = [int(t) for t in request.prompt]      # prompt followed by generated tokens
+        self.fed = 0                                                     # tokens[0:fed] are in the cache
+        self.result = EngineResult(id=jid, prompt_tokens=list(self.tokens))
+        self.key = ("job", jid)
+
+
+class Engine:
+    def __init__(self, runner: Runner, config: Optional[EngineConfig] = None, end_tokens: Iterable[int] = ()):
+        cfg = config or EngineConfig()
+        if cfg.max_running < 1:
+            raise ValueError("Engine: max_running must be >= 1")
+        if cfg.step_rows < 0 or cfg.prefill_chunk < 0:
+            raise ValueError("Engine: step_rows and prefill_chunk must be >= 0")
+        step_rows = cfg.step_rows if 0 < cfg.step_rows <= runner.max_rows else runner.max_rows
+        self.cfg = EngineConfig(min(cfg.max_running, runner.cache.max_requests), step_rows, cfg.prefill_chunk or step_rows)
+        self.runner = runner
+        self.end_tokens = set(int(t) for t in end_tokens)
+        self.jobs: List[_Job] = []
+        self.waiting: Deque[_Job] = deque()
+        self.running: List[_Job] = []                                    # in admission order
+        self.stats = EngineStats()
+
+    # ----------------------------------------------------------------------------- interface
+    def submit(self, request: EngineRequest) -> int:
+        context, vocab = self.runner.max_positions, self.runner.model.spec.vocab_size
+        if len(request.prompt) == 0:
+            raise ValueError("Engine.submit: prompt has no tokens")
+        if len(request.prompt) > context:
+            raise ValueError(f"Engine.submit: prompt of {len(request.prompt)} tokens does not fit in the context length {context}")
+        if any(not 0 <= int(t) < vocab for t in request.prompt):
+            raise ValueError("Engine.submit: token id out of range")
+        sampler = Sampler(request.sampler, vocab)                         # validates the configuration
+        steps = context if request.max_positions <= 0 else min(request.max_positions, context)
+        job = _Job(len(self.jobs), request, sampler, steps)
+        self.jobs.append(job)
+        self.waiting.append(job)
+        return job.id
+
+    def idle(self) -> bool:
+        return not self.waiting and not self.running
+
+    def result(self, jid: int) -> EngineResult:
+        if not 0 <= jid < len(self.jobs):
+            raise IndexError("Engine.result: unknown request id")
+        return self.jobs[jid].result
+
+    def run_until_idle(self) -> None:
+        while self.step():
+            pass
+
+    # ------------------------------------------------------------------------------ internals
+    def _admit(self) -> None:
+        while self.waiting and len(self.running) < self.cfg.max_running:
+            job = self.waiting.popleft()
+            self.runner.open(job.key)
+            job.fed = 0
+            self.running.append(job)
+        self.stats.max_running_seen = max(self.stats.max_running_seen, len(self.running))
+
+    def _finish(self, job: _Job, error: str = "") -> None:
+        job.result.finished, job.result.error, job.result.last_pass = True, error, self.stats.passes
+        self.runner.close(job.key)
+        self.running.remove(job)
+
+    def _preempt_youngest(self) -> None:
+        job = self.running.pop()
+        self.runner.close(job.key)
+        job.fed = 0
+        job.result.preemptions += 1
+        self.stats.preemptions += 1
+        self.waiting.appendleft(job)
+
+    def plan(self):
+        """The rows of the next step: [(job, n_rows)] in step order, decoding requests first.
+        Empty if not even one row fits in the free pages."""
+        cache = self.runner.cache
+        free = cache.free_pages()
+        budget = self.cfg.step_rows
+        taken = []
+        for phase in (0, 1):
+            for job in self.running:
+                pending = len(job.tokens) - job.fed
+                if (phase == 0) != (pending == 1):
+                    continue
+                take = min(pending, job.steps - job.fed, budget, 1 if phase == 0 else self.cfg.prefill_chunk)
+                while take > 0 and any(n > f for n, f in zip(cache.pages_needed(job.key, take), free)):
+                    take -= 1
+                if take <= 0:
+                    continue
+                free = [f - n for f, n in zip(free, cache.pages_needed(job.key, take))]
+                budget -= take
+                taken.append((job, take))
+        return taken
+
+    def step(self) -> bool:
+        """Runs one step.  False (and nothing done) if no request waits or runs."""
+        self._admit()
+        if not self.running:
+            return False
+        while True:
+            taken = self.plan()
+            if taken:
+                break
+            if len(self.running) == 1:
+                self._finish(self.running[0], POOL_TOO_SMALL)
+                return True
+            self._preempt_youngest()
+
+        entries, wanting = [], []
+        for job, n in taken:
+            last = job.fed + n == len(job.tokens)
+            entries.append(StepEntry(job.key, job.tokens[job.fed:job.fed + n], (n - 1,) if last else ()))
+            if last:
+                wanting.append(job)
+        logits = self.runner.step(entries)
+        st = self.stats
+        st.passes += 1
+        n_rows = sum(n for _, n in taken)
+        st.rows += n_rows
+        st.max_rows_in_pass = max(st.max_rows_in_pass, n_rows)
+        st.max_chunk = max(st.max_chunk, max(n for _, n in taken))
+
+        sampled = sample_rows(logits, [j.sampler for j in wanting]) if wanting else []
+        next_token = {j.id: t for j, t in zip(wanting, sampled)}
+        done = []
+        for job, n in taken:
+            if job.result.first_pass < 0:
+                job.result.first_pass = st.passes
+            job.fed += n
+            if job.id in next_token:
+                nxt = next_token[job.id]
+                st.logits_rows += 1
+                job.result.generated_tokens.append(nxt)
+                job.tokens.append(nxt)
+                if job.result.first_token_pass < 0:
+                    job.result.first_token_pass = st.passes
+                if nxt in self.end_tokens:
+                    job.result.stopped_by_end_token = True
+                    done.append(job)
+                    continue
+                if job.request.on_token is not None:
+                    job.request.on_token(nxt)
+            if job.fed >= job.steps:
+                done.append(job)
+        for job in done:
+            self._finish(job)
+        return True

@@ -1,0 +1,147 @@
+"""From logits to the next token: greedy, temperature, top-k, top-p, with the reference's random
+generator, so that a seed gives the same stream of uniform numbers as there.
+
+Rules (src/sampler/sampler.h:1-14, src/sampler/sampler.cpp:25-129):
+  1. temperature <= 0: the largest logit wins, the lowest index among equals; no randomness is used.
+  2. otherwise p = softmax(logits / temperature).
+  3. top-k keeps the k most likely tokens, top-p then the shortest prefix (by probability
+     descending, index ascending) whose mass reaches top_p times the kept mass.
+  4. a token is drawn by walking the kept tokens until the cumulative probability exceeds
+     u times the kept mass; without filtering the walk is in index order.
+Greedy and plain temperature sampling run on the device on the logits where the step left
+them; a request with top-k or top-p has its row brought to the host and filtered there, as the
+reference samples every row.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import List, Sequence
+
+import numpy as np
+import torch
+
+from ..kernels import ops
+
+_MASK = (1 << 64) - 1
+
+
+@dataclass(frozen=True)
+class SamplerConfig:
+    temperature: float = 0.8      # <= 0 means greedy
+    top_k: int = 0                # 0 = off
+    top_p: float = 1.0            # 1 = off; in (0, 1]
+    seed: int = 1
+
+    def validate(self, vocab_size: int) -> None:
+        if vocab_size <= 0:
+            raise ValueError("sampler: vocab_size must be positive")
+        if not self.temperature >= 0.0:                       # also refuses NaN
+            raise ValueError("sampler: temperature must be >= 0")
+        if self.top_k < 0:
+            raise ValueError("sampler: top_k must be >= 0")
+        if not 0.0 < self.top_p <= 1.0:
+            raise ValueError("sampler: top_p must be in (0, 1]")
+
+    @property
+    def greedy(self) -> bool:
+        return self.temperature <= 0.0
+
+    def filters(self, vocab_size: int) -> bool:
+        return 0 < self.top_k < vocab_size or self.top_p < 1.0
+
+
+def _splitmix64(x: int) -> int:
+    x = (x + 0x9E3779B97F4A7C15) & _MASK
+    x = ((x ^ (x >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    x = ((x ^ (x >> 27)) * 0x94D049BB133111EB) & _MASK
+    return x ^ (x >> 31)
+
+
+class UniformStream:
+    """xorshift64* started from splitmix64(seed); 24 random bits give u in [0, 1)."""
+
+    def __init__(self, seed: int):
+        self.state = _splitmix64(int(seed) & _MASK) or 1
+
+    def next_u32(self) -> int:
+        s = self.state
+        s ^= s >> 12
+        s ^= (s << 25) & _MASK
+        s ^= s >> 27
+        self.state = s
+        return ((s * 0x2545F4914F6CDD1D) & _MASK) >> 32
+
+    def next_uniform(self) -> float:
+        return (self.next_u32() >> 8) / 16777216.0
+
+
+def filtered_draw(logits: np.ndarray, cfg: SamplerConfig, u: float) -> int:
+    """Steps 2-4 on the host for one row (float32 probabilities, float64 sums)."""
+    logits = np.asarray(logits, dtype=np.float32)
+    n = logits.shape[0]
+    p = np.exp((logits - logits.max()) / np.float32(cfg.temperature), dtype=np.float32)
+    p *= np.float32(1.0 / float(p.sum(dtype=np.float64)))
+    order = np.arange(n)
+    if cfg.filters(n):
+        order = np.lexsort((order, -p))                       # probability descending, index ascending
+        if 0 < cfg.top_k < n:
+            order = order[:cfg.top_k]
+        if cfg.top_p < 1.0:
+            cum = np.cumsum(p[order], dtype=np.float64)
+            reached = np.nonzero(cum >= float(np.float32(cfg.top_p)) * cum[-1])[0]
+            if reached.size:
+                order = order[:reached[0] + 1]
+    cum = np.cumsum(p[order], dtype=np.float64)
+    hit = np.nonzero(float(np.float32(u)) * cum[-1] < cum)[0]
+    return int(order[hit[0]] if hit.size else order[-1])
+
+
+class Sampler:
+    """One request's sampler: its configuration and its own stream of uniform numbers."""
+
+    def __init__(self, config: SamplerConfig, vocab_size: int):
+        config.validate(vocab_size)
+        self.config, self.vocab_size = config, vocab_size
+        self.stream = UniformStream(config.seed)
+
+    def next_uniform(self) -> float:
+        return self.stream.next_uniform()
+
+    def sample(self, logits: torch.Tensor) -> int:
+        """One row of float32 logits on the device -> token id."""
+        return sample_rows(logits.reshape(1, -1), [self])[0]
+
+
+def sample_rows(logits: torch.Tensor, samplers: Sequence[Sampler]) -> List[int]:
+    """Row i of `logits` (float32 [n, vocab], on the device) is sampled with samplers[i].
+    A sampler draws one uniform number per call unless it is greedy."""
+    n, vocab = logits.shape
+    if n != len(samplers):
+        raise ValueError(f"{n} rows of logits for {len(samplers)} samplers")
+    out: List[int] = [0] * n
+    greedy = [i for i, s in enumerate(samplers) if s.config.greedy]
+    host = [i for i, s in enumerate(samplers) if not s.config.greedy and s.config.filters(vocab)]
+    plain = [i for i, s in enumerate(samplers) if not s.config.greedy and not s.config.filters(vocab)]
+    dev = logits.device
+    pending = []
+    if greedy:
+        rows = logits if len(greedy) == n else logits[torch.tensor(greedy, device=dev)]
+        res = torch.empty(len(greedy), dtype=torch.int32, device=dev)
+        ops.argmax(rows, res)
+        pending.append((greedy, res))
+    if plain:
+        rows = logits if len(plain) == n else logits[torch.tensor(plain, device=dev)]
+        temps = torch.tensor([samplers[i].config.temperature for i in plain], dtype=torch.float32).to(dev)
+        us = torch.tensor([samplers[i].next_uniform() for i in plain], dtype=torch.float32).to(dev)
+        res = torch.empty(len(plain), dtype=torch.int32, device=dev)
+        ops.sample_temperature(rows, temps, us, res)
+        pending.append((plain, res))
+    if host:
+        rows = logits[torch.tensor(host, device=dev)].cpu().numpy()
+        for i, row in zip(host, rows):
+            out[i] = filtered_draw(row, samplers[i].config, samplers[i].next_uniform())
+    for idx, res in pending:
+        for i, t in zip(idx, res.tolist()):
+            out[i] = int(t)
+    return out
