@@ -1,0 +1,252 @@
+// C[m, n] (=|+=) sum_k A[m, k] * W[n, k] with bfloat16 operands on the matrix cores, 32-bit sums.
+//
+// Both operands are row-major with k contiguous, so each lane's operand of a matrix instruction is
+// one 16-byte load of 8 consecutive k.  Two kernels:
+//
+//   tiled   a BM x 128 tile of C per workgroup of 4 waves, operands staged through LDS in
+//           k-blocks of 64 with the next block's global loads in flight during the products;
+//           v_mfma_f32_32x32x16_bf16.  For prompts (many rows).
+//   skinny  at most 64 rows of A (decode): weights stream from HBM straight into registers and
+//           are used once, activations go through LDS; v_mfma_f32_16x16x32_bf16.  k may be split
+//           over workgroups, partial sums are then added in a fixed order by a second kernel.
+//
+// Requirements (checked on the host): K a multiple of 8, rows of A and W 16-byte aligned.  The
+// output is float32 (stored or added onto what is there) or bfloat16 (stored).
+#include "common.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+enum Epilogue : int { EPI_STORE_F32 = 0, EPI_ADD_F32 = 1, EPI_STORE_BF16 = 2 };
+
+__device__ __forceinline__ uint4 load16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+template <int EPI>
+__device__ __forceinline__ void write_out(void* C, size_t o, float v) {
+    if constexpr (EPI == EPI_STORE_F32) ((float*)C)[o] = v;
+    else if constexpr (EPI == EPI_ADD_F32) ((float*)C)[o] += v;
+    else ((bf16_t*)C)[o] = f32_to_bf16(v);
+}
+
+// ------------------------------------------------------------------------------------------ tiled
+constexpr int BN = 128, BK = 64, LDS_STRIDE = BK + 8;     // +8 bf16 (16 bytes) of padding: conflict-free 16-byte reads
+
+template <int BM, int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
+                                                             int M, int N, int K, long lda, long ldw, long ldc) {
+    constexpr int WM = BM / 2;                 // rows of a wave's tile (waves sit 2 x 2)
+    constexpr int TM = WM / 32, TN = 2;        // 32x32 tiles per wave
+    constexpr int A_CHUNKS = BM * BK / 8 / 256, W_CHUNKS = BN * BK / 8 / 256;   // 16-byte chunks per thread
+    __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[BN * LDS_STRIDE];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * 64;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = floatx16{};
+
+    uint4 a_reg[A_CHUNKS], w_reg[W_CHUNKS];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int c = 0; c < A_CHUNKS; ++c) {
+            const int e = tid + 256 * c, row = e / (BK / 8), kc = (e % (BK / 8)) * 8;
+            const int m = m0 + row, k = k0 + kc;
+            a_reg[c] = (m < M && k < K) ? load16(A + (size_t)m * lda + k) : uint4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int c = 0; c < W_CHUNKS; ++c) {
+            const int e = tid + 256 * c, row = e / (BK / 8), kc = (e % (BK / 8)) * 8;
+            const int n = n0 + row, k = k0 + kc;
+            w_reg[c] = (n < N && k < K) ? load16(W + (size_t)n * ldw + k) : uint4{0, 0, 0, 0};
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int c = 0; c < A_CHUNKS; ++c) {
+            const int e = tid + 256 * c, row = e / (BK / 8), kc = (e % (BK / 8)) * 8;
+            *reinterpret_cast<uint4*>(&As[row * LDS_STRIDE + kc]) = a_reg[c];
+        }
+#pragma unroll
+        for (int c = 0; c < W_CHUNKS; ++c) {
+            const int e = tid + 256 * c, row = e / (BK / 8), kc = (e % (BK / 8)) * 8;
+            *reinterpret_cast<uint4*>(&Ws[row * LDS_STRIDE + kc]) = w_reg[c];
+        }
+    };
+
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        __syncthreads();                       // everyone has finished reading the previous block
+        stash();
+        __syncthreads();
+        if (k0 + BK < K) fetch(k0 + BK);       // in flight while the products below run
+        const int r = lane & 31, kq = (lane >> 5) * 8;
+#pragma unroll
+        for (int ks = 0; ks < BK; ks += 16) {
+            bf16x8 a[TM], b[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) a[i] = as_bf16x8(*reinterpret_cast<const uint4*>(&As[(wm + i * 32 + r) * LDS_STRIDE + ks + kq]));
+#pragma unroll
+            for (int j = 0; j < TN; ++j) b[j] = as_bf16x8(*reinterpret_cast<const uint4*>(&Ws[(wn + j * 32 + r) * LDS_STRIDE + ks + kq]));
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+    }
+    // Element v of a lane's 32x32 result: row 8*(v/4) + 4*(lane/32) + v%4, column lane%32.
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + wm + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3);
+                const int n = n0 + wn + j * 32 + (lane & 31);
+                if (m < M && n < N) write_out<EPI>(C, (size_t)m * ldc + n, acc[i][j][v]);
+            }
+}
+
+// ----------------------------------------------------------------------------------------- skinny
+// Workgroup: 4 waves, each a strip of 16 weight rows; the workgroup covers 64 weight rows and the
+// k range [k_begin, k_end) of its grid row.  Per block of 128 k, lane (r = lane%16, q = lane/16) of
+// a wave holds W[n0 + r][k0 + 32q + 8j .. +8] for j = 0..3: 64 contiguous bytes of a weight row.
+// The activations use the same assignment of k to lanes, so each product sums over the same k.
+constexpr int SK = 128, X_STRIDE = SK + 8;
+
+template <int MT>
+__global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, float* __restrict__ P,
+                                                              int M, int N, int K, long lda, long ldw, int k_per_split) {
+    __shared__ __attribute__((aligned(16))) bf16_t Xs[MT * 16 * X_STRIDE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 15, q = lane >> 4;
+    const int n = blockIdx.x * 64 + wave * 16 + r;
+    const int k_begin = blockIdx.y * k_per_split, k_end = min(K, k_begin + k_per_split);
+    const bf16_t* wrow = W + (size_t)min(n, N - 1) * ldw;
+
+    floatx4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = floatx4{};
+
+    uint4 w_next[4];
+    auto fetch_w = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int k = k0 + 32 * q + 8 * j;
+            w_next[j] = (k < k_end) ? load16(wrow + k) : uint4{0, 0, 0, 0};
+        }
+    };
+    fetch_w(k_begin);
+    for (int k0 = k_begin; k0 < k_end; k0 += SK) {
+        __syncthreads();
+        // activations of this k-block -> LDS (rows beyond M and k beyond the range are zero)
+        for (int e = tid; e < MT * 16 * (SK / 8); e += 256) {
+            const int row = e / (SK / 8), kc = (e % (SK / 8)) * 8;
+            const int k = k0 + kc;
+            *reinterpret_cast<uint4*>(&Xs[row * X_STRIDE + kc]) = (row < M && k < k_end) ? load16(A + (size_t)row * lda + k) : uint4{0, 0, 0, 0};
+        }
+        uint4 w_now[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w_now[j] = w_next[j];
+        if (k0 + SK < k_end) fetch_w(k0 + SK);
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bf16x8 b = as_bf16x8(w_now[j]);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(&Xs[(t * 16 + r) * X_STRIDE + 32 * q + 8 * j]));
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+            }
+        }
+    }
+    // Element v of a lane's 16x16 result: row (activation row) 4*(lane/16) + v, column (weight row) lane%16.
+    float* part = P + (size_t)blockIdx.y * M * N;
+    if (n < N) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int m = t * 16 + 4 * q + v;
+                if (m < M) part[(size_t)m * N + n] = acc[t][v];
+            }
+    }
+}
+
+// Adds the k-split partial sums [splits][M][N] in ascending split order and writes the result.
+template <int EPI>
+__global__ void skinny_reduce_kernel(const float* __restrict__ P, void* __restrict__ C, int M, int N, int splits, long ldc) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)M * N) return;
+    float s = 0.f;
+    for (int sp = 0; sp < splits; ++sp) s += P[(size_t)sp * M * N + i];
+    write_out<EPI>(C, (i / N) * ldc + (i % N), s);
+}
+
+int epilogue_of(int c_dtype, int accumulate) {
+    if (c_dtype == GI_F32) return accumulate ? EPI_ADD_F32 : EPI_STORE_F32;
+    if (c_dtype == GI_BF16 && !accumulate) return EPI_STORE_BF16;
+    return -1;
+}
+
+}  // namespace
+
+// Number of k-splits the skinny kernel would use, so that the caller can size the scratch
+// (splits * M * N floats).  Enough workgroups to cover the chip, each with at least 256 of k.
+GI_API int gi_gemm_bf16_skinny_splits(int N, int K) {
+    const int strips = (N + 63) / 64;
+    int splits = 1;
+    while (strips * splits < 512 && K / (splits * 2) >= 256) splits *= 2;
+    return splits;
+}
+
+GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int accumulate, int M, int N, int K, long lda, long ldw,
+                        long ldc, float* scratch, long scratch_floats, hipStream_t stream) {
+    GI_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: M %d, N %d, K %d must be positive", M, N, K);
+    GI_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_bf16: K %d and the row strides (%ld, %ld) must be multiples of 8", K, lda, ldw);
+    GI_REQUIRE(((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_bf16: operands must be 16-byte aligned");
+    GI_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm_bf16: leading dimensions too small");
+    const int epi = epilogue_of(c_dtype, accumulate);
+    GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
+
+    if (M <= 64) {
+        const int splits = gi_gemm_bf16_skinny_splits(N, K);
+        GI_REQUIRE(scratch != nullptr && scratch_floats >= (long)splits * M * N, "gemm_bf16: scratch of %ld floats needed, %ld given",
+                   (long)splits * M * N, scratch_floats);
+        int k_per_split = (K + splits - 1) / splits;
+        k_per_split = (k_per_split + SK - 1) / SK * SK;
+        dim3 grid((N + 63) / 64, splits);
+        const int mt = (M + 15) / 16;
+#define SKINNY(MT) gemm_bf16_skinny_kernel<MT><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, scratch, M, N, K, lda, ldw, k_per_split)
+        if (mt == 1) SKINNY(1); else if (mt == 2) SKINNY(2); else if (mt == 3) SKINNY(3); else SKINNY(4);
+#undef SKINNY
+        GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
+        const unsigned blocks = (unsigned)(((size_t)M * N + 255) / 256);
+        if (epi == EPI_STORE_F32) skinny_reduce_kernel<EPI_STORE_F32><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
+        else if (epi == EPI_ADD_F32) skinny_reduce_kernel<EPI_ADD_F32><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
+        else skinny_reduce_kernel<EPI_STORE_BF16><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
+        GI_CHECK_LAUNCH("gemm_bf16 (reduce)");
+        return 0;
+    }
+
+    GI_REQUIRE((M + 63) / 64 <= 65535, "gemm_bf16: M %d is too large", M);
+#define TILED(BM_, EPI_) gemm_bf16_tiled_kernel<BM_, EPI_><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
+    if (M <= 64 * 8 && (long)((M + 127) / 128) * ((N + BN - 1) / BN) < 256) {       // few rows: smaller tiles fill more of the chip
+        dim3 grid((N + BN - 1) / BN, (M + 63) / 64);
+        if (epi == EPI_STORE_F32) TILED(64, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(64, EPI_ADD_F32); else TILED(64, EPI_STORE_BF16);
+    } else {
+        dim3 grid((N + BN - 1) / BN, (M + 127) / 128);
+        if (epi == EPI_STORE_F32) TILED(128, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(128, EPI_ADD_F32); else TILED(128, EPI_STORE_BF16);
+    }
+#undef TILED
+    GI_CHECK_LAUNCH("gemm_bf16 (tiled)");
+    return 0;
+}

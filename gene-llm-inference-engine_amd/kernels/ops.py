@@ -30,6 +30,7 @@ _SIGNATURES = {
     "gi_gemm_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
                            c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
     "gi_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
 }
@@ -45,6 +46,8 @@ def lib():
             fn = getattr(l, name)
             fn.argtypes = sig
             fn.restype = c_int
+        l.gi_gemm_bf16_skinny_splits.argtypes = [c_int, c_int]
+        l.gi_gemm_bf16_skinny_splits.restype = c_int
         _lib = l
     return _lib
 
@@ -220,11 +223,28 @@ def attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window=None):
 
 
 def gemm_bf16_supports(a, w, out) -> bool:
-    return False
+    """Shapes and alignments the matrix-core kernels take; the exact kernel serves the rest."""
+    k = a.shape[1]
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and k % 8 == 0 and a.stride(1) == 1 and w.stride(1) == 1
+            and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and (out.dtype == torch.float32 or out.dtype == torch.bfloat16) and out.stride(1) == 1)
 
 
 def gemm_bf16(a, w, out, accumulate=False):
-    raise KernelError("no bfloat16 matrix-core kernel is built")
+    """out (=|+=) a @ w.T with bfloat16 operands on the matrix cores, float32 sums."""
+    _dev(a, w, out)
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape == (n, k), f"gemm: weight is {tuple(w.shape)}, activations are {tuple(a.shape)}")
+    _need(out.shape == (m, n), f"gemm: out is {tuple(out.shape)}, ({m}, {n}) is needed")
+    _need(gemm_bf16_supports(a, w, out), "gemm_bf16: operands must be bfloat16 with K and row strides multiples of 8, 16-byte aligned")
+    scratch, n_scratch = None, 0
+    if m <= 64:
+        n_scratch = lib().gi_gemm_bf16_skinny_splits(n, k) * m * n
+        scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device)
+    _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, m, n, k,
+          a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _stream())
+    return out
 
 
 def argmax(logits, out):
