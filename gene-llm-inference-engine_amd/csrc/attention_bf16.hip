@@ -1,0 +1,339 @@
+// Causal attention over the paged bfloat16 cache on the matrix cores: one kernel for portions of
+// prompts (many query rows of one request), one for single decoded rows.
+//
+// Cache of one layer, per page: keys [kv_head][place][HD], then values transposed
+// [kv_head][HD][place].  Page sizes must be multiples of 16.  Scores are scaled after the dot
+// product; softmax runs in 32-bit with a running maximum; probabilities are rounded to bfloat16
+// for the product with the values, their sum is kept unrounded.
+//
+// Both kernels use the freedom that a matrix instruction sums over its k index in any order as
+// long as both operands assign k to lanes in the same way: probabilities stay in the registers
+// in which the score product left them, and the value operand is loaded to match.
+#include "common.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint4 load16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ uint2 load8(const bf16_t* p) { return *reinterpret_cast<const uint2*>(p); }
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16); }
+
+// =========================================================================================== prompt
+// Workgroup: 4 waves, a tile of up to 128 consecutive rows of one request (32 per wave), one query
+// head.  Keys and values come in tiles of 64 positions through LDS.  The score product is taken
+// transposed, S^T[kv][q] = K * Q^T, so that each lane owns one query row (column lane%32) and the
+// softmax statistics of a row live in one lane (and its partner lane^32); the output is
+// accumulated transposed as well, O^T[d][q] = V^T * P^T.
+//
+// tiles[i] = {first row in the step, number of rows, position of the first row, request slot}.
+constexpr int KV_TILE = 64;
+
+template <int HD>
+__global__ __launch_bounds__(256) void attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
+                                                              bf16_t* __restrict__ out, const int4* __restrict__ tiles,
+                                                              const int* __restrict__ table, int table_stride, long page_stride,
+                                                              int page_size, int n_heads, int n_kv, int window, float scale) {
+    constexpr int K_STRIDE = HD + 8;            // bf16 elements; 16-byte reads of 32 rows hit distinct banks
+    constexpr int V_STRIDE = KV_TILE + 4;       // 8-byte reads of 32 rows hit distinct banks
+    constexpr int QSTEPS = HD / 16, DT = HD / 32;
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[KV_TILE * K_STRIDE];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[HD * V_STRIDE];
+
+    const int4 tile = tiles[blockIdx.x];
+    const int row0 = tile.x, n_rows = tile.y, pos0 = tile.z, slot = tile.w;
+    const int head = blockIdx.y, g = head / (n_heads / n_kv);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, hf = lane >> 5;
+    const int* tab = table + (size_t)slot * table_stride;
+
+    const int my_row = wave * 32 + col;                         // this lane's query row within the tile
+    const bool row_ok = my_row < n_rows;
+    const int my_pos = row_ok ? pos0 + my_row : -1;
+    const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+    const int wave_last = pos0 + min(n_rows, wave * 32 + 32) - 1;       // the last position this wave's rows see
+    const bool wave_ok = wave * 32 < n_rows;
+
+    bf16x8 qreg[QSTEPS];
+#pragma unroll
+    for (int s = 0; s < QSTEPS; ++s) {
+        uint4 v = {0, 0, 0, 0};
+        if (row_ok) v = load16(q + ((size_t)(row0 + my_row) * n_heads + head) * HD + 16 * s + 8 * hf);
+        qreg[s] = as_bf16x8(v);
+    }
+    floatx16 o[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i) o[i] = floatx16{};
+    float m = -INFINITY, l = 0.f;
+
+    const int last_pos = pos0 + n_rows - 1;
+    const int first_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+    const long v_plane = (long)n_kv * page_size * HD;
+    for (int kv0 = first_lo & ~(KV_TILE - 1); kv0 <= last_pos; kv0 += KV_TILE) {
+        __syncthreads();
+        // keys: 64 rows of HD, 16 bytes a thread at a time
+        for (int e = tid; e < KV_TILE * (HD / 8); e += 256) {
+            const int r = e / (HD / 8), c = (e % (HD / 8)) * 8, kv = kv0 + r;
+            uint4 v = {0, 0, 0, 0};
+            if (kv <= last_pos) {
+                const int page = tab[kv / page_size];
+                if (page >= 0) v = load16(cache + (long)page * page_stride + ((long)g * page_size + kv % page_size) * HD + c);
+            }
+            *reinterpret_cast<uint4*>(&Ks[r * K_STRIDE + c]) = v;
+        }
+        // values, already transposed in the cache: HD rows of 64 positions, 8 positions a thread at a time
+        for (int e = tid; e < HD * (KV_TILE / 8); e += 256) {
+            const int d = e % HD, c = (e / HD) * 8, kv = kv0 + c;
+            uint4 v = {0, 0, 0, 0};
+            if (kv <= last_pos) {
+                const int page = tab[kv / page_size];
+                if (page >= 0) v = load16(cache + (long)page * page_stride + v_plane + ((long)g * HD + d) * page_size + kv % page_size);
+            }
+            uint2* dst = reinterpret_cast<uint2*>(&Vs[d * V_STRIDE + c]);
+            dst[0] = uint2{v.x, v.y};
+            dst[1] = uint2{v.z, v.w};
+        }
+        __syncthreads();
+        if (!wave_ok) continue;
+#pragma unroll
+        for (int st = 0; st < KV_TILE / 32; ++st) {
+            const int kv_base = kv0 + 32 * st;
+            if (kv_base > wave_last) break;                               // beyond every row of this wave
+            floatx16 s = floatx16{};
+#pragma unroll
+            for (int ks = 0; ks < QSTEPS; ++ks) {
+                const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(&Ks[(32 * st + col) * K_STRIDE + 16 * ks + 8 * hf]));
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[ks], s, 0, 0, 0);
+            }
+            // element v of s: key position kv_base + 8*(v/4) + 4*hf + v%4, query row `col`
+            float mx = -INFINITY;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int kv = kv_base + 8 * (v / 4) + 4 * hf + (v & 3);
+                s[v] = (kv <= my_pos && kv >= my_lo) ? s[v] * scale : -INFINITY;
+                mx = fmaxf(mx, s[v]);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m, mx);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;      // a row that has seen nothing yet
+            const float corr = expf(m - m_use);
+            float sum = 0.f;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                s[v] = expf(s[v] - m_use);
+                sum += s[v];
+            }
+            sum += __shfl_xor(sum, 32, 64);
+            l = l * corr + sum;
+            m = m_new;
+#pragma unroll
+            for (int i = 0; i < DT; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o[i][v] *= corr;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {                                 // two groups of 16 key positions
+                const uint4 pb = {pack2(s[8 * t], s[8 * t + 1]), pack2(s[8 * t + 2], s[8 * t + 3]), pack2(s[8 * t + 4], s[8 * t + 5]),
+                                  pack2(s[8 * t + 6], s[8 * t + 7])};
+                // slot e of this lane is key position 32*st + 16*t + 8*(e/4) + 4*hf + e%4 of the tile
+#pragma unroll
+                for (int i = 0; i < DT; ++i) {
+                    const bf16_t* vrow = &Vs[(32 * i + col) * V_STRIDE + 32 * st + 16 * t + 4 * hf];
+                    const uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 8);
+                    o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(uint4{lo.x, lo.y, hi.x, hi.y}), as_bf16x8(pb), o[i], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (!row_ok) return;
+    const float inv = 1.0f / l;
+    bf16_t* orow = out + ((size_t)(row0 + my_row) * n_heads + head) * HD;
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) {                                  // element v: channel 32*i + 8*(v/4) + 4*hf + v%4
+            const int d = 32 * i + 8 * v4 + 4 * hf;
+            *reinterpret_cast<uint2*>(orow + d) = uint2{pack2(o[i][4 * v4] * inv, o[i][4 * v4 + 1] * inv),
+                                                        pack2(o[i][4 * v4 + 2] * inv, o[i][4 * v4 + 3] * inv)};
+        }
+}
+
+// =========================================================================================== decode
+// One wave per (row, key/value head, query-head group of up to 16, split of the context).  Keys and
+// values stream from global memory straight into the operands of v_mfma_f32_16x16x32_bf16; nothing
+// goes through LDS.  Scores: S[kv][head] = K * Q^T, 16 key positions at a time; output
+// O^T[d][head] = V^T * P^T, 32 key positions at a time.  Lane (r = lane%16, q4 = lane/16) owns
+// query head r of the group: its softmax statistics and its columns of S and O^T.
+// A split writes unnormalised partial results {m, l, O} to `part`; the combine kernel merges them.
+template <int HD>
+__global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
+                                                             float* __restrict__ part, const int* __restrict__ rows,
+                                                             const int* __restrict__ pos, const int* __restrict__ slots,
+                                                             const int* __restrict__ table, int table_stride, long page_stride,
+                                                             int page_size, int n_heads, int n_kv, int window, float scale,
+                                                             int n_splits, int split_len) {
+    constexpr int KSTEPS = HD / 32, DT = HD / 16;
+    const int group = n_heads / n_kv, hg_per_kv = (group + 15) / 16;
+    const int row = rows[blockIdx.x], g = blockIdx.y / hg_per_kv, hg = blockIdx.y % hg_per_kv, split = blockIdx.z;
+    const int lane = threadIdx.x, r = lane & 15, q4 = lane >> 4;
+    const int head_in_group = hg * 16 + r;
+    const bool head_ok = head_in_group < group;
+    const int head = g * group + head_in_group;
+    const int my_pos = pos[row];
+    const int lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+    const int* tab = table + (size_t)slots[row] * table_stride;
+    const int begin = (lo & ~31) + split * split_len, end = min(my_pos + 1, begin + split_len);     // split_len is a multiple of 32
+
+    bf16x8 qreg[KSTEPS];
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+        uint4 v = {0, 0, 0, 0};
+        if (head_ok) v = load16(q + ((size_t)row * n_heads + head) * HD + 32 * s + 8 * q4);
+        qreg[s] = as_bf16x8(v);
+    }
+    floatx4 o[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i) o[i] = floatx4{};
+    float m = -INFINITY, l = 0.f;
+    const long v_plane = (long)n_kv * page_size * HD;
+    const bf16_t* kbase = cache + (long)g * page_size * HD;
+    const bf16_t* vbase = cache + v_plane + (long)g * HD * page_size;
+
+    for (int kv0 = begin; kv0 < end; kv0 += 32) {
+        // scores of 32 key positions: two products of 16; an address beyond the row's own range is
+        // clamped into it (its score is masked below)
+        floatx4 s[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int kv = min(max(kv0 + 16 * t + r, lo), my_pos);
+            const bf16_t* krow = kbase + (long)tab[kv / page_size] * page_stride + (long)(kv % page_size) * HD;
+            s[t] = floatx4{};
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks)
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(load16(krow + 32 * ks + 8 * q4)), qreg[ks], s[t], 0, 0, 0);
+        }
+        // element v of s[t]: key position kv0 + 16*t + 4*q4 + v, query head r
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int kv = kv0 + 16 * t + 4 * q4 + v;
+                s[t][v] = (kv >= lo && kv < end) ? s[t][v] * scale : -INFINITY;
+                mx = fmaxf(mx, s[t][v]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = expf(m - m_use);
+        float sum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                s[t][v] = expf(s[t][v] - m_use);
+                sum += s[t][v];
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        l = l * corr + sum;
+        m = m_new;
+        // slot e of this lane is key position kv0 + 16*(e/4) + 4*q4 + e%4
+        const uint4 pb = {pack2(s[0][0], s[0][1]), pack2(s[0][2], s[0][3]), pack2(s[1][0], s[1][1]), pack2(s[1][2], s[1][3])};
+        const int kva = min(max(kv0 + 4 * q4, lo & ~3), my_pos & ~3), kvb = min(max(kv0 + 16 + 4 * q4, lo & ~3), my_pos & ~3);
+        const bf16_t* va = vbase + (long)tab[kva / page_size] * page_stride + kva % page_size;
+        const bf16_t* vb = vbase + (long)tab[kvb / page_size] * page_stride + kvb % page_size;
+#pragma unroll
+        for (int i = 0; i < DT; ++i) {
+            const uint2 x = load8(va + (long)(16 * i + r) * page_size), y = load8(vb + (long)(16 * i + r) * page_size);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) o[i][v] *= corr;
+            o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(uint4{x.x, x.y, y.x, y.y}), as_bf16x8(pb), o[i], 0, 0, 0);
+        }
+    }
+    if (!head_ok) return;
+    // part[row_index][head][split] = {m, l, O[HD]}; element v of o[i]: channel 16*i + 4*q4 + v, query head r
+    float* dst = part + (((size_t)blockIdx.x * n_heads + head) * n_splits + split) * (HD + 2);
+    if (q4 == 0) {
+        dst[0] = m;
+        dst[1] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) dst[2 + 16 * i + 4 * q4 + v] = o[i][v];
+}
+
+// Merges the splits of one (row, head) in split order: out = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s.
+__global__ void attention_decode_combine_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, const int* __restrict__ rows,
+                                                int n_heads, int hd, int n_splits) {
+    const int idx = blockIdx.x, head = blockIdx.y;
+    const float* src = part + ((size_t)idx * n_heads + head) * n_splits * (hd + 2);
+    float big = -INFINITY;
+    for (int s = 0; s < n_splits; ++s) big = fmaxf(big, src[(size_t)s * (hd + 2)]);
+    float denom = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+        const float ms = src[(size_t)s * (hd + 2)];
+        if (ms != -INFINITY) denom += expf(ms - big) * src[(size_t)s * (hd + 2) + 1];
+    }
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        float acc = 0.f;
+        for (int s = 0; s < n_splits; ++s) {
+            const float ms = src[(size_t)s * (hd + 2)];
+            if (ms != -INFINITY) acc += expf(ms - big) * src[(size_t)s * (hd + 2) + 2 + d];
+        }
+        out[((size_t)rows[idx] * n_heads + head) * hd + d] = f32_to_bf16(acc / denom);
+    }
+}
+
+}  // namespace
+
+GI_API int gi_attention_bf16_supports(int hd, int page_size, int prompt) {
+    if (page_size % 16 != 0) return 0;
+    if (prompt) return hd == 32 || hd == 64 || hd == 96 || hd == 128;
+    return hd == 32 || hd == 64 || hd == 96 || hd == 128 || hd == 256;
+}
+
+GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out, const int* tiles, int n_tiles, const int* table,
+                                    int table_stride, long page_stride, int page_size, int n_heads, int n_kv, int hd, int window,
+                                    float scale, hipStream_t stream) {
+    GI_REQUIRE(n_tiles > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_prompt: bad counts (%d tiles, %d heads, %d kv heads)",
+               n_tiles, n_heads, n_kv);
+    GI_REQUIRE(gi_attention_bf16_supports(hd, page_size, 1), "attention_prompt: head size %d with page size %d is not supported", hd, page_size);
+    GI_REQUIRE(page_stride >= 2L * n_kv * page_size * hd && page_stride % 8 == 0, "attention_prompt: bad page stride %ld", page_stride);
+    GI_REQUIRE(n_heads <= 65535, "attention_prompt: too many heads");
+    dim3 grid(n_tiles, n_heads);
+#define GO(HD) attention_prompt_kernel<HD><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, \
+                                                                     table, table_stride, page_stride, page_size, n_heads, n_kv, window, scale)
+    if (hd == 32) GO(32); else if (hd == 64) GO(64); else if (hd == 96) GO(96); else GO(128);
+#undef GO
+    GI_CHECK_LAUNCH("attention_prompt");
+    return 0;
+}
+
+GI_API int gi_attention_decode_bf16(const void* q, const void* cache, void* out, float* part, long part_floats, const int* rows, int n_rows,
+                                    const int* pos, const int* slots, const int* table, int table_stride, long page_stride, int page_size,
+                                    int n_heads, int n_kv, int hd, int window, float scale, int n_splits, int split_len,
+                                    hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_decode: bad counts (%d rows, %d heads, %d kv heads)",
+               n_rows, n_heads, n_kv);
+    GI_REQUIRE(gi_attention_bf16_supports(hd, page_size, 0), "attention_decode: head size %d with page size %d is not supported", hd, page_size);
+    GI_REQUIRE(page_stride >= 2L * n_kv * page_size * hd && page_stride % 8 == 0, "attention_decode: bad page stride %ld", page_stride);
+    GI_REQUIRE(n_splits >= 1 && n_splits <= 65535 && split_len > 0 && split_len % 32 == 0, "attention_decode: bad split (%d of %d)", n_splits, split_len);
+    GI_REQUIRE(part != nullptr && part_floats >= (long)n_rows * n_heads * n_splits * (hd + 2), "attention_decode: scratch too small");
+    const int hg = (n_heads / n_kv + 15) / 16;
+    GI_REQUIRE(n_kv * hg <= 65535, "attention_decode: too many heads");
+    dim3 grid(n_rows, n_kv * hg, n_splits);
+#define GO(HD) attention_decode_kernel<HD><<<grid, 64, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, part, rows, pos, slots, table, \
+                                                                   table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits, split_len)
+    if (hd == 32) GO(32); else if (hd == 64) GO(64); else if (hd == 96) GO(96); else if (hd == 128) GO(128); else GO(256);
+#undef GO
+    GI_CHECK_LAUNCH("attention_decode");
+    dim3 cgrid(n_rows, n_heads);
+    attention_decode_combine_kernel<<<cgrid, 64, 0, stream>>>(part, (bf16_t*)out, rows, n_heads, hd, n_splits);
+    GI_CHECK_LAUNCH("attention_decode (combine)");
+    return 0;
+}

@@ -9,8 +9,8 @@
 // The order of every sum depends on (pos, window, hd) only, so a row's result has the same bits
 // whatever else is in the batch and whichever pages hold its request.
 //
-// Cache of one layer: [page][K|V][kv_head][place][hd]; table[slot][i] is the page of positions
-// i*page_size .. (i+1)*page_size - 1.
+// Cache of one layer: per page the keys [kv_head][place][hd], then the values transposed
+// [kv_head][hd][place]; table[slot][i] is the page of positions i*page_size .. (i+1)*page_size - 1.
 #include "common.h"
 
 namespace {
@@ -40,9 +40,11 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
         const int j = j0 + lane;
         const bool valid = j <= p_row;
         float s = -INFINITY;
-        long off = 0;
+        long off = 0, voff = 0;
         if (valid) {
-            off = (long)tab[j / page_size] * page_stride + ((long)g * page_size + j % page_size) * hd;
+            const long page = (long)tab[j / page_size] * page_stride;
+            off = page + ((long)g * page_size + j % page_size) * hd;
+            voff = page + v_plane + (long)g * hd * page_size + j % page_size;
             float dot = 0.f;
             for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], load_f32(cache, off + d), dot);
             s = dot * scale;
@@ -54,7 +56,7 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
         m = m_new;
         __syncthreads();                         // the previous tile's p_s and v_off have been read
         p_s[lane] = p;
-        v_off[lane] = off + v_plane;
+        v_off[lane] = voff;
         __syncthreads();
         const int n_here = min(64, p_row - j0 + 1);
 #pragma unroll
@@ -65,7 +67,7 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
 #pragma unroll
             for (int i = 0; i < MAX_HD / 64; ++i) {
                 const int d = lane + 64 * i;
-                if (d < hd) acc[i] = fmaf(pj, load_f32(cache, vo + d), acc[i]);
+                if (d < hd) acc[i] = fmaf(pj, load_f32(cache, vo + (long)d * page_size), acc[i]);
             }
         }
     }

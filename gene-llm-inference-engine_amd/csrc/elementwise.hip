@@ -105,7 +105,9 @@ GI_API int gi_rope_cos_sin(const int* pos, const double* inv_freq, float* cos_ou
 //   k heads are rotated and, with the v heads as they are, written into the page
 //   table[slot[t]][pos / page_size] at place pos % page_size.
 // Pairs are (k, k + hd/2): a' = a*cos - b*sin, b' = a*sin + b*cos (src/kernels/kernels.cpp:165-180).
-// Cache of one layer: [page][K|V][kv_head][place][hd].  cos == nullptr means no rotation.
+// Cache of one layer: per page the keys [kv_head][place][hd], then the values transposed
+// [kv_head][hd][place] (so that consecutive positions of one value channel are contiguous, which is
+// what the matrix instructions of the attention kernels load).  cos == nullptr means no rotation.
 // k == nullptr means the layer reads another layer's cache and writes none.
 template <typename TQ, typename TC>
 __global__ void rope_store_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v, long ldq, long ldk,
@@ -137,8 +139,8 @@ __global__ void rope_store_kernel(const float* __restrict__ q, const float* __re
         const size_t o = ((size_t)g * page_size + place) * hd;
         store_f32(kbase, o + kk, a * cc - b * ss);
         store_f32(kbase, o + kk + half, a * ss + b * cc);
-        store_f32(vbase, o + kk, v[(size_t)t * ldv + g * hd + kk]);
-        store_f32(vbase, o + kk + half, v[(size_t)t * ldv + g * hd + kk + half]);
+        store_f32(vbase, ((size_t)g * hd + kk) * page_size + place, v[(size_t)t * ldv + g * hd + kk]);
+        store_f32(vbase, ((size_t)g * hd + kk + half) * page_size + place, v[(size_t)t * ldv + g * hd + kk + half]);
     }
 }
 

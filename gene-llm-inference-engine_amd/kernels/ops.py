@@ -31,6 +31,10 @@ _SIGNATURES = {
     "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
                            c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
+    "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
+                                 c_float, c_void_p],
+    "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long,
+                                 c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
     "gi_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
 }
@@ -46,6 +50,8 @@ def lib():
             fn = getattr(l, name)
             fn.argtypes = sig
             fn.restype = c_int
+        l.gi_attention_bf16_supports.argtypes = [c_int, c_int, c_int]
+        l.gi_attention_bf16_supports.restype = c_int
         l.gi_gemm_bf16_skinny_splits.argtypes = [c_int, c_int]
         l.gi_gemm_bf16_skinny_splits.restype = c_int
         _lib = l
@@ -135,6 +141,7 @@ def rope_cos_sin(positions, inv_freq, cos_out, sin_out):
 
 
 def _check_cache(cache, table, page_size, n_kv, hd, what):
+    # the last two axes of the value half hold [hd][place]: values are stored transposed
     _need(cache.dim() == 5 and tuple(cache.shape[1:]) == (2, n_kv, page_size, hd) and cache.is_contiguous(),
           f"{what}: the cache must be [pages, 2, {n_kv}, {page_size}, {hd}], contiguous; it is {tuple(cache.shape)}")
     _need(table.dim() == 2 and table.dtype == torch.int32 and table.stride(1) == 1, f"{what}: the page table must be int32 [slots, pages]")
@@ -217,8 +224,72 @@ def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, w
     return out
 
 
+class AttentionPlan:
+    """How a step's rows are shared between the two bfloat16 attention kernels: requests that bring
+    one row go to the decode kernel, portions of prompts are cut into tiles of up to 128 rows for
+    the prompt kernel.  Made once per step and used by every layer."""
+    TILE = 128
+
+    def __init__(self, seg_start, seg_len, seg_pos0, seg_slot, device):
+        dec, tiles, self.max_decode_context = [], [], 0
+        for start, n, pos0, slot in zip(seg_start, seg_len, seg_pos0, seg_slot):
+            if n == 1:
+                dec.append(start)
+                self.max_decode_context = max(self.max_decode_context, pos0 + 1)
+            else:
+                for off in range(0, n, self.TILE):
+                    tiles.append((start + off, min(self.TILE, n - off), pos0 + off, slot))
+        self.n_decode, self.n_tiles = len(dec), len(tiles)
+        both = torch.tensor(dec + [v for t in tiles for v in t], dtype=torch.int32).to(device)
+        self.decode_rows = both[:len(dec)]
+        self.tiles = both[len(dec):]
+
+
+def attention_bf16_supports(hd, page_size, prompt: bool) -> bool:
+    return bool(lib().gi_attention_bf16_supports(hd, page_size, 1 if prompt else 0))
+
+
+def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None,
+                   target_waves: int = 2048):
+    """Attention of a step's rows with the matrix-core kernels (bfloat16 q, cache and out)."""
+    _dev(q, cache, out, positions, slots, table)
+    n = q.shape[0]
+    for t, name in ((q, "q"), (cache, "cache"), (out, "out")):
+        _need(t.dtype == torch.bfloat16, f"attention_bf16: {name} must be bfloat16")
+    _need(q.shape == (n, n_heads * hd) and q.is_contiguous() and out.shape == q.shape and out.is_contiguous(),
+          "attention: q and out must be [n, heads*hd], contiguous")
+    page_size = cache.shape[3]
+    _check_cache(cache, table, page_size, n_kv, hd, "attention")
+    _i32(positions, "attention: positions", n)
+    _i32(slots, "attention: slots", n)
+    window = int(window or 0)
+    scale = float(scale if scale is not None else hd ** -0.5)
+    if plan.n_tiles:
+        _call("gi_attention_prompt_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles,
+              table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, _stream())
+    if plan.n_decode:
+        span = plan.max_decode_context if not window else min(plan.max_decode_context, window + 31)
+        waves = plan.n_decode * n_kv * ((n_heads // n_kv + 15) // 16)
+        n_splits = max(1, min(-(-target_waves // waves), -(-span // 64)))
+        split_len = -(-(-(-span // n_splits)) // 32) * 32
+        n_splits = -(-span // split_len)
+        n_part = plan.n_decode * n_heads * n_splits * (hd + 2)
+        part = torch.empty(n_part, dtype=torch.float32, device=q.device)
+        _call("gi_attention_decode_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), part.data_ptr(), n_part,
+              plan.decode_rows.data_ptr(), plan.n_decode, positions.data_ptr(), slots.data_ptr(), table.data_ptr(), table.stride(0),
+              cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits, split_len, _stream())
+    return out
+
+
 def attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window=None):
     """Attention of a step's rows; the kernel is chosen by the storage dtype and the batch's shape."""
+    page_size = cache.shape[3]
+    if q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16:
+        if "attention_plan" not in ctx.memo:
+            ctx.memo["attention_plan"] = AttentionPlan(ctx.seg_start, ctx.seg_len, ctx.seg_pos0, ctx.seg_slot, ctx.device)
+        plan = ctx.memo["attention_plan"]
+        if (not plan.n_tiles or attention_bf16_supports(hd, page_size, True)) and (not plan.n_decode or attention_bf16_supports(hd, page_size, False)):
+            return attention_bf16(q, cache, out, plan, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window)
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window)
 
 

@@ -150,3 +150,136 @@ def test_sample_temperature_matches_the_inverse_distribution():
                 p = torch.softmax(logits[i].double() / float(temps[i]), 0)
                 cum = torch.cumsum(p, 0)
                 assert abs(got - want) == 1 and float((cum - float(us[i])).abs().min()) < 1e-6, (vocab, i, got, want)
+
+
+# ------------------------------------------------------------------------------------- attention
+def build_paged(requests, n_kv, hd, page_size, dtype, seed, scale_one=None):
+    """Dense keys/values per request, written into a paged cache with scrambled pages and a rim of
+    NaN pages that nothing may touch.  requests: list of context lengths.  Returns cache, table, dense."""
+    g = torch.Generator().manual_seed(seed)
+    n_pages_needed = sum(-(-n // page_size) for n in requests)
+    n_pages = n_pages_needed + 3
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    cache = torch.full((n_pages, 2, n_kv, page_size, hd), float("nan"), dtype=dtype)
+    width = max(-(-n // page_size) for n in requests) + 2
+    table = torch.full((len(requests) + 1, width), -1, dtype=torch.int32)
+    dense, nxt = [], 0
+    for slot, n in enumerate(requests):
+        k = torch.randn(n, n_kv, hd, generator=g).to(dtype)
+        v = torch.randn(n, n_kv, hd, generator=g).to(dtype)
+        if scale_one is not None and n > scale_one[0]:
+            k[scale_one[0]] *= scale_one[1]                    # one far key that must stand out
+        dense.append((k, v))
+        for i in range(-(-n // page_size)):
+            page = perm[nxt]; nxt += 1
+            table[slot + 1, i] = page                          # slot 0 of the table stays unused (-1)
+            cache[page] = 0
+            m = min(page_size, n - i * page_size)
+            cache[page, 0, :, :m, :] = k[i * page_size:i * page_size + m].permute(1, 0, 2)
+            cache[page, 1].view(n_kv, hd, page_size)[:, :, :m] = v[i * page_size:i * page_size + m].permute(1, 2, 0)
+    return cache.to(DEV), table.to(DEV), dense
+
+
+def plain_attention_rows(q, dense, rows, n_heads, n_kv, hd, window):
+    """rows: (slot, pos) per row of q [n, heads*hd]; float64 softmax(q k / sqrt(hd)) v over keys <= pos."""
+    out = torch.zeros(q.shape[0], n_heads, hd, dtype=torch.float64)
+    qd = q.double().cpu().view(-1, n_heads, hd)
+    for i, (slot, pos) in enumerate(rows):
+        k, v = dense[slot]
+        lo = max(0, pos - window + 1) if window else 0
+        for h in range(n_heads):
+            kv = h // (n_heads // n_kv)
+            s = (k[lo:pos + 1, kv].double() @ qd[i, h]) / math.sqrt(hd)
+            out[i, h] = torch.softmax(s, 0) @ v[lo:pos + 1, kv].double()
+    return out.view(q.shape[0], n_heads * hd)
+
+
+ATT_CASES = [  # n_heads, n_kv, hd, page_size, window
+    (4, 2, 64, 16, None), (3, 1, 32, 16, None), (8, 8, 128, 32, None), (6, 2, 96, 16, None), (4, 4, 64, 16, 40), (32, 8, 64, 16, None),
+    (5, 5, 48, 16, None), (2, 1, 16, 4, 9),
+]
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,ps,window", ATT_CASES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_over_pages(n_heads, n_kv, hd, ps, window, dtype):
+    """Portions of prompts on top of an existing cache, beside single decoded rows, on scrambled pages."""
+    from geneinfer_amd.parts import StepContext
+    contexts = [300, 131, 1, 77, 530]
+    cache, table, dense = build_paged(contexts, n_kv, hd, ps, dtype, seed=hd + n_heads)
+    # request 0: rows at positions 150..299 (a portion on top of 150 cached positions); request 1: its last row;
+    # request 2: its only row; request 3: rows 0..76 (a whole prompt); request 4: its last row
+    segs = [(0, 150, 150), (1, 130, 1), (2, 0, 1), (3, 0, 77), (4, 529, 1)]
+    rows, seg_start, seg_len, seg_pos0, seg_slot = [], [], [], [], []
+    for slot, pos0, n in segs:
+        seg_start.append(len(rows)); seg_len.append(n); seg_pos0.append(pos0); seg_slot.append(slot + 1)
+        rows += [(slot, pos0 + i) for i in range(n)]
+    T = len(rows)
+    q = randn(T, n_heads * hd, dtype=dtype, seed=3)
+    pos = torch.tensor([p for _, p in rows], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([s + 1 for s, _ in rows], dtype=torch.int32, device=DEV)
+    ctx = StepContext(n_rows=T, dtype=dtype, device=torch.device(DEV), tokens=pos, row_pos=pos, row_slot=slots, seg_slot=seg_slot,
+                      seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0)
+    out = torch.full((T, n_heads * hd), float("nan"), dtype=dtype, device=DEV)
+    before = cache.clone()
+    ops().attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window)
+    want = plain_attention_rows(q, dense, rows, n_heads, n_kv, hd, window)
+    err = rel(out, want)
+    assert err < (2e-6 if dtype == torch.float32 else 8e-3), err
+    assert torch.equal(torch.nan_to_num(cache, nan=-1.0), torch.nan_to_num(before, nan=-1.0)), "attention wrote into the cache"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_finds_one_far_key(dtype):
+    """Among 700 keys one is scaled so that its score stands out: the output must be its value."""
+    from geneinfer_amd.parts import StepContext
+    n_heads, n_kv, hd, ps = 4, 2, 64, 16
+    cache, table, dense = build_paged([700], n_kv, hd, ps, dtype, seed=1)
+    k, v = dense[0]
+    target = 37
+    q = (k[target].float().repeat_interleave(n_heads // n_kv, 0) * 3.0).reshape(1, n_heads * hd).to(dtype).to(DEV)
+    pos = torch.tensor([699], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([1], dtype=torch.int32, device=DEV)
+    ctx = StepContext(n_rows=1, dtype=dtype, device=torch.device(DEV), tokens=pos, row_pos=pos, row_slot=slots, seg_slot=[1], seg_start=[0],
+                      seg_len=[1], seg_pos0=[699])
+    out = torch.empty(1, n_heads * hd, dtype=dtype, device=DEV)
+    ops().attention(q, cache, out, ctx, table, n_heads, n_kv, hd, None)
+    want = plain_attention_rows(q, dense, [(0, 699)], n_heads, n_kv, hd, None)
+    assert rel(out, want) < (2e-6 if dtype == torch.float32 else 8e-3)
+    assert rel(out.view(n_heads, hd)[0], v[target, 0]) < 2e-2          # the softmax is nearly one-hot on the target
+
+
+def test_rope_store_writes_the_right_places():
+    n_heads, n_kv, hd, ps = 4, 2, 32, 16
+    n_pages = 5
+    cache = torch.full((n_pages, 2, n_kv, ps, hd), -777.25, device=DEV)
+    table = torch.tensor([[-1, -1, -1], [3, 0, 4]], dtype=torch.int32, device=DEV)
+    T = 3
+    pos = torch.tensor([15, 16, 17], dtype=torch.int32, device=DEV)     # the last place of a page, then the next page
+    slots = torch.ones(T, dtype=torch.int32, device=DEV)
+    qkv = randn(T, (n_heads + 2 * n_kv) * hd, seed=20)
+    a, kvd = n_heads * hd, n_kv * hd
+    inv = torch.tensor([1.0 / (10000.0 ** (2 * k / hd)) for k in range(hd // 2)], dtype=torch.float64, device=DEV)
+    cos, sin = torch.empty(T, hd // 2, device=DEV), torch.empty(T, hd // 2, device=DEV)
+    ops().rope_cos_sin(pos, inv, cos, sin)
+    q_out = torch.empty(T, a, device=DEV)
+    ops().rope_store(qkv[:, :a], qkv[:, a:a + kvd], qkv[:, a + kvd:], cos, sin, pos, slots, table, q_out, cache, n_heads, n_kv, hd)
+
+    def rotate_half_form(x, heads):          # x*cos + rotate_half(x)*sin with cos/sin doubled over both halves (tests/verify_kernels.py:284-291)
+        x = x.double().cpu().view(T, heads, hd)
+        ang = pos.double().cpu()[:, None] * inv.cpu()[None, :]
+        c, s_ = torch.cat([ang.cos(), ang.cos()], -1)[:, None, :], torch.cat([ang.sin(), ang.sin()], -1)[:, None, :]
+        rot = torch.cat([-x[..., hd // 2:], x[..., :hd // 2]], -1)
+        return x * c + rot * s_
+
+    assert rel(q_out.view(T, n_heads, hd), rotate_half_form(qkv[:, :a], n_heads)) < 2e-6
+    k_want = rotate_half_form(qkv[:, a:a + kvd], n_kv)
+    v_want = qkv[:, a + kvd:].double().cpu().view(T, n_kv, hd)
+    for t, (page, place) in enumerate([(3, 15), (0, 0), (0, 1)]):
+        assert rel(cache[page, 0, :, place, :], k_want[t]) < 2e-6
+        assert rel(cache[page, 1].view(n_kv, hd, ps)[:, :, place], v_want[t]) < 1e-7
+    touched = torch.zeros_like(cache, dtype=torch.bool)
+    for page, place in [(3, 15), (0, 0), (0, 1)]:
+        touched[page, 0, :, place, :] = True
+        touched[page, 1].view(n_kv, hd, ps)[:, :, place] = True
+    assert torch.all(cache[~touched] == -777.25), "rope_store wrote outside its places"
