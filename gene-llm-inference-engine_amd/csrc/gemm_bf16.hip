@@ -6,9 +6,17 @@
 //   tiled   a BM x 128 tile of C per workgroup of 4 waves, operands staged through LDS in
 //           k-blocks of 64 with the next block's global loads in flight during the products;
 //           v_mfma_f32_32x32x16_bf16.  For prompts (many rows).
-//   skinny  at most 64 rows of A (decode): weights stream from HBM straight into registers and
-//           are used once, activations go through LDS; v_mfma_f32_16x16x32_bf16.  k may be split
-//           over workgroups, partial sums are then added in a fixed order by a second kernel.
+//   skinny  17..64 rows of A: weights stream from HBM straight into registers and are used
+//           once, activations go through LDS; v_mfma_f32_16x16x32_bf16.  k may be split over
+//           workgroups, partial sums are then added in a fixed order by a second kernel.
+//   slim    at most 16 rows of A (decode): a workgroup of 8 waves owns 16 (or 2 x 16) weight
+//           rows, its waves take interleaved blocks of k and add their sums through LDS in a
+//           fixed order, so one launch does the whole product and its epilogue.
+//
+// The "gated" epilogue serves SwiGLU: the weight is [gate; up] interleaved in groups of 16 rows
+// (16 gate rows, the 16 up rows of the same outputs, and so on), and the output column c of a
+// pair of groups is silu(gate_c) * up_c, stored as bfloat16: the stacked product never reaches
+// memory.
 //
 // Requirements (checked on the host): K a multiple of 8, rows of A and W 16-byte aligned.  The
 // output is float32 (stored or added onto what is there) or bfloat16 (stored).
@@ -20,7 +28,9 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-enum Epilogue : int { EPI_STORE_F32 = 0, EPI_ADD_F32 = 1, EPI_STORE_BF16 = 2 };
+enum Epilogue : int { EPI_STORE_F32 = 0, EPI_ADD_F32 = 1, EPI_STORE_BF16 = 2, EPI_GATED_BF16 = 3 };
+
+__device__ __forceinline__ float silu_gate(float g, float u) { return (g * (1.0f / (1.0f + expf(-g)))) * u; }
 
 __device__ __forceinline__ uint4 load16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
@@ -111,7 +121,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
             for (int v = 0; v < 16; ++v) {
                 const int m = m0 + wm + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3);
                 const int n = n0 + wn + j * 32 + (lane & 31);
-                if (m < M && n < N) write_out<EPI>(C, (size_t)m * ldc + n, acc[i][j][v]);
+                if constexpr (EPI == EPI_GATED_BF16) {
+                    // columns 32b .. 32b+15 are gates, 32b+16 .. 32b+31 the ups of outputs 16b .. 16b+15
+                    const float up = __shfl_xor(acc[i][j][v], 16, 64);
+                    if ((lane & 16) == 0 && m < M && n < N)
+                        ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(silu_gate(acc[i][j][v], up));
+                } else {
+                    if (m < M && n < N) write_out<EPI>(C, (size_t)m * ldc + n, acc[i][j][v]);
+                }
             }
 }
 
@@ -191,6 +208,76 @@ __global__ void skinny_reduce_kernel(const float* __restrict__ P, void* __restri
     write_out<EPI>(C, (i / N) * ldc + (i % N), s);
 }
 
+// ------------------------------------------------------------------------------------------- slim
+// At most 16 rows of A.  Workgroup: 8 waves = STRIPS strips of 16 weight rows x (8 / STRIPS) slices
+// of k; slice s takes the 128-wide blocks of k numbered s, s + slices, ...  Both operands go from
+// global memory straight into registers (the activations are few and stay in cache); lane
+// (r = lane%16, q = lane/16) holds 64 contiguous bytes of weight row r and of activation row r per
+// block.  The slices' sums meet in LDS and are added in slice order.
+template <int STRIPS, int EPI>
+__global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
+                                                            int M, int N, int K, long lda, long ldw, long ldc) {
+    constexpr int SLICES = 8 / STRIPS;
+    __shared__ float red[8][64][4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int strip = wave % STRIPS, slice = wave / STRIPS;
+    const int r = lane & 15, q = lane >> 4;
+    const int n = (blockIdx.x * STRIPS + strip) * 16 + r;
+    const bf16_t* wrow = W + (size_t)min(n, N - 1) * ldw + 32 * q;
+    const bf16_t* xrow = A + (size_t)min(r, M - 1) * lda + 32 * q;
+    const bool x_ok = r < M;
+
+    floatx4 acc = floatx4{};
+    uint4 w_cur[4], x_cur[4], w_nxt[4], x_nxt[4];
+    auto fetch = [&](int k0, uint4* w, uint4* x) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool in = k0 + 32 * q + 8 * j < K;
+            w[j] = in ? load16(wrow + k0 + 8 * j) : uint4{0, 0, 0, 0};
+            x[j] = (in && x_ok) ? load16(xrow + k0 + 8 * j) : uint4{0, 0, 0, 0};
+        }
+    };
+    int k0 = slice * SK;
+    if (k0 < K) fetch(k0, w_cur, x_cur);
+    for (; k0 < K; k0 += SLICES * SK) {
+        const int k1 = k0 + SLICES * SK;
+        if (k1 < K) fetch(k1, w_nxt, x_nxt);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x_cur[j]), as_bf16x8(w_cur[j]), acc, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            w_cur[j] = w_nxt[j];
+            x_cur[j] = x_nxt[j];
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave][lane][v] = acc[v];
+    __syncthreads();
+    // Element v of a lane's result: activation row 4*q + v, weight row r of the strip.
+    if (tid < 256 * (EPI == EPI_GATED_BF16 ? 1 : STRIPS)) {
+        const int st = tid >> 8, e = tid & 255, m = e >> 4, c = e & 15;
+        const int src_lane = c + 16 * (m >> 2), v = m & 3;
+        if (m < M) {
+            if constexpr (EPI == EPI_GATED_BF16) {
+                float gate = 0.f, up = 0.f;
+#pragma unroll
+                for (int s = 0; s < SLICES; ++s) {
+                    gate += red[s * STRIPS + 0][src_lane][v];
+                    up += red[s * STRIPS + 1][src_lane][v];
+                }
+                const int col = blockIdx.x * 16 + c;
+                if (col * 2 < N) ((bf16_t*)C)[(size_t)m * ldc + col] = f32_to_bf16(silu_gate(gate, up));
+            } else {
+                float sum = 0.f;
+#pragma unroll
+                for (int s = 0; s < SLICES; ++s) sum += red[s * STRIPS + st][src_lane][v];
+                const int col = (blockIdx.x * STRIPS + st) * 16 + c;
+                if (col < N) write_out<EPI>(C, (size_t)m * ldc + col, sum);
+            }
+        }
+    }
+}
+
 int epilogue_of(int c_dtype, int accumulate) {
     if (c_dtype == GI_F32) return accumulate ? EPI_ADD_F32 : EPI_STORE_F32;
     if (c_dtype == GI_BF16 && !accumulate) return EPI_STORE_BF16;
@@ -208,16 +295,36 @@ GI_API int gi_gemm_bf16_skinny_splits(int N, int K) {
     return splits;
 }
 
-GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int accumulate, int M, int N, int K, long lda, long ldw,
-                        long ldc, float* scratch, long scratch_floats, hipStream_t stream) {
+// `gated` != 0: W is [gate; up] interleaved in groups of 16 rows (N rows in all, a multiple of 32)
+// and C is bfloat16 [M, N/2] = silu(gate) * up.
+GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int accumulate, int gated, int M, int N, int K, long lda,
+                        long ldw, long ldc, float* scratch, long scratch_floats, hipStream_t stream) {
     GI_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: M %d, N %d, K %d must be positive", M, N, K);
     GI_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_bf16: K %d and the row strides (%ld, %ld) must be multiples of 8", K, lda, ldw);
     GI_REQUIRE(((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_bf16: operands must be 16-byte aligned");
-    GI_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm_bf16: leading dimensions too small");
-    const int epi = epilogue_of(c_dtype, accumulate);
+    GI_REQUIRE(lda >= K && ldw >= K && ldc >= (gated ? N / 2 : N), "gemm_bf16: leading dimensions too small");
+    int epi = epilogue_of(c_dtype, accumulate);
+    if (gated) {
+        GI_REQUIRE(N % 32 == 0 && c_dtype == GI_BF16 && !accumulate, "gemm_bf16: the gated product needs N %% 32 == 0 and a bfloat16 output");
+        epi = EPI_GATED_BF16;
+    }
     GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
 
-    if (M <= 64) {
+    if (M <= 16) {
+#define SLIM(STRIPS_, EPI_) gemm_bf16_slim_kernel<STRIPS_, EPI_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
+        if (epi == EPI_GATED_BF16) {
+            dim3 grid(N / 32);
+            SLIM(2, EPI_GATED_BF16);
+        } else {
+            dim3 grid((N + 15) / 16);
+            if (epi == EPI_STORE_F32) SLIM(1, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, EPI_ADD_F32); else SLIM(1, EPI_STORE_BF16);
+        }
+#undef SLIM
+        GI_CHECK_LAUNCH("gemm_bf16 (slim)");
+        return 0;
+    }
+
+    if (M <= 64 && !gated) {
         const int splits = gi_gemm_bf16_skinny_splits(N, K);
         GI_REQUIRE(scratch != nullptr && scratch_floats >= (long)splits * M * N, "gemm_bf16: scratch of %ld floats needed, %ld given",
                    (long)splits * M * N, scratch_floats);
@@ -241,10 +348,12 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
 #define TILED(BM_, EPI_) gemm_bf16_tiled_kernel<BM_, EPI_><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
     if (M <= 64 * 8 && (long)((M + 127) / 128) * ((N + BN - 1) / BN) < 256) {       // few rows: smaller tiles fill more of the chip
         dim3 grid((N + BN - 1) / BN, (M + 63) / 64);
-        if (epi == EPI_STORE_F32) TILED(64, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(64, EPI_ADD_F32); else TILED(64, EPI_STORE_BF16);
+        if (epi == EPI_STORE_F32) TILED(64, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(64, EPI_ADD_F32);
+        else if (epi == EPI_STORE_BF16) TILED(64, EPI_STORE_BF16); else TILED(64, EPI_GATED_BF16);
     } else {
         dim3 grid((N + BN - 1) / BN, (M + 127) / 128);
-        if (epi == EPI_STORE_F32) TILED(128, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(128, EPI_ADD_F32); else TILED(128, EPI_STORE_BF16);
+        if (epi == EPI_STORE_F32) TILED(128, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(128, EPI_ADD_F32);
+        else if (epi == EPI_STORE_BF16) TILED(128, EPI_STORE_BF16); else TILED(128, EPI_GATED_BF16);
     }
 #undef TILED
     GI_CHECK_LAUNCH("gemm_bf16 (tiled)");

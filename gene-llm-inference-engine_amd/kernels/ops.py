@@ -30,7 +30,7 @@ _SIGNATURES = {
     "gi_gemm_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
                            c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
-    "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
+    "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
     "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_void_p],
     "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long,
@@ -301,21 +301,29 @@ def gemm_bf16_supports(a, w, out) -> bool:
             and (out.dtype == torch.float32 or out.dtype == torch.bfloat16) and out.stride(1) == 1)
 
 
-def gemm_bf16(a, w, out, accumulate=False):
-    """out (=|+=) a @ w.T with bfloat16 operands on the matrix cores, float32 sums."""
+def gemm_bf16(a, w, out, accumulate=False, gated=False):
+    """out (=|+=) a @ w.T with bfloat16 operands on the matrix cores, float32 sums.
+    gated: w is [gate; up] interleaved in groups of 16 rows and out = silu(a @ gate.T) * (a @ up.T), bfloat16 [m, n/2]."""
     _dev(a, w, out)
     m, k = a.shape
     n = w.shape[0]
     _need(w.shape == (n, k), f"gemm: weight is {tuple(w.shape)}, activations are {tuple(a.shape)}")
-    _need(out.shape == (m, n), f"gemm: out is {tuple(out.shape)}, ({m}, {n}) is needed")
+    _need(out.shape == (m, n // 2 if gated else n), f"gemm: out is {tuple(out.shape)}, ({m}, {n // 2 if gated else n}) is needed")
     _need(gemm_bf16_supports(a, w, out), "gemm_bf16: operands must be bfloat16 with K and row strides multiples of 8, 16-byte aligned")
     scratch, n_scratch = None, 0
-    if m <= 64:
+    if 16 < m <= 64 and not gated:
         n_scratch = lib().gi_gemm_bf16_skinny_splits(n, k) * m * n
         scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device)
-    _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, m, n, k,
-          a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _stream())
+    _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,
+          m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _stream())
     return out
+
+
+def interleave_gate_up(gate, up):
+    """[gate; up] in groups of 16 rows: 16 gate rows, the 16 up rows of the same outputs, and so on."""
+    i, d = gate.shape
+    _need(i % 16 == 0 and up.shape == gate.shape, "interleave_gate_up: the intermediate size must be a multiple of 16")
+    return torch.stack([gate.view(i // 16, 16, d), up.view(i // 16, 16, d)], dim=1).reshape(2 * i, d).contiguous()
 
 
 def argmax(logits, out):

@@ -14,10 +14,14 @@ from .linear import activation_dtype_for, linear
 class SwiGlu(FeedForward):
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
-        self.w_gate_up = torch.cat([tensors[spec.gate_proj], tensors[spec.up_proj]], dim=0).contiguous()
+        gate, up = tensors[spec.gate_proj], tensors[spec.up_proj]
         self.w_down = tensors[spec.down_proj]
-        self.in_dtype = activation_dtype_for(self.w_gate_up, dtype)
+        self.in_dtype = activation_dtype_for(gate, dtype)
         self.mid_dtype = activation_dtype_for(self.w_down, dtype)
+        # bfloat16 throughout: the gate is applied inside the product (weights interleaved for it)
+        self.fused = (self.in_dtype == torch.bfloat16 and self.mid_dtype == torch.bfloat16 and up.dtype == torch.bfloat16
+                      and spec.intermediate_size % 16 == 0 and spec.hidden_size % 8 == 0)
+        self.w_gate_up = ops.interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], dim=0).contiguous()
 
     @classmethod
     def tensor_needs(cls, spec):
@@ -26,6 +30,11 @@ class SwiGlu(FeedForward):
 
     def forward(self, h, residual, ctx):
         T, inter = ctx.n_rows, self.spec.intermediate_size
+        if self.fused:
+            mid = torch.empty((T, inter), dtype=torch.bfloat16, device=ctx.device)
+            ops.gemm_bf16(h, self.w_gate_up, mid, gated=True)
+            linear(mid, self.w_down, residual, accumulate=True)
+            return
         gate_up = torch.empty((T, 2 * inter), dtype=torch.float32, device=ctx.device)
         linear(h, self.w_gate_up, gate_up)
         mid = torch.empty((T, inter), dtype=self.mid_dtype, device=ctx.device)

@@ -65,6 +65,18 @@ def test_gemm_bf16(m, n, k, out_dtype, accumulate):
     assert torch.equal(out[:, n:], base[:, n:])
 
 
+@pytest.mark.parametrize("m,inter,k", [(1, 16, 8), (5, 48, 136), (16, 160, 96), (17, 176, 64), (64, 32, 264), (70, 192, 128), (300, 8192 // 16, 2048 // 8)])
+def test_gemm_bf16_gated(m, inter, k):
+    a = randn(m, k, dtype=torch.bfloat16, seed=15)
+    gate, up = randn(inter, k, dtype=torch.bfloat16, seed=16, scale=0.3), randn(inter, k, dtype=torch.bfloat16, seed=17, scale=0.3)
+    w = ops().interleave_gate_up(gate, up)
+    out = torch.full((m, inter + 2), 3.0, dtype=torch.bfloat16, device=DEV)
+    ops().gemm_bf16(a, w, out[:, :inter], gated=True)
+    want = torch.nn.functional.silu(a.double() @ gate.double().T) * (a.double() @ up.double().T)
+    assert rel(out[:, :inter], want) < 6e-3
+    assert torch.all(out[:, inter:] == 3.0)
+
+
 def test_gemm_bf16_refuses_what_it_cannot_do():
     o = ops()
     a, w = randn(4, 12, dtype=torch.bfloat16), randn(6, 12, dtype=torch.bfloat16)
