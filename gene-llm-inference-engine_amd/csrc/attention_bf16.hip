@@ -173,7 +173,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
                                                              const int* __restrict__ pos, const int* __restrict__ slots,
                                                              const int* __restrict__ table, int table_stride, long page_stride,
                                                              int page_size, int n_heads, int n_kv, int window, float scale,
-                                                             int n_splits, int split_len) {
+                                                             int n_splits) {
     constexpr int KSTEPS = HD / 32, DT = HD / 16;
     const int group = n_heads / n_kv, hg_per_kv = (group + 15) / 16;
     const int row = rows[blockIdx.x], g = blockIdx.y / hg_per_kv, hg = blockIdx.y % hg_per_kv, split = blockIdx.z;
@@ -184,7 +184,10 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
     const int my_pos = pos[row];
     const int lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
     const int* tab = table + (size_t)slots[row] * table_stride;
-    const int begin = (lo & ~31) + split * split_len, end = min(my_pos + 1, begin + split_len);     // split_len is a multiple of 32
+    // every row cuts its own range into n_splits pieces (multiples of 32); short rows leave later pieces empty
+    const int span = my_pos + 1 - (lo & ~31);
+    const int split_len = (((span + n_splits - 1) / n_splits) + 31) & ~31;
+    const int begin = (lo & ~31) + split * split_len, end = min(my_pos + 1, begin + split_len);
 
     bf16x8 qreg[KSTEPS];
 #pragma unroll
@@ -201,18 +204,39 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
     const bf16_t* kbase = cache + (long)g * page_size * HD;
     const bf16_t* vbase = cache + v_plane + (long)g * HD * page_size;
 
-    for (int kv0 = begin; kv0 < end; kv0 += 32) {
-        // scores of 32 key positions: two products of 16; an address beyond the row's own range is
-        // clamped into it (its score is masked below)
-        floatx4 s[2];
+    // Loads run ahead of the products: the keys of the next 32 positions and the values of these 32
+    // are requested before the scores of these 32 are taken.  An address beyond the row's own range
+    // is clamped into it; what it brings is masked below.
+    uint4 k_cur[2][KSTEPS], k_nxt[2][KSTEPS];
+    auto load_keys = [&](int kv0, uint4 (&dst)[2][KSTEPS]) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int kv = min(max(kv0 + 16 * t + r, lo), my_pos);
-            const bf16_t* krow = kbase + (long)tab[kv / page_size] * page_stride + (long)(kv % page_size) * HD;
+            const bf16_t* krow = kbase + (long)tab[kv / page_size] * page_stride + (long)(kv % page_size) * HD + 8 * q4;
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) dst[t][ks] = load16(krow + 32 * ks);
+        }
+    };
+    if (begin < end) load_keys(begin, k_cur);
+    for (int kv0 = begin; kv0 < end; kv0 += 32) {
+        // slot e of this lane in the value product is key position kv0 + 16*(e/4) + 4*q4 + e%4
+        const int kva = min(max(kv0 + 4 * q4, lo & ~3), my_pos & ~3), kvb = min(max(kv0 + 16 + 4 * q4, lo & ~3), my_pos & ~3);
+        const bf16_t* va = vbase + (long)tab[kva / page_size] * page_stride + kva % page_size + (long)r * page_size;
+        const bf16_t* vb = vbase + (long)tab[kvb / page_size] * page_stride + kvb % page_size + (long)r * page_size;
+        uint2 vx[DT], vy[DT];
+#pragma unroll
+        for (int i = 0; i < DT; ++i) {
+            vx[i] = load8(va + (long)(16 * i) * page_size);
+            vy[i] = load8(vb + (long)(16 * i) * page_size);
+        }
+        if (kv0 + 32 < end) load_keys(kv0 + 32, k_nxt);
+
+        floatx4 s[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
             s[t] = floatx4{};
 #pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks)
-                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(load16(krow + 32 * ks + 8 * q4)), qreg[ks], s[t], 0, 0, 0);
+            for (int ks = 0; ks < KSTEPS; ++ks) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(k_cur[t][ks]), qreg[ks], s[t], 0, 0, 0);
         }
         // element v of s[t]: key position kv0 + 16*t + 4*q4 + v, query head r
         float mx = -INFINITY;
@@ -241,18 +265,17 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
         sum += __shfl_xor(sum, 32, 64);
         l = l * corr + sum;
         m = m_new;
-        // slot e of this lane is key position kv0 + 16*(e/4) + 4*q4 + e%4
         const uint4 pb = {pack2(s[0][0], s[0][1]), pack2(s[0][2], s[0][3]), pack2(s[1][0], s[1][1]), pack2(s[1][2], s[1][3])};
-        const int kva = min(max(kv0 + 4 * q4, lo & ~3), my_pos & ~3), kvb = min(max(kv0 + 16 + 4 * q4, lo & ~3), my_pos & ~3);
-        const bf16_t* va = vbase + (long)tab[kva / page_size] * page_stride + kva % page_size;
-        const bf16_t* vb = vbase + (long)tab[kvb / page_size] * page_stride + kvb % page_size;
 #pragma unroll
         for (int i = 0; i < DT; ++i) {
-            const uint2 x = load8(va + (long)(16 * i + r) * page_size), y = load8(vb + (long)(16 * i + r) * page_size);
 #pragma unroll
             for (int v = 0; v < 4; ++v) o[i][v] *= corr;
-            o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(uint4{x.x, x.y, y.x, y.y}), as_bf16x8(pb), o[i], 0, 0, 0);
+            o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(uint4{vx[i].x, vx[i].y, vy[i].x, vy[i].y}), as_bf16x8(pb), o[i], 0, 0, 0);
         }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) k_cur[t][ks] = k_nxt[t][ks];
     }
     if (!head_ok) return;
     // part[row_index][head][split] = {m, l, O[HD]}; element v of o[i]: channel 16*i + 4*q4 + v, query head r
@@ -267,25 +290,44 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
         for (int v = 0; v < 4; ++v) dst[2 + 16 * i + 4 * q4 + v] = o[i][v];
 }
 
-// Merges the splits of one (row, head) in split order: out = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s.
-__global__ void attention_decode_combine_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, const int* __restrict__ rows,
-                                                int n_heads, int hd, int n_splits) {
-    const int idx = blockIdx.x, head = blockIdx.y;
+// Merges the splits of one (row, head): out = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s, the sums
+// taken in split order.  One wave: lane s first fetches split s's {m, l} (all splits at once), then
+// lane d adds channel d over the splits with the weights read from LDS.
+constexpr int MAX_SPLITS = 256;
+
+__global__ __launch_bounds__(64) void attention_decode_combine_kernel(const float* __restrict__ part, bf16_t* __restrict__ out,
+                                                                     const int* __restrict__ rows, int n_heads, int hd, int n_splits) {
+    __shared__ float weight[MAX_SPLITS], weighted_l[MAX_SPLITS];
+    const int idx = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const float* src = part + ((size_t)idx * n_heads + head) * n_splits * (hd + 2);
+    float mine_m[MAX_SPLITS / 64], mine_l[MAX_SPLITS / 64];
     float big = -INFINITY;
-    for (int s = 0; s < n_splits; ++s) big = fmaxf(big, src[(size_t)s * (hd + 2)]);
-    float denom = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-        const float ms = src[(size_t)s * (hd + 2)];
-        if (ms != -INFINITY) denom += expf(ms - big) * src[(size_t)s * (hd + 2) + 1];
+#pragma unroll
+    for (int i = 0; i < MAX_SPLITS / 64; ++i) {
+        const int s = lane + 64 * i;
+        mine_m[i] = s < n_splits ? src[(size_t)s * (hd + 2)] : -INFINITY;
+        mine_l[i] = s < n_splits ? src[(size_t)s * (hd + 2) + 1] : 0.f;
+        big = fmaxf(big, mine_m[i]);
     }
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-        float acc = 0.f;
-        for (int s = 0; s < n_splits; ++s) {
-            const float ms = src[(size_t)s * (hd + 2)];
-            if (ms != -INFINITY) acc += expf(ms - big) * src[(size_t)s * (hd + 2) + 2 + d];
+    big = wave_max(big);
+#pragma unroll
+    for (int i = 0; i < MAX_SPLITS / 64; ++i) {
+        const int s = lane + 64 * i;
+        if (s < n_splits) {
+            const float w = (mine_m[i] == -INFINITY) ? 0.f : expf(mine_m[i] - big);
+            weight[s] = w;
+            weighted_l[s] = w * mine_l[i];
         }
-        out[((size_t)rows[idx] * n_heads + head) * hd + d] = f32_to_bf16(acc / denom);
+    }
+    __syncthreads();
+    float denom = 0.f;
+    for (int s = 0; s < n_splits; ++s) denom += weighted_l[s];
+    const float inv = 1.0f / denom;
+    for (int d = lane; d < hd; d += 64) {
+        float acc = 0.f;
+#pragma unroll 8
+        for (int s = 0; s < n_splits; ++s) acc = fmaf(weight[s], src[(size_t)s * (hd + 2) + 2 + d], acc);
+        out[((size_t)rows[idx] * n_heads + head) * hd + d] = f32_to_bf16(acc * inv);
     }
 }
 
@@ -316,19 +358,18 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
 
 GI_API int gi_attention_decode_bf16(const void* q, const void* cache, void* out, float* part, long part_floats, const int* rows, int n_rows,
                                     const int* pos, const int* slots, const int* table, int table_stride, long page_stride, int page_size,
-                                    int n_heads, int n_kv, int hd, int window, float scale, int n_splits, int split_len,
-                                    hipStream_t stream) {
+                                    int n_heads, int n_kv, int hd, int window, float scale, int n_splits, hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_decode: bad counts (%d rows, %d heads, %d kv heads)",
                n_rows, n_heads, n_kv);
     GI_REQUIRE(gi_attention_bf16_supports(hd, page_size, 0), "attention_decode: head size %d with page size %d is not supported", hd, page_size);
     GI_REQUIRE(page_stride >= 2L * n_kv * page_size * hd && page_stride % 8 == 0, "attention_decode: bad page stride %ld", page_stride);
-    GI_REQUIRE(n_splits >= 1 && n_splits <= 65535 && split_len > 0 && split_len % 32 == 0, "attention_decode: bad split (%d of %d)", n_splits, split_len);
+    GI_REQUIRE(n_splits >= 1 && n_splits <= MAX_SPLITS, "attention_decode: the number of splits %d is outside 1..%d", n_splits, MAX_SPLITS);
     GI_REQUIRE(part != nullptr && part_floats >= (long)n_rows * n_heads * n_splits * (hd + 2), "attention_decode: scratch too small");
     const int hg = (n_heads / n_kv + 15) / 16;
     GI_REQUIRE(n_kv * hg <= 65535, "attention_decode: too many heads");
     dim3 grid(n_rows, n_kv * hg, n_splits);
 #define GO(HD) attention_decode_kernel<HD><<<grid, 64, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, part, rows, pos, slots, table, \
-                                                                   table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits, split_len)
+                                                                   table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits)
     if (hd == 32) GO(32); else if (hd == 64) GO(64); else if (hd == 96) GO(96); else if (hd == 128) GO(128); else GO(256);
 #undef GO
     GI_CHECK_LAUNCH("attention_decode");

@@ -209,45 +209,46 @@ __global__ void skinny_reduce_kernel(const float* __restrict__ P, void* __restri
 }
 
 // ------------------------------------------------------------------------------------------- slim
-// At most 16 rows of A.  Workgroup: 8 waves = STRIPS strips of 16 weight rows x (8 / STRIPS) slices
-// of k; slice s takes the 128-wide blocks of k numbered s, s + slices, ...  Both operands go from
-// global memory straight into registers (the activations are few and stay in cache); lane
-// (r = lane%16, q = lane/16) holds 64 contiguous bytes of weight row r and of activation row r per
-// block.  The slices' sums meet in LDS and are added in slice order.
-template <int STRIPS, int EPI>
+// At most 16 rows of A.  Workgroup: 8 waves = STRIPS strips of ROWS weight rows x (8 / STRIPS)
+// slices of k; slice s takes the 128-wide blocks of k numbered s, s + slices, ...  Both operands go
+// from global memory straight into registers (the activations are few and stay in cache): for the
+// j-th product of a block, lane (r = lane%16, q = lane/16) holds k0 + 32j + 8q .. +8 of weight row r
+// and of activation row r, so the four lanes of a row read 64 contiguous bytes per load.  Loads run
+// two blocks ahead of the products.  The slices' sums meet in LDS and are added in slice order.
+// ROWS = 8 leaves half of each product idle and doubles the number of workgroups for narrow outputs.
+template <int STRIPS, int ROWS, int EPI>
 __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
                                                             int M, int N, int K, long lda, long ldw, long ldc) {
-    constexpr int SLICES = 8 / STRIPS;
+    constexpr int SLICES = 8 / STRIPS, STEP = SLICES * SK, DEPTH = 3;
     __shared__ float red[8][64][4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int strip = wave % STRIPS, slice = wave / STRIPS;
     const int r = lane & 15, q = lane >> 4;
-    const int n = (blockIdx.x * STRIPS + strip) * 16 + r;
-    const bf16_t* wrow = W + (size_t)min(n, N - 1) * ldw + 32 * q;
-    const bf16_t* xrow = A + (size_t)min(r, M - 1) * lda + 32 * q;
-    const bool x_ok = r < M;
+    const int n = (blockIdx.x * STRIPS + strip) * ROWS + r;
+    const bool w_ok = r < ROWS && n < N, x_ok = r < M;
+    const bf16_t* wrow = W + (size_t)(w_ok ? n : 0) * ldw + 8 * q;
+    const bf16_t* xrow = A + (size_t)(x_ok ? r : 0) * lda + 8 * q;
 
     floatx4 acc = floatx4{};
-    uint4 w_cur[4], x_cur[4], w_nxt[4], x_nxt[4];
+    uint4 w_buf[DEPTH][4], x_buf[DEPTH][4];
     auto fetch = [&](int k0, uint4* w, uint4* x) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const bool in = k0 + 32 * q + 8 * j < K;
-            w[j] = in ? load16(wrow + k0 + 8 * j) : uint4{0, 0, 0, 0};
-            x[j] = (in && x_ok) ? load16(xrow + k0 + 8 * j) : uint4{0, 0, 0, 0};
+            const bool in = k0 + 32 * j + 8 * q < K;
+            w[j] = (in && w_ok) ? load16(wrow + k0 + 32 * j) : uint4{0, 0, 0, 0};
+            x[j] = (in && x_ok) ? load16(xrow + k0 + 32 * j) : uint4{0, 0, 0, 0};
         }
     };
-    int k0 = slice * SK;
-    if (k0 < K) fetch(k0, w_cur, x_cur);
-    for (; k0 < K; k0 += SLICES * SK) {
-        const int k1 = k0 + SLICES * SK;
-        if (k1 < K) fetch(k1, w_nxt, x_nxt);
+    const int k_first = slice * SK;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x_cur[j]), as_bf16x8(w_cur[j]), acc, 0, 0, 0);
+    for (int d = 0; d < DEPTH - 1; ++d) fetch(k_first + d * STEP, w_buf[d], x_buf[d]);      // beyond K: zeros, no loads
+    for (int k0 = k_first; k0 < K; k0 += DEPTH * STEP) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            w_cur[j] = w_nxt[j];
-            x_cur[j] = x_nxt[j];
+        for (int d = 0; d < DEPTH; ++d) {                     // buffer d holds block k0 + d*STEP
+            fetch(k0 + (d + DEPTH - 1) * STEP, w_buf[(d + DEPTH - 1) % DEPTH], x_buf[(d + DEPTH - 1) % DEPTH]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x_buf[d][j]), as_bf16x8(w_buf[d][j]), acc, 0, 0, 0);
         }
     }
 #pragma unroll
@@ -257,7 +258,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
     if (tid < 256 * (EPI == EPI_GATED_BF16 ? 1 : STRIPS)) {
         const int st = tid >> 8, e = tid & 255, m = e >> 4, c = e & 15;
         const int src_lane = c + 16 * (m >> 2), v = m & 3;
-        if (m < M) {
+        if (m < M && c < ROWS) {
             if constexpr (EPI == EPI_GATED_BF16) {
                 float gate = 0.f, up = 0.f;
 #pragma unroll
@@ -265,13 +266,12 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
                     gate += red[s * STRIPS + 0][src_lane][v];
                     up += red[s * STRIPS + 1][src_lane][v];
                 }
-                const int col = blockIdx.x * 16 + c;
-                if (col * 2 < N) ((bf16_t*)C)[(size_t)m * ldc + col] = f32_to_bf16(silu_gate(gate, up));
+                ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 16 + c] = f32_to_bf16(silu_gate(gate, up));
             } else {
                 float sum = 0.f;
 #pragma unroll
                 for (int s = 0; s < SLICES; ++s) sum += red[s * STRIPS + st][src_lane][v];
-                const int col = (blockIdx.x * STRIPS + st) * 16 + c;
+                const int col = (blockIdx.x * STRIPS + st) * ROWS + c;
                 if (col < N) write_out<EPI>(C, (size_t)m * ldc + col, sum);
             }
         }
@@ -311,13 +311,17 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
 
     if (M <= 16) {
-#define SLIM(STRIPS_, EPI_) gemm_bf16_slim_kernel<STRIPS_, EPI_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
+#define SLIM(STRIPS_, ROWS_, EPI_) \
+    gemm_bf16_slim_kernel<STRIPS_, ROWS_, EPI_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
         if (epi == EPI_GATED_BF16) {
             dim3 grid(N / 32);
-            SLIM(2, EPI_GATED_BF16);
-        } else {
+            SLIM(2, 16, EPI_GATED_BF16);
+        } else if ((N + 15) / 16 >= 256) {
             dim3 grid((N + 15) / 16);
-            if (epi == EPI_STORE_F32) SLIM(1, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, EPI_ADD_F32); else SLIM(1, EPI_STORE_BF16);
+            if (epi == EPI_STORE_F32) SLIM(1, 16, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 16, EPI_ADD_F32); else SLIM(1, 16, EPI_STORE_BF16);
+        } else {                                   // a narrow output: strips of 8 rows, twice the workgroups
+            dim3 grid((N + 7) / 8);
+            if (epi == EPI_STORE_F32) SLIM(1, 8, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 8, EPI_ADD_F32); else SLIM(1, 8, EPI_STORE_BF16);
         }
 #undef SLIM
         GI_CHECK_LAUNCH("gemm_bf16 (slim)");

@@ -56,10 +56,11 @@ class Runner:
     max_requests live requests (request slots)
     max_rows     most rows one step may hold
     max_positions longest request; defaults to the model's limit
+    use_graphs   replay decode steps (one token per request, all logits wanted) from captured HIP graphs
     """
 
     def __init__(self, model: DecoderModel, *, page_size: int = 16, max_tokens: int = 4096, max_requests: int = 8,
-                 max_rows: int = 4096, max_positions: Optional[int] = None):
+                 max_rows: int = 4096, max_positions: Optional[int] = None, use_graphs: bool = True):
         self.model = model
         self.page_size = int(page_size)
         self.max_rows = int(max_rows)
@@ -70,6 +71,8 @@ class Runner:
                                   max_positions=self.max_positions, dtype=model.dtype, device=model.device)
         self._view = _CacheView(self.cache, needs, reads_from)
         self.steps_run = 0
+        self.use_graphs = bool(use_graphs)
+        self._graphs = {}
 
     # -------------------------------------------------------------------------------- requests
     def open(self, request: Hashable) -> None:
@@ -112,12 +115,12 @@ class Runner:
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Runs the batch; returns float32 logits [wanted, vocab] on the device in the order of the
-        entries and of each entry's `want`, or None if nothing was wanted."""
+        entries and of each entry's `want`, or None if nothing was wanted.  The tensor is valid
+        until the next step."""
         n_rows = self._validate(entries)
         self.cache.reserve([(e.request, len(e.tokens)) for e in entries])       # OutOfPages: nothing changed
         self.cache.sync()
 
-        dev = self.model.device
         meta = np.empty((3, n_rows), dtype=np.int32)                            # tokens, positions, slots
         seg_slot, seg_start, seg_len, seg_pos0, logit_rows = [], [], [], [], []
         row = 0
@@ -129,12 +132,67 @@ class Runner:
             seg_slot.append(slot); seg_start.append(row); seg_len.append(n); seg_pos0.append(pos0)
             logit_rows += [row + int(w) for w in e.want]
             row += n
-        meta_dev = torch.from_numpy(meta).to(dev)
-        rows_dev = torch.tensor(logit_rows, dtype=torch.int32).to(dev) if logit_rows else None
-        ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
-                          row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0)
-        logits = self.model.forward(ctx, self._view, rows_dev, len(logit_rows))
+
+        if self.use_graphs and n_rows == len(entries) and logit_rows == list(range(n_rows)):
+            logits = self._decode_step(meta, seg_slot, seg_pos0)
+        else:
+            dev = self.model.device
+            meta_dev = torch.from_numpy(meta).to(dev)
+            rows_dev = torch.tensor(logit_rows, dtype=torch.int32).to(dev) if logit_rows else None
+            ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
+                              row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0)
+            logits = self.model.forward(ctx, self._view, rows_dev, len(logit_rows))
         for e in entries:
             self.cache.advance(e.request, len(e.tokens))
         self.steps_run += 1
         return logits
+
+    # --------------------------------------------------------------------------- captured decode
+    def _decode_step(self, meta: np.ndarray, seg_slot, seg_pos0) -> torch.Tensor:
+        """A step in which every request brings one token and wants its logits runs as a replay of a
+        HIP graph captured once per batch size: the launches of the whole pass cost one call.  The
+        graph reads tokens, positions and slots from fixed device buffers that are filled before
+        every replay; nothing else in it depends on the step."""
+        batch = meta.shape[1]
+        g = self._graphs.get(batch)
+        if g is None:
+            g = self._graphs[batch] = _DecodeGraph(self, batch)
+        return g.run(meta, seg_slot, seg_pos0)
+
+
+class _DecodeGraph:
+    def __init__(self, runner: Runner, batch: int):
+        from ..kernels.ops import AttentionPlan
+        self.runner, self.batch = runner, batch
+        dev = runner.model.device
+        self.meta = torch.zeros((3, batch), dtype=torch.int32, device=dev)
+        self.staging = torch.zeros((3, batch), dtype=torch.int32).pin_memory()
+        self.logit_rows = torch.arange(batch, dtype=torch.int32, device=dev)
+        self.plan = AttentionPlan.all_decode(batch, runner.max_positions, dev)
+        self.graph = None
+        self.logits = None
+        self.calls = 0
+
+    def _context(self, seg_slot, seg_pos0) -> StepContext:
+        m, b = self.runner.model, self.batch
+        ctx = StepContext(n_rows=b, dtype=m.dtype, device=m.device, tokens=self.meta[0], row_pos=self.meta[1], row_slot=self.meta[2],
+                          seg_slot=list(seg_slot), seg_start=list(range(b)), seg_len=[1] * b, seg_pos0=list(seg_pos0))
+        ctx.memo["attention_plan"] = self.plan
+        return ctx
+
+    def run(self, meta: np.ndarray, seg_slot, seg_pos0) -> torch.Tensor:
+        self.staging.numpy()[:] = meta
+        self.meta.copy_(self.staging, non_blocking=True)
+        r = self.runner
+        self.calls += 1
+        if self.graph is None:
+            if self.calls < 2:          # the first step of a batch size runs as it is; a size that comes again is captured
+                return r.model.forward(self._context(seg_slot, seg_pos0), r._view, self.logit_rows, self.batch)
+            # Capturing records the launches without running them, so this step runs once more below, by replay.
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self.logits = r.model.forward(self._context(seg_slot, seg_pos0), r._view, self.logit_rows, self.batch)
+            self.graph = graph
+        self.graph.replay()
+        return self.logits

@@ -34,7 +34,7 @@ _SIGNATURES = {
     "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_void_p],
     "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long,
-                                 c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
+                                 c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     "gi_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
 }
@@ -230,6 +230,15 @@ class AttentionPlan:
     the prompt kernel.  Made once per step and used by every layer."""
     TILE = 128
 
+    @classmethod
+    def all_decode(cls, n_rows, max_context, device):
+        """Every row is a request's single new row (what a captured decode step uses: nothing in it depends on the step)."""
+        plan = cls.__new__(cls)
+        plan.n_decode, plan.n_tiles, plan.max_decode_context = n_rows, 0, max_context
+        plan.decode_rows = torch.arange(n_rows, dtype=torch.int32, device=device)
+        plan.tiles = plan.decode_rows[:0]
+        return plan
+
     def __init__(self, seg_start, seg_len, seg_pos0, seg_slot, device):
         dec, tiles, self.max_decode_context = [], [], 0
         for start, n, pos0, slot in zip(seg_start, seg_len, seg_pos0, seg_slot):
@@ -270,14 +279,12 @@ def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, 
     if plan.n_decode:
         span = plan.max_decode_context if not window else min(plan.max_decode_context, window + 31)
         waves = plan.n_decode * n_kv * ((n_heads // n_kv + 15) // 16)
-        n_splits = max(1, min(-(-target_waves // waves), -(-span // 64)))
-        split_len = -(-(-(-span // n_splits)) // 32) * 32
-        n_splits = -(-span // split_len)
+        n_splits = max(1, min(-(-target_waves // waves), -(-span // 64), 256))
         n_part = plan.n_decode * n_heads * n_splits * (hd + 2)
         part = torch.empty(n_part, dtype=torch.float32, device=q.device)
         _call("gi_attention_decode_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), part.data_ptr(), n_part,
               plan.decode_rows.data_ptr(), plan.n_decode, positions.data_ptr(), slots.data_ptr(), table.data_ptr(), table.stride(0),
-              cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits, split_len, _stream())
+              cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits, _stream())
     return out
 
 
