@@ -71,7 +71,9 @@ class PageGroup:
         self.first_live[slot] = max(int(self.first_live[slot]), i)
 
     def release_all(self, slot: int) -> None:
-        for i in range(int(self.first_live[slot]), int(self.n_held[slot])):
+        # last page first, as the reference's truncate (src/model/kv_cache.cpp:100-109): the request's
+        # first page is then the next one handed out
+        for i in range(int(self.n_held[slot]) - 1, int(self.first_live[slot]) - 1, -1):
             self.pool.release(int(self.table_host[slot, i]))
         self.table_host[slot, :] = -1
         self.first_live[slot] = 0
@@ -207,11 +209,13 @@ class CacheManager:
         """The reserved positions have been written: the request is n_new longer; pages behind a
         window are given back."""
         slot = self.slot(request)
-        self._length[request] += n_new
+        new_length = self._length[request] + n_new
         for g in self.groups:
-            if self._length[request] > int(g.n_held[slot]) * g.page_size:
+            if new_length > int(g.n_held[slot]) * g.page_size:
                 raise CacheError(f"request {request!r} advanced beyond its reserved pages")
-            g.drop_behind_window(slot, self._length[request])
+        self._length[request] = new_length
+        for g in self.groups:
+            g.drop_behind_window(slot, new_length)
 
     def sync(self) -> None:
         """Brings the device copies of changed page tables up to date."""

@@ -39,8 +39,8 @@ def config_class_for(cfg: dict) -> type:
     else:
         name = _BY_MODEL_TYPE.get(cfg.get("model_type"))
     if name not in _BY_ARCHITECTURE:
-        shown = name if name is not None else f"model_type {cfg.get('model_type')!r}"
-        raise ConfigError(f"unknown architecture {shown!r}; registered: {', '.join(registered_architectures())}")
+        shown = repr(name) if name is not None else f"(model_type {cfg.get('model_type')!r}, no 'architectures')"
+        raise ConfigError(f"unknown architecture {shown}; registered: {', '.join(registered_architectures())}")
     return _BY_ARCHITECTURE[name]
 
 

@@ -28,7 +28,8 @@ class GenerateResult:
 
 def generate(runner: Runner, sampler: Sampler, prompt_tokens: Sequence[int], max_positions: int = 0,
              end_tokens: Iterable[int] = (), on_token: Optional[Callable[[int], None]] = None,
-             prefill_rows: Optional[int] = None, request="generate") -> GenerateResult:
+             prefill_rows: Optional[int] = None, request="generate", sample=None) -> GenerateResult:
+    """`sample(logits_row, sampler) -> token` replaces the sampler's own device sampling (tests without a GPU use it)."""
     prompt = [int(t) for t in prompt_tokens]
     if not prompt:
         raise ValueError("generate: prompt has no tokens")
@@ -52,7 +53,7 @@ def generate(runner: Runner, sampler: Sampler, prompt_tokens: Sequence[int], max
         token = prompt[pos] if pos < len(prompt) else None
         while pos < steps:
             logits = runner.step([StepEntry(request, [token], (0,))])
-            nxt = sampler.sample(logits[0])                  # brings the token to the host: the step has finished
+            nxt = sampler.sample(logits[0]) if sample is None else sample(logits[0], sampler)     # the token reaches the host: the step has finished
             result.generated_tokens.append(nxt)
             if len(result.generated_tokens) == 1:
                 t_first = time.perf_counter()

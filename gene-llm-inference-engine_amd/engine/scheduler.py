@@ -79,8 +79,10 @@ class _Job:
 
 
 class Engine:
-    def __init__(self, runner: Runner, config: Optional[EngineConfig] = None, end_tokens: Iterable[int] = ()):
+    def __init__(self, runner: Runner, config: Optional[EngineConfig] = None, end_tokens: Iterable[int] = (), sample=sample_rows):
+        """`sample(logits, samplers) -> tokens` draws one token per row of logits with that row's sampler."""
         cfg = config or EngineConfig()
+        self._sample = sample
         if cfg.max_running < 1:
             raise ValueError("Engine: max_running must be >= 1")
         if cfg.step_rows < 0 or cfg.prefill_chunk < 0:
@@ -194,7 +196,7 @@ class Engine:
         st.max_rows_in_pass = max(st.max_rows_in_pass, n_rows)
         st.max_chunk = max(st.max_chunk, max(n for _, n in taken))
 
-        sampled = sample_rows(logits, [j.sampler for j in wanting]) if wanting else []
+        sampled = self._sample(logits, [j.sampler for j in wanting]) if wanting else []
         next_token = {j.id: t for j, t in zip(wanting, sampled)}
         done = []
         for job, n in taken:

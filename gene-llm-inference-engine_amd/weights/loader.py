@@ -94,6 +94,7 @@ def load_tensors(folder, needs: Iterable[TensorNeed], compute_dtype: torch.dtype
     out = {}
     for name, need in wanted.items():
         src = st.tensor(name)
-        out[name] = _converted(src, st.entries[name].dtype_name, need.role, compute_dtype).to(device).contiguous()
+        t = _converted(src, st.entries[name].dtype_name, need.role, compute_dtype).to(device).contiguous()
+        out[name] = t.clone() if t.data_ptr() == src.data_ptr() else t       # never a view of the read-only mapping
     st.close()
     return out

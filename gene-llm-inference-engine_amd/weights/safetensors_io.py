@@ -108,11 +108,8 @@ class SafetensorsFile:
         return flat.reshape(e.shape)
 
     def close(self):
-        # Views handed out keep the mapping alive through the buffer protocol; closing is best effort.
-        try:
-            self._map.close()
-        except BufferError:
-            pass
+        """Closes the file.  The mapping itself lives as long as any tensor made from it (tensors keep
+        a reference to it), so it is never unmapped under a tensor."""
         self._file.close()
 
 

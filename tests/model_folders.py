@@ -64,7 +64,7 @@ def random_weights(cfg: dict, seed: int, std: float = 0.2):
     return w
 
 
-_NAMES = {torch.float32: "F32", torch.bfloat16: "BF16", torch.float16: "F16", torch.int32: "I32", torch.float64: "F64"}
+_NAMES = {torch.float32: "F32", torch.bfloat16: "BF16", torch.float16: "F16", torch.int32: "I32", torch.int64: "I64", torch.float64: "F64"}
 
 
 def write_safetensors_by_hand(path, tensors: dict, shuffle_seed=None, header_pad=0):

@@ -1,0 +1,186 @@
+"""The cache manager without a GPU: the page pool's order and errors, and the manager's books under
+random orders of requests (no page lost, held twice or freed twice), windows, groups and state slots."""
+import random
+
+import pytest
+import torch
+
+from geneinfer_amd.cache import CacheError, CacheManager, OutOfPages, PagedKvNeed, PageError, PagePool, StateNeed
+
+
+def test_pool_hands_out_page_0_first_and_the_last_freed_next():          # src/model/kv_cache.cpp:22-56, tests/verify_kvpool.py:24-45
+    pool = PagePool(4)
+    assert [pool.allocate() for _ in range(3)] == [0, 1, 2]
+    pool.release(1)
+    pool.release(0)
+    assert pool.allocate() == 0 and pool.allocate() == 1 and pool.allocate() == 3
+    with pytest.raises(OutOfPages):
+        pool.allocate()
+    assert pool.free_count == 0
+
+
+def test_pool_misuse_raises():
+    pool = PagePool(2)
+    p = pool.allocate()
+    pool.retain(p)
+    pool.release(p)
+    assert pool.ref_count(p) == 1 and pool.free_count == 1
+    pool.release(p)
+    with pytest.raises(PageError, match="already free"):
+        pool.release(p)
+    with pytest.raises(PageError, match="cannot be retained"):
+        pool.retain(p)
+    with pytest.raises(PageError, match="does not exist"):
+        pool.release(5)
+
+
+FULL = PagedKvNeed(2, 16)
+WINDOW = PagedKvNeed(2, 16, window=10)
+
+
+def manager(needs, reads=None, n_pages=12, page_size=4, max_requests=4, max_positions=64):
+    return CacheManager(needs, reads or [None] * len(needs), page_size=page_size, n_pages=n_pages, max_requests=max_requests,
+                        max_positions=max_positions, allocate_storage=False)
+
+
+def test_layers_with_equal_needs_share_a_group():
+    m = manager([FULL, WINDOW, FULL, None, StateNeed((3,)), WINDOW], [None, None, None, None, None, 1])
+    assert len(m.groups) == 2
+    assert m.groups[0].entries == [0, 2] and m.groups[1].entries == [1]       # entry 5 reads entry 1's pages
+    assert m._entry_group[5] == m._entry_group[1]
+    with pytest.raises(CacheError, match="whose need differs"):
+        manager([FULL, WINDOW], [None, 0])
+
+
+def test_reserve_is_all_or_nothing():
+    m = manager([FULL], n_pages=5)
+    m.open("a"); m.open("b")
+    m.reserve([("a", 9)])                                                      # 3 pages
+    m.advance("a", 9)
+    before = (m.free_pages(), list(m.groups[0].table_host[m.slot("b")]))
+    with pytest.raises(OutOfPages):
+        m.reserve([("a", 4), ("b", 5)])                                        # 1 + 2 pages > 2 free
+    assert (m.free_pages(), list(m.groups[0].table_host[m.slot("b")])) == before
+    m.reserve([("a", 3), ("b", 5)])                                            # 0 + 2 pages
+    m.check_consistency()
+    assert m.free_pages() == [0]
+
+
+def test_positions_map_to_pages_and_close_gives_everything_back():
+    m = manager([FULL], n_pages=6)
+    m.open("a")
+    m.reserve([("a", 5)]); m.advance("a", 5)
+    m.reserve([("a", 4)]); m.advance("a", 4)
+    g = m.groups[0]
+    assert g.held_pages(m.slot("a")) == [0, 1, 2] and m.length("a") == 9
+    m.open("b")
+    m.reserve([("b", 1)]); m.advance("b", 1)
+    m.close("a")
+    assert m.free_pages() == [5]
+    m.open("c")
+    m.reserve([("c", 8)])
+    assert g.held_pages(m.slot("c")) == [0, 1]                                 # the pages freed last are used again first
+    m.check_consistency()
+
+
+def test_window_pages_are_given_back_as_the_request_moves_on():
+    m = manager([WINDOW], n_pages=5, page_size=4)                              # window 10: at most ceil((10 + 3) / 4) + 1 pages live
+    m.open("a")
+    g, slot = m.groups[0], None
+    for step in range(40):
+        m.reserve([("a", 1)])
+        m.advance("a", 1)
+        slot = m.slot("a")
+        length = m.length("a")
+        live = g.held_pages(slot)
+        first_visible = max(0, length - 10 + 1)                                # what the next row still sees
+        assert int(g.first_live[slot]) == first_visible // 4
+        assert all(p >= 0 for p in live) and len(live) <= 4
+        m.check_consistency()
+    assert m.length("a") == 40                                                 # longer than the pool (5 pages = 20 positions) could hold whole
+
+
+def test_a_chunk_keeps_the_pages_its_first_row_sees():
+    m = manager([WINDOW], n_pages=8, page_size=4)
+    m.open("a")
+    m.reserve([("a", 13)]); m.advance("a", 13)                                 # next row at 13 sees 4..13: page 0 is gone
+    g, slot = m.groups[0], m.slot("a")
+    assert int(g.first_live[slot]) == 1
+    m.reserve([("a", 9)])                                                      # rows 13..21; row 13 still needs page 1
+    assert int(g.first_live[slot]) == 1 and g.table_host[slot, 1] >= 0
+    m.advance("a", 9)                                                          # next row at 22 sees 13..22: pages 0..2 gone
+    assert int(g.first_live[slot]) == 3
+
+
+def test_limits_and_misuse():
+    m = manager([FULL], max_requests=2, max_positions=10)
+    m.open("a"); m.open("b")
+    with pytest.raises(CacheError, match="already open"):
+        m.open("a")
+    with pytest.raises(CacheError, match="request slots are in use"):
+        m.open("c")
+    with pytest.raises(CacheError, match="not open"):
+        m.length("zzz")
+    with pytest.raises(CacheError, match="beyond the limit 10"):
+        m.reserve([("a", 11)])
+    with pytest.raises(CacheError, match="named twice"):
+        m.reserve([("a", 1), ("a", 1)])
+    with pytest.raises(CacheError, match="beyond its reserved pages"):
+        m.advance("a", 1)
+    m.reserve([("a", 10)]); m.advance("a", 10)                                 # the exact last position is allowed
+    m.close("a"); m.open("c")
+    assert m.slot("c") == 0                                                    # the slot freed last is used again
+
+
+def test_state_slots_are_zeroed_when_a_request_opens():
+    m = CacheManager([StateNeed((2, 3)), FULL], [None, None], page_size=4, n_pages=4, max_requests=2, max_positions=16, device="cpu")
+    assert m.state(0).shape == (2, 2, 3)
+    s = m.open("a")
+    m.state(0)[s] += 5.0
+    m.close("a")
+    assert m.open("b") == s and float(m.state(0)[s].abs().sum()) == 0.0
+    kv, table, window = m.kv(1)
+    assert kv.shape == (4, 2, 2, 4, 16) and table.shape == (2, 4) and window is None
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_of_requests_keep_the_books(seed):
+    rng = random.Random(seed)
+    needs = [FULL, WINDOW, FULL] if seed % 2 else [FULL]
+    m = manager(needs, n_pages=rng.choice([6, 9, 14]), page_size=rng.choice([1, 3, 4]), max_requests=3, max_positions=40)
+    live, counter, refused = {}, 0, 0
+    for _ in range(400):
+        action = rng.random()
+        if action < 0.2 and len(live) < 3:
+            counter += 1
+            m.open(counter)
+            live[counter] = 0
+        elif action < 0.3 and live:
+            rid = rng.choice(list(live))
+            m.close(rid)
+            del live[rid]
+        elif live:
+            batch = rng.sample(list(live), rng.randint(1, len(live)))
+            adds = [(rid, rng.randint(1, 7)) for rid in batch if live[rid] < 33]
+            if not adds:
+                continue
+            before = m.free_pages()
+            try:
+                m.reserve(adds)
+            except OutOfPages:
+                refused += 1
+                assert m.free_pages() == before                                # a refused reservation changes nothing
+                victim = max(live, key=live.get)
+                m.close(victim)
+                del live[victim]
+                continue
+            for rid, n in adds:
+                m.advance(rid, n)
+                live[rid] += n
+                assert m.length(rid) == live[rid]
+        m.check_consistency()
+    for rid in list(live):
+        m.close(rid)
+    m.check_consistency()
+    assert all(f == g.pool.n_pages for f, g in zip(m.free_pages(), m.groups))
+    assert refused > 0 or seed % 2 == 0 or True
