@@ -33,6 +33,7 @@ class DecoderModel:
         self.final_norm = norm_class(spec.final_norm)(spec.final_norm, tensors, dtype, device)
         self.head_in_dtype = activation_dtype_for(self.lm_head, dtype)
         self.run_order = spec.run_order
+        self.graph_safe = all(getattr(l, "graph_safe", False) for l in self.layers) and getattr(self.final_norm, "graph_safe", False)
 
     # ----------------------------------------------------------------------------- what it needs
     def cache_needs(self):

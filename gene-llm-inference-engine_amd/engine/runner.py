@@ -56,7 +56,8 @@ class Runner:
     max_requests live requests (request slots)
     max_rows     most rows one step may hold
     max_positions longest request; defaults to the model's limit
-    use_graphs   replay decode steps (one token per request, all logits wanted) from captured HIP graphs
+    use_graphs   replay decode steps (one token per request, all logits wanted) from captured HIP graphs,
+                 if every part of the model allows it (`graph_safe`)
     """
 
     def __init__(self, model: DecoderModel, *, page_size: int = 16, max_tokens: int = 4096, max_requests: int = 8,
@@ -71,7 +72,7 @@ class Runner:
                                   max_positions=self.max_positions, dtype=model.dtype, device=model.device)
         self._view = _CacheView(self.cache, needs, reads_from)
         self.steps_run = 0
-        self.use_graphs = bool(use_graphs)
+        self.use_graphs = bool(use_graphs) and model.graph_safe
         self._graphs = {}
 
     # -------------------------------------------------------------------------------- requests

@@ -16,6 +16,8 @@ from .linear import activation_dtype_for, linear
 
 
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
         s = spec

@@ -62,7 +62,14 @@ class LayerCache:
 
 
 class Part:
-    """Common construction: `spec`, `tensors` (by name, on the device), compute dtype, device."""
+    """Common construction: `spec`, `tensors` (by name, on the device), compute dtype, device.
+
+    `graph_safe` says that everything in the part's work that changes from step to step is read on
+    the device (from the context's tensors, the page tables and the cache), never from the
+    context's host-side lists: only then may a decode step be captured once and replayed.  It is
+    False unless a part says otherwise, and one part that is not makes the runner launch every
+    step anew."""
+    graph_safe = False
 
     def __init__(self, spec, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device):
         self.spec, self.dtype, self.device = spec, dtype, device

@@ -12,6 +12,8 @@ from .linear import activation_dtype_for, linear
 
 
 class SwiGlu(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
         gate, up = tensors[spec.gate_proj], tensors[spec.up_proj]

@@ -10,6 +10,8 @@ from .base import Norm, register_norm
 
 
 class RmsNorm(Norm):
+    graph_safe = True
+
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
         self.weight = tensors[spec.weight]

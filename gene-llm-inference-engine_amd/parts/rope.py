@@ -35,6 +35,8 @@ def inverse_frequencies(head_dim: int, theta: float, scaling=None):
 
 
 class RotaryHalfSplit(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
         if spec.head_dim % 2:

@@ -1,0 +1,184 @@
+"""Each part of a layer alone against the plain functions, and a toy architecture defined in the
+tests (windowed and full attention, a mixer with state of its own, a layer run twice, a layer that
+reads another's cache) built and stepped through the framework as it is."""
+import random
+
+import pytest
+import torch
+
+import toy_architecture as toy
+import traces
+from model_folders import relative_error
+from plain_llama import causal_attention, read_model_folder, rms_norm, rope_inverse_frequencies, rope_rotate, swiglu
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def step_context(segs, dtype):
+    """segs: (slot, pos0, n) per request."""
+    from geneinfer_amd.parts import StepContext
+    pos, slots, seg_start = [], [], []
+    for slot, pos0, n in segs:
+        seg_start.append(len(pos))
+        pos += list(range(pos0, pos0 + n))
+        slots += [slot] * n
+    t = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    return StepContext(n_rows=len(pos), dtype=dtype, device=torch.device(DEV), tokens=t(pos), row_pos=t(pos), row_slot=t(slots),
+                       seg_slot=[s for s, _, _ in segs], seg_start=seg_start, seg_len=[n for _, _, n in segs], seg_pos0=[p for _, p, _ in segs])
+
+
+def randn(*shape, seed=0, scale=1.0):
+    return scale * torch.randn(*shape, generator=torch.Generator().manual_seed(seed))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from geneinfer_amd.config import RmsNormSpec
+    from geneinfer_amd.parts import norm_class
+    spec = RmsNormSpec(size=72, eps=0.02, weight="n.w")
+    w = (1 + 0.1 * randn(72, seed=1)).to(dtype)
+    part = norm_class(spec)(spec, {"n.w": w.to(DEV)}, dtype, DEV)
+    assert [(n.name, n.shape, n.role) for n in part.tensor_needs(spec)] == [("n.w", (72,), "norm")]
+    x = randn(9, 72, seed=2, scale=4.0)
+    got = part(x.to(DEV), dtype)
+    assert got.dtype == dtype and relative_error(got, rms_norm(x.double(), w.double(), 0.02)) < (2e-6 if dtype == torch.float32 else 5e-3)
+
+
+def test_rotary_part_tables_are_shared_within_a_step():
+    from geneinfer_amd.config import Llama3Scaling, RotarySpec
+    from geneinfer_amd.parts import position_class
+    spec = RotarySpec(32, 500000.0, Llama3Scaling(4.0, 1.0, 4.0, 32))
+    part = position_class(spec)(spec, {}, torch.float32, DEV)
+    ctx = step_context([(0, 35, 4), (1, 0, 1)], torch.float32)
+    cos, sin = part.prepare(ctx)
+    inv = rope_inverse_frequencies(32, 500000.0, dict(factor=4.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=32))
+    ang = ctx.row_pos.cpu().double()[:, None] * inv[None, :]
+    assert (cos.cpu().double() - ang.cos()).abs().max() < 1e-7 and (sin.cpu().double() - ang.sin()).abs().max() < 1e-7
+    again = position_class(spec)(spec, {}, torch.float32, DEV).prepare(ctx)
+    assert again[0] is cos                                            # a second layer with the same spec reuses the step's tables
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [None, 5])
+def test_attention_part_over_two_steps(dtype, window):
+    """A portion, then its continuation beside another request's first rows: the part alone with a cache manager."""
+    from geneinfer_amd.cache import CacheManager
+    from geneinfer_amd.config import AttentionSpec, RotarySpec
+    from geneinfer_amd.parts import LayerCache, mixer_class
+    D, H, KV, hd = 40, 4, 2, 32
+    spec = AttentionSpec(D, H, KV, hd, "q", "k", "v", "o", position=RotarySpec(hd, 10000.0), window=window)
+    w = {"q": randn(H * hd, D, seed=1, scale=0.2), "k": randn(KV * hd, D, seed=2, scale=0.2), "v": randn(KV * hd, D, seed=3, scale=0.2),
+         "o": randn(D, H * hd, seed=4, scale=0.2)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    cls = mixer_class(spec)
+    part = cls(spec, {k: v.to(DEV) for k, v in w.items()}, dtype, DEV)
+    assert {n.name: n.shape for n in cls.tensor_needs(spec)} == {"q": (128, 40), "k": (64, 40), "v": (64, 40), "o": (40, 128)}
+    need = cls.cache_need(spec)
+    assert (need.n_kv_heads, need.head_dim, need.window) == (KV, hd, window)
+    cache = CacheManager([need], [None], page_size=16, n_pages=6, max_requests=2, max_positions=64, dtype=dtype, device=DEV)
+    kv, table, _ = cache.kv(0)
+    hs = {"a": randn(23, D, seed=5).to(dtype), "b": randn(7, D, seed=6).to(dtype)}
+    got = {"a": [], "b": []}
+    for step in ([("a", 0, 17)], [("a", 17, 6), ("b", 0, 7)]):
+        for r, _, _ in step:
+            if not cache.is_open(r):
+                cache.open(r)
+        cache.reserve([(r, n) for r, _, n in step]); cache.sync()
+        ctx = step_context([(cache.slot(r), p0, n) for r, p0, n in step], dtype)
+        h = torch.cat([hs[r][p0:p0 + n] for r, p0, n in step]).to(DEV)
+        residual = torch.zeros(h.shape[0], D, device=DEV)
+        part.forward(h, residual, ctx, LayerCache(kv=kv, table=table, writes=True))
+        row = 0
+        for r, _, n in step:
+            got[r].append(residual[row:row + n].cpu()); row += n
+            cache.advance(r, n)
+    inv = rope_inverse_frequencies(hd, 10000.0)
+    store = (lambda t: t.to(torch.bfloat16).double()) if dtype == torch.bfloat16 else (lambda t: t)
+    for r, h in hs.items():
+        T, hx = h.shape[0], h.double()
+        wd = {k: v.double() for k, v in w.items()}
+        q = store(rope_rotate((hx @ wd["q"].T).reshape(T, H, hd), torch.arange(T), inv))
+        k = store(rope_rotate((hx @ wd["k"].T).reshape(T, KV, hd), torch.arange(T), inv))
+        v = store((hx @ wd["v"].T).reshape(T, KV, hd))
+        want = store(causal_attention(q, k, v, window)).reshape(T, H * hd) @ wd["o"].T
+        assert relative_error(torch.cat(got[r]), want) < (3e-6 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part(dtype):
+    from geneinfer_amd.config import SwiGluSpec
+    from geneinfer_amd.parts import feed_forward_class
+    D, I = 40, 112
+    spec = SwiGluSpec(D, I, "g", "u", "d")
+    w = {"g": randn(I, D, seed=1, scale=0.3).to(dtype), "u": randn(I, D, seed=2, scale=0.3).to(dtype), "d": randn(D, I, seed=3, scale=0.3).to(dtype)}
+    part = feed_forward_class(spec)(spec, {k: v.to(DEV) for k, v in w.items()}, dtype, DEV)
+    for rows in (1, 5, 70):                                           # decode-sized and prompt-sized batches take different kernels
+        h = randn(rows, D, seed=rows).to(dtype)
+        base = randn(rows, D, seed=rows + 1)
+        residual = base.clone().to(DEV)
+        part.forward(h.to(DEV), residual, step_context([(0, 0, rows)], dtype), )
+        store = (lambda t: t.to(torch.bfloat16).double()) if dtype == torch.bfloat16 else (lambda t: t)
+        want = base.double() + swiglu(h.double(), w["g"].double(), w["u"].double(), w["d"].double(), store)
+        assert relative_error(residual, want) < (3e-6 if dtype == torch.float32 else 8e-3), rows
+
+
+def test_registries_refuse_unknown_kinds_and_double_registration():
+    from geneinfer_amd.parts import Mixer, mixer_class, register_mixer
+    class Nothing:
+        kind = "no_such_mixer"
+    with pytest.raises(KeyError, match="no mixer of kind 'no_such_mixer' is registered; known: .*attention"):
+        mixer_class(Nothing())
+    with pytest.raises(ValueError, match="already registered"):
+        register_mixer("attention", Mixer)
+
+
+# ------------------------------------------------------------------------------------ toy model
+@pytest.fixture(scope="module")
+def toy_model(tmp_path_factory):
+    from geneinfer_amd.weights import write_random_model
+    toy.register()
+    toy.register()                                                    # registering the same classes again is harmless
+    cfg = toy.ToyConfig()
+    folder = tmp_path_factory.mktemp("toy")
+    write_random_model(folder, cfg, seed=5, dtype="bfloat16", std=0.2)
+    _, weights = read_model_folder(folder)
+    rng = random.Random(4)
+    requests = {f"t{i}": [rng.randrange(cfg.vocab_size) for _ in range(n)] for i, n in enumerate([40, 9, 63, 21, 34])}
+    return cfg, folder, weights, requests
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", ["whole", "tail_singly", "portions", "mixed"])
+def test_toy_architecture_under_every_cut(toy_model, dtype, mode):
+    from geneinfer_amd.cache import PagedKvNeed, StateNeed
+    from geneinfer_amd.engine import Runner, StepEntry, load_model
+    cfg, folder, weights, requests = toy_model
+    model = load_model(folder, dtype, DEV)                            # config.json names the toy architecture; nothing else does
+    assert type(model.config) is toy.ToyConfig
+    steps = {"whole": traces.whole, "tail_singly": lambda r: traces.tail_singly(r, 32), "portions": traces.portions,
+             "mixed": lambda r: traces.mixed(r, seed=8)}[mode](requests)
+    runner = Runner(model, page_size=16 if dtype == "bfloat16" else 4, max_tokens=traces.peak_tokens(steps, 16), max_requests=4)
+    groups = runner.cache.groups
+    assert [(g.need.window, g.entries) for g in groups] == [(None, [0, 3]), (cfg.window, [1])]      # entry 4 reads entry 1's pages
+    assert list(runner.cache.states) == [2] and runner.cache.state(2).shape == (4, cfg.hidden_size)
+    where, got = traces.wanted_positions(steps), {}
+    for s in steps:
+        for e in s["entries"]:
+            if not runner.is_open(e["id"]):
+                runner.open(e["id"])
+        logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        for row, key in zip(logits.cpu(), where[s["step"]]):
+            got[key] = row
+        for rid in s["end"]:
+            runner.close(rid)
+        runner.cache.check_consistency()
+        held = [sum(len(g.held_pages(runner.cache.slot(r))) for r in runner.cache.open_requests()) for g in groups]
+        assert held[1] <= len(runner.cache.open_requests()) * (2 + (cfg.window + 8) // runner.page_size + 1)     # windowed pages are given back
+    assert runner.cache.free_pages() == [g.pool.n_pages for g in groups]
+    store = (lambda t: t.to(torch.bfloat16).double()) if dtype == "bfloat16" else (lambda t: t)
+    worst = 0.0
+    for rid, toks in requests.items():
+        want = toy.plain_logits(cfg, weights, toks, store=store)
+        worst = max(worst, max(relative_error(got[(rid, p)], want[p]) for p in range(len(toks))))
+    assert worst < (2e-5 if dtype == "float32" else 2e-2), worst

@@ -1,0 +1,135 @@
+"""A toy architecture that exists only in the tests, to show that parts, layer order and cache
+needs are data: it is registered, built, loaded and stepped through the framework's public
+interfaces without a change to the framework's files.
+
+Layers: 0 full attention, 1 windowed attention, 2 a "decay" mixer with a state of its own
+(s <- decay * s + h per row, out = W s), each followed by SwiGLU.  Run order: 0, 1, 2, then layer
+0 once more (a cache of its own) and layer 1 once more reading the pages of its first run.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import ClassVar
+
+import torch
+
+from geneinfer_amd.cache import StateNeed
+from geneinfer_amd.config import (AttentionSpec, LayerSpec, ModelSpec, RmsNormSpec, RotarySpec, RunEntry, SwiGluSpec,
+                                  register_architecture)
+from geneinfer_amd.parts import Mixer, register_mixer
+from geneinfer_amd.weights import TensorNeed
+from plain_llama import causal_attention, rms_norm, rope_inverse_frequencies, rope_rotate, swiglu
+
+
+@dataclass(frozen=True)
+class DecaySpec:
+    kind: ClassVar[str] = "toy_decay"
+    hidden_size: int
+    decay: float
+    weight: str
+
+
+class DecayMixer(Mixer):
+    """State per request: s [hidden] in 32-bit.  Rows of a request are taken in order; the state is
+    read at the start of the request's rows and written back after them."""
+
+    def __init__(self, spec, tensors, dtype, device):
+        super().__init__(spec, tensors, dtype, device)
+        self.w = tensors[spec.weight].float()
+        self.in_dtype = torch.float32
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        return [TensorNeed(spec.weight, (spec.hidden_size, spec.hidden_size))]
+
+    @classmethod
+    def cache_need(cls, spec):
+        return StateNeed((spec.hidden_size,), torch.float32)
+
+    def forward(self, h, residual, ctx, cache):
+        for slot, start, n in zip(ctx.seg_slot, ctx.seg_start, ctx.seg_len):
+            s = cache.state[slot].clone()
+            for i in range(start, start + n):
+                s = self.spec.decay * s + h[i].float()
+                residual[i] += self.w @ s
+            cache.state[slot] = s
+
+
+@dataclass(frozen=True)
+class ToyConfig:
+    hidden_size: int = 48
+    intermediate_size: int = 80
+    num_attention_heads: int = 3
+    num_key_value_heads: int = 1
+    head_dim: int = 16
+    vocab_size: int = 200
+    window: int = 6
+    decay: float = 0.7
+    rms_norm_eps: float = 1e-5
+    rope_theta: float = 10000.0
+    max_position_embeddings: int = 256
+
+    architecture = "ToyMixedForCausalLM"
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(**{k: d[k] for k in cls.__dataclass_fields__ if k in d})
+
+    def to_dict(self):
+        return {"architectures": [self.architecture], "model_type": "toy_mixed", **{k: getattr(self, k) for k in self.__dataclass_fields__}}
+
+    def model_spec(self) -> ModelSpec:
+        d, rot = self.hidden_size, RotarySpec(self.head_dim, self.rope_theta, None)
+        def attention(l, window):
+            p = f"layers.{l}.attn."
+            return AttentionSpec(d, self.num_attention_heads, self.num_key_value_heads, self.head_dim, p + "q", p + "k", p + "v", p + "o",
+                                 position=rot, window=window)
+        def rest(l, mixer):
+            p = f"layers.{l}."
+            return LayerSpec(mixer=mixer, feed_forward=SwiGluSpec(d, self.intermediate_size, p + "ff.gate", p + "ff.up", p + "ff.down"),
+                             mixer_norm=RmsNormSpec(d, self.rms_norm_eps, p + "norm1"), feed_forward_norm=RmsNormSpec(d, self.rms_norm_eps, p + "norm2"))
+        layers = (rest(0, attention(0, None)), rest(1, attention(1, self.window)), rest(2, DecaySpec(d, self.decay, "layers.2.decay.w")))
+        order = (RunEntry(0), RunEntry(1), RunEntry(2), RunEntry(0), RunEntry(1, cache_of=1))
+        return ModelSpec(architecture=self.architecture, vocab_size=self.vocab_size, hidden_size=d, max_positions=self.max_position_embeddings,
+                         embedding="embed", final_norm=RmsNormSpec(d, self.rms_norm_eps, "final_norm"), lm_head="head", layers=layers,
+                         run_order=order)
+
+
+def register():
+    """Idempotent: the registries refuse a second class under a name, not the same class again."""
+    register_mixer("toy_decay", DecayMixer)
+    register_architecture(ToyConfig.architecture, ToyConfig, model_type="toy_mixed")
+
+
+def plain_logits(cfg: ToyConfig, w: dict, tokens, dtype=torch.float64, store=lambda t: t):
+    """The toy model over a whole sequence with the plain parts (no cache, no state slots)."""
+    w = {k: v.to(dtype) for k, v in w.items()}
+    T, H, KV, hd = len(tokens), cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    pos = torch.arange(T)
+    inv = rope_inverse_frequencies(hd, cfg.rope_theta)
+    x = w["embed"][torch.tensor(tokens)]
+    spec = cfg.model_spec()
+    kept = {}
+    for i, entry in enumerate(spec.run_order):
+        l, p = entry.layer, f"layers.{entry.layer}."
+        xb = rms_norm(x, w[p + "norm1"], cfg.rms_norm_eps)
+        if l == 2:
+            s, outs = torch.zeros(cfg.hidden_size, dtype=dtype), []
+            for t in range(T):
+                s = cfg.decay * s + xb[t]
+                outs.append(w["layers.2.decay.w"] @ s)
+            x = x + torch.stack(outs)
+        else:
+            xb = store(xb)
+            q = store(rope_rotate((xb @ w[p + "attn.q"].T).reshape(T, H, hd), pos, inv))
+            if entry.cache_of is None:
+                k = store(rope_rotate((xb @ w[p + "attn.k"].T).reshape(T, KV, hd), pos, inv))
+                v = store((xb @ w[p + "attn.v"].T).reshape(T, KV, hd))
+                kept[i] = (k, v)
+            else:
+                k, v = kept[entry.cache_of]
+            att = store(causal_attention(q, k, v, cfg.window if l == 1 else None)).reshape(T, H * hd)
+            x = x + att @ w[p + "attn.o"].T
+        xb = store(rms_norm(x, w[p + "norm2"], cfg.rms_norm_eps))
+        x = x + swiglu(xb, w[p + "ff.gate"], w[p + "ff.up"], w[p + "ff.down"], store)
+    return store(rms_norm(x, w["final_norm"], cfg.rms_norm_eps)) @ w["head"].T
