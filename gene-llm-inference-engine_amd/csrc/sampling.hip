@@ -10,30 +10,46 @@ namespace {
 
 constexpr int NT = 1024;
 
-__global__ __launch_bounds__(NT) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab, long stride) {
-    __shared__ float best_v[NT / 64];
-    __shared__ int best_i[NT / 64];
-    const float* row = logits + (size_t)blockIdx.x * stride;
+// Arg max in two stages so that a few rows still fill the chip: stage one takes runs of CHUNK
+// logits (one workgroup each), stage two the winners of a row.  Among equal values the lowest index
+// wins at every comparison, so the result is the lowest index of the maximum.
+constexpr int CHUNK = 4096;
+
+__device__ __forceinline__ void better(float& bv, int& bi, float ov, int oi) {
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+}
+
+__global__ __launch_bounds__(256) void argmax_chunks_kernel(const float* __restrict__ logits, float* __restrict__ part_v, int* __restrict__ part_i,
+                                                            int vocab, long stride, int n_chunks) {
+    __shared__ float sv[4];
+    __shared__ int si[4];
+    const float* row = logits + (size_t)blockIdx.y * stride;
+    const int begin = blockIdx.x * CHUNK, end = min(vocab, begin + CHUNK);
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += NT) {
+    for (int i = begin + threadIdx.x; i < end; i += 256) {
         const float v = row[i];
         if (v > bv || bi == 0x7fffffff) { bv = v; bi = i; }      // ascending i: strict > keeps the lowest index
     }
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(bv, off, 64);
-        const int oi = __shfl_xor(bi, off, 64);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    if (lane == 0) { best_v[wave] = bv; best_i[wave] = bi; }
+    for (int off = 32; off > 0; off >>= 1) better(bv, bi, __shfl_xor(bv, off, 64), __shfl_xor(bi, off, 64));
+    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = bv; si[threadIdx.x >> 6] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < NT / 64; ++w)
-            if (best_v[w] > bv || (best_v[w] == bv && best_i[w] < bi)) { bv = best_v[w]; bi = best_i[w]; }
-        out[blockIdx.x] = bi;
+        for (int w = 1; w < 4; ++w) better(bv, bi, sv[w], si[w]);
+        part_v[(size_t)blockIdx.y * n_chunks + blockIdx.x] = bv;
+        part_i[(size_t)blockIdx.y * n_chunks + blockIdx.x] = bi;
     }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ part_v, const int* __restrict__ part_i, int* __restrict__ out,
+                                                          int n_chunks) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int c = threadIdx.x; c < n_chunks; c += 64) better(bv, bi, part_v[(size_t)blockIdx.x * n_chunks + c], part_i[(size_t)blockIdx.x * n_chunks + c]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) better(bv, bi, __shfl_xor(bv, off, 64), __shfl_xor(bi, off, 64));
+    if (threadIdx.x == 0) out[blockIdx.x] = bi;
 }
 
 // Each thread owns a contiguous run of tokens, so that cumulative sums follow index order.
@@ -95,10 +111,17 @@ __global__ __launch_bounds__(NT) void sample_temperature_kernel(const float* __r
 
 }  // namespace
 
-GI_API int gi_argmax(const float* logits, int* out, int n_rows, int vocab, long stride, hipStream_t stream) {
-    GI_REQUIRE(n_rows > 0 && vocab > 0 && stride >= vocab, "argmax: bad sizes (rows %d, vocab %d, stride %ld)", n_rows, vocab, stride);
-    argmax_kernel<<<n_rows, NT, 0, stream>>>(logits, out, vocab, stride);
-    GI_CHECK_LAUNCH("argmax");
+// Chunks per row, so that the caller can size the scratch: n_rows * chunks floats and as many ints.
+GI_API int gi_argmax_chunks(int vocab) { return (vocab + CHUNK - 1) / CHUNK; }
+
+GI_API int gi_argmax(const float* logits, int* out, float* part_v, int* part_i, int n_rows, int vocab, long stride, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && n_rows <= 65535 && vocab > 0 && stride >= vocab, "argmax: bad sizes (rows %d, vocab %d, stride %ld)", n_rows, vocab, stride);
+    GI_REQUIRE(part_v != nullptr && part_i != nullptr, "argmax: scratch is missing");
+    const int n_chunks = gi_argmax_chunks(vocab);
+    argmax_chunks_kernel<<<dim3(n_chunks, n_rows), 256, 0, stream>>>(logits, part_v, part_i, vocab, stride, n_chunks);
+    GI_CHECK_LAUNCH("argmax (chunks)");
+    argmax_final_kernel<<<n_rows, 64, 0, stream>>>(part_v, part_i, out, n_chunks);
+    GI_CHECK_LAUNCH("argmax (final)");
     return 0;
 }
 

@@ -62,10 +62,12 @@ class DecoderModel:
             self.layers[entry.layer].forward(x, ctx, cache.layer_cache(i))
         if n_logit_rows == 0:
             return None
-        picked = torch.empty((n_logit_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device)
-        ops.gather_rows(x, logit_rows, picked)
-        normed = self.final_norm(picked, self.head_in_dtype)
         logits = torch.empty((n_logit_rows, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        if hasattr(self.final_norm, "deferred"):
+            normed = self.final_norm.deferred(x, self.head_in_dtype, rows=logit_rows)
+        else:
+            picked = torch.empty((n_logit_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device)
+            normed = self.final_norm(ops.gather_rows(x, logit_rows, picked), self.head_in_dtype)
         linear(normed, self.lm_head, logits)
         return logits
 

@@ -35,7 +35,9 @@ _SIGNATURES = {
                                  c_float, c_void_p],
     "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long,
                                  c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
-    "gi_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
+    "gi_gemm_bf16_normed": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                            c_long, c_long, c_void_p],
+    "gi_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
 }
 
@@ -50,6 +52,10 @@ def lib():
             fn = getattr(l, name)
             fn.argtypes = sig
             fn.restype = c_int
+        l.gi_gemm_bf16_normed_supports.argtypes = [c_int, c_int]
+        l.gi_gemm_bf16_normed_supports.restype = c_int
+        l.gi_argmax_chunks.argtypes = [c_int]
+        l.gi_argmax_chunks.restype = c_int
         l.gi_attention_bf16_supports.argtypes = [c_int, c_int, c_int]
         l.gi_attention_bf16_supports.restype = c_int
         l.gi_gemm_bf16_skinny_splits.argtypes = [c_int, c_int]
@@ -326,6 +332,31 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False):
     return out
 
 
+def gemm_bf16_normed_supports(x, norm_weight, w, out, n_rows) -> bool:
+    k = x.shape[1]
+    return (x.dtype == torch.float32 and x.stride(1) == 1 and x.stride(0) % 4 == 0 and x.data_ptr() % 16 == 0 and w.dtype == torch.bfloat16
+            and w.stride(1) == 1 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0 and norm_weight.data_ptr() % 16 == 0
+            and norm_weight.dtype in _CODE and out.stride(1) == 1 and bool(lib().gi_gemm_bf16_normed_supports(n_rows, k)))
+
+
+def gemm_bf16_normed(x, norm_weight, eps, w, out, accumulate=False, gated=False, rows=None):
+    """out (=|+=) rmsnorm(x[rows]) @ w.T for at most 16 rows, the norm applied inside the product's kernel.
+    x float32 [n, k]; rows: int32 indices of the rows to take (all of x if None)."""
+    _dev(x, norm_weight, w, out, rows)
+    k = x.shape[1]
+    m = x.shape[0] if rows is None else rows.numel()
+    n = w.shape[0]
+    _need(w.shape == (n, k) and norm_weight.shape == (k,) and norm_weight.is_contiguous(), "gemm_normed: shapes of the weights do not fit the rows")
+    _need(out.shape == (m, n // 2 if gated else n), f"gemm_normed: out is {tuple(out.shape)}, ({m}, {n // 2 if gated else n}) is needed")
+    _need(gemm_bf16_normed_supports(x, norm_weight, w, out, m), "gemm_normed: unsupported operands (float32 rows, bfloat16 weights, at most 16 rows)")
+    if rows is not None:
+        _i32(rows, "gemm_normed: rows", m)
+    _call("gi_gemm_bf16_normed", x.data_ptr(), x.stride(0), _ptr(rows), norm_weight.data_ptr(), _code(norm_weight, "gemm_normed: norm weight"),
+          float(eps), w.data_ptr(), out.data_ptr(), _code(out, "gemm_normed: out"), 1 if accumulate else 0, 1 if gated else 0, m, n, k,
+          w.stride(0), out.stride(0), _stream())
+    return out
+
+
 def interleave_gate_up(gate, up):
     """[gate; up] in groups of 16 rows: 16 gate rows, the 16 up rows of the same outputs, and so on."""
     i, d = gate.shape
@@ -338,7 +369,10 @@ def argmax(logits, out):
     n, vocab = logits.shape
     _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "argmax: logits must be float32 with unit inner stride")
     _i32(out, "argmax: out", n)
-    _call("gi_argmax", logits.data_ptr(), out.data_ptr(), n, vocab, logits.stride(0), _stream())
+    chunks = lib().gi_argmax_chunks(vocab)
+    part_v = torch.empty(n * chunks, dtype=torch.float32, device=logits.device)
+    part_i = torch.empty(n * chunks, dtype=torch.int32, device=logits.device)
+    _call("gi_argmax", logits.data_ptr(), out.data_ptr(), part_v.data_ptr(), part_i.data_ptr(), n, vocab, logits.stride(0), _stream())
     return out
 
 

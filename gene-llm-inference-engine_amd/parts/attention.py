@@ -17,6 +17,7 @@ from .linear import activation_dtype_for, linear
 
 class Attention(Mixer):
     graph_safe = True
+    accepts_deferred_norm = True      # its input goes into `linear` only
 
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)

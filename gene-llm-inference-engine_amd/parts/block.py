@@ -30,11 +30,17 @@ class PreNormBlock:
     def cache_need(cls, spec):
         return mixer_class(spec.mixer).cache_need(spec.mixer)
 
+    @staticmethod
+    def _normed(norm, part, x, ctx):
+        """The part's input: the normed rows, or the norm handed on unapplied if both sides can."""
+        dtype = getattr(part, "in_dtype", ctx.dtype)
+        if getattr(part, "accepts_deferred_norm", False) and hasattr(norm, "deferred"):
+            return norm.deferred(x, dtype)
+        return norm(x, dtype)
+
     def forward(self, x, ctx, cache):
-        h = self.mixer_norm(x, getattr(self.mixer, "in_dtype", ctx.dtype))
-        self.mixer.forward(h, x, ctx, cache)
-        h = self.feed_forward_norm(x, getattr(self.feed_forward, "in_dtype", ctx.dtype))
-        self.feed_forward.forward(h, x, ctx)
+        self.mixer.forward(self._normed(self.mixer_norm, self.mixer, x, ctx), x, ctx, cache)
+        self.feed_forward.forward(self._normed(self.feed_forward_norm, self.feed_forward, x, ctx), x, ctx)
 
 
 register_block("prenorm", PreNormBlock)

@@ -1,17 +1,26 @@
 """Matrix products of the parts: out (=|+=) a @ weight.T with weights [out_features, in_features]
 as checkpoints store them (no bias).  The kernel is chosen by the operands' storage: 32-bit
 operands take the exact kernel; bfloat16 operands take the matrix-core kernels where their
-shape rules allow and the exact kernel otherwise."""
+shape rules allow and the exact kernel otherwise.  `a` may be a norm not yet applied
+(`NormedRows`): for a few rows it is applied inside the product's kernel."""
 from __future__ import annotations
 
 import torch
 
 from ..kernels import ops
+from .norm import NormedRows
 
 
-def linear(a: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
+def linear(a, weight: torch.Tensor, out: torch.Tensor, accumulate: bool = False, gated: bool = False) -> torch.Tensor:
+    """gated: weight is [gate; up] interleaved by `ops.interleave_gate_up` and out = silu(gate) * up (bfloat16 only)."""
+    if isinstance(a, NormedRows):
+        if a.out_dtype == torch.bfloat16 and ops.gemm_bf16_normed_supports(a.x, a.norm.weight, weight, out, a.n_rows):
+            return ops.gemm_bf16_normed(a.x, a.norm.weight, a.norm.eps, weight, out, accumulate, gated, a.rows)
+        a = a.materialize()
     if a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and ops.gemm_bf16_supports(a, weight, out):
-        return ops.gemm_bf16(a, weight, out, accumulate)
+        return ops.gemm_bf16(a, weight, out, accumulate, gated)
+    if gated:
+        raise ops.KernelError("the gated product exists for bfloat16 operands only")
     return ops.gemm_exact(a, weight, out, accumulate)
 
 

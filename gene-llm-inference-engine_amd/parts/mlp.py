@@ -13,6 +13,7 @@ from .linear import activation_dtype_for, linear
 
 class SwiGlu(FeedForward):
     graph_safe = True
+    accepts_deferred_norm = True      # its input goes into `linear` only
 
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
@@ -34,7 +35,7 @@ class SwiGlu(FeedForward):
         T, inter = ctx.n_rows, self.spec.intermediate_size
         if self.fused:
             mid = torch.empty((T, inter), dtype=torch.bfloat16, device=ctx.device)
-            ops.gemm_bf16(h, self.w_gate_up, mid, gated=True)
+            linear(h, self.w_gate_up, mid, gated=True)
             linear(mid, self.w_down, residual, accumulate=True)
             return
         gate_up = torch.empty((T, 2 * inter), dtype=torch.float32, device=ctx.device)

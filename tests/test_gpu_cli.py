@@ -1,0 +1,56 @@
+"""The command line: bin/gi_generate with the reference's options, bin/make_random_model."""
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+import torch
+
+from model_folders import CONFIGS, full_config, write_model
+from plain_llama import PlainLlama
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+@pytest.mark.gpu
+def test_gi_generate_greedy_dumps_the_plain_tokens(tmp_path):
+    write_model(tmp_path / "m", CONFIGS["A"], seed=9)
+    prompt = [17, 4, 200, 33, 91]
+    dump = tmp_path / "tokens.txt"
+    r = subprocess.run([str(ROOT / "bin" / "gi_generate"), "--model", str(tmp_path / "m"), "--prompt-ids", " ".join(map(str, prompt)),
+                        "--steps", str(len(prompt) + 7), "--temperature", "0", "--weights", "f32", "--dump-tokens", str(dump), "--page-size", "4"],
+                       capture_output=True, text=True, timeout=170)
+    assert r.returncode == 0, r.stderr
+    lines = dump.read_text().splitlines()
+    want = PlainLlama(tmp_path / "m").greedy(prompt, 8)
+    assert [int(t) for t in lines[0].split()] == prompt and [int(t) for t in lines[1].split()] == want
+    assert r.stdout.split() == [str(t) for t in prompt + want]                 # echo of the prompt, then the tokens as they come
+    assert "prompt: 5 tokens" in r.stderr and "generated: 8 tokens" in r.stderr and "temperature 0.00" in r.stderr
+    quiet = subprocess.run([str(ROOT / "bin" / "gi_generate"), "--model", str(tmp_path / "m"), "--prompt-ids", "1,2,3", "--steps", "6", "--seed", "5",
+                            "--no-echo", "--quiet"], capture_output=True, text=True, timeout=170)
+    assert quiet.returncode == 0 and len(quiet.stdout.split()) == 4 and "prompt:" not in quiet.stderr and "gpu:" not in quiet.stderr
+    again = subprocess.run([str(ROOT / "bin" / "gi_generate"), "--model", str(tmp_path / "m"), "--prompt-ids", "1,2,3", "--steps", "6", "--seed", "5",
+                            "--no-echo", "--quiet"], capture_output=True, text=True, timeout=170)
+    assert again.stdout == quiet.stdout                                         # the same seed, the same tokens
+
+
+def test_gi_generate_usage_errors(tmp_path):
+    exe = str(ROOT / "bin" / "gi_generate")
+    for args, msg in (([], "--model is required"), (["--model", "x", "--weights", "int8"], "--weights must be native or f32"),
+                      (["--model", "x", "--frobnicate"], "unknown option --frobnicate"), (["--model"], "missing value for --model"),
+                      (["--model", "x", "--steps", "ten"], "invalid integer for --steps"), (["--model", "x", "--device", "cpu"], "only gpu exists")):
+        r = subprocess.run([exe, *args], capture_output=True, text=True, timeout=60)
+        assert r.returncode == 2 and msg in r.stderr and "usage: gi_generate" in r.stderr
+    r = subprocess.run([exe, "--model", str(tmp_path), "--prompt-ids", "1"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 1 and r.stderr.startswith("error:")                  # no config.json there
+
+
+def test_make_random_model_writes_a_loadable_folder(tmp_path):
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(full_config(CONFIGS["C"])))
+    r = subprocess.run([str(ROOT / "bin" / "make_random_model"), "--config", str(cfg), "--out", str(tmp_path / "m"), "--seed", "3", "--dtype", "float32"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    logits = PlainLlama(tmp_path / "m").logits([1, 2, 3])
+    assert logits.shape == (3, 301) and torch.isfinite(logits).all()
