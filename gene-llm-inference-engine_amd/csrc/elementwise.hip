@@ -63,11 +63,60 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict
     for (int d = threadIdx.x; d < dim; d += 256) store_f32(orow, d, load_f32(w, d) * (scale * xr[d]));
 }
 
-GI_API int gi_rmsnorm(const float* x, const void* w, int w_dtype, void* out, int out_dtype, int n_rows, int dim, float eps,
+// The same for rows whose length is a multiple of 4 and at most 4096, 16-byte aligned: every thread
+// loads its (at most four) groups of four values at once and keeps them for the second pass, so the
+// kernel waits for memory once.  `rows` (optional) gathers the input rows.
+__device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) { *reinterpret_cast<float4*>(p) = float4{a, b, c, d}; }
+__device__ __forceinline__ void store4(bf16_t* p, float a, float b, float c, float d) {
+    *reinterpret_cast<uint2*>(p) = uint2{(uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16), (uint32_t)f32_to_bf16(c) | ((uint32_t)f32_to_bf16(d) << 16)};
+}
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16_t* p) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    return float4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u)};
+}
+
+template <typename TW, typename TO>
+__global__ __launch_bounds__(256) void rmsnorm_fast_kernel(const float* __restrict__ x, const int* __restrict__ rows, const TW* __restrict__ w,
+                                                          TO* __restrict__ out, int dim, float eps, size_t x_stride, size_t out_stride) {
+    __shared__ float red[4];
+    const float* xr = x + (size_t)(rows ? rows[blockIdx.x] : blockIdx.x) * x_stride;
+    TO* orow = out + (size_t)blockIdx.x * out_stride;
+    const int n4 = dim / 4;
+    float4 v[4], wv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = threadIdx.x + 256 * i;
+        v[i] = c < n4 ? load4(xr + 4 * c) : float4{0.f, 0.f, 0.f, 0.f};
+        wv[i] = c < n4 ? load4(w + 4 * c) : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        ss = fmaf(v[i].x, v[i].x, ss); ss = fmaf(v[i].y, v[i].y, ss); ss = fmaf(v[i].z, v[i].z, ss); ss = fmaf(v[i].w, v[i].w, ss);
+    }
+    ss = block_sum<256>(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)dim + eps);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = threadIdx.x + 256 * i;
+        if (c < n4) store4(orow + 4 * c, wv[i].x * (scale * v[i].x), wv[i].y * (scale * v[i].y), wv[i].z * (scale * v[i].z), wv[i].w * (scale * v[i].w));
+    }
+}
+
+// rows != nullptr: out[i] = norm(x[rows[i]]) (needs the fast kernel's conditions: dim a multiple of 4, at most 4096, aligned rows).
+GI_API int gi_rmsnorm(const float* x, const int* rows, const void* w, int w_dtype, void* out, int out_dtype, int n_rows, int dim, float eps,
                       long x_stride, long out_stride, hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && dim > 0, "rmsnorm: n_rows %d and dim %d must be positive", n_rows, dim);
     GI_REQUIRE(x_stride >= dim && out_stride >= dim, "rmsnorm: row strides must be at least dim");
-#define LAUNCH(TW, TO) rmsnorm_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(x, (const TW*)w, (TO*)out, dim, eps, (size_t)x_stride, (size_t)out_stride)
+    const bool fast = dim % 4 == 0 && dim <= 4096 && x_stride % 4 == 0 && out_stride % 4 == 0 && ((uintptr_t)x & 15) == 0 &&
+                      ((uintptr_t)w & 15) == 0 && ((uintptr_t)out & 15) == 0;
+    GI_REQUIRE(rows == nullptr || fast, "rmsnorm: gathering rows needs a row length that is a multiple of 4 and at most 4096, and aligned operands");
+#define LAUNCH(TW, TO)                                                                                                                   \
+    do {                                                                                                                                 \
+        if (fast) rmsnorm_fast_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(x, rows, (const TW*)w, (TO*)out, dim, eps, (size_t)x_stride, (size_t)out_stride); \
+        else rmsnorm_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(x, (const TW*)w, (TO*)out, dim, eps, (size_t)x_stride, (size_t)out_stride);              \
+    } while (0)
     if (w_dtype == GI_F32 && out_dtype == GI_F32) LAUNCH(float, float);
     else if (w_dtype == GI_F32 && out_dtype == GI_BF16) LAUNCH(float, bf16_t);
     else if (w_dtype == GI_BF16 && out_dtype == GI_F32) LAUNCH(bf16_t, float);
@@ -114,34 +163,32 @@ __global__ void rope_store_kernel(const float* __restrict__ q, const float* __re
                                   long ldv, const float* __restrict__ cos_t, const float* __restrict__ sin_t, const int* __restrict__ pos,
                                   const int* __restrict__ slot, const int* __restrict__ table, int table_stride, TQ* __restrict__ q_out,
                                   TC* __restrict__ cache, long page_stride, int page_size, int n_heads, int n_kv, int hd) {
+    // One thread per pair: items 0 .. n_heads*half-1 are query pairs, the rest key pairs (which also carry the two values).
     const int t = blockIdx.x, half = hd / 2;
-    const float* c = cos_t ? cos_t + (size_t)t * half : nullptr;
-    const float* s = sin_t ? sin_t + (size_t)t * half : nullptr;
-    const int n_q_items = n_heads * half;
-    for (int i = threadIdx.x; i < n_q_items; i += blockDim.x) {
-        const int h = i / half, kk = i % half;
+    const int i = blockIdx.y * blockDim.x + threadIdx.x;
+    const int n_q_items = n_heads * half, n_k_items = k ? n_kv * half : 0;
+    if (i >= n_q_items + n_k_items) return;
+    const bool is_q = i < n_q_items;
+    const int j = is_q ? i : i - n_q_items, h = j / half, kk = j % half;
+    const float cc = cos_t ? cos_t[(size_t)t * half + kk] : 1.f, ss = sin_t ? sin_t[(size_t)t * half + kk] : 0.f;
+    if (is_q) {
         const float a = q[(size_t)t * ldq + h * hd + kk], b = q[(size_t)t * ldq + h * hd + kk + half];
-        const float cc = c ? c[kk] : 1.f, ss = s ? s[kk] : 0.f;
         store_f32(q_out, (size_t)t * n_heads * hd + h * hd + kk, a * cc - b * ss);
         store_f32(q_out, (size_t)t * n_heads * hd + h * hd + kk + half, a * ss + b * cc);
+        return;
     }
-    if (k == nullptr) return;
+    const float a = k[(size_t)t * ldk + h * hd + kk], b = k[(size_t)t * ldk + h * hd + kk + half];
+    const float va = v[(size_t)t * ldv + h * hd + kk], vb = v[(size_t)t * ldv + h * hd + kk + half];
     const int p = pos[t];
     const long page = table[(size_t)slot[t] * table_stride + p / page_size];
     const int place = p % page_size;
     TC* kbase = cache + page * page_stride;
     TC* vbase = kbase + (size_t)n_kv * page_size * hd;
-    const int n_k_items = n_kv * half;
-    for (int i = threadIdx.x; i < n_k_items; i += blockDim.x) {
-        const int g = i / half, kk = i % half;
-        const float a = k[(size_t)t * ldk + g * hd + kk], b = k[(size_t)t * ldk + g * hd + kk + half];
-        const float cc = c ? c[kk] : 1.f, ss = s ? s[kk] : 0.f;
-        const size_t o = ((size_t)g * page_size + place) * hd;
-        store_f32(kbase, o + kk, a * cc - b * ss);
-        store_f32(kbase, o + kk + half, a * ss + b * cc);
-        store_f32(vbase, ((size_t)g * hd + kk) * page_size + place, v[(size_t)t * ldv + g * hd + kk]);
-        store_f32(vbase, ((size_t)g * hd + kk + half) * page_size + place, v[(size_t)t * ldv + g * hd + kk + half]);
-    }
+    const size_t o = ((size_t)h * page_size + place) * hd;
+    store_f32(kbase, o + kk, a * cc - b * ss);
+    store_f32(kbase, o + kk + half, a * ss + b * cc);
+    store_f32(vbase, ((size_t)h * hd + kk) * page_size + place, va);
+    store_f32(vbase, ((size_t)h * hd + kk + half) * page_size + place, vb);
 }
 
 GI_API int gi_rope_store(const float* q, const float* k, const float* v, long ldq, long ldk, long ldv, const float* cos_t,
@@ -154,8 +201,11 @@ GI_API int gi_rope_store(const float* q, const float* k, const float* v, long ld
     GI_REQUIRE(k == nullptr || (v != nullptr && cache != nullptr && table != nullptr && page_size > 0 &&
                                 page_stride >= 2L * n_kv * page_size * hd),
                "rope_store: cache write needs v, a cache, a table and a page stride of at least 2*n_kv*page_size*hd");
+    const int items = (n_heads + (k ? n_kv : 0)) * (hd / 2);
+    dim3 grid(n_rows, (items + 255) / 256);
+    GI_REQUIRE(grid.y <= 65535, "rope_store: too many heads");
 #define LAUNCH(TQ, TC)                                                                                                       \
-    rope_store_kernel<TQ, TC><<<n_rows, 256, 0, stream>>>(q, k, v, ldq, ldk, ldv, cos_t, sin_t, pos, slot, table, table_stride, \
+    rope_store_kernel<TQ, TC><<<grid, 256, 0, stream>>>(q, k, v, ldq, ldk, ldv, cos_t, sin_t, pos, slot, table, table_stride, \
                                                           (TQ*)q_out, (TC*)cache, page_stride, page_size, n_heads, n_kv, hd)
     if (q_dtype == GI_F32 && cache_dtype == GI_F32) LAUNCH(float, float);
     else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t);

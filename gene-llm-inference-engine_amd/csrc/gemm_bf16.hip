@@ -216,27 +216,18 @@ __global__ void skinny_reduce_kernel(const float* __restrict__ P, void* __restri
 // and of activation row r, so the four lanes of a row read 64 contiguous bytes per load.  Loads run
 // two blocks ahead of the products.  The slices' sums meet in LDS and are added in slice order.
 // ROWS = 8 leaves half of each product idle and doubles the number of workgroups for narrow outputs.
-// NORM: the activations are not given as bfloat16 rows but as the 32-bit residual rows X (optionally
-// gathered through `x_rows`) with an RMS norm still to apply: each wave first normalises one or two
-// rows, out = w * (x * rsqrt(mean(x^2) + eps)) rounded to bfloat16, into LDS, and the products read
-// their activation operand from there.  The weights' first loads are already in flight meanwhile.
-template <int STRIPS, int ROWS, int EPI, bool NORM>
+template <int STRIPS, int ROWS, int EPI>
 __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
-                                                            int M, int N, int K, long lda, long ldw, long ldc,
-                                                            const float* __restrict__ X, long ldx, const int* __restrict__ x_rows,
-                                                            const void* __restrict__ norm_w, int norm_w_bf16, float eps) {
+                                                            int M, int N, int K, long lda, long ldw, long ldc) {
     constexpr int SLICES = 8 / STRIPS, STEP = SLICES * SK, DEPTH = 3;
     __shared__ float red[8][64][4];
-    extern __shared__ __attribute__((aligned(16))) unsigned char dyn_lds[];
-    bf16_t* hs = reinterpret_cast<bf16_t*>(dyn_lds);
-    const int hstride = K + 8;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int strip = wave % STRIPS, slice = wave / STRIPS;
     const int r = lane & 15, q = lane >> 4;
     const int n = (blockIdx.x * STRIPS + strip) * ROWS + r;
     const bool w_ok = r < ROWS && n < N, x_ok = r < M;
     const bf16_t* wrow = W + (size_t)(w_ok ? n : 0) * ldw + 8 * q;
-    const bf16_t* xrow = NORM ? hs + (size_t)(x_ok ? r : 0) * hstride + 8 * q : A + (size_t)(x_ok ? r : 0) * lda + 8 * q;
+    const bf16_t* xrow = A + (size_t)(x_ok ? r : 0) * lda + 8 * q;
 
     floatx4 acc = floatx4{};
     uint4 w_buf[DEPTH][4], x_buf[DEPTH][4];
@@ -245,55 +236,19 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
         for (int j = 0; j < 4; ++j) {
             const bool in = k0 + 32 * j + 8 * q < K;
             w[j] = (in && w_ok) ? load16(wrow + k0 + 32 * j) : uint4{0, 0, 0, 0};
-            if constexpr (!NORM) x[j] = (in && x_ok) ? load16(xrow + k0 + 32 * j) : uint4{0, 0, 0, 0};
+            x[j] = (in && x_ok) ? load16(xrow + k0 + 32 * j) : uint4{0, 0, 0, 0};
         }
     };
     const int k_first = slice * SK;
 #pragma unroll
     for (int d = 0; d < DEPTH - 1; ++d) fetch(k_first + d * STEP, w_buf[d], x_buf[d]);      // beyond K: zeros, no loads
-    if constexpr (NORM) {
-        for (int m = wave; m < M; m += 8) {
-            const float* xr = X + (size_t)(x_rows ? x_rows[m] : m) * ldx;
-            float ss = 0.f;
-            for (int c = lane; c < K / 4; c += 64) {
-                const float4 v = *reinterpret_cast<const float4*>(xr + 4 * c);
-                ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
-            }
-            ss = wave_sum(ss);
-            const float rstd = 1.0f / sqrtf(ss / (float)K + eps);
-            for (int c = lane; c < K / 4; c += 64) {
-                const float4 v = *reinterpret_cast<const float4*>(xr + 4 * c);
-                float w0, w1, w2, w3;
-                if (norm_w_bf16) {
-                    const uint2 wv = *reinterpret_cast<const uint2*>((const bf16_t*)norm_w + 4 * c);
-                    w0 = __uint_as_float(wv.x << 16); w1 = __uint_as_float(wv.x & 0xffff0000u);
-                    w2 = __uint_as_float(wv.y << 16); w3 = __uint_as_float(wv.y & 0xffff0000u);
-                } else {
-                    const float4 wv = *reinterpret_cast<const float4*>((const float*)norm_w + 4 * c);
-                    w0 = wv.x; w1 = wv.y; w2 = wv.z; w3 = wv.w;
-                }
-                const uint32_t lo = (uint32_t)f32_to_bf16(w0 * (rstd * v.x)) | ((uint32_t)f32_to_bf16(w1 * (rstd * v.y)) << 16);
-                const uint32_t hi = (uint32_t)f32_to_bf16(w2 * (rstd * v.z)) | ((uint32_t)f32_to_bf16(w3 * (rstd * v.w)) << 16);
-                *reinterpret_cast<uint2*>(hs + (size_t)m * hstride + 4 * c) = uint2{lo, hi};
-            }
-        }
-        __syncthreads();
-    }
     for (int k0 = k_first; k0 < K; k0 += DEPTH * STEP) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {                     // buffer d holds block k0 + d*STEP
             fetch(k0 + (d + DEPTH - 1) * STEP, w_buf[(d + DEPTH - 1) % DEPTH], x_buf[(d + DEPTH - 1) % DEPTH]);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                uint4 xa;
-                if constexpr (NORM) {
-                    const int k = k0 + d * STEP + 32 * j + 8 * q;
-                    xa = (x_ok && k < K) ? *reinterpret_cast<const uint4*>(xrow + k0 + d * STEP + 32 * j) : uint4{0, 0, 0, 0};
-                } else {
-                    xa = x_buf[d][j];
-                }
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xa), as_bf16x8(w_buf[d][j]), acc, 0, 0, 0);
-            }
+            for (int j = 0; j < 4; ++j)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x_buf[d][j]), as_bf16x8(w_buf[d][j]), acc, 0, 0, 0);
         }
     }
 #pragma unroll
@@ -321,48 +276,6 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
             }
         }
     }
-}
-
-constexpr size_t SLIM_NORM_LDS_MAX = 120 * 1024;
-
-template <int STRIPS, int ROWS, int EPI, bool NORM>
-int launch_slim_one(dim3 grid, size_t lds, const void* A, const void* W, void* C, int M, int N, int K, long lda, long ldw, long ldc,
-                    const float* X, long ldx, const int* x_rows, const void* norm_w, int norm_w_bf16, float eps, hipStream_t stream) {
-    auto kernel = gemm_bf16_slim_kernel<STRIPS, ROWS, EPI, NORM>;
-    static size_t granted = 32 * 1024;         // per instantiation: the most dynamic LDS asked for so far
-    if (lds > granted) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)SLIM_NORM_LDS_MAX);
-        if (e != hipSuccess) return gi_fail("gemm_bf16 (slim): %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
-        granted = SLIM_NORM_LDS_MAX;
-    }
-    kernel<<<grid, 512, lds, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, X, ldx, x_rows, norm_w, norm_w_bf16, eps);
-    GI_CHECK_LAUNCH("gemm_bf16 (slim)");
-    return 0;
-}
-
-// X == nullptr: A holds the bfloat16 activations.  Otherwise A is unused and X (with norm_w, eps) is normalised in the kernel.
-int launch_slim(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, const float* X, long ldx,
-                const int* x_rows, const void* norm_w, int norm_w_bf16, float eps, hipStream_t stream) {
-    const bool norm = X != nullptr;
-    const size_t lds = norm ? (size_t)M * (K + 8) * sizeof(bf16_t) : 0;
-#define ARGS A, W, C, M, N, K, lda, ldw, ldc, X, ldx, x_rows, norm_w, norm_w_bf16, eps, stream
-#define PICK(STRIPS_, ROWS_, EPI_) (norm ? launch_slim_one<STRIPS_, ROWS_, EPI_, true>(grid, lds, ARGS) : launch_slim_one<STRIPS_, ROWS_, EPI_, false>(grid, lds, ARGS))
-    if (epi == EPI_GATED_BF16) {
-        dim3 grid(N / 32);
-        return PICK(2, 16, EPI_GATED_BF16);
-    }
-    if ((N + 15) / 16 >= 256) {
-        dim3 grid((N + 15) / 16);
-        if (epi == EPI_STORE_F32) return PICK(1, 16, EPI_STORE_F32);
-        if (epi == EPI_ADD_F32) return PICK(1, 16, EPI_ADD_F32);
-        return PICK(1, 16, EPI_STORE_BF16);
-    }
-    dim3 grid((N + 7) / 8);                    // a narrow output: strips of 8 rows, twice the workgroups
-    if (epi == EPI_STORE_F32) return PICK(1, 8, EPI_STORE_F32);
-    if (epi == EPI_ADD_F32) return PICK(1, 8, EPI_ADD_F32);
-    return PICK(1, 8, EPI_STORE_BF16);
-#undef PICK
-#undef ARGS
 }
 
 int epilogue_of(int c_dtype, int accumulate) {
@@ -397,7 +310,23 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     }
     GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
 
-    if (M <= 16) return launch_slim(A, W, C, epi, M, N, K, lda, ldw, ldc, nullptr, 0, nullptr, nullptr, 0, 0.f, stream);
+    if (M <= 16) {
+#define SLIM(STRIPS_, ROWS_, EPI_) \
+    gemm_bf16_slim_kernel<STRIPS_, ROWS_, EPI_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
+        if (epi == EPI_GATED_BF16) {
+            dim3 grid(N / 32);
+            SLIM(2, 16, EPI_GATED_BF16);
+        } else if ((N + 15) / 16 >= 256) {
+            dim3 grid((N + 15) / 16);
+            if (epi == EPI_STORE_F32) SLIM(1, 16, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 16, EPI_ADD_F32); else SLIM(1, 16, EPI_STORE_BF16);
+        } else {                                   // a narrow output: strips of 8 rows, twice the workgroups
+            dim3 grid((N + 7) / 8);
+            if (epi == EPI_STORE_F32) SLIM(1, 8, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 8, EPI_ADD_F32); else SLIM(1, 8, EPI_STORE_BF16);
+        }
+#undef SLIM
+        GI_CHECK_LAUNCH("gemm_bf16 (slim)");
+        return 0;
+    }
 
     if (M <= 64 && !gated) {
         const int splits = gi_gemm_bf16_skinny_splits(N, K);
@@ -433,26 +362,4 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
 #undef TILED
     GI_CHECK_LAUNCH("gemm_bf16 (tiled)");
     return 0;
-}
-
-// The same product for at most 16 rows with the RMS norm of the 32-bit rows X applied inside the kernel:
-// C (=|+=) rmsnorm(X[x_rows], norm_w, eps) @ W.T.  Returns 1 from the *_supports call if the shape fits.
-GI_API int gi_gemm_bf16_normed_supports(int M, int K) {
-    return M >= 1 && M <= 16 && K % 8 == 0 && (size_t)M * (K + 8) * sizeof(bf16_t) <= SLIM_NORM_LDS_MAX;
-}
-
-GI_API int gi_gemm_bf16_normed(const float* X, long ldx, const int* x_rows, const void* norm_w, int norm_w_dtype, float eps, const void* W, void* C,
-                               int c_dtype, int accumulate, int gated, int M, int N, int K, long ldw, long ldc, hipStream_t stream) {
-    GI_REQUIRE(gi_gemm_bf16_normed_supports(M, K), "gemm_bf16_normed: %d rows of %d are not supported (at most 16 rows, K a multiple of 8)", M, K);
-    GI_REQUIRE(N > 0 && ldw % 8 == 0 && ldw >= K && ldx >= K && ldx % 4 == 0, "gemm_bf16_normed: bad sizes or strides");
-    GI_REQUIRE(((uintptr_t)X & 15) == 0 && ((uintptr_t)W & 15) == 0 && ((uintptr_t)norm_w & 15) == 0, "gemm_bf16_normed: operands must be 16-byte aligned");
-    GI_REQUIRE(norm_w_dtype == GI_F32 || norm_w_dtype == GI_BF16, "gemm_bf16_normed: unknown norm weight dtype %d", norm_w_dtype);
-    GI_REQUIRE(ldc >= (gated ? N / 2 : N), "gemm_bf16_normed: leading dimension of the output too small");
-    int epi = epilogue_of(c_dtype, accumulate);
-    if (gated) {
-        GI_REQUIRE(N % 32 == 0 && c_dtype == GI_BF16 && !accumulate, "gemm_bf16_normed: the gated product needs N %% 32 == 0 and a bfloat16 output");
-        epi = EPI_GATED_BF16;
-    }
-    GI_REQUIRE(epi >= 0, "gemm_bf16_normed: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
-    return launch_slim(nullptr, W, C, epi, M, N, K, 0, ldw, ldc, X, ldx, x_rows, norm_w, norm_w_dtype == GI_BF16 ? 1 : 0, eps, stream);
 }

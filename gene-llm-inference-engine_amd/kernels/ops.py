@@ -21,7 +21,7 @@ class KernelError(RuntimeError):
 
 _SIGNATURES = {
     "gi_embed": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
-    "gi_rmsnorm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_long, c_long, c_void_p],
+    "gi_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_long, c_long, c_void_p],
     "gi_rope_cos_sin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "gi_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                       c_int, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -35,8 +35,6 @@ _SIGNATURES = {
                                  c_float, c_void_p],
     "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long,
                                  c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
-    "gi_gemm_bf16_normed": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                            c_long, c_long, c_void_p],
     "gi_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
 }
@@ -52,8 +50,6 @@ def lib():
             fn = getattr(l, name)
             fn.argtypes = sig
             fn.restype = c_int
-        l.gi_gemm_bf16_normed_supports.argtypes = [c_int, c_int]
-        l.gi_gemm_bf16_normed_supports.restype = c_int
         l.gi_argmax_chunks.argtypes = [c_int]
         l.gi_argmax_chunks.restype = c_int
         l.gi_attention_bf16_supports.argtypes = [c_int, c_int, c_int]
@@ -123,14 +119,24 @@ def embed(table, tokens, out):
     return out
 
 
-def rmsnorm(x, weight, eps, out):
-    """out = weight * (x * rsqrt(mean(x^2) + eps)) per row; x float32 [n, dim]."""
-    _dev(x, weight, out)
-    n, dim = x.shape
+def rmsnorm_can_gather(x, weight, out) -> bool:
+    dim = x.shape[1]
+    return (dim % 4 == 0 and dim <= 4096 and x.stride(0) % 4 == 0 and out.stride(0) % 4 == 0 and x.data_ptr() % 16 == 0
+            and weight.data_ptr() % 16 == 0 and out.data_ptr() % 16 == 0)
+
+
+def rmsnorm(x, weight, eps, out, rows=None):
+    """out = weight * (x * rsqrt(mean(x^2) + eps)) per row; x float32 [n, dim].  rows: int32 indices, out[i] = norm(x[rows[i]])."""
+    _dev(x, weight, out, rows)
+    dim = x.shape[1]
+    n = x.shape[0] if rows is None else rows.numel()
     _need(x.dtype == torch.float32 and x.stride(1) == 1, "rmsnorm: x must be float32 with unit inner stride")
-    _need(out.shape == x.shape and out.stride(1) == 1, "rmsnorm: out must have x's shape and unit inner stride")
+    _need(out.shape == (n, dim) and out.stride(1) == 1, "rmsnorm: out must be [rows, dim] with unit inner stride")
     _need(weight.shape == (dim,) and weight.is_contiguous(), "rmsnorm: weight must be [dim]")
-    _call("gi_rmsnorm", x.data_ptr(), weight.data_ptr(), _code(weight, "rmsnorm: weight"), out.data_ptr(), _code(out, "rmsnorm: out"),
+    if rows is not None:
+        _i32(rows, "rmsnorm: rows", n)
+        _need(rmsnorm_can_gather(x, weight, out), "rmsnorm: these operands cannot be gathered in the kernel")
+    _call("gi_rmsnorm", x.data_ptr(), _ptr(rows), weight.data_ptr(), _code(weight, "rmsnorm: weight"), out.data_ptr(), _code(out, "rmsnorm: out"),
           n, dim, float(eps), x.stride(0), out.stride(0), _stream())
     return out
 
@@ -329,31 +335,6 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False):
         scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device)
     _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,
           m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _stream())
-    return out
-
-
-def gemm_bf16_normed_supports(x, norm_weight, w, out, n_rows) -> bool:
-    k = x.shape[1]
-    return (x.dtype == torch.float32 and x.stride(1) == 1 and x.stride(0) % 4 == 0 and x.data_ptr() % 16 == 0 and w.dtype == torch.bfloat16
-            and w.stride(1) == 1 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0 and norm_weight.data_ptr() % 16 == 0
-            and norm_weight.dtype in _CODE and out.stride(1) == 1 and bool(lib().gi_gemm_bf16_normed_supports(n_rows, k)))
-
-
-def gemm_bf16_normed(x, norm_weight, eps, w, out, accumulate=False, gated=False, rows=None):
-    """out (=|+=) rmsnorm(x[rows]) @ w.T for at most 16 rows, the norm applied inside the product's kernel.
-    x float32 [n, k]; rows: int32 indices of the rows to take (all of x if None)."""
-    _dev(x, norm_weight, w, out, rows)
-    k = x.shape[1]
-    m = x.shape[0] if rows is None else rows.numel()
-    n = w.shape[0]
-    _need(w.shape == (n, k) and norm_weight.shape == (k,) and norm_weight.is_contiguous(), "gemm_normed: shapes of the weights do not fit the rows")
-    _need(out.shape == (m, n // 2 if gated else n), f"gemm_normed: out is {tuple(out.shape)}, ({m}, {n // 2 if gated else n}) is needed")
-    _need(gemm_bf16_normed_supports(x, norm_weight, w, out, m), "gemm_normed: unsupported operands (float32 rows, bfloat16 weights, at most 16 rows)")
-    if rows is not None:
-        _i32(rows, "gemm_normed: rows", m)
-    _call("gi_gemm_bf16_normed", x.data_ptr(), x.stride(0), _ptr(rows), norm_weight.data_ptr(), _code(norm_weight, "gemm_normed: norm weight"),
-          float(eps), w.data_ptr(), out.data_ptr(), _code(out, "gemm_normed: out"), 1 if accumulate else 0, 1 if gated else 0, m, n, k,
-          w.stride(0), out.stride(0), _stream())
     return out
 
 

@@ -2,7 +2,9 @@
 as checkpoints store them (no bias).  The kernel is chosen by the operands' storage: 32-bit
 operands take the exact kernel; bfloat16 operands take the matrix-core kernels where their
 shape rules allow and the exact kernel otherwise.  `a` may be a norm not yet applied
-(`NormedRows`): for a few rows it is applied inside the product's kernel."""
+(`NormedRows`); it is applied here, by the norm's own kernel (which also gathers the rows it names).
+Applying it inside the product's kernel was measured and did not pay: as a prologue it costs what the
+separate kernel costs, and commuted into the epilogue it makes the product's loop twice as slow."""
 from __future__ import annotations
 
 import torch
@@ -14,8 +16,6 @@ from .norm import NormedRows
 def linear(a, weight: torch.Tensor, out: torch.Tensor, accumulate: bool = False, gated: bool = False) -> torch.Tensor:
     """gated: weight is [gate; up] interleaved by `ops.interleave_gate_up` and out = silu(gate) * up (bfloat16 only)."""
     if isinstance(a, NormedRows):
-        if a.out_dtype == torch.bfloat16 and ops.gemm_bf16_normed_supports(a.x, a.norm.weight, weight, out, a.n_rows):
-            return ops.gemm_bf16_normed(a.x, a.norm.weight, a.norm.eps, weight, out, accumulate, gated, a.rows)
         a = a.materialize()
     if a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and ops.gemm_bf16_supports(a, weight, out):
         return ops.gemm_bf16(a, weight, out, accumulate, gated)

@@ -1,9 +1,9 @@
 """RMS norm: out = w * (x * rsqrt(mean(x^2) + eps)), eps inside the root, the weight as stored
 (reference: src/kernels/kernels.cpp:72-83).
 
-A norm may be handed on *unapplied* (`deferred`): `NormedRows` names the rows, the weight and eps,
-and the matrix product that consumes it applies the norm inside its own kernel when the batch is
-small enough for that (decode), or asks for the rows (`materialize`) otherwise."""
+A norm may be handed on *unapplied* (`deferred`): `NormedRows` names the rows (optionally a
+selection of them), the weight and eps; whoever consumes it asks for the rows (`materialize`), and
+the norm's kernel gathers the selection itself."""
 from __future__ import annotations
 
 import torch
@@ -23,10 +23,7 @@ class NormedRows:
 
     def materialize(self) -> torch.Tensor:
         if self._value is None:
-            x = self.x
-            if self.rows is not None:
-                x = ops.gather_rows(self.x, self.rows, torch.empty((self.n_rows, self.x.shape[1]), dtype=torch.float32, device=self.x.device))
-            self._value = self.norm(x, self.out_dtype)
+            self._value = self.norm(self.x, self.out_dtype, self.rows)
         return self._value
 
 
@@ -42,9 +39,13 @@ class RmsNorm(Norm):
     def tensor_needs(cls, spec):
         return [TensorNeed(spec.weight, (spec.size,), "norm")]
 
-    def __call__(self, x, out_dtype):
-        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
-        return ops.rmsnorm(x, self.weight, self.eps, out)
+    def __call__(self, x, out_dtype, rows=None):
+        """The normed rows of x, or of x[rows]."""
+        n = x.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, x.shape[1]), dtype=out_dtype, device=x.device)
+        if rows is not None and not ops.rmsnorm_can_gather(x, self.weight, out):
+            x, rows = ops.gather_rows(x, rows, torch.empty((n, x.shape[1]), dtype=torch.float32, device=x.device)), None
+        return ops.rmsnorm(x, self.weight, self.eps, out, rows)
 
     def deferred(self, x, out_dtype, rows=None) -> NormedRows:
         return NormedRows(self, x, out_dtype, rows)

@@ -101,3 +101,21 @@ def relative_error(got, want) -> float:
     got = torch.as_tensor(got).double().cpu()
     want = torch.as_tensor(want).double().cpu()
     return float((got - want).abs().max() / want.abs().max().clamp_min(1e-30))
+
+
+def assert_within_bfloat16_noise(got: dict, exact, rounded, what=""):
+    """The criterion for whole-model logits in bfloat16.
+
+    `got[key]` are the engine's rows, `exact(key)` the 64-bit plain model's, `rounded(key)` those of the
+    plain model that rounds to bfloat16 where the engine stores bfloat16.  One value that falls on the
+    other side of a rounding edge changes everything after it by the size of the rounding noise, so the
+    rounding plain model is no tighter a reference than the exact one; what can be asked is that the
+    engine is as close to the exact model as rounding alone explains: its mean error within 1.5x and
+    its worst error within 2x of the rounding plain model's.  A fault of masking, paging or order shows
+    as errors many times the noise."""
+    errors = [relative_error(row, exact(key)) for key, row in got.items()]
+    noise = [relative_error(rounded(key), exact(key)) for key in got]
+    mean_e, mean_n = sum(errors) / len(errors), sum(noise) / len(noise)
+    assert mean_e < 1.5 * mean_n + 1e-4, f"{what}: mean error {mean_e:.3e} against rounding noise {mean_n:.3e}"
+    assert max(errors) < 2.0 * max(noise) + 1e-4, f"{what}: worst error {max(errors):.3e} against rounding noise {max(noise):.3e}"
+    return mean_e, mean_n

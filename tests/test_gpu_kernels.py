@@ -295,31 +295,3 @@ def test_rope_store_writes_the_right_places():
         touched[page, 0, :, place, :] = True
         touched[page, 1].view(n_kv, hd, ps)[:, :, place] = True
     assert torch.all(cache[~touched] == -777.25), "rope_store wrote outside its places"
-
-
-@pytest.mark.parametrize("m,n,k", [(1, 16, 8), (3, 100, 136), (8, 3072, 2048), (16, 130, 264), (5, 64, 96), (13, 4096, 4096)])
-@pytest.mark.parametrize("w_dtype", [torch.float32, torch.bfloat16])
-def test_gemm_bf16_with_the_norm_inside(m, n, k, w_dtype):
-    o = ops()
-    x = randn(m + 3, k, seed=21, scale=3.0)
-    nw = (1 + 0.1 * randn(k, seed=22)).to(w_dtype)
-    w = randn(n, k, dtype=torch.bfloat16, seed=23, scale=0.2)
-    rows = torch.arange(m + 2, 2 - 1, -1, dtype=torch.int32, device=DEV)[:m]            # some rows, backwards
-    for eps in (1e-6, 0.05):
-        xd = x[rows.long()].double()
-        h = (nw.double() * (xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + eps))).to(torch.bfloat16).double()
-        out = torch.empty(m, n, device=DEV)
-        o.gemm_bf16_normed(x, nw, eps, w, out, rows=rows)
-        assert rel(out, h @ w.double().T) < 3e-3, (m, n, k)        # the norm's own rounding to bfloat16 may differ by one step here and there
-    base = randn(m, n, seed=24)
-    out = base.clone()
-    o.gemm_bf16_normed(x[:m], nw, 1e-5, w, out, accumulate=True)
-    xd = x[:m].double()
-    h = (nw.double() * (xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + 1e-5))).to(torch.bfloat16).double()
-    assert rel(out, base.double() + h @ w.double().T) < 3e-3
-    if n % 32 == 0:
-        gate_up = o.interleave_gate_up(w[:n // 2].contiguous(), w[n // 2:].contiguous())
-        mid = torch.empty(m, n // 2, dtype=torch.bfloat16, device=DEV)
-        o.gemm_bf16_normed(x[:m], nw, 1e-5, gate_up, mid, gated=True)
-        want = torch.nn.functional.silu(h @ w[:n // 2].double().T) * (h @ w[n // 2:].double().T)
-        assert rel(mid, want) < 8e-3

@@ -8,7 +8,7 @@ import torch
 
 import toy_architecture as toy
 import traces
-from model_folders import relative_error
+from model_folders import assert_within_bfloat16_noise, relative_error
 from plain_llama import causal_attention, read_model_folder, rms_norm, rope_inverse_frequencies, rope_rotate, swiglu
 
 pytestmark = pytest.mark.gpu
@@ -176,9 +176,11 @@ def test_toy_architecture_under_every_cut(toy_model, dtype, mode):
         held = [sum(len(g.held_pages(runner.cache.slot(r))) for r in runner.cache.open_requests()) for g in groups]
         assert held[1] <= len(runner.cache.open_requests()) * (2 + (cfg.window + 8) // runner.page_size + 1)     # windowed pages are given back
     assert runner.cache.free_pages() == [g.pool.n_pages for g in groups]
-    store = (lambda t: t.to(torch.bfloat16).double()) if dtype == "bfloat16" else (lambda t: t)
-    worst = 0.0
-    for rid, toks in requests.items():
-        want = toy.plain_logits(cfg, weights, toks, store=store)
-        worst = max(worst, max(relative_error(got[(rid, p)], want[p]) for p in range(len(toks))))
-    assert worst < (2e-5 if dtype == "float32" else 2e-2), worst
+    exact = {rid: toy.plain_logits(cfg, weights, toks) for rid, toks in requests.items()}
+    if dtype == "float32":
+        worst = max(relative_error(row, exact[rid][p]) for (rid, p), row in got.items())
+        assert worst < 2e-5, worst
+    else:
+        rounded = {rid: toy.plain_logits(cfg, weights, toks, store=lambda t: t.to(torch.bfloat16).double()) for rid, toks in requests.items()}
+        assert_within_bfloat16_noise(got, lambda k: exact[k[0]][k[1]], lambda k: rounded[k[0]][k[1]], mode)
+    assert runner.use_graphs is False                                 # the toy mixer reads host-side step data: no step of this model is captured

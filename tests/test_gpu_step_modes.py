@@ -7,17 +7,15 @@ import pytest
 import torch
 
 import traces
-from model_folders import CONFIGS, PAGE_SIZE, relative_error, write_model
+from model_folders import CONFIGS, PAGE_SIZE, assert_within_bfloat16_noise, relative_error, write_model
 from plain_llama import PlainLlama
 
 pytestmark = pytest.mark.gpu
 
-# float32 is compared with the plain model in 64-bit.  bfloat16 is compared with the plain model
-# rounding to bfloat16 at the same places as the engine (a tight bound: what is left is the order
-# of 32-bit sums and values that fall on the other side of a rounding edge), and with the exact
-# 64-bit model under a loose bound that only says the logits are the same function.
-TOLERANCE = {"float32": 2e-5, "bfloat16": 1.5e-2}
-LOOSE_BF16 = 0.12
+# float32 is compared with the plain model in 64-bit.  bfloat16 is held against the rounding noise
+# of a plain model that rounds to bfloat16 where the engine stores bfloat16 (see
+# `assert_within_bfloat16_noise`).
+TOLERANCE = {"float32": 2e-5}
 LENGTHS = {"A": [5, 11, 17, 70, 45], "B": [1, 9, 33, 40, 75, 51], "C": [3, 66, 37, 50]}
 
 
@@ -90,12 +88,12 @@ def test_step_modes(case, dtype, mode):
     max_tokens = traces.peak_tokens(steps, round_to=ps)          # so few pages that they are used again
     got = replay(folder, dtype, steps, ps, max_tokens)
     assert len(got) == sum(len(t) for t in requests.values())
-    worst = check(got, want[dtype], dtype)
-    if dtype == "bfloat16":
-        loose = max(relative_error(row, want["float32"][rid][pos]) for (rid, pos), row in got.items())
-        assert loose < LOOSE_BF16, f"bfloat16 against the exact model: {loose:.3e}"
-        print(f"  against the exact model: {loose:.2e}")
-    print(f"{name} {dtype} {mode}: worst relative error {worst:.2e}, {len(steps)} steps, pool of {max_tokens} positions")
+    if dtype == "float32":
+        worst = check(got, want[dtype], dtype)
+        print(f"{name} {dtype} {mode}: worst relative error {worst:.2e}, {len(steps)} steps, pool of {max_tokens} positions")
+    else:
+        mean_e, mean_n = assert_within_bfloat16_noise(got, lambda k: want["float32"][k[0]][k[1]], lambda k: want["bfloat16"][k[0]][k[1]], f"{name} {mode}")
+        print(f"{name} {dtype} {mode}: mean error {mean_e:.2e} (rounding noise {mean_n:.2e}), {len(steps)} steps, pool of {max_tokens} positions")
     if dtype == "float32":
         ref = _WHOLE.setdefault((name, "ref"), got if mode == "whole" else replay(folder, dtype, traces.whole(requests), ps, 4096))
         for key, row in got.items():
