@@ -20,7 +20,10 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 load16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ __forceinline__ uint2 load8(const bf16_t* p) { return *reinterpret_cast<const uint2*>(p); }
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
-__device__ __forceinline__ uint32_t pack2(float a, float b) { return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16); }
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return f32x2_to_bf16x2(a, b); }
+// e^x as 2^(x * log2 e): one multiply and the hardware's exp2.
+constexpr float LOG2E = 1.4426950408889634f;
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // =========================================================================================== prompt
 // Workgroup: 4 waves, a tile of up to 128 consecutive rows of one request (32 per wave), one query
@@ -32,18 +35,21 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) { return (uint32_t)f
 // tiles[i] = {first row in the step, number of rows, position of the first row, request slot}.
 constexpr int KV_TILE = 64;
 
-template <int HD>
-__global__ __launch_bounds__(256) void attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
-                                                              bf16_t* __restrict__ out, const int4* __restrict__ tiles,
-                                                              const int* __restrict__ table, int table_stride, long page_stride,
-                                                              int page_size, int n_heads, int n_kv, int window, float scale) {
+template <int HD, int NW>
+__global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
+                                                                  bf16_t* __restrict__ out, const int4* __restrict__ tiles,
+                                                                  const int* __restrict__ table, int table_stride, long page_stride,
+                                                                  int page_size, int n_heads, int n_kv, int window, float scale) {
+    constexpr int NT = 64 * NW;                 // threads; the tile has 32 * NW query rows
     constexpr int K_STRIDE = HD + 8;            // bf16 elements; 16-byte reads of 32 rows hit distinct banks
     constexpr int V_STRIDE = KV_TILE + 4;       // 8-byte reads of 32 rows hit distinct banks
     constexpr int QSTEPS = HD / 16, DT = HD / 32;
+    constexpr int CHUNKS = KV_TILE * HD / 8 / NT;           // 16-byte pieces of the keys (and of the values) per thread and tile
+    static_assert(KV_TILE * HD / 8 % NT == 0, "the tile must divide among the threads");
     __shared__ __attribute__((aligned(16))) bf16_t Ks[KV_TILE * K_STRIDE];
     __shared__ __attribute__((aligned(16))) bf16_t Vs[HD * V_STRIDE];
 
-    const int4 tile = tiles[blockIdx.x];
+    const int4 tile = tiles[gridDim.x - 1 - blockIdx.x];     // later tiles of a prompt see more keys: they start first
     const int row0 = tile.x, n_rows = tile.y, pos0 = tile.z, slot = tile.w;
     const int head = blockIdx.y, g = head / (n_heads / n_kv);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -56,6 +62,10 @@ __global__ __launch_bounds__(256) void attention_prompt_kernel(const bf16_t* __r
     const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
     const int wave_last = pos0 + min(n_rows, wave * 32 + 32) - 1;       // the last position this wave's rows see
     const bool wave_ok = wave * 32 < n_rows;
+    const bool wave_full = wave * 32 + 32 <= n_rows;
+    const int wave_first = wave_full ? pos0 + wave * 32 : -1;           // keys up to here are seen by every row of the wave (none if rows are missing)
+    const int wave_lo_max = window > 0 ? max(0, wave_last - window + 1) : 0;      // ... and keys from here on
+    const float scale2 = scale * LOG2E;
 
     bf16x8 qreg[QSTEPS];
 #pragma unroll
@@ -72,31 +82,61 @@ __global__ __launch_bounds__(256) void attention_prompt_kernel(const bf16_t* __r
     const int last_pos = pos0 + n_rows - 1;
     const int first_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
     const long v_plane = (long)n_kv * page_size * HD;
-    for (int kv0 = first_lo & ~(KV_TILE - 1); kv0 <= last_pos; kv0 += KV_TILE) {
-        __syncthreads();
-        // keys: 64 rows of HD, 16 bytes a thread at a time
-        for (int e = tid; e < KV_TILE * (HD / 8); e += 256) {
-            const int r = e / (HD / 8), c = (e % (HD / 8)) * 8, kv = kv0 + r;
-            uint4 v = {0, 0, 0, 0};
-            if (kv <= last_pos) {
-                const int page = tab[kv / page_size];
-                if (page >= 0) v = load16(cache + (long)page * page_stride + ((long)g * page_size + kv % page_size) * HD + c);
-            }
-            *reinterpret_cast<uint4*>(&Ks[r * K_STRIDE + c]) = v;
+
+    // A tile of 64 key positions travels global memory -> registers -> LDS; the next tile's loads are
+    // issued before the products of this one, and the page numbers they need one tile earlier still,
+    // so that neither the table lookup nor the load itself is waited for.
+    const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+    auto page_index = [&](int kv) { return page_shift >= 0 ? kv >> page_shift : kv / page_size; };
+    auto place_of = [&](int kv) { return page_shift >= 0 ? kv & (page_size - 1) : kv % page_size; };
+    uint4 k_reg[CHUNKS], v_reg[CHUNKS];
+    int k_page[CHUNKS], v_page[CHUNKS];
+    auto fetch_pages = [&](int kv0) {
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            const int e = tid + NT * i;
+            const int kv_k = kv0 + e / (HD / 8), kv_v = kv0 + (e / HD) * 8;
+            k_page[i] = kv_k <= last_pos ? tab[page_index(kv_k)] : -1;
+            v_page[i] = kv_v <= last_pos ? tab[page_index(kv_v)] : -1;
         }
-        // values, already transposed in the cache: HD rows of 64 positions, 8 positions a thread at a time
-        for (int e = tid; e < HD * (KV_TILE / 8); e += 256) {
-            const int d = e % HD, c = (e / HD) * 8, kv = kv0 + c;
-            uint4 v = {0, 0, 0, 0};
-            if (kv <= last_pos) {
-                const int page = tab[kv / page_size];
-                if (page >= 0) v = load16(cache + (long)page * page_stride + v_plane + ((long)g * HD + d) * page_size + kv % page_size);
+    };
+    auto fetch = [&](int kv0) {                 // with the pages that fetch_pages(kv0) brought
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            const int e = tid + NT * i;
+            {   // keys: 64 rows of HD
+                const int r = e / (HD / 8), c = (e % (HD / 8)) * 8, kv = kv0 + r;
+                k_reg[i] = k_page[i] >= 0 ? load16(cache + (long)k_page[i] * page_stride + ((long)g * page_size + place_of(kv)) * HD + c) : uint4{0, 0, 0, 0};
             }
-            uint2* dst = reinterpret_cast<uint2*>(&Vs[d * V_STRIDE + c]);
-            dst[0] = uint2{v.x, v.y};
-            dst[1] = uint2{v.z, v.w};
+            {   // values, already transposed in the cache: HD rows of 64 positions, 8 positions a piece
+                const int d = e % HD, c = (e / HD) * 8, kv = kv0 + c;
+                v_reg[i] = v_page[i] >= 0 ? load16(cache + (long)v_page[i] * page_stride + v_plane + ((long)g * HD + d) * page_size + place_of(kv)) : uint4{0, 0, 0, 0};
+            }
         }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int i = 0; i < CHUNKS; ++i) {
+            const int e = tid + NT * i;
+            *reinterpret_cast<uint4*>(&Ks[(e / (HD / 8)) * K_STRIDE + (e % (HD / 8)) * 8]) = k_reg[i];
+            uint2* dst = reinterpret_cast<uint2*>(&Vs[(e % HD) * V_STRIDE + (e / HD) * 8]);
+            dst[0] = uint2{v_reg[i].x, v_reg[i].y};
+            dst[1] = uint2{v_reg[i].z, v_reg[i].w};
+        }
+    };
+
+    const int kv_first = first_lo & ~(KV_TILE - 1);
+    fetch_pages(kv_first);
+    fetch(kv_first);
+    fetch_pages(kv_first + KV_TILE);            // beyond the last position: no lookups
+    for (int kv0 = kv_first; kv0 <= last_pos; kv0 += KV_TILE) {
+        __syncthreads();                        // the previous tile has been read by everyone
+        stash();
         __syncthreads();
+        if (kv0 + KV_TILE <= last_pos) {
+            fetch(kv0 + KV_TILE);
+            fetch_pages(kv0 + 2 * KV_TILE);
+        }
         if (!wave_ok) continue;
 #pragma unroll
         for (int st = 0; st < KV_TILE / 32; ++st) {
@@ -108,31 +148,41 @@ __global__ __launch_bounds__(256) void attention_prompt_kernel(const bf16_t* __r
                 const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(&Ks[(32 * st + col) * K_STRIDE + 16 * ks + 8 * hf]));
                 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[ks], s, 0, 0, 0);
             }
-            // element v of s: key position kv_base + 8*(v/4) + 4*hf + v%4, query row `col`
+            // element v of s: key position kv_base + 8*(v/4) + 4*hf + v%4, query row `col`.  Scores are kept
+            // in units of log2 e (scale2 = scale * log2 e), so that e^(s - m) is one exp2.
+            const bool inside = kv_base + 31 <= wave_first && kv_base >= wave_lo_max;     // every key of the tile is seen by every row of the wave
             float mx = -INFINITY;
+            if (inside) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int kv = kv_base + 8 * (v / 4) + 4 * hf + (v & 3);
-                s[v] = (kv <= my_pos && kv >= my_lo) ? s[v] * scale : -INFINITY;
-                mx = fmaxf(mx, s[v]);
+                for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[v]);
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int kv = kv_base + 8 * (v / 4) + 4 * hf + (v & 3);
+                    s[v] = (kv <= my_pos && kv >= my_lo) ? s[v] : -INFINITY;
+                    mx = fmaxf(mx, s[v]);
+                }
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale2;             // scale2 > 0: the maximum of the scaled scores
             const float m_new = fmaxf(m, mx);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;      // a row that has seen nothing yet
-            const float corr = expf(m - m_use);
             float sum = 0.f;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                s[v] = expf(s[v] - m_use);
+                s[v] = exp2_fast(fmaf(s[v], scale2, -m_use));
                 sum += s[v];
             }
             sum += __shfl_xor(sum, 32, 64);
-            l = l * corr + sum;
-            m = m_new;
+            if (__any(m_new != m)) {                                      // some row's maximum rose: rescale what was gathered so far
+                const float corr = exp2_fast(m - m_use);
+                l *= corr;
 #pragma unroll
-            for (int i = 0; i < DT; ++i)
+                for (int i = 0; i < DT; ++i)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) o[i][v] *= corr;
+                    for (int v = 0; v < 16; ++v) o[i][v] *= corr;
+                m = m_new;
+            }
+            l += sum;
 #pragma unroll
             for (int t = 0; t < 2; ++t) {                                 // two groups of 16 key positions
                 const uint4 pb = {pack2(s[8 * t], s[8 * t + 1]), pack2(s[8 * t + 2], s[8 * t + 3]), pack2(s[8 * t + 4], s[8 * t + 5]),
@@ -188,6 +238,10 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
     const int span = my_pos + 1 - (lo & ~31);
     const int split_len = (((span + n_splits - 1) / n_splits) + 31) & ~31;
     const int begin = (lo & ~31) + split * split_len, end = min(my_pos + 1, begin + split_len);
+    const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+    auto page_index = [&](int kv) { return page_shift >= 0 ? kv >> page_shift : kv / page_size; };
+    auto place_of = [&](int kv) { return page_shift >= 0 ? kv & (page_size - 1) : kv % page_size; };
+    const float scale2 = scale * LOG2E;            // scores are kept in units of log2 e: e^(s - m) is one exp2
 
     bf16x8 qreg[KSTEPS];
 #pragma unroll
@@ -212,7 +266,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int kv = min(max(kv0 + 16 * t + r, lo), my_pos);
-            const bf16_t* krow = kbase + (long)tab[kv / page_size] * page_stride + (long)(kv % page_size) * HD + 8 * q4;
+            const bf16_t* krow = kbase + (long)tab[page_index(kv)] * page_stride + (long)place_of(kv) * HD + 8 * q4;
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) dst[t][ks] = load16(krow + 32 * ks);
         }
@@ -221,8 +275,8 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
     for (int kv0 = begin; kv0 < end; kv0 += 32) {
         // slot e of this lane in the value product is key position kv0 + 16*(e/4) + 4*q4 + e%4
         const int kva = min(max(kv0 + 4 * q4, lo & ~3), my_pos & ~3), kvb = min(max(kv0 + 16 + 4 * q4, lo & ~3), my_pos & ~3);
-        const bf16_t* va = vbase + (long)tab[kva / page_size] * page_stride + kva % page_size + (long)r * page_size;
-        const bf16_t* vb = vbase + (long)tab[kvb / page_size] * page_stride + kvb % page_size + (long)r * page_size;
+        const bf16_t* va = vbase + (long)tab[page_index(kva)] * page_stride + place_of(kva) + (long)r * page_size;
+        const bf16_t* vb = vbase + (long)tab[page_index(kvb)] * page_stride + place_of(kvb) + (long)r * page_size;
         uint2 vx[DT], vy[DT];
 #pragma unroll
         for (int i = 0; i < DT; ++i) {
@@ -245,20 +299,20 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int kv = kv0 + 16 * t + 4 * q4 + v;
-                s[t][v] = (kv >= lo && kv < end) ? s[t][v] * scale : -INFINITY;
+                s[t][v] = (kv >= lo && kv < end) ? s[t][v] * scale2 : -INFINITY;
                 mx = fmaxf(mx, s[t][v]);
             }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m, mx);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float corr = expf(m - m_use);
+        const float corr = exp2_fast(m - m_use);
         float sum = 0.f;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                s[t][v] = expf(s[t][v] - m_use);
+                s[t][v] = exp2_fast(s[t][v] - m_use);
                 sum += s[t][v];
             }
         sum += __shfl_xor(sum, 16, 64);
@@ -314,7 +368,7 @@ __global__ __launch_bounds__(64) void attention_decode_combine_kernel(const floa
     for (int i = 0; i < MAX_SPLITS / 64; ++i) {
         const int s = lane + 64 * i;
         if (s < n_splits) {
-            const float w = (mine_m[i] == -INFINITY) ? 0.f : expf(mine_m[i] - big);
+            const float w = (mine_m[i] == -INFINITY) ? 0.f : exp2_fast(mine_m[i] - big);      // the splits' maxima are in units of log2 e
             weight[s] = w;
             weighted_l[s] = w * mine_l[i];
         }
@@ -339,17 +393,26 @@ GI_API int gi_attention_bf16_supports(int hd, int page_size, int prompt) {
     return hd == 32 || hd == 64 || hd == 96 || hd == 128 || hd == 256;
 }
 
-GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out, const int* tiles, int n_tiles, const int* table,
-                                    int table_stride, long page_stride, int page_size, int n_heads, int n_kv, int hd, int window,
-                                    float scale, hipStream_t stream) {
+// tiles hold at most `rows_per_tile` rows each (64 or 128).
+GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out, const int* tiles, int n_tiles, int rows_per_tile,
+                                    const int* table, int table_stride, long page_stride, int page_size, int n_heads, int n_kv, int hd,
+                                    int window, float scale, hipStream_t stream) {
+    GI_REQUIRE(rows_per_tile == 64 || rows_per_tile == 128, "attention_prompt: tiles of %d rows are not supported (64 or 128)", rows_per_tile);
     GI_REQUIRE(n_tiles > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_prompt: bad counts (%d tiles, %d heads, %d kv heads)",
                n_tiles, n_heads, n_kv);
     GI_REQUIRE(gi_attention_bf16_supports(hd, page_size, 1), "attention_prompt: head size %d with page size %d is not supported", hd, page_size);
     GI_REQUIRE(page_stride >= 2L * n_kv * page_size * hd && page_stride % 8 == 0, "attention_prompt: bad page stride %ld", page_stride);
     GI_REQUIRE(n_heads <= 65535, "attention_prompt: too many heads");
     dim3 grid(n_tiles, n_heads);
-#define GO(HD) attention_prompt_kernel<HD><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, \
-                                                                     table, table_stride, page_stride, page_size, n_heads, n_kv, window, scale)
+#define GO(HD)                                                                                                                          \
+    do {                                                                                                                                \
+        if (rows_per_tile == 64)                                                                                                        \
+            attention_prompt_kernel<HD, 2><<<grid, 128, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
+                                                                     table_stride, page_stride, page_size, n_heads, n_kv, window, scale); \
+        else                                                                                                                            \
+            attention_prompt_kernel<HD, 4><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
+                                                                     table_stride, page_stride, page_size, n_heads, n_kv, window, scale); \
+    } while (0)
     if (hd == 32) GO(32); else if (hd == 64) GO(64); else if (hd == 96) GO(96); else GO(128);
 #undef GO
     GI_CHECK_LAUNCH("attention_prompt");

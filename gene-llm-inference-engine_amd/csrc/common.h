@@ -30,13 +30,14 @@ int gi_fail(const char* fmt, ...);
 
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
-// Round to nearest, ties to even; NaN stays NaN.
-__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
+// Round to nearest, ties to even; NaN stays NaN.  gfx950 converts in hardware (v_cvt_pk_bf16_f32).
+typedef __bf16 gi_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float gi_floatx2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
+    const gi_floatx2 f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, gi_bf16x2));
 }
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) { return (bf16_t)(f32x2_to_bf16x2(f, 0.f) & 0xffffu); }
 
 __device__ __forceinline__ float load_f32(const float* p, size_t i) { return p[i]; }
 __device__ __forceinline__ float load_f32(const bf16_t* p, size_t i) { return bf16_to_f32(p[i]); }

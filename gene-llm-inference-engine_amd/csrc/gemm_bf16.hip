@@ -288,6 +288,10 @@ int epilogue_of(int c_dtype, int accumulate) {
 
 // Number of k-splits the skinny kernel would use, so that the caller can size the scratch
 // (splits * M * N floats).  Enough workgroups to cover the chip, each with at least 256 of k.
+// Tuning knob: 0 lets the entry point choose the tile height of the tiled kernel, 64 or 128 forces it.
+static int g_force_bm = 0;
+GI_API void gi_gemm_bf16_set_tile(int bm) { g_force_bm = bm; }
+
 GI_API int gi_gemm_bf16_skinny_splits(int N, int K) {
     const int strips = (N + 63) / 64;
     int splits = 1;
@@ -350,7 +354,7 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
 
     GI_REQUIRE((M + 63) / 64 <= 65535, "gemm_bf16: M %d is too large", M);
 #define TILED(BM_, EPI_) gemm_bf16_tiled_kernel<BM_, EPI_><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
-    if (M <= 64 * 8 && (long)((M + 127) / 128) * ((N + BN - 1) / BN) < 256) {       // few rows: smaller tiles fill more of the chip
+    if (g_force_bm == 64 || (g_force_bm == 0 && (long)((M + 127) / 128) * ((N + BN - 1) / BN) < 512)) {   // few tiles: smaller ones fill more of the chip
         dim3 grid((N + BN - 1) / BN, (M + 63) / 64);
         if (epi == EPI_STORE_F32) TILED(64, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(64, EPI_ADD_F32);
         else if (epi == EPI_STORE_BF16) TILED(64, EPI_STORE_BF16); else TILED(64, EPI_GATED_BF16);

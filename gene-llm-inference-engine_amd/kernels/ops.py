@@ -31,7 +31,7 @@ _SIGNATURES = {
     "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
                            c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
-    "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
+    "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_void_p],
     "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long,
                                  c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
@@ -240,7 +240,7 @@ class AttentionPlan:
     """How a step's rows are shared between the two bfloat16 attention kernels: requests that bring
     one row go to the decode kernel, portions of prompts are cut into tiles of up to 128 rows for
     the prompt kernel.  Made once per step and used by every layer."""
-    TILE = 128
+    TILE = int(__import__("os").environ.get("GI_ATTENTION_TILE", "128"))      # rows of a prompt tile: 64 or 128
 
     @classmethod
     def all_decode(cls, n_rows, max_context, device):
@@ -286,7 +286,7 @@ def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, 
     window = int(window or 0)
     scale = float(scale if scale is not None else hd ** -0.5)
     if plan.n_tiles:
-        _call("gi_attention_prompt_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles,
+        _call("gi_attention_prompt_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles, plan.TILE,
               table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, _stream())
     if plan.n_decode:
         span = plan.max_decode_context if not window else min(plan.max_decode_context, window + 31)
