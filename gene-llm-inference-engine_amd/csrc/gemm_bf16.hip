@@ -208,6 +208,22 @@ __global__ void skinny_reduce_kernel(const float* __restrict__ P, void* __restri
     write_out<EPI>(C, (i / N) * ldc + (i % N), s);
 }
 
+// The same for the gated product: columns 32b .. 32b+15 of the partial sums are gates, 32b+16 .. 32b+31 the ups of
+// outputs 16b .. 16b+15; the output [M, N/2] is silu(gate) * up in bfloat16.
+__global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* __restrict__ C, int M, int N, int splits, long ldc) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int half = N / 2;
+    if (i >= (size_t)M * half) return;
+    const size_t m = i / half;
+    const int c = (int)(i % half), col = (c >> 4) * 32 + (c & 15);
+    float gate = 0.f, up = 0.f;
+    for (int sp = 0; sp < splits; ++sp) {
+        gate += P[((size_t)sp * M + m) * N + col];
+        up += P[((size_t)sp * M + m) * N + col + 16];
+    }
+    C[m * ldc + c] = f32_to_bf16(silu_gate(gate, up));
+}
+
 // ------------------------------------------------------------------------------------------- slim
 // At most 16 rows of A.  Workgroup: 8 waves = STRIPS strips of ROWS weight rows x (8 / STRIPS)
 // slices of k; slice s takes the 128-wide blocks of k numbered s, s + slices, ...  Both operands go
@@ -332,7 +348,7 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
         return 0;
     }
 
-    if (M <= 64 && !gated) {
+    if (M <= 64) {
         const int splits = gi_gemm_bf16_skinny_splits(N, K);
         GI_REQUIRE(scratch != nullptr && scratch_floats >= (long)splits * M * N, "gemm_bf16: scratch of %ld floats needed, %ld given",
                    (long)splits * M * N, scratch_floats);
@@ -345,7 +361,8 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
 #undef SKINNY
         GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
         const unsigned blocks = (unsigned)(((size_t)M * N + 255) / 256);
-        if (epi == EPI_STORE_F32) skinny_reduce_kernel<EPI_STORE_F32><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
+        if (epi == EPI_GATED_BF16) skinny_reduce_gated_kernel<<<(unsigned)(((size_t)M * (N / 2) + 255) / 256), 256, 0, stream>>>(scratch, (bf16_t*)C, M, N, splits, ldc);
+        else if (epi == EPI_STORE_F32) skinny_reduce_kernel<EPI_STORE_F32><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
         else if (epi == EPI_ADD_F32) skinny_reduce_kernel<EPI_ADD_F32><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
         else skinny_reduce_kernel<EPI_STORE_BF16><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
         GI_CHECK_LAUNCH("gemm_bf16 (reduce)");
