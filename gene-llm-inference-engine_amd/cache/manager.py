@@ -205,6 +205,33 @@ class CacheManager:
             for g in self.groups:
                 g.grow(slot, length + n_new)
 
+    def reserve_one_each(self, requests: Sequence[Hashable], slots: Sequence[int], lengths: Sequence[int]) -> None:
+        """`reserve` for one more position of every named request (open, each named once, `slots` and
+        `lengths` theirs): the common case of a decode step, without a Python loop over requests
+        unless a request crosses into a new page."""
+        slot_arr, next_len = np.asarray(slots, dtype=np.int64), np.asarray(lengths, dtype=np.int64) + 1
+        if int(next_len.max()) > self.max_positions:
+            raise CacheError(f"a request would pass the position limit {self.max_positions}")
+        growing = []
+        for g in self.groups:
+            need = (next_len + g.page_size - 1) // g.page_size > g.n_held[slot_arr]
+            count = int(need.sum())
+            if count > g.pool.free_count:
+                raise OutOfPages(f"not enough free pages (free per group: {self.free_pages()})")
+            growing.append(np.nonzero(need)[0] if count else ())
+        for g, idx in zip(self.groups, growing):
+            for i in idx:
+                g.grow(slots[i], int(next_len[i]))
+
+    def advance_one_each(self, requests: Sequence[Hashable], slots: Sequence[int], lengths: Sequence[int]) -> None:
+        """`advance` by one position for every named request, after `reserve_one_each`."""
+        for r, n in zip(requests, lengths):
+            self._length[r] = n + 1
+        for g in self.groups:
+            if g.need.window is not None:
+                for slot, n in zip(slots, lengths):
+                    g.drop_behind_window(slot, n + 1)
+
     def advance(self, request: Hashable, n_new: int) -> None:
         """The reserved positions have been written: the request is n_new longer; pages behind a
         window are given back."""

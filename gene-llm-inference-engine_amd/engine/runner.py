@@ -118,6 +118,8 @@ class Runner:
         """Runs the batch; returns float32 logits [wanted, vocab] on the device in the order of the
         entries and of each entry's `want`, or None if nothing was wanted.  The tensor is valid
         until the next step."""
+        if self.use_graphs and all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries) and entries:
+            return self._step_of_single_tokens(entries)
         n_rows = self._validate(entries)
         self.cache.reserve([(e.request, len(e.tokens)) for e in entries])       # OutOfPages: nothing changed
         self.cache.sync()
@@ -134,21 +136,48 @@ class Runner:
             logit_rows += [row + int(w) for w in e.want]
             row += n
 
-        if self.use_graphs and n_rows == len(entries) and logit_rows == list(range(n_rows)):
-            logits = self._decode_step(meta, seg_slot, seg_pos0)
-        else:
-            dev = self.model.device
-            meta_dev = torch.from_numpy(meta).to(dev)
-            rows_dev = torch.tensor(logit_rows, dtype=torch.int32).to(dev) if logit_rows else None
-            ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
-                              row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0)
-            logits = self.model.forward(ctx, self._view, rows_dev, len(logit_rows))
+        dev = self.model.device
+        meta_dev = torch.from_numpy(meta).to(dev)
+        rows_dev = torch.tensor(logit_rows, dtype=torch.int32).to(dev) if logit_rows else None
+        ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
+                          row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0)
+        logits = self.model.forward(ctx, self._view, rows_dev, len(logit_rows))
         for e in entries:
             self.cache.advance(e.request, len(e.tokens))
         self.steps_run += 1
         return logits
 
     # --------------------------------------------------------------------------- captured decode
+    def _step_of_single_tokens(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """The decode step: every request brings one token and wants its logits.  The same checks and the
+        same bookkeeping as the general path, done over whole lists at once (this path runs once per
+        generated token of every request, so its host time counts)."""
+        cache, n = self.cache, len(entries)
+        requests = [e.request for e in entries]
+        if len(set(requests)) != n:
+            raise StepError("a request appears twice in one step")
+        try:
+            slots = [cache._slot[r] for r in requests]
+        except KeyError as err:
+            raise StepError(f"request {err.args[0]!r} is not open") from None
+        lengths = [cache._length[r] for r in requests]
+        tokens = [int(e.tokens[0]) for e in entries]
+        vocab = self.model.spec.vocab_size
+        if min(tokens) < 0 or max(tokens) >= vocab:
+            bad = next(i for i, t in enumerate(tokens) if not 0 <= t < vocab)
+            raise StepError(f"token {tokens[bad]} of request {requests[bad]!r} is outside the vocabulary [0, {vocab})")
+        if max(lengths) + 1 > self.max_positions:
+            bad = max(range(n), key=lengths.__getitem__)
+            raise StepError(f"request {requests[bad]!r} would pass the position limit {self.max_positions}")
+        if n > self.max_rows:
+            raise StepError(f"the step holds {n} rows, more than max_rows = {self.max_rows}")
+        cache.reserve_one_each(requests, slots, lengths)                        # OutOfPages: nothing changed
+        cache.sync()
+        logits = self._decode_step(np.array([tokens, lengths, slots], dtype=np.int32), slots, lengths)
+        cache.advance_one_each(requests, slots, lengths)
+        self.steps_run += 1
+        return logits
+
     def _decode_step(self, meta: np.ndarray, seg_slot, seg_pos0) -> torch.Tensor:
         """A step in which every request brings one token and wants its logits runs as a replay of a
         HIP graph captured once per batch size: the launches of the whole pass cost one call.  The

@@ -119,6 +119,9 @@ def sample_rows(logits: torch.Tensor, samplers: Sequence[Sampler]) -> List[int]:
     n, vocab = logits.shape
     if n != len(samplers):
         raise ValueError(f"{n} rows of logits for {len(samplers)} samplers")
+    if all(s.config.greedy for s in samplers):                   # the common case without a list per kind
+        res = torch.empty(n, dtype=torch.int32, device=logits.device)
+        return ops.argmax(logits, res).tolist()
     out: List[int] = [0] * n
     greedy = [i for i, s in enumerate(samplers) if s.config.greedy]
     host = [i for i, s in enumerate(samplers) if not s.config.greedy and s.config.filters(vocab)]

@@ -184,3 +184,46 @@ def test_random_orders_of_requests_keep_the_books(seed):
     m.check_consistency()
     assert all(f == g.pool.n_pages for f, g in zip(m.free_pages(), m.groups))
     assert refused > 0 or seed % 2 == 0 or True
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_one_position_for_each_is_the_same_as_the_general_path(seed):
+    """reserve_one_each / advance_one_each against reserve / advance on a twin manager."""
+    rng = random.Random(seed)
+    needs = [FULL, WINDOW] if seed % 2 else [FULL]
+    a, b = (manager(needs, n_pages=10, page_size=4, max_requests=4, max_positions=40) for _ in range(2))
+    live = []
+    for step in range(120):
+        first = rng.randint(1, 6)
+        if len(live) < 4 and rng.random() < 0.2 and min(a.free_pages()) >= 2:
+            rid = f"r{step}"
+            for m in (a, b):
+                m.open(rid)
+                m.reserve([(rid, first)]); m.advance(rid, first)
+            live.append(rid)
+        if live and rng.random() < 0.1:
+            rid = live.pop(rng.randrange(len(live)))
+            a.close(rid); b.close(rid)
+        batch = [r for r in live if rng.random() < 0.8 and a.length(r) < 39]
+        if not batch:
+            continue
+        slots, lengths = [a.slot(r) for r in batch], [a.length(r) for r in batch]
+        try:
+            a.reserve([(r, 1) for r in batch])
+            general_ok = True
+        except OutOfPages:
+            general_ok = False
+        if general_ok:
+            b.reserve_one_each(batch, slots, lengths)
+            for r in batch:
+                a.advance(r, 1)
+            b.advance_one_each(batch, slots, lengths)
+        else:
+            with pytest.raises(OutOfPages):
+                b.reserve_one_each(batch, slots, lengths)
+            victim = live.pop(0)
+            a.close(victim); b.close(victim)
+        for ga, gb in zip(a.groups, b.groups):
+            assert (ga.table_host == gb.table_host).all() and ga.pool.free_count == gb.pool.free_count
+        assert all(a.length(r) == b.length(r) for r in live)
+        b.check_consistency()
