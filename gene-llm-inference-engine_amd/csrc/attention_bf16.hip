@@ -211,52 +211,113 @@ __global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t*
 }
 
 // =========================================================================================== decode
-// One wave per (row, key/value head, query-head group of up to 16, split of the context).  Keys and
-// values stream from global memory straight into the operands of v_mfma_f32_16x16x32_bf16; nothing
-// goes through LDS.  Scores: S[kv][head] = K * Q^T, 16 key positions at a time; output
-// O^T[d][head] = V^T * P^T, 32 key positions at a time.  Lane (r = lane%16, q4 = lane/16) owns
-// query head r of the group: its softmax statistics and its columns of S and O^T.
-// A split writes unnormalised partial results {m, l, O} to `part`; the combine kernel merges them.
+// One workgroup per (row, key/value head, query-head group of up to 16, split of the context); its
+// waves cut the split's range further, one piece each.  Keys and values stream from global memory
+// straight into the operands of v_mfma_f32_16x16x32_bf16.  Scores: S[kv][head] = K * Q^T, 16 key
+// positions at a time; output O^T[d][head] = V^T * P^T, 32 key positions at a time.  Lane
+// (r = lane%16, q4 = lane/16) owns query head r of the group: its softmax statistics and its
+// columns of S and O^T.  The waves' unnormalised results {m, l, O} meet in LDS and are merged in
+// wave order; with one split the workgroup writes the attention output itself, otherwise it writes
+// one partial result to `part` and the combine kernel merges the splits.
+//
+// FUSED: the queries, keys and values come unrotated in 32-bit, as the input product left them.
+// Every wave rotates its own queries.  The row's own key and value are not in the cache yet: the
+// wave whose piece ends at the row's position rotates the key, puts key and value into its
+// operands in place of what the cache holds there, and writes both to the row's page for later
+// steps (one store per element, by the first query-head group).
 template <int HD>
-__global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
-                                                             float* __restrict__ part, const int* __restrict__ rows,
-                                                             const int* __restrict__ pos, const int* __restrict__ slots,
-                                                             const int* __restrict__ table, int table_stride, long page_stride,
-                                                             int page_size, int n_heads, int n_kv, int window, float scale,
-                                                             int n_splits) {
+struct DecodeShape {                                      // waves a workgroup may have, by the registers a wave needs
+    static constexpr int MAX_WAVES = HD <= 128 ? 8 : 4;
+};
+
+// Channels c .. c+7 of a head and what their rotation needs, as loaded (`src` points at the head's
+// channel 0): the loads are issued early and the rotation is taken when the values are needed.
+struct Unrotated8 {
+    float4 a[2], b[2], cs[2], sn[2];
+    bool low;
+};
+__device__ __forceinline__ Unrotated8 load_unrotated8(const float* __restrict__ src, const float* __restrict__ cos_row,
+                                                      const float* __restrict__ sin_row, int c, int half) {
+    Unrotated8 u;
+    u.low = c < half;
+    const int cl = u.low ? c : c - half;
+#pragma unroll
+    for (int h4 = 0; h4 < 2; ++h4) {
+        u.a[h4] = *reinterpret_cast<const float4*>(src + cl + 4 * h4);
+        u.b[h4] = *reinterpret_cast<const float4*>(src + cl + half + 4 * h4);
+        u.cs[h4] = cos_row ? *reinterpret_cast<const float4*>(cos_row + cl + 4 * h4) : float4{1.f, 1.f, 1.f, 1.f};
+        u.sn[h4] = sin_row ? *reinterpret_cast<const float4*>(sin_row + cl + 4 * h4) : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    return u;
+}
+__device__ __forceinline__ float rotate1(bool low, float a, float b, float c, float s) { return low ? a * c - b * s : a * s + b * c; }
+__device__ __forceinline__ uint4 rotated8(const Unrotated8& u) {
+    uint32_t w[4];
+#pragma unroll
+    for (int h4 = 0; h4 < 2; ++h4) {
+        w[2 * h4] = pack2(rotate1(u.low, u.a[h4].x, u.b[h4].x, u.cs[h4].x, u.sn[h4].x), rotate1(u.low, u.a[h4].y, u.b[h4].y, u.cs[h4].y, u.sn[h4].y));
+        w[2 * h4 + 1] = pack2(rotate1(u.low, u.a[h4].z, u.b[h4].z, u.cs[h4].z, u.sn[h4].z), rotate1(u.low, u.a[h4].w, u.b[h4].w, u.cs[h4].w, u.sn[h4].w));
+    }
+    return uint4{w[0], w[1], w[2], w[3]};
+}
+
+template <int HD, bool FUSED>
+__global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_decode_kernel(
+    const bf16_t* __restrict__ q, const float* __restrict__ qf, const float* __restrict__ kf, const float* __restrict__ vf, long ldq, long ldk,
+    long ldv, const float* __restrict__ cos_t, const float* __restrict__ sin_t, bf16_t* __restrict__ cache, float* __restrict__ part,
+    bf16_t* __restrict__ out, const int* __restrict__ rows, const int* __restrict__ pos, const int* __restrict__ slots,
+    const int* __restrict__ table, int table_stride, long page_stride, int page_size, int n_heads, int n_kv, int window, float scale,
+    int n_splits, int gh) {
     constexpr int KSTEPS = HD / 32, DT = HD / 16;
+    extern __shared__ float merged[];                        // [wave][gh][HD + 2]
     const int group = n_heads / n_kv, hg_per_kv = (group + 15) / 16;
-    const int row = rows[blockIdx.x], g = blockIdx.y / hg_per_kv, hg = blockIdx.y % hg_per_kv, split = blockIdx.z;
-    const int lane = threadIdx.x, r = lane & 15, q4 = lane >> 4;
+    const int row = rows ? rows[blockIdx.x] : blockIdx.x, g = blockIdx.y / hg_per_kv, hg = blockIdx.y % hg_per_kv, split = blockIdx.z;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+    const int r = lane & 15, q4 = lane >> 4;
     const int head_in_group = hg * 16 + r;
     const bool head_ok = head_in_group < group;
     const int head = g * group + head_in_group;
+    // The unrotated queries depend on the row alone: their loads go out first, ahead of the chain
+    // position -> page table -> keys.
+    [[maybe_unused]] Unrotated8 q_raw[KSTEPS];
+    [[maybe_unused]] const float* cos_row = nullptr;
+    [[maybe_unused]] const float* sin_row = nullptr;
+    if constexpr (FUSED) {
+        cos_row = cos_t ? cos_t + (size_t)row * (HD / 2) : nullptr;
+        sin_row = sin_t ? sin_t + (size_t)row * (HD / 2) : nullptr;
+        if (head_ok) {
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s) q_raw[s] = load_unrotated8(qf + (size_t)row * ldq + (size_t)head * HD, cos_row, sin_row, 32 * s + 8 * q4, HD / 2);
+        }
+    }
     const int my_pos = pos[row];
     const int lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
     const int* tab = table + (size_t)slots[row] * table_stride;
-    // every row cuts its own range into n_splits pieces (multiples of 32); short rows leave later pieces empty
+    // every row cuts its own range into pieces (multiples of 32), one per wave of every split; short rows leave later pieces empty
+    const int n_pieces = n_splits * n_waves, piece = split * n_waves + wave;
     const int span = my_pos + 1 - (lo & ~31);
-    const int split_len = (((span + n_splits - 1) / n_splits) + 31) & ~31;
-    const int begin = (lo & ~31) + split * split_len, end = min(my_pos + 1, begin + split_len);
+    const int piece_len = (((span + n_pieces - 1) / n_pieces) + 31) & ~31;
+    const int begin = (lo & ~31) + piece * piece_len, end = min(my_pos + 1, begin + piece_len);
     const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
     auto page_index = [&](int kv) { return page_shift >= 0 ? kv >> page_shift : kv / page_size; };
     auto place_of = [&](int kv) { return page_shift >= 0 ? kv & (page_size - 1) : kv % page_size; };
     const float scale2 = scale * LOG2E;            // scores are kept in units of log2 e: e^(s - m) is one exp2
-
-    bf16x8 qreg[KSTEPS];
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-        uint4 v = {0, 0, 0, 0};
-        if (head_ok) v = load16(q + ((size_t)row * n_heads + head) * HD + 32 * s + 8 * q4);
-        qreg[s] = as_bf16x8(v);
-    }
-    floatx4 o[DT];
-#pragma unroll
-    for (int i = 0; i < DT; ++i) o[i] = floatx4{};
-    float m = -INFINITY, l = 0.f;
     const long v_plane = (long)n_kv * page_size * HD;
     const bf16_t* kbase = cache + (long)g * page_size * HD;
     const bf16_t* vbase = cache + v_plane + (long)g * HD * page_size;
+
+    // the row's own key and value, likewise before the page table is read
+    const bool has_own = FUSED && kf != nullptr && begin < end && end == my_pos + 1;     // this wave's piece holds the row's own position
+    [[maybe_unused]] Unrotated8 k_raw[KSTEPS];
+    [[maybe_unused]] float v_raw[DT];
+    if constexpr (FUSED) {
+        if (has_own) {
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) k_raw[ks] = load_unrotated8(kf + (size_t)row * ldk + (size_t)g * HD, cos_row, sin_row, 32 * ks + 8 * q4, HD / 2);
+#pragma unroll
+            for (int i = 0; i < DT; ++i) v_raw[i] = vf[(size_t)row * ldv + (size_t)g * HD + 16 * i + r];
+        }
+    }
 
     // Loads run ahead of the products: the keys of the next 32 positions and the values of these 32
     // are requested before the scores of these 32 are taken.  An address beyond the row's own range
@@ -272,6 +333,41 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
         }
     };
     if (begin < end) load_keys(begin, k_cur);
+
+    bf16x8 qreg[KSTEPS];
+    uint4 own_key[KSTEPS];
+    bf16_t own_value[DT];
+    if constexpr (FUSED) {
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) qreg[s] = as_bf16x8(head_ok ? rotated8(q_raw[s]) : uint4{0, 0, 0, 0});
+        if (has_own) {
+            bf16_t* page = cache + (long)tab[page_index(my_pos)] * page_stride;
+            const int place = place_of(my_pos);
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+                own_key[ks] = rotated8(k_raw[ks]);
+                if (r == 0 && hg == 0)
+                    *reinterpret_cast<uint4*>(page + (long)g * page_size * HD + (long)place * HD + 32 * ks + 8 * q4) = own_key[ks];
+            }
+#pragma unroll
+            for (int i = 0; i < DT; ++i) {
+                own_value[i] = f32_to_bf16(v_raw[i]);
+                if ((i & 3) == q4 && hg == 0) page[v_plane + ((long)g * HD + 16 * i + r) * page_size + place] = own_value[i];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+            uint4 v = {0, 0, 0, 0};
+            if (head_ok) v = load16(q + ((size_t)row * n_heads + head) * HD + 32 * s + 8 * q4);
+            qreg[s] = as_bf16x8(v);
+        }
+    }
+
+    floatx4 o[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i) o[i] = floatx4{};
+    float m = -INFINITY, l = 0.f;
     for (int kv0 = begin; kv0 < end; kv0 += 32) {
         // slot e of this lane in the value product is key position kv0 + 16*(e/4) + 4*q4 + e%4
         const int kva = min(max(kv0 + 4 * q4, lo & ~3), my_pos & ~3), kvb = min(max(kv0 + 16 + 4 * q4, lo & ~3), my_pos & ~3);
@@ -284,6 +380,30 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
             vy[i] = load8(vb + (long)(16 * i) * page_size);
         }
         if (kv0 + 32 < end) load_keys(kv0 + 32, k_nxt);
+        if constexpr (FUSED) {
+            if (has_own && kv0 + 32 >= end) {             // the last block of the piece: the row's own key and value go in
+                const int off = my_pos - kv0;             // 0 .. 31
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    if ((off >> 4) == t && (off & 15) == r) {
+#pragma unroll
+                        for (int ks = 0; ks < KSTEPS; ++ks) k_cur[t][ks] = own_key[ks];
+                    }
+                if (((off & 15) >> 2) == q4) {
+                    const int e = off & 3;
+                    const bool second = (off >> 4) != 0;
+#pragma unroll
+                    for (int i = 0; i < DT; ++i) {
+                        const uint2 had = second ? vy[i] : vx[i];
+                        const uint32_t val = own_value[i];
+                        const uint32_t x = e == 0 ? (had.x & 0xffff0000u) | val : e == 1 ? (had.x & 0x0000ffffu) | (val << 16) : had.x;
+                        const uint32_t y = e == 2 ? (had.y & 0xffff0000u) | val : e == 3 ? (had.y & 0x0000ffffu) | (val << 16) : had.y;
+                        vx[i] = second ? vx[i] : uint2{x, y};
+                        vy[i] = second ? uint2{x, y} : vy[i];
+                    }
+                }
+            }
+        }
 
         floatx4 s[2];
 #pragma unroll
@@ -331,17 +451,46 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(const bf16_t* __re
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) k_cur[t][ks] = k_nxt[t][ks];
     }
-    if (!head_ok) return;
-    // part[row_index][head][split] = {m, l, O[HD]}; element v of o[i]: channel 16*i + 4*q4 + v, query head r
-    float* dst = part + (((size_t)blockIdx.x * n_heads + head) * n_splits + split) * (HD + 2);
-    if (q4 == 0) {
-        dst[0] = m;
-        dst[1] = l;
+
+    // The waves' results meet in LDS: element v of o[i] is channel 16*i + 4*q4 + v of query head r.
+    if (r < gh) {
+        float* mine = merged + ((size_t)wave * gh + r) * (HD + 2);
+        if (q4 == 0) {
+            mine[0] = m;
+            mine[1] = l;
+        }
+#pragma unroll
+        for (int i = 0; i < DT; ++i)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) mine[2 + 16 * i + 4 * q4 + v] = o[i][v];
     }
-#pragma unroll
-    for (int i = 0; i < DT; ++i)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) dst[2 + 16 * i + 4 * q4 + v] = o[i][v];
+    __syncthreads();
+    for (int e = threadIdx.x; e < gh * HD; e += blockDim.x) {
+        const int hh = e / HD, d = e % HD;
+        if (hg * 16 + hh >= group) continue;
+        const int out_head = g * group + hg * 16 + hh;
+        const float* first = merged + (size_t)hh * (HD + 2);
+        const size_t wave_stride = (size_t)gh * (HD + 2);
+        float big = -INFINITY;
+        for (int w = 0; w < n_waves; ++w) big = fmaxf(big, first[w * wave_stride]);
+        float denom = 0.f, acc = 0.f;
+        for (int w = 0; w < n_waves; ++w) {                  // in wave order
+            const float mw = first[w * wave_stride];
+            const float weight = (mw == -INFINITY) ? 0.f : exp2_fast(mw - big);
+            denom = fmaf(weight, first[w * wave_stride + 1], denom);
+            acc = fmaf(weight, first[w * wave_stride + 2 + d], acc);
+        }
+        if (n_splits == 1) {
+            out[((size_t)row * n_heads + out_head) * HD + d] = f32_to_bf16(acc / denom);
+        } else {                                             // part[row_index][head][split] = {m, l, O[HD]}
+            float* dst = part + (((size_t)blockIdx.x * n_heads + out_head) * n_splits + split) * (HD + 2);
+            if (d == 0) {
+                dst[0] = big;
+                dst[1] = denom;
+            }
+            dst[2 + d] = acc;
+        }
+    }
 }
 
 // Merges the splits of one (row, head): out = sum_s e^(m_s - M) O_s / sum_s e^(m_s - M) l_s, the sums
@@ -381,7 +530,7 @@ __global__ __launch_bounds__(64) void attention_decode_combine_kernel(const floa
         float acc = 0.f;
 #pragma unroll 8
         for (int s = 0; s < n_splits; ++s) acc = fmaf(weight[s], src[(size_t)s * (hd + 2) + 2 + d], acc);
-        out[((size_t)rows[idx] * n_heads + head) * hd + d] = f32_to_bf16(acc * inv);
+        out[((size_t)(rows ? rows[idx] : idx) * n_heads + head) * hd + d] = f32_to_bf16(acc * inv);
     }
 }
 
@@ -419,25 +568,64 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
     return 0;
 }
 
-GI_API int gi_attention_decode_bf16(const void* q, const void* cache, void* out, float* part, long part_floats, const int* rows, int n_rows,
-                                    const int* pos, const int* slots, const int* table, int table_stride, long page_stride, int page_size,
-                                    int n_heads, int n_kv, int hd, int window, float scale, int n_splits, hipStream_t stream) {
+// Waves a workgroup of the decode kernel may have for this head size.
+GI_API int gi_attention_decode_max_waves(int hd) { return hd <= 128 ? 8 : 4; }
+
+// Rows `rows[0 .. n_rows)` of the step (`rows` null: rows 0 .. n_rows-1), one new position each.  Either `q` holds their rotated
+// queries in bfloat16 and the cache already holds their keys and values, or (`qf` given) `qf`,
+// `kf`, `vf` hold the unrotated 32-bit products, `cos_t`/`sin_t` the rotation (or null for none),
+// and the kernel rotates, attends and writes the new keys and values to the cache itself (`kf`
+// null: the pages belong to another layer and hold them already).  `n_waves` pieces per workgroup,
+// `n_splits` workgroups per row and head group; `part` is needed for n_splits > 1.
+GI_API int gi_attention_decode_bf16(const void* q, const float* qf, const float* kf, const float* vf, long ldq, long ldk, long ldv,
+                                    const float* cos_t, const float* sin_t, void* cache, void* out, float* part, long part_floats,
+                                    const int* rows, int n_rows, const int* pos, const int* slots, const int* table, int table_stride,
+                                    long page_stride, int page_size, int n_heads, int n_kv, int hd, int window, float scale, int n_splits,
+                                    int n_waves, hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_decode: bad counts (%d rows, %d heads, %d kv heads)",
                n_rows, n_heads, n_kv);
     GI_REQUIRE(gi_attention_bf16_supports(hd, page_size, 0), "attention_decode: head size %d with page size %d is not supported", hd, page_size);
     GI_REQUIRE(page_stride >= 2L * n_kv * page_size * hd && page_stride % 8 == 0, "attention_decode: bad page stride %ld", page_stride);
     GI_REQUIRE(n_splits >= 1 && n_splits <= MAX_SPLITS, "attention_decode: the number of splits %d is outside 1..%d", n_splits, MAX_SPLITS);
-    GI_REQUIRE(part != nullptr && part_floats >= (long)n_rows * n_heads * n_splits * (hd + 2), "attention_decode: scratch too small");
-    const int hg = (n_heads / n_kv + 15) / 16;
+    GI_REQUIRE(n_waves >= 1 && n_waves <= gi_attention_decode_max_waves(hd), "attention_decode: %d waves per workgroup are outside 1..%d",
+               n_waves, gi_attention_decode_max_waves(hd));
+    GI_REQUIRE(n_splits == 1 || (part != nullptr && part_floats >= (long)n_rows * n_heads * n_splits * (hd + 2)), "attention_decode: scratch too small");
+    GI_REQUIRE((q != nullptr) != (qf != nullptr), "attention_decode: give either rotated bfloat16 queries or the unrotated 32-bit products");
+    if (qf) {
+        GI_REQUIRE((kf == nullptr) == (vf == nullptr), "attention_decode: keys and values come together");
+        GI_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attention_decode: cos and sin must both be given or both be absent");
+        GI_REQUIRE(ldq % 4 == 0 && ((uintptr_t)qf & 15) == 0 && (!kf || (ldk % 4 == 0 && ((uintptr_t)kf & 15) == 0)) &&
+                       (!cos_t || ((((uintptr_t)cos_t | (uintptr_t)sin_t) & 15) == 0)),
+                   "attention_decode: the 32-bit inputs must be 16-byte aligned with row strides that are multiples of 4");
+        GI_REQUIRE(ldq >= (long)n_heads * hd && (!kf || (ldk >= (long)n_kv * hd && ldv >= (long)n_kv * hd)), "attention_decode: row strides too small");
+    }
+    const int group = n_heads / n_kv, hg = (group + 15) / 16, gh = group < 16 ? group : 16;
     GI_REQUIRE(n_kv * hg <= 65535, "attention_decode: too many heads");
+    size_t lds = (size_t)n_waves * gh * (hd + 2) * sizeof(float);
+    while (lds > 64 * 1024 && n_waves > 1) {                  // many wide heads: fewer waves so that their results fit
+        n_waves /= 2;
+        lds = (size_t)n_waves * gh * (hd + 2) * sizeof(float);
+    }
+    GI_REQUIRE(lds <= 64 * 1024, "attention_decode: %d heads of size %d per key/value head do not fit", gh, hd);
     dim3 grid(n_rows, n_kv * hg, n_splits);
-#define GO(HD) attention_decode_kernel<HD><<<grid, 64, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, part, rows, pos, slots, table, \
-                                                                   table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits)
+#define GO2(HD, FUSED_)                                                                                                                    \
+    attention_decode_kernel<HD, FUSED_><<<grid, 64 * n_waves, lds, stream>>>((const bf16_t*)q, qf, kf, vf, ldq, ldk, ldv, cos_t, sin_t,   \
+                                                                             (bf16_t*)cache, part, (bf16_t*)out, rows, pos, slots, table, \
+                                                                             table_stride, page_stride, page_size, n_heads, n_kv, window,  \
+                                                                             scale, n_splits, gh)
+#define GO(HD)                    \
+    do {                          \
+        if (qf) GO2(HD, true);    \
+        else GO2(HD, false);      \
+    } while (0)
     if (hd == 32) GO(32); else if (hd == 64) GO(64); else if (hd == 96) GO(96); else if (hd == 128) GO(128); else GO(256);
 #undef GO
+#undef GO2
     GI_CHECK_LAUNCH("attention_decode");
-    dim3 cgrid(n_rows, n_heads);
-    attention_decode_combine_kernel<<<cgrid, 64, 0, stream>>>(part, (bf16_t*)out, rows, n_heads, hd, n_splits);
-    GI_CHECK_LAUNCH("attention_decode (combine)");
+    if (n_splits > 1) {
+        dim3 cgrid(n_rows, n_heads);
+        attention_decode_combine_kernel<<<cgrid, 64, 0, stream>>>(part, (bf16_t*)out, rows, n_heads, hd, n_splits);
+        GI_CHECK_LAUNCH("attention_decode (combine)");
+    }
     return 0;
 }

@@ -33,8 +33,9 @@ _SIGNATURES = {
     "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
     "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_void_p],
-    "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long,
-                                 c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                 c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
+                                 c_float, c_int, c_int, c_void_p],
     "gi_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
 }
@@ -247,8 +248,8 @@ class AttentionPlan:
         """Every row is a request's single new row (what a captured decode step uses: nothing in it depends on the step)."""
         plan = cls.__new__(cls)
         plan.n_decode, plan.n_tiles, plan.max_decode_context = n_rows, 0, max_context
-        plan.decode_rows = torch.arange(n_rows, dtype=torch.int32, device=device)
-        plan.tiles = plan.decode_rows[:0]
+        plan.decode_rows = None                                  # rows 0 .. n_rows-1
+        plan.tiles = torch.empty(0, dtype=torch.int32, device=device)
         return plan
 
     def __init__(self, seg_start, seg_len, seg_pos0, seg_slot, device):
@@ -262,7 +263,7 @@ class AttentionPlan:
                     tiles.append((start + off, min(self.TILE, n - off), pos0 + off, slot))
         self.n_decode, self.n_tiles = len(dec), len(tiles)
         both = torch.tensor(dec + [v for t in tiles for v in t], dtype=torch.int32).to(device)
-        self.decode_rows = both[:len(dec)]
+        self.decode_rows = both[:len(dec)] if tiles else None      # no prompt rows: the decode rows are all rows, in order
         self.tiles = both[len(dec):]
 
 
@@ -270,14 +271,31 @@ def attention_bf16_supports(hd, page_size, prompt: bool) -> bool:
     return bool(lib().gi_attention_bf16_supports(hd, page_size, 1 if prompt else 0))
 
 
+def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096):
+    """(splits, waves per workgroup) of the decode kernel: about `target_waves` waves in all and pieces of
+    at least 64 positions; a single split (no combine kernel) when a workgroup's waves cover them."""
+    groups = n_decode * n_kv * ((n_heads // n_kv + 15) // 16)
+    pieces = max(1, min(-(-target_waves // groups), -(-span // 64)))
+    max_waves = min(8, lib().gi_attention_decode_max_waves(hd))
+    if pieces <= max_waves:
+        return 1, pieces
+    n_waves = min(4, max_waves)
+    return min(-(-pieces // n_waves), 256), n_waves
+
+
 def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None,
-                   target_waves: int = 2048):
-    """Attention of a step's rows with the matrix-core kernels (bfloat16 q, cache and out)."""
+                   target_waves: int = 4096, products=None):
+    """Attention of a step's rows with the matrix-core kernels (bfloat16 cache and out).
+
+    `q` holds the rotated queries in bfloat16 and the cache the rows' keys and values; or, for a step
+    of single decoded rows only, `q` is None and `products = (q, k, v, cos, sin)` holds the unrotated
+    float32 products and the rotation's tables (k, v None: the pages are another layer's; cos, sin
+    None: no rotation): the decode kernel then rotates, writes the cache and attends in one launch."""
+    n = out.shape[0]
     _dev(q, cache, out, positions, slots, table)
-    n = q.shape[0]
     for t, name in ((q, "q"), (cache, "cache"), (out, "out")):
-        _need(t.dtype == torch.bfloat16, f"attention_bf16: {name} must be bfloat16")
-    _need(q.shape == (n, n_heads * hd) and q.is_contiguous() and out.shape == q.shape and out.is_contiguous(),
+        _need(t is None or t.dtype == torch.bfloat16, f"attention_bf16: {name} must be bfloat16")
+    _need(out.shape == (n, n_heads * hd) and out.is_contiguous() and (q is None or (q.shape == out.shape and q.is_contiguous())),
           "attention: q and out must be [n, heads*hd], contiguous")
     page_size = cache.shape[3]
     _check_cache(cache, table, page_size, n_kv, hd, "attention")
@@ -285,31 +303,69 @@ def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, 
     _i32(slots, "attention: slots", n)
     window = int(window or 0)
     scale = float(scale if scale is not None else hd ** -0.5)
+    _need((q is None) != (products is None), "attention_bf16: give rotated queries or the unrotated products")
+    qf = kf = vf = cos = sin = None
+    if products is not None:
+        _need(plan.n_tiles == 0, "attention_bf16: unrotated products serve steps of single decoded rows only")
+        qf, kf, vf, cos, sin = products
+        _dev(qf, kf, vf, cos, sin)
+        _need(qf.dtype == torch.float32 and qf.shape == (n, n_heads * hd) and qf.stride(1) == 1, "attention: q must be float32 [n, heads*hd]")
+        for t, name in ((kf, "k"), (vf, "v")):
+            _need(t is None or (t.dtype == torch.float32 and t.shape == (n, n_kv * hd) and t.stride(1) == 1),
+                  f"attention: {name} must be float32 [n, kv_heads*hd]")
+        for t in (cos, sin):
+            _need(t is None or (t.dtype == torch.float32 and t.shape == (n, hd // 2) and t.is_contiguous()), "attention: cos/sin must be float32 [n, hd/2]")
     if plan.n_tiles:
         _call("gi_attention_prompt_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles, plan.TILE,
               table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, _stream())
     if plan.n_decode:
         span = plan.max_decode_context if not window else min(plan.max_decode_context, window + 31)
-        waves = plan.n_decode * n_kv * ((n_heads // n_kv + 15) // 16)
-        n_splits = max(1, min(-(-target_waves // waves), -(-span // 64), 256))
-        n_part = plan.n_decode * n_heads * n_splits * (hd + 2)
-        part = torch.empty(n_part, dtype=torch.float32, device=q.device)
-        _call("gi_attention_decode_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), part.data_ptr(), n_part,
-              plan.decode_rows.data_ptr(), plan.n_decode, positions.data_ptr(), slots.data_ptr(), table.data_ptr(), table.stride(0),
-              cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits, _stream())
+        n_splits, n_waves = decode_attention_shape(plan.n_decode, n_heads, n_kv, hd, span, target_waves)
+        n_part = plan.n_decode * n_heads * n_splits * (hd + 2) if n_splits > 1 else 0
+        part = torch.empty(n_part, dtype=torch.float32, device=out.device) if n_part else None
+        _call("gi_attention_decode_bf16", _ptr(q), _ptr(qf), _ptr(kf), _ptr(vf), qf.stride(0) if qf is not None else 0,
+              kf.stride(0) if kf is not None else 0, vf.stride(0) if vf is not None else 0, _ptr(cos), _ptr(sin), cache.data_ptr(),
+              out.data_ptr(), _ptr(part), n_part, _ptr(plan.decode_rows), plan.n_decode, positions.data_ptr(), slots.data_ptr(),
+              table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits, n_waves, _stream())
     return out
+
+
+def _plan_of(ctx):
+    if "attention_plan" not in ctx.memo:
+        ctx.memo["attention_plan"] = AttentionPlan(ctx.seg_start, ctx.seg_len, ctx.seg_pos0, ctx.seg_slot, ctx.device)
+    return ctx.memo["attention_plan"]
 
 
 def attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window=None):
     """Attention of a step's rows; the kernel is chosen by the storage dtype and the batch's shape."""
     page_size = cache.shape[3]
     if q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16:
-        if "attention_plan" not in ctx.memo:
-            ctx.memo["attention_plan"] = AttentionPlan(ctx.seg_start, ctx.seg_len, ctx.seg_pos0, ctx.seg_slot, ctx.device)
-        plan = ctx.memo["attention_plan"]
+        plan = _plan_of(ctx)
         if (not plan.n_tiles or attention_bf16_supports(hd, page_size, True)) and (not plan.n_decode or attention_bf16_supports(hd, page_size, False)):
             return attention_bf16(q, cache, out, plan, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window)
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window)
+
+
+# With many rows the chip is full of waves and the fused kernel's extra registers cost more than the
+# rotation kernel's launch (measured at the Llama-3.2-1B shape: +2..3 % at 1 and 8 rows, -10 % at 64).
+FUSED_DECODE_MAX_ROWS = 16
+
+
+def attention_from_products(q, k, v, cos, sin, cache, out, ctx, table, n_heads, n_kv, hd, window=None) -> bool:
+    """Rotation, cache write and attention in one launch, from the unrotated float32 products, when
+    every row of the step is a request's single new row, the rows are few and the matrix-core decode
+    kernel takes the sizes.  Returns False (nothing done) otherwise: the caller then rotates and stores first."""
+    if not (cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.dtype == torch.float32):
+        return False
+    plan = _plan_of(ctx)
+    if plan.n_tiles or not plan.n_decode or not attention_bf16_supports(hd, cache.shape[3], False):
+        return False
+    if plan.n_decode > FUSED_DECODE_MAX_ROWS:
+        return False
+    if q.stride(0) % 4 or q.data_ptr() % 16 or (k is not None and (k.stride(0) % 4 or k.data_ptr() % 16)):
+        return False
+    attention_bf16(None, cache, out, plan, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, products=(q, k, v, cos, sin))
+    return True
 
 
 def gemm_bf16_supports(a, w, out) -> bool:

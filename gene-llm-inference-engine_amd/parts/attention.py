@@ -44,18 +44,19 @@ class Attention(Mixer):
     def forward(self, h, residual, ctx, cache):
         s, T = self.spec, ctx.n_rows
         cos, sin = self.position.prepare(ctx) if self.position is not None else (None, None)
-        q_rot = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
+        att = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
         if cache.writes:
             qkv = torch.empty((T, self.a_dim + 2 * self.kv_dim), dtype=torch.float32, device=ctx.device)
             linear(h, self.w_qkv, qkv)
             q, k, v = qkv[:, :self.a_dim], qkv[:, self.a_dim:self.a_dim + self.kv_dim], qkv[:, self.a_dim + self.kv_dim:]
-            ops.rope_store(q, k, v, cos, sin, ctx.row_pos, ctx.row_slot, cache.table, q_rot, cache.kv, s.n_heads, s.n_kv_heads, s.head_dim)
         else:                       # the pages are another layer's: only the queries are made
-            q = torch.empty((T, self.a_dim), dtype=torch.float32, device=ctx.device)
+            q, k, v = torch.empty((T, self.a_dim), dtype=torch.float32, device=ctx.device), None, None
             linear(h, self.w_qkv[:self.a_dim], q)
-            ops.rope_store(q, None, None, cos, sin, ctx.row_pos, ctx.row_slot, cache.table, q_rot, cache.kv, s.n_heads, s.n_kv_heads, s.head_dim)
-        att = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
-        ops.attention(q_rot, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, s.window)
+        # a step of single decoded rows: one kernel rotates, writes the pages and attends
+        if not ops.attention_from_products(q, k, v, cos, sin, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, s.window):
+            q_rot = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
+            ops.rope_store(q, k, v, cos, sin, ctx.row_pos, ctx.row_slot, cache.table, q_rot, cache.kv, s.n_heads, s.n_kv_heads, s.head_dim)
+            ops.attention(q_rot, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, s.window)
         if att.dtype != self.att_dtype:
             att = att.to(self.att_dtype)
         linear(att, self.w_o, residual, accumulate=True)

@@ -261,6 +261,61 @@ def test_attention_finds_one_far_key(dtype):
     assert rel(out.view(n_heads, hd)[0], v[target, 0]) < 2e-2          # the softmax is nearly one-hot on the target
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd,ps,window", ATT_CASES)
+@pytest.mark.parametrize("target_waves", [4096, 64])
+def test_decode_attention_from_unrotated_products(n_heads, n_kv, hd, ps, window, target_waves, monkeypatch):
+    """Single decoded rows whose keys and values are not in the cache yet: one kernel rotates q and k,
+    attends (its own position included) and writes k and v to the right places, in one split and in several."""
+    from geneinfer_amd.parts import StepContext
+    shape = ops().decode_attention_shape
+    monkeypatch.setattr(ops(), "decode_attention_shape", lambda *a, **k: shape(*a[:5], target_waves=target_waves))
+    contexts = [300, 131, 1, 77, 530, 16, 17, 1200, 32, 33]           # the new row's position is the last of each
+    cache, table, dense = build_paged(contexts, n_kv, hd, ps, torch.bfloat16, seed=hd + n_heads + 1)
+    T = len(contexts)
+    pos = torch.tensor([n - 1 for n in contexts], dtype=torch.int32, device=DEV)
+    slots = torch.arange(1, T + 1, dtype=torch.int32, device=DEV)
+    a, kvd = n_heads * hd, n_kv * hd
+    qkv = randn(T, a + 2 * kvd, seed=31)
+    inv = torch.tensor([1.0 / (10000.0 ** (2 * k / hd)) for k in range(hd // 2)], dtype=torch.float64, device=DEV)
+    cos, sin = torch.empty(T, hd // 2, device=DEV), torch.empty(T, hd // 2, device=DEV)
+    ops().rope_cos_sin(pos, inv, cos, sin)
+
+    def rotated(x, heads):
+        x = x.double().cpu().view(T, heads, hd)
+        c, s_ = torch.cat([cos, cos], -1).double().cpu()[:, None, :], torch.cat([sin, sin], -1).double().cpu()[:, None, :]
+        return x * c + torch.cat([-x[..., hd // 2:], x[..., :hd // 2]], -1) * s_
+
+    q_rot = rotated(qkv[:, :a], n_heads).to(torch.bfloat16).view(T, a)
+    k_rot = rotated(qkv[:, a:a + kvd], n_kv).to(torch.bfloat16)
+    v_new = qkv[:, a + kvd:].cpu().view(T, n_kv, hd).to(torch.bfloat16)
+    want_cache = cache.clone()
+    for i, n in enumerate(contexts):                                   # the row's own place: empty before, k and v after
+        dense[i][0][n - 1], dense[i][1][n - 1] = k_rot[i], v_new[i]
+        page, place = int(table[i + 1, (n - 1) // ps]), (n - 1) % ps
+        cache[page, 0, :, place, :] = 0
+        cache[page, 1].view(n_kv, hd, ps)[:, :, place] = 0
+        want_cache[page, 0, :, place, :] = k_rot[i].to(DEV)
+        want_cache[page, 1].view(n_kv, hd, ps)[:, :, place] = v_new[i].to(DEV)
+    ctx = StepContext(n_rows=T, dtype=torch.bfloat16, device=torch.device(DEV), tokens=pos, row_pos=pos, row_slot=slots,
+                      seg_slot=list(range(1, T + 1)), seg_start=list(range(T)), seg_len=[1] * T, seg_pos0=[n - 1 for n in contexts])
+    out = torch.full((T, a), float("nan"), dtype=torch.bfloat16, device=DEV)
+    done = ops().attention_from_products(qkv[:, :a], qkv[:, a:a + kvd], qkv[:, a + kvd:], cos, sin, cache, out, ctx, table, n_heads, n_kv, hd, window)
+    if not ops().attention_bf16_supports(hd, ps, False):
+        assert done is False and bool(torch.isnan(out.float()).all())    # refused: the caller rotates and stores first
+        return
+    assert done is True
+    want = plain_attention_rows(q_rot, dense, [(i, n - 1) for i, n in enumerate(contexts)], n_heads, n_kv, hd, window)
+    assert rel(out, want) < 8e-3, rel(out, want)
+    got_c, want_c = torch.nan_to_num(cache.float(), nan=-1.0), torch.nan_to_num(want_cache.float(), nan=-1.0)
+    assert rel(got_c, want_c) < 1e-3                                  # a rotated key may round the other way in 32-bit
+    assert float(((got_c - want_c).abs() > 0.02 * want_c.abs() + 1e-6).sum()) == 0
+    # read-only use of another layer's pages (which now hold the rows' keys and values): the same output, the cache untouched
+    out2, before = torch.full_like(out, float("nan")), cache.clone()
+    assert ops().attention_from_products(qkv[:, :a], None, None, cos, sin, cache, out2, ctx, table, n_heads, n_kv, hd, window)
+    assert rel(out2, want) < 8e-3
+    assert torch.equal(torch.nan_to_num(cache, nan=-1.0), torch.nan_to_num(before, nan=-1.0))
+
+
 def test_rope_store_writes_the_right_places():
     n_heads, n_kv, hd, ps = 4, 2, 32, 16
     n_pages = 5
