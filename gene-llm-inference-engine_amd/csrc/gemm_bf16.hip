@@ -133,67 +133,119 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
 }
 
 // ----------------------------------------------------------------------------------------- skinny
-// Workgroup: 4 waves, each a strip of 16 weight rows; the workgroup covers 64 weight rows and the
-// k range [k_begin, k_end) of its grid row.  Per block of 128 k, lane (r = lane%16, q = lane/16) of
-// a wave holds W[n0 + r][k0 + 32q + 8j .. +8] for j = 0..3: 64 contiguous bytes of a weight row.
-// The activations use the same assignment of k to lanes, so each product sums over the same k.
-constexpr int SK = 128, X_STRIDE = SK + 8;
+// Workgroup: 8 waves = 4 strips of 16 weight rows x 2 halves of each 256-wide block of k; the
+// workgroup covers 64 weight rows and the k range [k_begin, k_end) of its grid row.  Weights stream
+// from HBM straight into registers, two blocks ahead of their use: for the j-th product of a
+// block, lane (r = lane%16, q = lane/16) holds k0 + 128*half + 32j + 8q .. +8 of weight row r, so
+// the four lanes of a row read 64 contiguous bytes per load.  The activations of a block go
+// through LDS (they are shared by the strips) and are fetched into registers one block ahead.
+// The halves' sums meet in LDS.  PARTIAL: the sums of the k range go to P[split][M][N] and a
+// second kernel adds the splits in order; otherwise the workgroup saw all of k and writes the
+// result with its epilogue itself.
+constexpr int SK = 128;                               // k per product group of a wave (4 products of 32)
+constexpr int KB = 2 * SK, X_STRIDE = KB + 8;         // k per block of the workgroup; +8 bf16 of padding
 
-template <int MT>
-__global__ __launch_bounds__(256) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, float* __restrict__ P,
-                                                              int M, int N, int K, long lda, long ldw, int k_per_split) {
+template <int MT, int EPI, bool PARTIAL>
+__global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
+                                                              float* __restrict__ P, int M, int N, int K, long lda, long ldw, long ldc,
+                                                              int k_per_split) {
     __shared__ __attribute__((aligned(16))) bf16_t Xs[MT * 16 * X_STRIDE];
+    __shared__ float other[4][MT][64][4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int strip = wave & 3, half = wave >> 2;
     const int r = lane & 15, q = lane >> 4;
-    const int n = blockIdx.x * 64 + wave * 16 + r;
+    const int n = blockIdx.x * 64 + strip * 16 + r;
     const int k_begin = blockIdx.y * k_per_split, k_end = min(K, k_begin + k_per_split);
-    const bf16_t* wrow = W + (size_t)min(n, N - 1) * ldw;
+    const bf16_t* wrow = W + (size_t)min(n, N - 1) * ldw + SK * half + 8 * q;
 
     floatx4 acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = floatx4{};
 
-    uint4 w_next[4];
-    auto fetch_w = [&](int k0) {
+    uint4 w_buf[3][4], x_reg[MT];
+    auto fetch_w = [&](int k0, uint4* w) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int k = k0 + 32 * q + 8 * j;
-            w_next[j] = (k < k_end) ? load16(wrow + k) : uint4{0, 0, 0, 0};
+        for (int j = 0; j < 4; ++j) w[j] = (k0 + SK * half + 32 * j + 8 * q < k_end) ? load16(wrow + k0 + 32 * j) : uint4{0, 0, 0, 0};
+    };
+    auto fetch_x = [&](int k0) {                      // rows beyond M and k beyond the range are zero
+#pragma unroll
+        for (int c = 0; c < MT; ++c) {
+            const int e = tid + 512 * c, row = e / (KB / 8), k = k0 + (e % (KB / 8)) * 8;
+            x_reg[c] = (row < M && k < k_end) ? load16(A + (size_t)row * lda + k) : uint4{0, 0, 0, 0};
         }
     };
-    fetch_w(k_begin);
-    for (int k0 = k_begin; k0 < k_end; k0 += SK) {
-        __syncthreads();
-        // activations of this k-block -> LDS (rows beyond M and k beyond the range are zero)
-        for (int e = tid; e < MT * 16 * (SK / 8); e += 256) {
-            const int row = e / (SK / 8), kc = (e % (SK / 8)) * 8;
-            const int k = k0 + kc;
-            *reinterpret_cast<uint4*>(&Xs[row * X_STRIDE + kc]) = (row < M && k < k_end) ? load16(A + (size_t)row * lda + k) : uint4{0, 0, 0, 0};
-        }
-        uint4 w_now[4];
+    fetch_x(k_begin);
+    fetch_w(k_begin, w_buf[0]);
+    fetch_w(k_begin + KB, w_buf[1]);
+    for (int k0 = k_begin; k0 < k_end; k0 += 3 * KB) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) w_now[j] = w_next[j];
-        if (k0 + SK < k_end) fetch_w(k0 + SK);
-        __syncthreads();
+        for (int d = 0; d < 3; ++d) {                 // buffer d holds the weights of block k0 + d*KB
+            const int kk = k0 + d * KB;
+            if (kk < k_end) {                         // the same for every thread of the workgroup
+                __syncthreads();                      // everyone has finished reading the previous block
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const bf16x8 b = as_bf16x8(w_now[j]);
+                for (int c = 0; c < MT; ++c) {
+                    const int e = tid + 512 * c;
+                    *reinterpret_cast<uint4*>(&Xs[(e / (KB / 8)) * X_STRIDE + (e % (KB / 8)) * 8]) = x_reg[c];
+                }
+                __syncthreads();
+                fetch_x(kk + KB);
+                fetch_w(kk + 2 * KB, w_buf[(d + 2) % 3]);
 #pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(&Xs[(t * 16 + r) * X_STRIDE + 32 * q + 8 * j]));
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+                for (int j = 0; j < 4; ++j) {
+                    const bf16x8 b = as_bf16x8(w_buf[d][j]);
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) {
+                        const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(&Xs[(t * 16 + r) * X_STRIDE + SK * half + 32 * j + 8 * q]));
+                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
+                    }
+                }
             }
         }
     }
+    // the second half's sums join the first's
+    if (half == 1) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) other[strip][t][lane][v] = acc[t][v];
+    }
+    __syncthreads();
+    if (half == 0) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[t][v] += other[strip][t][lane][v];
+    }
     // Element v of a lane's 16x16 result: row (activation row) 4*(lane/16) + v, column (weight row) lane%16.
-    float* part = P + (size_t)blockIdx.y * M * N;
-    if (n < N) {
+    if constexpr (EPI == EPI_GATED_BF16 && !PARTIAL) {
+        // strips 0 and 2 hold gates, strips 1 and 3 the ups of the same outputs: the ups cross over through LDS
+        __syncthreads();
+        if (half == 0 && (strip & 1)) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) other[strip][t][lane][v] = acc[t][v];
+        }
+        __syncthreads();
+        if (half == 0 && !(strip & 1) && n < N) {
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int m = t * 16 + 4 * q + v;
+                    if (m < M) ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 32 + (strip >> 1) * 16 + r] = f32_to_bf16(silu_gate(acc[t][v], other[strip + 1][t][lane][v]));
+                }
+        }
+    } else if (half == 0 && n < N) {
 #pragma unroll
         for (int t = 0; t < MT; ++t)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int m = t * 16 + 4 * q + v;
-                if (m < M) part[(size_t)m * N + n] = acc[t][v];
+                if (m >= M) continue;
+                if constexpr (PARTIAL) P[((size_t)blockIdx.y * M + m) * N + n] = acc[t][v];
+                else write_out<EPI>(C, (size_t)m * ldc + n, acc[t][v]);
             }
     }
 }
@@ -308,10 +360,15 @@ int epilogue_of(int c_dtype, int accumulate) {
 static int g_force_bm = 0;
 GI_API void gi_gemm_bf16_set_tile(int bm) { g_force_bm = bm; }
 
+
+// Number of k-splits of the skinny kernel for a product with 17..64 rows, so that the caller can size
+// the scratch (splits * M * N floats); 0: the output is wide enough to fill the chip without a split,
+// no scratch is needed.  Enough workgroups to cover the chip, each with at least one block of k.
 GI_API int gi_gemm_bf16_skinny_splits(int N, int K) {
     const int strips = (N + 63) / 64;
+    if (strips >= 192) return 0;
     int splits = 1;
-    while (strips * splits < 512 && K / (splits * 2) >= 256) splits *= 2;
+    while (strips * splits < 384 && K / (splits * 2) >= KB) splits *= 2;
     return splits;
 }
 
@@ -330,7 +387,12 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     }
     GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
 
-    if (M <= 16) {
+    // Up to 16 rows the slim kernel (no LDS staging, one launch) is the faster one, except for wide outputs with more
+    // than a few rows, where its per-workgroup reading of the activations costs more than the skinny kernel's staging
+    // (measured crossovers at K = 2048: 12 rows for 256 strips of 64 columns, 5 rows for 2004 strips).
+    const int strips64 = (N + 63) / 64;
+    const bool wide_skinny = gi_gemm_bf16_skinny_splits(N, K) == 0 && (M >= 12 || (M >= 5 && strips64 >= 1024));
+    if (M <= 16 && !wide_skinny) {
 #define SLIM(STRIPS_, ROWS_, EPI_) \
     gemm_bf16_slim_kernel<STRIPS_, ROWS_, EPI_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
         if (epi == EPI_GATED_BF16) {
@@ -349,16 +411,29 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     }
 
     if (M <= 64) {
-        const int splits = gi_gemm_bf16_skinny_splits(N, K);
+        const int splits = gi_gemm_bf16_skinny_splits(N, K), mt = (M + 15) / 16;
+#define SKINNY_MT(EPI_, PARTIAL_)                                                                                                   \
+    do {                                                                                                                            \
+        if (mt == 1) gemm_bf16_skinny_kernel<1, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split); \
+        else if (mt == 2) gemm_bf16_skinny_kernel<2, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split); \
+        else if (mt == 3) gemm_bf16_skinny_kernel<3, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split); \
+        else gemm_bf16_skinny_kernel<4, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split); \
+    } while (0)
+        if (splits == 0) {                             // a wide output: every workgroup sees all of k and finishes its columns
+            const int k_per_split = K;
+            dim3 grid((N + 63) / 64, 1);
+            if (epi == EPI_GATED_BF16) SKINNY_MT(EPI_GATED_BF16, false); else if (epi == EPI_STORE_F32) SKINNY_MT(EPI_STORE_F32, false);
+            else if (epi == EPI_ADD_F32) SKINNY_MT(EPI_ADD_F32, false); else SKINNY_MT(EPI_STORE_BF16, false);
+            GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
+            return 0;
+        }
         GI_REQUIRE(scratch != nullptr && scratch_floats >= (long)splits * M * N, "gemm_bf16: scratch of %ld floats needed, %ld given",
                    (long)splits * M * N, scratch_floats);
         int k_per_split = (K + splits - 1) / splits;
-        k_per_split = (k_per_split + SK - 1) / SK * SK;
+        k_per_split = (k_per_split + KB - 1) / KB * KB;
         dim3 grid((N + 63) / 64, splits);
-        const int mt = (M + 15) / 16;
-#define SKINNY(MT) gemm_bf16_skinny_kernel<MT><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, scratch, M, N, K, lda, ldw, k_per_split)
-        if (mt == 1) SKINNY(1); else if (mt == 2) SKINNY(2); else if (mt == 3) SKINNY(3); else SKINNY(4);
-#undef SKINNY
+        SKINNY_MT(EPI_STORE_F32, true);
+#undef SKINNY_MT
         GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
         const unsigned blocks = (unsigned)(((size_t)M * N + 255) / 256);
         if (epi == EPI_GATED_BF16) skinny_reduce_gated_kernel<<<(unsigned)(((size_t)M * (N / 2) + 255) / 256), 256, 0, stream>>>(scratch, (bf16_t*)C, M, N, splits, ldc);

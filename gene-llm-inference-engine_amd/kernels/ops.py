@@ -386,7 +386,7 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False):
     _need(out.shape == (m, n // 2 if gated else n), f"gemm: out is {tuple(out.shape)}, ({m}, {n // 2 if gated else n}) is needed")
     _need(gemm_bf16_supports(a, w, out), "gemm_bf16: operands must be bfloat16 with K and row strides multiples of 8, 16-byte aligned")
     scratch, n_scratch = None, 0
-    if 16 < m <= 64:
+    if m <= 64:
         n_scratch = lib().gi_gemm_bf16_skinny_splits(n, k) * m * n
         scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device)
     _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,
