@@ -1,14 +1,17 @@
 // C[m, n] (=|+=) sum_k A[m, k] * W[n, k] with bfloat16 operands on the matrix cores, 32-bit sums.
 //
 // Both operands are row-major with k contiguous, so each lane's operand of a matrix instruction is
-// one 16-byte load of 8 consecutive k.  Two kernels:
+// one 16-byte load of 8 consecutive k.  Four kernels:
 //
-//   tiled   a BM x 128 tile of C per workgroup of 4 waves, operands staged through LDS in
-//           k-blocks of 64 with the next block's global loads in flight during the products;
-//           v_mfma_f32_32x32x16_bf16.  For prompts (many rows).
-//   skinny  17..64 rows of A: weights stream from HBM straight into registers and are used
-//           once, activations go through LDS; v_mfma_f32_16x16x32_bf16.  k may be split over
-//           workgroups, partial sums are then added in a fixed order by a second kernel.
+//   piped   prompts (128 rows or more, K a multiple of 64): tiles of 128 x 128 or 256 x 256,
+//           operands loaded from global memory straight into a ring of LDS stages, several
+//           blocks of k in flight; v_mfma_f32_32x32x16_bf16.
+//   tiled   the other shapes above 64 rows: a BM x 128 tile of C per workgroup of 4 waves,
+//           operands staged through registers into LDS in k-blocks of 64.
+//   skinny  up to 64 rows of A: weights stream from HBM straight into registers and are used
+//           once, activations go through LDS; v_mfma_f32_16x16x32_bf16.  Wide outputs are
+//           finished by the workgroup that sees all of k; for narrow ones k is split over
+//           workgroups and the partial sums are added in a fixed order by a second kernel.
 //   slim    at most 16 rows of A (decode): a workgroup of 8 waves owns 16 (or 2 x 16) weight
 //           rows, its waves take interleaved blocks of k and add their sums through LDS in a
 //           fixed order, so one launch does the whole product and its epilogue.
@@ -123,6 +126,110 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
                 const int n = n0 + wn + j * 32 + (lane & 31);
                 if constexpr (EPI == EPI_GATED_BF16) {
                     // columns 32b .. 32b+15 are gates, 32b+16 .. 32b+31 the ups of outputs 16b .. 16b+15
+                    const float up = __shfl_xor(acc[i][j][v], 16, 64);
+                    if ((lane & 16) == 0 && m < M && n < N)
+                        ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(silu_gate(acc[i][j][v], up));
+                } else {
+                    if (m < M && n < N) write_out<EPI>(C, (size_t)m * ldc + n, acc[i][j][v]);
+                }
+            }
+}
+
+// ------------------------------------------------------------------------------------------ piped
+// The same product for large shapes, with the operands going from global memory straight into LDS
+// (global_load_lds_dwordx4: no registers in between) through a ring of blocks of 64 k, so that
+// several blocks are in flight while one is multiplied.  Workgroup: 4 waves (2 x 2), a tile of
+// BM x BN; a wave owns (BM/2) x (BN/2).  A stage holds BM rows of A, then BN rows of W, 128 bytes
+// (a cache line) each; a wave-wide load fills 8 rows.  The 16-byte chunk c of row `row` lies at
+// chunk position c ^ ((row >> 1) & 7): the loads write LDS contiguously, and the 16-byte reads
+// of 16 consecutive rows (what one clock serves: 64 banks of 4 bytes) hit 16 different slots,
+// without padding (a load cannot pad).  Needs K % 64 == 0; rows beyond M or N are read from the
+// last valid row and their results are dropped.
+constexpr int PK = 64;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int EPI>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
+                                                             int M, int N, int K, long lda, long ldw, long ldc) {
+    constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
+    constexpr int ROWS = BM + BN, STAGE_BYTES = ROWS * 128, LOADS = ROWS / 8 / (WAVES_M * WAVES_N);      // loads per wave and stage
+    static_assert(ROWS % (8 * WAVES_M * WAVES_N) == 0, "the rows of a stage must divide among the waves' loads");
+    static_assert(STAGES >= 2 && STAGES <= 4, "the counted waits below cover 2 to 4 stages");
+    extern __shared__ __attribute__((aligned(16))) unsigned char ring[];               // STAGES * STAGE_BYTES
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+    const bf16_t* src[LOADS];                  // this lane's source of each of its wave's loads, at k = 0
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int row = (wave * LOADS + i) * 8 + (lane >> 3), c = (lane & 7) ^ ((row >> 1) & 7);
+        src[i] = row < BM ? A + (size_t)min(m0 + row, M - 1) * lda + 8 * c : W + (size_t)min(n0 + row - BM, N - 1) * ldw + 8 * c;
+    }
+    // The loads are written as assembly so that the compiler does not see them: it would otherwise wait for all of
+    // them before every read of LDS and at every barrier, and nothing would stay in flight.  What orders them against
+    // the reads is below: the counted wait, then the barrier.
+    const unsigned ring_base = (unsigned)(size_t)(lds_ptr_t)ring;
+    auto issue = [&](int slot, int k0) {
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const unsigned dst = __builtin_amdgcn_readfirstlane(ring_base + slot * STAGE_BYTES + (wave * LOADS + i) * 1024);   // the wave's 1 KB; lane l lands at + 16 l
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(dst), "v"(src[i] + k0) : "memory", "m0");
+        }
+    };
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = floatx16{};
+
+    const int n_k = K / PK;
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s)
+        if (s < n_k) issue(s, s * PK);
+    const int r = lane & 31, swz = (r >> 1) & 7;
+    const unsigned char* a_rows = ring + (wm + r) * 128;
+    const unsigned char* b_rows = ring + (BM + wn + r) * 128;
+    for (int it = 0; it < n_k; ++it) {
+        // this wave's part of block `it` has landed when at most the loads of the blocks after it are outstanding
+        const int ahead = min(n_k - 1 - it, STAGES - 2);
+        if (ahead >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * LOADS) : "memory");
+        else if (ahead == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();          // everyone's part has landed, and everyone has finished block it-1
+        asm volatile("" ::: "memory");
+        if (it + STAGES - 1 < n_k) issue((it + STAGES - 1) % STAGES, (it + STAGES - 1) * PK);      // into the slot of block it-1
+        const int stage_off = (it % STAGES) * STAGE_BYTES;
+        // operands of the next 16 k are read while the products of these 16 run
+        bf16x8 a[2][TM], b[2][TN];
+        auto read_operands = [&](int ks, bf16x8* av, bf16x8* bv) {
+            const int chunk = (((ks >> 3) + (lane >> 5)) ^ swz) * 16;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) av[i] = as_bf16x8(*reinterpret_cast<const uint4*>(a_rows + stage_off + i * 32 * 128 + chunk));
+#pragma unroll
+            for (int j = 0; j < TN; ++j) bv[j] = as_bf16x8(*reinterpret_cast<const uint4*>(b_rows + stage_off + j * 32 * 128 + chunk));
+        };
+        read_operands(0, a[0], b[0]);
+#pragma unroll
+        for (int step = 0; step < PK / 16; ++step) {
+            if (step + 1 < PK / 16) read_operands(16 * (step + 1), a[(step + 1) & 1], b[(step + 1) & 1]);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[step & 1][i], b[step & 1][j], acc[i][j], 0, 0, 0);
+        }
+    }
+    // Element v of a lane's 32x32 result: row 8*(v/4) + 4*(lane/32) + v%4, column lane%32.
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = m0 + wm + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3);
+                const int n = n0 + wn + j * 32 + (lane & 31);
+                if constexpr (EPI == EPI_GATED_BF16) {
                     const float up = __shfl_xor(acc[i][j][v], 16, 64);
                     if ((lane & 16) == 0 && m < M && n < N)
                         ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(silu_gate(acc[i][j][v], up));
@@ -357,8 +464,10 @@ int epilogue_of(int c_dtype, int accumulate) {
 // Number of k-splits the skinny kernel would use, so that the caller can size the scratch
 // (splits * M * N floats).  Enough workgroups to cover the chip, each with at least 256 of k.
 // Tuning knob: 0 lets the entry point choose the tile height of the tiled kernel, 64 or 128 forces it.
-static int g_force_bm = 0;
+static int g_force_bm = 0, g_piped = 1;
 GI_API void gi_gemm_bf16_set_tile(int bm) { g_force_bm = bm; }
+// Tuning knob: 0 sends large products to the register-staged tiled kernel instead of the LDS-ring kernel.
+GI_API void gi_gemm_bf16_set_piped(int on) { g_piped = on; }
 
 
 // Number of k-splits of the skinny kernel for a product with 17..64 rows, so that the caller can size
@@ -445,6 +554,36 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     }
 
     GI_REQUIRE((M + 63) / 64 <= 65535, "gemm_bf16: M %d is too large", M);
+    if (K % PK == 0 && M >= 128 && N >= 128 && g_piped) {
+#define PIPED(BM_, BN_, WM_, WN_, ST_, EPI_)                                                                                                      \
+    do {                                                                                                                                \
+        constexpr int bytes = ST_ * (BM_ + BN_) * 128;                                                                                  \
+        static bool raised = false;                                                                                                     \
+        if (!raised) {                                                                                                                  \
+            if (hipFuncSetAttribute((const void*)gemm_bf16_piped_kernel<BM_, BN_, WM_, WN_, ST_, EPI_>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) \
+                return gi_fail("gemm_bf16: cannot reserve %d bytes of LDS", bytes);                                                     \
+            raised = true;                                                                                                              \
+        }                                                                                                                               \
+        dim3 grid((N + BN_ - 1) / BN_, (M + BM_ - 1) / BM_);                                                                            \
+        gemm_bf16_piped_kernel<BM_, BN_, WM_, WN_, ST_, EPI_><<<grid, 64 * WM_ * WN_, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+    } while (0)
+#define PIPED_EPI(BM_, BN_, WM_, WN_, ST_)                                                                                              \
+    do {                                                                                                                                \
+        if (epi == EPI_STORE_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_F32); else if (epi == EPI_ADD_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_ADD_F32);  \
+        else if (epi == EPI_STORE_BF16) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_BF16); else PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_BF16);                \
+    } while (0)
+        // Measured at 2,048 rows (K = 2048 and 8192): where 256 x 256 tiles still give every compute unit two, they halve
+        // the traffic into LDS; otherwise 128 x 128, two workgroups per unit with two stages each when there are enough
+        // tiles, else one workgroup of eight waves with four stages.
+        const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128), tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+        if (tiles256 >= 512) PIPED_EPI(256, 256, 4, 2, 2);
+        else if (tiles128 > 256) PIPED_EPI(128, 128, 2, 2, 2);
+        else PIPED_EPI(128, 128, 2, 4, 4);
+#undef PIPED_EPI
+#undef PIPED
+        GI_CHECK_LAUNCH("gemm_bf16 (piped)");
+        return 0;
+    }
 #define TILED(BM_, EPI_) gemm_bf16_tiled_kernel<BM_, EPI_><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
     if (g_force_bm == 64 || (g_force_bm == 0 && (long)((M + 127) / 128) * ((N + BN - 1) / BN) < 512)) {   // few tiles: smaller ones fill more of the chip
         dim3 grid((N + BN - 1) / BN, (M + 63) / 64);

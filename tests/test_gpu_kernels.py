@@ -52,7 +52,11 @@ def test_gemm_exact_rows_alone_have_the_same_bits():
 
 @pytest.mark.parametrize("m,n,k", [(1, 16, 8), (1, 2048, 2048), (3, 100, 136), (8, 130, 264), (16, 64, 128), (17, 1000, 520),
                                    (33, 48, 72), (64, 515, 1032), (65, 128, 64), (100, 300, 200), (128, 128, 128), (200, 257, 96),
-                                   (513, 384, 1024), (2048, 96, 160)])
+                                   (513, 384, 1024), (2048, 96, 160),
+                                   # the LDS-ring kernel: one block of k, edge tiles, each of its three tile choices
+                                   (256, 160, 64), (130, 129, 192), (2100, 2200, 192), (4000, 8200, 128),
+                                   # wide outputs finished by the skinny kernel itself, from 12 rows and from 5
+                                   (12, 12300, 520), (40, 12300, 264), (5, 65600, 72), (16, 12288, 256)])
 @pytest.mark.parametrize("out_dtype,accumulate", [(torch.float32, False), (torch.float32, True), (torch.bfloat16, False)])
 def test_gemm_bf16(m, n, k, out_dtype, accumulate):
     a, w = randn(m, k, dtype=torch.bfloat16, seed=5), randn(n, k, dtype=torch.bfloat16, seed=6)
@@ -65,7 +69,8 @@ def test_gemm_bf16(m, n, k, out_dtype, accumulate):
     assert torch.equal(out[:, n:], base[:, n:])
 
 
-@pytest.mark.parametrize("m,inter,k", [(1, 16, 8), (5, 48, 136), (16, 160, 96), (17, 176, 64), (64, 32, 264), (70, 192, 128), (300, 8192 // 16, 2048 // 8)])
+@pytest.mark.parametrize("m,inter,k", [(1, 16, 8), (5, 48, 136), (16, 160, 96), (17, 176, 64), (64, 32, 264), (70, 192, 128), (300, 8192 // 16, 2048 // 8),
+                                       (40, 6144, 264), (13, 6160, 72), (64, 8192, 512), (2048, 1024, 192), (600, 288, 64)])
 def test_gemm_bf16_gated(m, inter, k):
     a = randn(m, k, dtype=torch.bfloat16, seed=15)
     gate, up = randn(inter, k, dtype=torch.bfloat16, seed=16, scale=0.3), randn(inter, k, dtype=torch.bfloat16, seed=17, scale=0.3)
