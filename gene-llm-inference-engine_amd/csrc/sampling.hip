@@ -3,7 +3,8 @@
 // number per row.  Rules as the reference's host sampler states them
 // (src/sampler/sampler.cpp:54-80, 119-128): p_i = exp((l_i - max) / T) in 32-bit, sums in 64-bit,
 // tokens walked in index order, the first with r = u * total < cumulative sum wins, the last
-// token if rounding lets none win.
+// token if rounding lets none win.  (The 64-bit sums are taken in a tree, not one by one: the draw
+// can differ from the reference's only where r falls within rounding of a boundary.)
 #include "common.h"
 
 namespace {
@@ -52,58 +53,98 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restric
     if (threadIdx.x == 0) out[blockIdx.x] = bi;
 }
 
-// Each thread owns a contiguous run of tokens, so that cumulative sums follow index order.
-__global__ __launch_bounds__(NT) void sample_temperature_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
-                                                                const float* __restrict__ uniform, int* __restrict__ out, int vocab,
-                                                                long stride) {
-    __shared__ float red_f[NT / 64];
-    __shared__ double run_start[NT];
-    __shared__ double total_s;
+// Temperature sampling in three stages, so that a few rows still fill the chip: the maxima of runs of
+// CHUNK logits (one workgroup each); with the row's maximum known, the runs' sums of p = exp((l - max) / T)
+// in 64-bit; then one workgroup per row finds the run that holds r = u * total (runs in index order),
+// gives each of its threads 16 consecutive tokens of that run, finds the thread by a prefix sum, and that
+// thread walks its tokens one by one.  Cumulative sums follow index order up to the rounding of 64-bit sums.
+__global__ __launch_bounds__(256) void chunk_max_kernel(const float* __restrict__ logits, float* __restrict__ part_m, int vocab, long stride,
+                                                        int n_chunks) {
+    __shared__ float red[4];
+    const float* row = logits + (size_t)blockIdx.y * stride;
+    const int begin = blockIdx.x * CHUNK, end = min(vocab, begin + CHUNK);
+    float mx = -INFINITY;
+    for (int i = begin + threadIdx.x; i < end; i += 256) mx = fmaxf(mx, row[i]);
+    mx = wave_max(mx);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+    __syncthreads();
+    if (threadIdx.x == 0) part_m[(size_t)blockIdx.y * n_chunks + blockIdx.x] = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ float row_max(const float* __restrict__ part_m, int n_chunks) {       // the same value in every thread
+    float mx = -INFINITY;
+    for (int c = 0; c < n_chunks; ++c) mx = fmaxf(mx, part_m[c]);
+    return mx;
+}
+
+__global__ __launch_bounds__(256) void chunk_sum_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                        const float* __restrict__ part_m, double* __restrict__ part_s, int vocab,
+                                                        long stride, int n_chunks) {
+    __shared__ double red[4];
+    const float* row = logits + (size_t)blockIdx.y * stride;
+    const float temp = temperature[blockIdx.y], mx = row_max(part_m + (size_t)blockIdx.y * n_chunks, n_chunks);
+    const int begin = blockIdx.x * CHUNK, end = min(vocab, begin + CHUNK);
+    double sum = 0.0;
+    for (int i = begin + threadIdx.x; i < end; i += 256) sum += (double)expf((row[i] - mx) / temp);
+    sum = wave_sum_f64(sum);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) part_s[(size_t)blockIdx.y * n_chunks + blockIdx.x] = ((red[0] + red[1]) + red[2]) + red[3];
+}
+
+constexpr int RUN = CHUNK / 256;            // tokens a thread of the last stage owns
+
+__global__ __launch_bounds__(256) void sample_pick_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+                                                          const float* __restrict__ uniform, const float* __restrict__ part_m,
+                                                          const double* __restrict__ part_s, int* __restrict__ out, int vocab, long stride,
+                                                          int n_chunks) {
+    __shared__ double wave_total[4];
     __shared__ int winner;
     const float* row = logits + (size_t)blockIdx.x * stride;
-    const float temp = temperature[blockIdx.x];
-    const int tid = threadIdx.x;
-
-    float mx = -INFINITY;
-    for (int i = tid; i < vocab; i += NT) mx = fmaxf(mx, row[i]);
-    mx = wave_max(mx);
-    if ((tid & 63) == 0) red_f[tid >> 6] = mx;
-    __syncthreads();
-    mx = red_f[0];
-    for (int w = 1; w < NT / 64; ++w) mx = fmaxf(mx, red_f[w]);
-
-    const int per = (vocab + NT - 1) / NT;
-    const int begin = min(vocab, tid * per), end = min(vocab, begin + per);
-    double mine = 0.0;
-    for (int i = begin; i < end; ++i) mine += (double)expf((row[i] - mx) / temp);
-    run_start[tid] = mine;
-    if (tid == 0) winner = vocab - 1;       // if rounding lets no token win, the last one does
-    __syncthreads();
-    if (tid == 0) {                         // prefix sums of the 1024 run totals, in index order
-        double c = 0.0;
-        for (int i = 0; i < NT; ++i) {
-            const double s = run_start[i];
-            run_start[i] = c;
-            c += s;
-        }
-        total_s = c;
-    }
-    __syncthreads();
+    const float temp = temperature[blockIdx.x], mx = row_max(part_m + (size_t)blockIdx.x * n_chunks, n_chunks);
+    const double* sums = part_s + (size_t)blockIdx.x * n_chunks;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // The reference normalises p by a 32-bit 1/sum before it draws; the draw compares u * sum(p) with
     // cumulative p, which is the same comparison scaled by a constant, so it is made on the
     // unnormalised values here.
-    const double r = (double)uniform[blockIdx.x] * total_s;
-    const double start = run_start[tid];
-    const double stop = (tid == NT - 1) ? total_s : run_start[tid + 1];
-    if (begin < end && r >= start && r < stop) {
-        double c = start;
-        int pick = -1;
-        for (int i = begin; i < end; ++i) {
-            c += (double)expf((row[i] - mx) / temp);
-            if (r < c) { pick = i; break; }
+    double total = 0.0;
+    for (int c = 0; c < n_chunks; ++c) total += sums[c];
+    const double r = (double)uniform[blockIdx.x] * total;
+    int chunk = n_chunks - 1;                // the run that holds r (the last one if rounding lets none hold it)
+    double before = 0.0;
+    for (int c = 0; c < n_chunks - 1; ++c) {
+        if (r < before + sums[c]) { chunk = c; break; }
+        before += sums[c];
+    }
+    const int begin = chunk * CHUNK, end = min(vocab, begin + CHUNK);
+    const int lo = min(end, begin + tid * RUN), hi = min(end, lo + RUN);
+    double mine = 0.0;
+    for (int i = lo; i < hi; ++i) mine += (double)expf((row[i] - mx) / temp);
+    double c = mine;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {                  // inclusive prefix sum over the lanes of a wave
+        const double below = __shfl_up(c, off, 64);
+        if (lane >= off) c += below;
+    }
+    if (lane == 63) wave_total[wave] = c;
+    if (tid == 0) winner = min(end, vocab - 1);              // if rounding leaves r beyond the run: the next token in index order
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) before += wave_total[w];
+    const double run_stop = before + c, run_start = run_stop - mine;
+    if (lo < hi && r >= run_start && r < run_stop) {          // at most one thread
+        double walk = run_start;
+        int pick = min(hi, vocab - 1);
+        for (int i = lo; i < hi; ++i) {
+            walk += (double)expf((row[i] - mx) / temp);
+            if (r < walk) { pick = i; break; }
         }
-        // Rounding may leave r just beyond this run's last partial sum: the next token in index order wins.
-        winner = pick >= 0 ? pick : min(end, vocab - 1);
+        winner = pick;
     }
     __syncthreads();
     if (tid == 0) out[blockIdx.x] = winner;
@@ -125,10 +166,17 @@ GI_API int gi_argmax(const float* logits, int* out, float* part_v, int* part_i, 
     return 0;
 }
 
-GI_API int gi_sample_temperature(const float* logits, const float* temperature, const float* uniform, int* out, int n_rows, int vocab,
-                                 long stride, hipStream_t stream) {
-    GI_REQUIRE(n_rows > 0 && vocab > 0 && stride >= vocab, "sample_temperature: bad sizes (rows %d, vocab %d, stride %ld)", n_rows, vocab, stride);
-    sample_temperature_kernel<<<n_rows, NT, 0, stream>>>(logits, temperature, uniform, out, vocab, stride);
-    GI_CHECK_LAUNCH("sample_temperature");
+// part_m: n_rows * gi_argmax_chunks(vocab) floats, part_s: as many doubles.
+GI_API int gi_sample_temperature(const float* logits, const float* temperature, const float* uniform, int* out, float* part_m, double* part_s,
+                                 int n_rows, int vocab, long stride, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && n_rows <= 65535 && vocab > 0 && stride >= vocab, "sample_temperature: bad sizes (rows %d, vocab %d, stride %ld)", n_rows, vocab, stride);
+    GI_REQUIRE(part_m != nullptr && part_s != nullptr, "sample_temperature: scratch is missing");
+    const int n_chunks = gi_argmax_chunks(vocab);
+    chunk_max_kernel<<<dim3(n_chunks, n_rows), 256, 0, stream>>>(logits, part_m, vocab, stride, n_chunks);
+    GI_CHECK_LAUNCH("sample_temperature (maxima)");
+    chunk_sum_kernel<<<dim3(n_chunks, n_rows), 256, 0, stream>>>(logits, temperature, part_m, part_s, vocab, stride, n_chunks);
+    GI_CHECK_LAUNCH("sample_temperature (sums)");
+    sample_pick_kernel<<<n_rows, 256, 0, stream>>>(logits, temperature, uniform, part_m, part_s, out, vocab, stride, n_chunks);
+    GI_CHECK_LAUNCH("sample_temperature (pick)");
     return 0;
 }

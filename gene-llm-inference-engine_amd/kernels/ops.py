@@ -37,7 +37,7 @@ _SIGNATURES = {
                                  c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_int, c_int, c_void_p],
     "gi_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
-    "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
+    "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
 }
 
 _lib = None
@@ -420,6 +420,9 @@ def sample_temperature(logits, temperature, uniform, out):
     for t, name in ((temperature, "temperature"), (uniform, "uniform")):
         _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= n, f"sample: {name} must be float32 [n]")
     _i32(out, "sample: out", n)
-    _call("gi_sample_temperature", logits.data_ptr(), temperature.data_ptr(), uniform.data_ptr(), out.data_ptr(), n, vocab,
-          logits.stride(0), _stream())
+    chunks = lib().gi_argmax_chunks(vocab)
+    part_m = torch.empty(n * chunks, dtype=torch.float32, device=logits.device)
+    part_s = torch.empty(n * chunks, dtype=torch.float64, device=logits.device)
+    _call("gi_sample_temperature", logits.data_ptr(), temperature.data_ptr(), uniform.data_ptr(), out.data_ptr(), part_m.data_ptr(),
+          part_s.data_ptr(), n, vocab, logits.stride(0), _stream())
     return out

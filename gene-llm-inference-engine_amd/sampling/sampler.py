@@ -104,6 +104,9 @@ class Sampler:
         config.validate(vocab_size)
         self.config, self.vocab_size = config, vocab_size
         self.stream = UniformStream(config.seed)
+        # where this sampler's rows go in `sample_rows`: arg max, plain temperature (both on the device), filtered (host)
+        self.kind = "greedy" if config.greedy else "filtered" if config.filters(vocab_size) else "plain"
+        self.temperature = float(config.temperature)
 
     def next_uniform(self) -> float:
         return self.stream.next_uniform()
@@ -119,14 +122,17 @@ def sample_rows(logits: torch.Tensor, samplers: Sequence[Sampler]) -> List[int]:
     n, vocab = logits.shape
     if n != len(samplers):
         raise ValueError(f"{n} rows of logits for {len(samplers)} samplers")
-    if all(s.config.greedy for s in samplers):                   # the common case without a list per kind
-        res = torch.empty(n, dtype=torch.int32, device=logits.device)
-        return ops.argmax(logits, res).tolist()
-    out: List[int] = [0] * n
-    greedy = [i for i, s in enumerate(samplers) if s.config.greedy]
-    host = [i for i, s in enumerate(samplers) if not s.config.greedy and s.config.filters(vocab)]
-    plain = [i for i, s in enumerate(samplers) if not s.config.greedy and not s.config.filters(vocab)]
     dev = logits.device
+    kinds = {s.kind for s in samplers}
+    if kinds == {"greedy"}:                                      # the two common cases without a list per kind
+        return ops.argmax(logits, torch.empty(n, dtype=torch.int32, device=dev)).tolist()
+    if kinds == {"plain"}:
+        both = torch.tensor([[s.temperature for s in samplers], [s.stream.next_uniform() for s in samplers]], dtype=torch.float32).to(dev)
+        return ops.sample_temperature(logits, both[0], both[1], torch.empty(n, dtype=torch.int32, device=dev)).tolist()
+    out: List[int] = [0] * n
+    greedy = [i for i, s in enumerate(samplers) if s.kind == "greedy"]
+    host = [i for i, s in enumerate(samplers) if s.kind == "filtered"]
+    plain = [i for i, s in enumerate(samplers) if s.kind == "plain"]
     pending = []
     if greedy:
         rows = logits if len(greedy) == n else logits[torch.tensor(greedy, device=dev)]
@@ -135,10 +141,10 @@ def sample_rows(logits: torch.Tensor, samplers: Sequence[Sampler]) -> List[int]:
         pending.append((greedy, res))
     if plain:
         rows = logits if len(plain) == n else logits[torch.tensor(plain, device=dev)]
-        temps = torch.tensor([samplers[i].config.temperature for i in plain], dtype=torch.float32).to(dev)
-        us = torch.tensor([samplers[i].next_uniform() for i in plain], dtype=torch.float32).to(dev)
+        both = torch.tensor([[samplers[i].temperature for i in plain], [samplers[i].next_uniform() for i in plain]],
+                            dtype=torch.float32).to(dev)                       # one copy for temperatures and uniform numbers
         res = torch.empty(len(plain), dtype=torch.int32, device=dev)
-        ops.sample_temperature(rows, temps, us, res)
+        ops.sample_temperature(rows, both[0], both[1], res)
         pending.append((plain, res))
     if host:
         rows = logits[torch.tensor(host, device=dev)].cpu().numpy()
