@@ -83,12 +83,17 @@ class PageGroup:
     def held_pages(self, slot: int) -> List[int]:
         return [int(p) for p in self.table_host[slot, int(self.first_live[slot]):int(self.n_held[slot])]]
 
-    def sync(self) -> None:
+    def sync(self, upload=None) -> None:
         if self.table_dev is None or not self.dirty:
             self.dirty.clear()
             return
         rows = sorted(self.dirty)
         self.dirty.clear()
+        if upload is not None:                 # int32 array -> device tensor without waiting for the device
+            idx = upload(np.asarray(rows, dtype=np.int32))
+            data = upload(self.table_host[rows]).view(len(rows), self.table_host.shape[1])
+            self.table_dev.index_copy_(0, idx.long(), data)
+            return
         idx = torch.tensor(rows, dtype=torch.int64)
         data = torch.from_numpy(self.table_host[rows])
         self.table_dev.index_copy_(0, idx.to(self.table_dev.device), data.to(self.table_dev.device))
@@ -244,10 +249,11 @@ class CacheManager:
         for g in self.groups:
             g.drop_behind_window(slot, new_length)
 
-    def sync(self) -> None:
-        """Brings the device copies of changed page tables up to date."""
+    def sync(self, upload=None) -> None:
+        """Brings the device copies of changed page tables up to date.  `upload(int32 array) -> device tensor`
+        is the caller's way of copying without waiting for the device (it must take a snapshot at once)."""
         for g in self.groups:
-            g.sync()
+            g.sync(upload)
 
     # --------------------------------------------------------------------------------- views
     def kv(self, entry: int):

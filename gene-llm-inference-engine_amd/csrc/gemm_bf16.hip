@@ -144,13 +144,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
 // chunk position c ^ ((row >> 1) & 7): the loads write LDS contiguously, and the 16-byte reads
 // of 16 consecutive rows (what one clock serves: 64 banks of 4 bytes) hit 16 different slots,
 // without padding (a load cannot pad).  Needs K % 64 == 0; rows beyond M or N are read from the
-// last valid row and their results are dropped.
+// last valid row and their results are dropped.  With few tiles, k is split over the grid's z: each
+// workgroup then writes the sums of its share to its own [M, N] slab of 32-bit partial results, and the
+// reduce kernel below adds the slabs in order and applies the epilogue.
 constexpr int PK = 64;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int EPI>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
-                                                             int M, int N, int K, long lda, long ldw, long ldc) {
+                                                             int M, int N, int K, long lda, long ldw, long ldc, int k_per_split,
+                                                             long split_stride) {
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int ROWS = BM + BN, STAGE_BYTES = ROWS * 128, LOADS = ROWS / 8 / (WAVES_M * WAVES_N);      // loads per wave and stage
     static_assert(ROWS % (8 * WAVES_M * WAVES_N) == 0, "the rows of a stage must divide among the waves' loads");
@@ -165,7 +168,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
     for (int i = 0; i < LOADS; ++i) {
         const int row = (wave * LOADS + i) * 8 + (lane >> 3), c = (lane & 7) ^ ((row >> 1) & 7);
         src[i] = row < BM ? A + (size_t)min(m0 + row, M - 1) * lda + 8 * c : W + (size_t)min(n0 + row - BM, N - 1) * ldw + 8 * c;
+        src[i] += (size_t)blockIdx.z * k_per_split;           // this workgroup's share of k (all of it without a split)
     }
+    if (split_stride) C = (float*)C + (size_t)blockIdx.z * split_stride;       // ... and its own partial result
     // The loads are written as assembly so that the compiler does not see them: it would otherwise wait for all of
     // them before every read of LDS and at every barrier, and nothing would stay in flight.  What orders them against
     // the reads is below: the counted wait, then the barrier.
@@ -184,7 +189,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = floatx16{};
 
-    const int n_k = K / PK;
+    const int n_k = min(K - (int)blockIdx.z * k_per_split, k_per_split) / PK;
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
         if (s < n_k) issue(s, s * PK);
@@ -481,6 +486,33 @@ GI_API int gi_gemm_bf16_skinny_splits(int N, int K) {
     return splits;
 }
 
+// Splits of k for the LDS-ring kernel (more than 64 rows): with fewer than 192 tiles of 128 x 128 the tiles alone
+// leave compute units idle and the weights stream too slowly; every share keeps at least 256 of k.
+GI_API int gi_gemm_bf16_piped_splits(int M, int N, int K) {
+    if (M <= 64 || K % PK != 0 || N < 128) return 1;
+    const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+    int splits = 1;
+    while (tiles * splits < 192 && K % (splits * 2 * PK) == 0 && K / (splits * 2) >= 256) splits *= 2;
+    return splits;
+}
+
+// Floats of scratch a product of these sizes needs (partial sums of k-splits), 0 if none.
+GI_API long gi_gemm_bf16_scratch_floats(int M, int N, int K) {
+    if (M <= 64) return (long)gi_gemm_bf16_skinny_splits(N, K) * M * N;
+    const int splits = gi_gemm_bf16_piped_splits(M, N, K);
+    return splits > 1 ? (long)splits * M * N : 0;
+}
+
+static int reduce_partials(const float* scratch, void* C, int epi, int M, int N, int splits, long ldc, hipStream_t stream) {
+    const unsigned blocks = (unsigned)(((size_t)M * N + 255) / 256);
+    if (epi == EPI_GATED_BF16) skinny_reduce_gated_kernel<<<(unsigned)(((size_t)M * (N / 2) + 255) / 256), 256, 0, stream>>>(scratch, (bf16_t*)C, M, N, splits, ldc);
+    else if (epi == EPI_STORE_F32) skinny_reduce_kernel<EPI_STORE_F32><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
+    else if (epi == EPI_ADD_F32) skinny_reduce_kernel<EPI_ADD_F32><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
+    else skinny_reduce_kernel<EPI_STORE_BF16><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
+    GI_CHECK_LAUNCH("gemm_bf16 (reduce)");
+    return 0;
+}
+
 // `gated` != 0: W is [gate; up] interleaved in groups of 16 rows (N rows in all, a multiple of 32)
 // and C is bfloat16 [M, N/2] = silu(gate) * up.
 GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int accumulate, int gated, int M, int N, int K, long lda,
@@ -544,18 +576,12 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
         SKINNY_MT(EPI_STORE_F32, true);
 #undef SKINNY_MT
         GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
-        const unsigned blocks = (unsigned)(((size_t)M * N + 255) / 256);
-        if (epi == EPI_GATED_BF16) skinny_reduce_gated_kernel<<<(unsigned)(((size_t)M * (N / 2) + 255) / 256), 256, 0, stream>>>(scratch, (bf16_t*)C, M, N, splits, ldc);
-        else if (epi == EPI_STORE_F32) skinny_reduce_kernel<EPI_STORE_F32><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
-        else if (epi == EPI_ADD_F32) skinny_reduce_kernel<EPI_ADD_F32><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
-        else skinny_reduce_kernel<EPI_STORE_BF16><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
-        GI_CHECK_LAUNCH("gemm_bf16 (reduce)");
-        return 0;
+        return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream);
     }
 
     GI_REQUIRE((M + 63) / 64 <= 65535, "gemm_bf16: M %d is too large", M);
-    if (K % PK == 0 && M >= 128 && N >= 128 && g_piped) {
-#define PIPED(BM_, BN_, WM_, WN_, ST_, EPI_)                                                                                                      \
+    if (K % PK == 0 && N >= 128 && g_piped) {
+#define PIPED(BM_, BN_, WM_, WN_, ST_, EPI_, OUT_, LDC_, SPLITS_, KPS_, SLAB_)                                                          \
     do {                                                                                                                                \
         constexpr int bytes = ST_ * (BM_ + BN_) * 128;                                                                                  \
         static bool raised = false;                                                                                                     \
@@ -564,14 +590,26 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
                 return gi_fail("gemm_bf16: cannot reserve %d bytes of LDS", bytes);                                                     \
             raised = true;                                                                                                              \
         }                                                                                                                               \
-        dim3 grid((N + BN_ - 1) / BN_, (M + BM_ - 1) / BM_);                                                                            \
-        gemm_bf16_piped_kernel<BM_, BN_, WM_, WN_, ST_, EPI_><<<grid, 64 * WM_ * WN_, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+        dim3 grid((N + BN_ - 1) / BN_, (M + BM_ - 1) / BM_, SPLITS_);                                                                   \
+        gemm_bf16_piped_kernel<BM_, BN_, WM_, WN_, ST_, EPI_><<<grid, 64 * WM_ * WN_, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, OUT_, M, N, K, lda, \
+                                                                                                        ldw, LDC_, KPS_, SLAB_);        \
     } while (0)
 #define PIPED_EPI(BM_, BN_, WM_, WN_, ST_)                                                                                              \
     do {                                                                                                                                \
-        if (epi == EPI_STORE_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_F32); else if (epi == EPI_ADD_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_ADD_F32);  \
-        else if (epi == EPI_STORE_BF16) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_BF16); else PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_BF16);                \
+        if (epi == EPI_STORE_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_F32, C, ldc, 1, K, 0L);                                      \
+        else if (epi == EPI_ADD_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_ADD_F32, C, ldc, 1, K, 0L);                                     \
+        else if (epi == EPI_STORE_BF16) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_BF16, C, ldc, 1, K, 0L);                               \
+        else PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_BF16, C, ldc, 1, K, 0L);                                                          \
     } while (0)
+        const int splits = gi_gemm_bf16_piped_splits(M, N, K);
+        if (splits > 1) {                              // few tiles: k is shared out, the sums are finished by the reduce kernel
+            GI_REQUIRE(scratch != nullptr && scratch_floats >= (long)splits * M * N, "gemm_bf16: scratch of %ld floats needed, %ld given",
+                       (long)splits * M * N, scratch_floats);
+            const int k_per_split = K / splits;
+            PIPED(128, 128, 2, 2, 2, EPI_STORE_F32, scratch, (long)N, splits, k_per_split, (long)M * N);
+            GI_CHECK_LAUNCH("gemm_bf16 (piped, split)");
+            return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream);
+        }
         // Measured at 2,048 rows (K = 2048 and 8192): where 256 x 256 tiles still give every compute unit two, they halve
         // the traffic into LDS; otherwise 128 x 128, two workgroups per unit with two stages each when there are enough
         // tiles, else one workgroup of eight waves with four stages.

@@ -74,6 +74,7 @@ class Runner:
         self.steps_run = 0
         self.use_graphs = bool(use_graphs) and model.graph_safe
         self._graphs = {}
+        self._uploads = _StepUploads(model.device, min(8 * self.max_rows + 1024, 1 << 18))       # at most 1 MiB a buffer; what is larger is copied the ordinary way
 
     # -------------------------------------------------------------------------------- requests
     def open(self, request: Hashable) -> None:
@@ -122,7 +123,8 @@ class Runner:
             return self._step_of_single_tokens(entries)
         n_rows = self._validate(entries)
         self.cache.reserve([(e.request, len(e.tokens)) for e in entries])       # OutOfPages: nothing changed
-        self.cache.sync()
+        self._uploads.begin_step()
+        self.cache.sync(self._uploads.put)
 
         meta = np.empty((3, n_rows), dtype=np.int32)                            # tokens, positions, slots
         seg_slot, seg_start, seg_len, seg_pos0, logit_rows = [], [], [], [], []
@@ -137,11 +139,13 @@ class Runner:
             row += n
 
         dev = self.model.device
-        meta_dev = torch.from_numpy(meta).to(dev)
-        rows_dev = torch.tensor(logit_rows, dtype=torch.int32).to(dev) if logit_rows else None
+        meta_dev = self._uploads.put(meta).view(3, n_rows)
+        rows_dev = self._uploads.put(np.asarray(logit_rows, dtype=np.int32)) if logit_rows else None
         ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
-                          row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0)
+                          row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0,
+                          upload=self._uploads.put)
         logits = self.model.forward(ctx, self._view, rows_dev, len(logit_rows))
+        self._uploads.end_step()
         for e in entries:
             self.cache.advance(e.request, len(e.tokens))
         self.steps_run += 1
@@ -172,7 +176,10 @@ class Runner:
         if n > self.max_rows:
             raise StepError(f"the step holds {n} rows, more than max_rows = {self.max_rows}")
         cache.reserve_one_each(requests, slots, lengths)                        # OutOfPages: nothing changed
-        cache.sync()
+        if any(g.dirty for g in cache.groups):
+            self._uploads.begin_step()
+            cache.sync(self._uploads.put)
+            self._uploads.end_step()
         logits = self._decode_step(np.array([tokens, lengths, slots], dtype=np.int32), slots, lengths)
         cache.advance_one_each(requests, slots, lengths)
         self.steps_run += 1
@@ -188,6 +195,46 @@ class Runner:
         if g is None:
             g = self._graphs[batch] = _DecodeGraph(self, batch)
         return g.run(meta, seg_slot, seg_pos0)
+
+
+class _StepUploads:
+    """The int32 data a step makes on the host (tokens, positions, slots, row lists, tile lists) goes to
+    the device through pinned memory with copies that do not wait: a ring of buffers, one per step in
+    flight; a buffer is taken again only after the copies of its last use have finished.  What `put`
+    returns is valid while the step runs."""
+    DEPTH = 4
+
+    def __init__(self, device, capacity: int):
+        self.device, self.capacity = device, capacity
+        on_gpu = torch.device(device).type == "cuda"
+        self.host = [torch.empty(capacity, dtype=torch.int32, pin_memory=on_gpu) for _ in range(self.DEPTH)]
+        self.dev = [torch.empty(capacity, dtype=torch.int32, device=device) for _ in range(self.DEPTH)]
+        self.done = [None] * self.DEPTH
+        self.turn, self.used = 0, 0
+
+    def begin_step(self) -> None:
+        self.turn = (self.turn + 1) % self.DEPTH
+        self.used = 0
+        if self.done[self.turn] is not None:
+            self.done[self.turn].synchronize()
+
+    def put(self, values: np.ndarray) -> torch.Tensor:
+        flat = np.ascontiguousarray(values, dtype=np.int32).reshape(-1)
+        n = flat.size
+        if self.used + n > self.capacity:                       # more than the ring was made for: an ordinary copy
+            return torch.from_numpy(flat.copy()).to(self.device)
+        a, b = self.used, self.used + n
+        self.used = (b + 3) & ~3                                # pieces start at multiples of 16 bytes
+        self.host[self.turn][a:b] = torch.from_numpy(flat)
+        piece = self.dev[self.turn][a:b]
+        piece.copy_(self.host[self.turn][a:b], non_blocking=True)
+        return piece
+
+    def end_step(self) -> None:
+        if torch.device(self.device).type == "cuda":
+            ev = self.done[self.turn] or torch.cuda.Event()
+            ev.record()
+            self.done[self.turn] = ev
 
 
 class _DecodeGraph:

@@ -55,20 +55,32 @@ def lib():
         l.gi_argmax_chunks.restype = c_int
         l.gi_attention_bf16_supports.argtypes = [c_int, c_int, c_int]
         l.gi_attention_bf16_supports.restype = c_int
-        l.gi_gemm_bf16_skinny_splits.argtypes = [c_int, c_int]
-        l.gi_gemm_bf16_skinny_splits.restype = c_int
+        l.gi_gemm_bf16_scratch_floats.argtypes = [c_int, c_int, c_int]
+        l.gi_gemm_bf16_scratch_floats.restype = c_long
         _lib = l
     return _lib
 
 
+_FUNCTIONS = {}
+
+
 def _call(name, *args):
-    l = lib()
-    rc = getattr(l, name)(*args)
-    if rc != 0:
-        raise KernelError(l.gi_last_error().decode())
+    fn = _FUNCTIONS.get(name)
+    if fn is None:
+        fn = _FUNCTIONS[name] = getattr(lib(), name)
+    if fn(*args) != 0:
+        raise KernelError(lib().gi_last_error().decode())
+
+
+# The current stream's handle, asked for at every launch (it changes under graph capture).  torch's
+# public way costs several microseconds a call, and a step makes over a hundred launches.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
 def _stream():
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -79,21 +91,18 @@ def _code(t: torch.Tensor, what: str) -> int:
         raise KernelError(f"{what} has dtype {t.dtype}; float32 or bfloat16 is needed") from None
 
 
-def _need(cond, msg):
-    if not cond:
-        raise KernelError(msg)
-
-
 def _dev(*tensors):
     for t in tensors:
-        if t is not None:
-            _need(t.is_cuda, "kernel operands must lie in device memory")
+        if t is not None and not t.is_cuda:
+            raise KernelError("kernel operands must lie in device memory")
 
 
 def _i32(t, what, n=None):
-    _need(t.dtype == torch.int32 and t.is_contiguous(), f"{what} must be a contiguous int32 tensor")
+    if not (t.dtype == torch.int32 and t.is_contiguous()):
+        raise KernelError(f"{what} must be a contiguous int32 tensor")
     if n is not None:
-        _need(t.numel() >= n, f"{what} holds {t.numel()} entries, {n} are needed")
+        if not (t.numel() >= n):
+            raise KernelError(f"{what} holds {t.numel()} entries, {n} are needed")
 
 
 def _ptr(t):
@@ -113,8 +122,10 @@ def embed(table, tokens, out):
     """out[t, :] = table[tokens[t], :] widened to float32."""
     _dev(table, tokens, out)
     n, dim = out.shape
-    _need(table.dim() == 2 and table.shape[1] == dim and table.is_contiguous(), "embed: table must be [vocab, dim], contiguous")
-    _need(out.dtype == torch.float32 and out.is_contiguous(), "embed: out must be contiguous float32")
+    if not (table.dim() == 2 and table.shape[1] == dim and table.is_contiguous()):
+        raise KernelError("embed: table must be [vocab, dim], contiguous")
+    if not (out.dtype == torch.float32 and out.is_contiguous()):
+        raise KernelError("embed: out must be contiguous float32")
     _i32(tokens, "embed: tokens", n)
     _call("gi_embed", table.data_ptr(), _code(table, "embed: table"), tokens.data_ptr(), out.data_ptr(), n, dim, _stream())
     return out
@@ -131,12 +142,16 @@ def rmsnorm(x, weight, eps, out, rows=None):
     _dev(x, weight, out, rows)
     dim = x.shape[1]
     n = x.shape[0] if rows is None else rows.numel()
-    _need(x.dtype == torch.float32 and x.stride(1) == 1, "rmsnorm: x must be float32 with unit inner stride")
-    _need(out.shape == (n, dim) and out.stride(1) == 1, "rmsnorm: out must be [rows, dim] with unit inner stride")
-    _need(weight.shape == (dim,) and weight.is_contiguous(), "rmsnorm: weight must be [dim]")
+    if not (x.dtype == torch.float32 and x.stride(1) == 1):
+        raise KernelError("rmsnorm: x must be float32 with unit inner stride")
+    if not (out.shape == (n, dim) and out.stride(1) == 1):
+        raise KernelError("rmsnorm: out must be [rows, dim] with unit inner stride")
+    if not (weight.shape == (dim,) and weight.is_contiguous()):
+        raise KernelError("rmsnorm: weight must be [dim]")
     if rows is not None:
         _i32(rows, "rmsnorm: rows", n)
-        _need(rmsnorm_can_gather(x, weight, out), "rmsnorm: these operands cannot be gathered in the kernel")
+        if not (rmsnorm_can_gather(x, weight, out)):
+            raise KernelError("rmsnorm: these operands cannot be gathered in the kernel")
     _call("gi_rmsnorm", x.data_ptr(), _ptr(rows), weight.data_ptr(), _code(weight, "rmsnorm: weight"), out.data_ptr(), _code(out, "rmsnorm: out"),
           n, dim, float(eps), x.stride(0), out.stride(0), _stream())
     return out
@@ -147,17 +162,20 @@ def rope_cos_sin(positions, inv_freq, cos_out, sin_out):
     _dev(positions, inv_freq, cos_out, sin_out)
     n, half = cos_out.shape
     _i32(positions, "rope_cos_sin: positions", n)
-    _need(inv_freq.dtype == torch.float64 and inv_freq.shape == (half,) and inv_freq.is_contiguous(), "rope_cos_sin: inv_freq must be float64 [half]")
+    if not (inv_freq.dtype == torch.float64 and inv_freq.shape == (half,) and inv_freq.is_contiguous()):
+        raise KernelError("rope_cos_sin: inv_freq must be float64 [half]")
     for t in (cos_out, sin_out):
-        _need(t.dtype == torch.float32 and t.is_contiguous() and t.shape == (n, half), "rope_cos_sin: outputs must be float32 [n, half]")
+        if not (t.dtype == torch.float32 and t.is_contiguous() and t.shape == (n, half)):
+            raise KernelError("rope_cos_sin: outputs must be float32 [n, half]")
     _call("gi_rope_cos_sin", positions.data_ptr(), inv_freq.data_ptr(), cos_out.data_ptr(), sin_out.data_ptr(), n, half, _stream())
 
 
 def _check_cache(cache, table, page_size, n_kv, hd, what):
     # the last two axes of the value half hold [hd][place]: values are stored transposed
-    _need(cache.dim() == 5 and tuple(cache.shape[1:]) == (2, n_kv, page_size, hd) and cache.is_contiguous(),
-          f"{what}: the cache must be [pages, 2, {n_kv}, {page_size}, {hd}], contiguous; it is {tuple(cache.shape)}")
-    _need(table.dim() == 2 and table.dtype == torch.int32 and table.stride(1) == 1, f"{what}: the page table must be int32 [slots, pages]")
+    if not (cache.dim() == 5 and tuple(cache.shape[1:]) == (2, n_kv, page_size, hd) and cache.is_contiguous()):
+        raise KernelError( f"{what}: the cache must be [pages, 2, {n_kv}, {page_size}, {hd}], contiguous; it is {tuple(cache.shape)}")
+    if not (table.dim() == 2 and table.dtype == torch.int32 and table.stride(1) == 1):
+        raise KernelError(f"{what}: the page table must be int32 [slots, pages]")
 
 
 def rope_store(q, k, v, cos, sin, positions, slots, table, q_out, cache, n_heads, n_kv, hd):
@@ -165,16 +183,20 @@ def rope_store(q, k, v, cos, sin, positions, slots, table, q_out, cache, n_heads
     q, k, v are float32 views [n, heads*hd] with unit inner stride (columns of one product are fine)."""
     _dev(q, k, v, cos, sin, positions, slots, table, q_out, cache)
     n = q.shape[0]
-    _need(q.dtype == torch.float32 and q.shape[1] == n_heads * hd and q.stride(1) == 1, "rope_store: q must be float32 [n, heads*hd]")
-    _need(q_out.shape == (n, n_heads * hd) and q_out.is_contiguous(), "rope_store: q_out must be [n, heads*hd], contiguous")
+    if not (q.dtype == torch.float32 and q.shape[1] == n_heads * hd and q.stride(1) == 1):
+        raise KernelError("rope_store: q must be float32 [n, heads*hd]")
+    if not (q_out.shape == (n, n_heads * hd) and q_out.is_contiguous()):
+        raise KernelError("rope_store: q_out must be [n, heads*hd], contiguous")
     if cos is not None:
         for t in (cos, sin):
-            _need(t.dtype == torch.float32 and t.shape == (n, hd // 2) and t.is_contiguous(), "rope_store: cos/sin must be float32 [n, hd/2]")
+            if not (t.dtype == torch.float32 and t.shape == (n, hd // 2) and t.is_contiguous()):
+                raise KernelError("rope_store: cos/sin must be float32 [n, hd/2]")
     page_size = page_stride = 0
     cache_code = _code(q_out, "rope_store: q_out")
     if k is not None:
         for t, name in ((k, "k"), (v, "v")):
-            _need(t.dtype == torch.float32 and t.shape == (n, n_kv * hd) and t.stride(1) == 1, f"rope_store: {name} must be float32 [n, kv_heads*hd]")
+            if not (t.dtype == torch.float32 and t.shape == (n, n_kv * hd) and t.stride(1) == 1):
+                raise KernelError(f"rope_store: {name} must be float32 [n, kv_heads*hd]")
         page_size = cache.shape[3]
         _check_cache(cache, table, page_size, n_kv, hd, "rope_store")
         page_stride = cache.stride(0)
@@ -192,8 +214,10 @@ def silu_mul(gate_up, out):
     """out[t, i] = silu(gate_up[t, i]) * gate_up[t, inter + i]."""
     _dev(gate_up, out)
     n, inter = out.shape
-    _need(gate_up.dtype == torch.float32 and gate_up.shape == (n, 2 * inter) and gate_up.is_contiguous(), "silu_mul: gate_up must be float32 [n, 2*inter]")
-    _need(out.is_contiguous(), "silu_mul: out must be contiguous")
+    if not (gate_up.dtype == torch.float32 and gate_up.shape == (n, 2 * inter) and gate_up.is_contiguous()):
+        raise KernelError("silu_mul: gate_up must be float32 [n, 2*inter]")
+    if not (out.is_contiguous()):
+        raise KernelError("silu_mul: out must be contiguous")
     _call("gi_silu_mul", gate_up.data_ptr(), out.data_ptr(), _code(out, "silu_mul: out"), n, inter, _stream())
     return out
 
@@ -201,8 +225,10 @@ def silu_mul(gate_up, out):
 def gather_rows(x, rows, out):
     _dev(x, rows, out)
     k, dim = out.shape
-    _need(x.dtype == torch.float32 and x.is_contiguous() and x.shape[1] == dim, "gather_rows: x must be contiguous float32 [n, dim]")
-    _need(out.dtype == torch.float32 and out.is_contiguous(), "gather_rows: out must be contiguous float32")
+    if not (x.dtype == torch.float32 and x.is_contiguous() and x.shape[1] == dim):
+        raise KernelError("gather_rows: x must be contiguous float32 [n, dim]")
+    if not (out.dtype == torch.float32 and out.is_contiguous()):
+        raise KernelError("gather_rows: out must be contiguous float32")
     _i32(rows, "gather_rows: rows", k)
     _call("gi_gather_rows", x.data_ptr(), rows.data_ptr(), out.data_ptr(), k, dim, _stream())
     return out
@@ -213,9 +239,12 @@ def gemm_exact(a, w, out, accumulate=False):
     _dev(a, w, out)
     m, k = a.shape
     n = w.shape[0]
-    _need(w.shape == (n, k), f"gemm: weight is {tuple(w.shape)}, activations are {tuple(a.shape)}")
-    _need(out.shape == (m, n), f"gemm: out is {tuple(out.shape)}, ({m}, {n}) is needed")
-    _need(a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, "gemm: operands need unit inner stride")
+    if not (w.shape == (n, k)):
+        raise KernelError(f"gemm: weight is {tuple(w.shape)}, activations are {tuple(a.shape)}")
+    if not (out.shape == (m, n)):
+        raise KernelError(f"gemm: out is {tuple(out.shape)}, ({m}, {n}) is needed")
+    if not (a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1):
+        raise KernelError("gemm: operands need unit inner stride")
     _call("gi_gemm_exact", a.data_ptr(), _code(a, "gemm: a"), w.data_ptr(), _code(w, "gemm: w"), out.data_ptr(), _code(out, "gemm: out"),
           1 if accumulate else 0, m, n, k, a.stride(0), w.stride(0), out.stride(0), _stream())
     return out
@@ -225,8 +254,8 @@ def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, w
     """Each row attends over its request's cached keys up to its own position."""
     _dev(q, cache, out, positions, slots, table)
     n = q.shape[0]
-    _need(q.shape == (n, n_heads * hd) and q.is_contiguous() and out.shape == q.shape and out.is_contiguous(),
-          "attention: q and out must be [n, heads*hd], contiguous")
+    if not (q.shape == (n, n_heads * hd) and q.is_contiguous() and out.shape == q.shape and out.is_contiguous()):
+        raise KernelError( "attention: q and out must be [n, heads*hd], contiguous")
     page_size = cache.shape[3]
     _check_cache(cache, table, page_size, n_kv, hd, "attention")
     _i32(positions, "attention: positions", n)
@@ -252,7 +281,7 @@ class AttentionPlan:
         plan.tiles = torch.empty(0, dtype=torch.int32, device=device)
         return plan
 
-    def __init__(self, seg_start, seg_len, seg_pos0, seg_slot, device):
+    def __init__(self, seg_start, seg_len, seg_pos0, seg_slot, device, to_device=None):
         dec, tiles, self.max_decode_context = [], [], 0
         for start, n, pos0, slot in zip(seg_start, seg_len, seg_pos0, seg_slot):
             if n == 1:
@@ -262,9 +291,10 @@ class AttentionPlan:
                 for off in range(0, n, self.TILE):
                     tiles.append((start + off, min(self.TILE, n - off), pos0 + off, slot))
         self.n_decode, self.n_tiles = len(dec), len(tiles)
-        both = torch.tensor(dec + [v for t in tiles for v in t], dtype=torch.int32).to(device)
-        self.decode_rows = both[:len(dec)] if tiles else None      # no prompt rows: the decode rows are all rows, in order
-        self.tiles = both[len(dec):]
+        put = to_device if to_device is not None else (lambda values: torch.tensor(values, dtype=torch.int32).to(device))
+        flat_tiles = [v for t in tiles for v in t]
+        self.decode_rows = put(dec) if dec and tiles else None      # no prompt rows: the decode rows are all rows, in order
+        self.tiles = put(flat_tiles) if tiles else torch.empty(0, dtype=torch.int32, device=device)      # read 16 bytes at a time: its own piece
 
 
 def attention_bf16_supports(hd, page_size, prompt: bool) -> bool:
@@ -294,27 +324,32 @@ def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, 
     n = out.shape[0]
     _dev(q, cache, out, positions, slots, table)
     for t, name in ((q, "q"), (cache, "cache"), (out, "out")):
-        _need(t is None or t.dtype == torch.bfloat16, f"attention_bf16: {name} must be bfloat16")
-    _need(out.shape == (n, n_heads * hd) and out.is_contiguous() and (q is None or (q.shape == out.shape and q.is_contiguous())),
-          "attention: q and out must be [n, heads*hd], contiguous")
+        if not (t is None or t.dtype == torch.bfloat16):
+            raise KernelError(f"attention_bf16: {name} must be bfloat16")
+    if not (out.shape == (n, n_heads * hd) and out.is_contiguous() and (q is None or (q.shape == out.shape and q.is_contiguous()))):
+        raise KernelError( "attention: q and out must be [n, heads*hd], contiguous")
     page_size = cache.shape[3]
     _check_cache(cache, table, page_size, n_kv, hd, "attention")
     _i32(positions, "attention: positions", n)
     _i32(slots, "attention: slots", n)
     window = int(window or 0)
     scale = float(scale if scale is not None else hd ** -0.5)
-    _need((q is None) != (products is None), "attention_bf16: give rotated queries or the unrotated products")
+    if not ((q is None) != (products is None)):
+        raise KernelError("attention_bf16: give rotated queries or the unrotated products")
     qf = kf = vf = cos = sin = None
     if products is not None:
-        _need(plan.n_tiles == 0, "attention_bf16: unrotated products serve steps of single decoded rows only")
+        if not (plan.n_tiles == 0):
+            raise KernelError("attention_bf16: unrotated products serve steps of single decoded rows only")
         qf, kf, vf, cos, sin = products
         _dev(qf, kf, vf, cos, sin)
-        _need(qf.dtype == torch.float32 and qf.shape == (n, n_heads * hd) and qf.stride(1) == 1, "attention: q must be float32 [n, heads*hd]")
+        if not (qf.dtype == torch.float32 and qf.shape == (n, n_heads * hd) and qf.stride(1) == 1):
+            raise KernelError("attention: q must be float32 [n, heads*hd]")
         for t, name in ((kf, "k"), (vf, "v")):
-            _need(t is None or (t.dtype == torch.float32 and t.shape == (n, n_kv * hd) and t.stride(1) == 1),
-                  f"attention: {name} must be float32 [n, kv_heads*hd]")
+            if not (t is None or (t.dtype == torch.float32 and t.shape == (n, n_kv * hd) and t.stride(1) == 1)):
+                raise KernelError( f"attention: {name} must be float32 [n, kv_heads*hd]")
         for t in (cos, sin):
-            _need(t is None or (t.dtype == torch.float32 and t.shape == (n, hd // 2) and t.is_contiguous()), "attention: cos/sin must be float32 [n, hd/2]")
+            if not (t is None or (t.dtype == torch.float32 and t.shape == (n, hd // 2) and t.is_contiguous())):
+                raise KernelError("attention: cos/sin must be float32 [n, hd/2]")
     if plan.n_tiles:
         _call("gi_attention_prompt_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles, plan.TILE,
               table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, _stream())
@@ -332,7 +367,7 @@ def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, 
 
 def _plan_of(ctx):
     if "attention_plan" not in ctx.memo:
-        ctx.memo["attention_plan"] = AttentionPlan(ctx.seg_start, ctx.seg_len, ctx.seg_pos0, ctx.seg_slot, ctx.device)
+        ctx.memo["attention_plan"] = AttentionPlan(ctx.seg_start, ctx.seg_len, ctx.seg_pos0, ctx.seg_slot, ctx.device, ctx.to_device)
     return ctx.memo["attention_plan"]
 
 
@@ -376,19 +411,20 @@ def gemm_bf16_supports(a, w, out) -> bool:
             and (out.dtype == torch.float32 or out.dtype == torch.bfloat16) and out.stride(1) == 1)
 
 
-def gemm_bf16(a, w, out, accumulate=False, gated=False):
+def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False):
     """out (=|+=) a @ w.T with bfloat16 operands on the matrix cores, float32 sums.
     gated: w is [gate; up] interleaved in groups of 16 rows and out = silu(a @ gate.T) * (a @ up.T), bfloat16 [m, n/2]."""
     _dev(a, w, out)
     m, k = a.shape
     n = w.shape[0]
-    _need(w.shape == (n, k), f"gemm: weight is {tuple(w.shape)}, activations are {tuple(a.shape)}")
-    _need(out.shape == (m, n // 2 if gated else n), f"gemm: out is {tuple(out.shape)}, ({m}, {n // 2 if gated else n}) is needed")
-    _need(gemm_bf16_supports(a, w, out), "gemm_bf16: operands must be bfloat16 with K and row strides multiples of 8, 16-byte aligned")
-    scratch, n_scratch = None, 0
-    if m <= 64:
-        n_scratch = lib().gi_gemm_bf16_skinny_splits(n, k) * m * n
-        scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device)
+    if not (w.shape == (n, k)):
+        raise KernelError(f"gemm: weight is {tuple(w.shape)}, activations are {tuple(a.shape)}")
+    if not (out.shape == (m, n // 2 if gated else n)):
+        raise KernelError(f"gemm: out is {tuple(out.shape)}, ({m}, {n // 2 if gated else n}) is needed")
+    if not (checked or gemm_bf16_supports(a, w, out)):
+        raise KernelError("gemm_bf16: operands must be bfloat16 with K and row strides multiples of 8, 16-byte aligned")
+    n_scratch = lib().gi_gemm_bf16_scratch_floats(m, n, k)           # partial sums where k is split over workgroups
+    scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device) if n_scratch else None
     _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,
           m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _stream())
     return out
@@ -397,14 +433,16 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False):
 def interleave_gate_up(gate, up):
     """[gate; up] in groups of 16 rows: 16 gate rows, the 16 up rows of the same outputs, and so on."""
     i, d = gate.shape
-    _need(i % 16 == 0 and up.shape == gate.shape, "interleave_gate_up: the intermediate size must be a multiple of 16")
+    if not (i % 16 == 0 and up.shape == gate.shape):
+        raise KernelError("interleave_gate_up: the intermediate size must be a multiple of 16")
     return torch.stack([gate.view(i // 16, 16, d), up.view(i // 16, 16, d)], dim=1).reshape(2 * i, d).contiguous()
 
 
 def argmax(logits, out):
     _dev(logits, out)
     n, vocab = logits.shape
-    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "argmax: logits must be float32 with unit inner stride")
+    if not (logits.dtype == torch.float32 and logits.stride(1) == 1):
+        raise KernelError("argmax: logits must be float32 with unit inner stride")
     _i32(out, "argmax: out", n)
     chunks = lib().gi_argmax_chunks(vocab)
     part_v = torch.empty(n * chunks, dtype=torch.float32, device=logits.device)
@@ -416,9 +454,11 @@ def argmax(logits, out):
 def sample_temperature(logits, temperature, uniform, out):
     _dev(logits, temperature, uniform, out)
     n, vocab = logits.shape
-    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "sample: logits must be float32 with unit inner stride")
+    if not (logits.dtype == torch.float32 and logits.stride(1) == 1):
+        raise KernelError("sample: logits must be float32 with unit inner stride")
     for t, name in ((temperature, "temperature"), (uniform, "uniform")):
-        _need(t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= n, f"sample: {name} must be float32 [n]")
+        if not (t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= n):
+            raise KernelError(f"sample: {name} must be float32 [n]")
     _i32(out, "sample: out", n)
     chunks = lib().gi_argmax_chunks(vocab)
     part_m = torch.empty(n * chunks, dtype=torch.float32, device=logits.device)

@@ -22,6 +22,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Any, Callable, Dict, List, Optional
 
+import numpy as np
 import torch
 
 from ..weights.loader import TensorNeed
@@ -42,6 +43,14 @@ class StepContext:
     seg_len: List[int]                       # number of rows,
     seg_pos0: List[int]                      # position of the first row
     memo: Dict[Any, Any] = field(default_factory=dict)     # per-step tables shared by layers (rotary cos/sin)
+    upload: Optional[Callable[[np.ndarray], torch.Tensor]] = None      # the runner's way of bringing int32 step data to the device
+
+    def to_device(self, values) -> torch.Tensor:
+        """int32 data made on the host for this step (row lists, tile lists) as a device tensor, valid during the step."""
+        arr = np.ascontiguousarray(values, dtype=np.int32)
+        if self.upload is not None:
+            return self.upload(arr)
+        return torch.from_numpy(arr).to(self.device)
 
     @property
     def max_seg_len(self) -> int:

@@ -18,7 +18,7 @@ def linear(a, weight: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
     if isinstance(a, NormedRows):
         a = a.materialize()
     if a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and ops.gemm_bf16_supports(a, weight, out):
-        return ops.gemm_bf16(a, weight, out, accumulate, gated)
+        return ops.gemm_bf16(a, weight, out, accumulate, gated, checked=True)
     if gated:
         raise ops.KernelError("the gated product exists for bfloat16 operands only")
     return ops.gemm_exact(a, weight, out, accumulate)

@@ -55,6 +55,8 @@ def test_gemm_exact_rows_alone_have_the_same_bits():
                                    (513, 384, 1024), (2048, 96, 160),
                                    # the LDS-ring kernel: one block of k, edge tiles, each of its three tile choices
                                    (256, 160, 64), (130, 129, 192), (2100, 2200, 192), (4000, 8200, 128),
+                                   # ... and with k shared out over workgroups because the tiles are few
+                                   (72, 256, 1024), (300, 2048, 2048), (65, 130, 512),
                                    # wide outputs finished by the skinny kernel itself, from 12 rows and from 5
                                    (12, 12300, 520), (40, 12300, 264), (5, 65600, 72), (16, 12288, 256)])
 @pytest.mark.parametrize("out_dtype,accumulate", [(torch.float32, False), (torch.float32, True), (torch.bfloat16, False)])
@@ -70,7 +72,7 @@ def test_gemm_bf16(m, n, k, out_dtype, accumulate):
 
 
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 8), (5, 48, 136), (16, 160, 96), (17, 176, 64), (64, 32, 264), (70, 192, 128), (300, 8192 // 16, 2048 // 8),
-                                       (40, 6144, 264), (13, 6160, 72), (64, 8192, 512), (2048, 1024, 192), (600, 288, 64)])
+                                       (40, 6144, 264), (13, 6160, 72), (64, 8192, 512), (2048, 1024, 192), (600, 288, 64), (200, 512, 1024)])
 def test_gemm_bf16_gated(m, inter, k):
     a = randn(m, k, dtype=torch.bfloat16, seed=15)
     gate, up = randn(inter, k, dtype=torch.bfloat16, seed=16, scale=0.3), randn(inter, k, dtype=torch.bfloat16, seed=17, scale=0.3)
