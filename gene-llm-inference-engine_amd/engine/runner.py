@@ -9,6 +9,8 @@ keeps the same promises, src/model/model.h:63-76, src/model/transformer.cpp:483-
 """
 from __future__ import annotations
 
+import gc
+
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
 
@@ -176,16 +178,16 @@ class Runner:
         if n > self.max_rows:
             raise StepError(f"the step holds {n} rows, more than max_rows = {self.max_rows}")
         cache.reserve_one_each(requests, slots, lengths)                        # OutOfPages: nothing changed
-        if any(g.dirty for g in cache.groups):
-            self._uploads.begin_step()
-            cache.sync(self._uploads.put)
-            self._uploads.end_step()
-        logits = self._decode_step(np.array([tokens, lengths, slots], dtype=np.int32), slots, lengths)
+        self._uploads.begin_step()
+        cache.sync(self._uploads.put)
+        meta = self._uploads.stage(np.array([tokens, lengths, slots], dtype=np.int32)).view(3, n)
+        logits = self._decode_step(meta, slots, lengths)
+        self._uploads.end_step()
         cache.advance_one_each(requests, slots, lengths)
         self.steps_run += 1
         return logits
 
-    def _decode_step(self, meta: np.ndarray, seg_slot, seg_pos0) -> torch.Tensor:
+    def _decode_step(self, meta: torch.Tensor, seg_slot, seg_pos0) -> torch.Tensor:
         """A step in which every request brings one token and wants its logits runs as a replay of a
         HIP graph captured once per batch size: the launches of the whole pass cost one call.  The
         graph reads tokens, positions and slots from fixed device buffers that are filled before
@@ -193,7 +195,7 @@ class Runner:
         batch = meta.shape[1]
         g = self._graphs.get(batch)
         if g is None:
-            g = self._graphs[batch] = _DecodeGraph(self, batch)
+            g = self._graphs[batch] = _DecodeGraph(self.model, self._view, self.max_positions, batch)
         return g.run(meta, seg_slot, seg_pos0)
 
 
@@ -230,6 +232,17 @@ class _StepUploads:
         piece.copy_(self.host[self.turn][a:b], non_blocking=True)
         return piece
 
+    def stage(self, values: np.ndarray) -> torch.Tensor:
+        """The values in this step's pinned buffer only (for a copy the caller makes itself, into its own device memory)."""
+        flat = np.ascontiguousarray(values, dtype=np.int32).reshape(-1)
+        n = flat.size
+        if self.used + n > self.capacity:
+            return torch.from_numpy(flat.copy())
+        a, b = self.used, self.used + n
+        self.used = (b + 3) & ~3
+        self.host[self.turn][a:b] = torch.from_numpy(flat)
+        return self.host[self.turn][a:b]
+
     def end_step(self) -> None:
         if torch.device(self.device).type == "cuda":
             ev = self.done[self.turn] or torch.cuda.Event()
@@ -238,38 +251,48 @@ class _StepUploads:
 
 
 class _DecodeGraph:
-    def __init__(self, runner: Runner, batch: int):
+    """The captured pass of one batch size.  It holds the model and the cache view, not the runner: a runner and
+    its graphs must not form a reference cycle, or they would be freed by the cycle collector at a moment of its
+    choosing, possibly while another graph is being captured, which the HIP runtime answers by aborting."""
+
+    def __init__(self, model: DecoderModel, view, max_positions: int, batch: int):
         from ..kernels.ops import AttentionPlan
-        self.runner, self.batch = runner, batch
-        dev = runner.model.device
+        self.model, self.view, self.batch = model, view, batch
+        dev = model.device
         self.meta = torch.zeros((3, batch), dtype=torch.int32, device=dev)
-        self.staging = torch.zeros((3, batch), dtype=torch.int32).pin_memory()
         self.logit_rows = torch.arange(batch, dtype=torch.int32, device=dev)
-        self.plan = AttentionPlan.all_decode(batch, runner.max_positions, dev)
+        self.plan = AttentionPlan.all_decode(batch, max_positions, dev)
         self.graph = None
         self.logits = None
         self.calls = 0
 
     def _context(self, seg_slot, seg_pos0) -> StepContext:
-        m, b = self.runner.model, self.batch
+        m, b = self.model, self.batch
         ctx = StepContext(n_rows=b, dtype=m.dtype, device=m.device, tokens=self.meta[0], row_pos=self.meta[1], row_slot=self.meta[2],
                           seg_slot=list(seg_slot), seg_start=list(range(b)), seg_len=[1] * b, seg_pos0=list(seg_pos0))
         ctx.memo["attention_plan"] = self.plan
         return ctx
 
-    def run(self, meta: np.ndarray, seg_slot, seg_pos0) -> torch.Tensor:
-        self.staging.numpy()[:] = meta
-        self.meta.copy_(self.staging, non_blocking=True)
-        r = self.runner
+    def run(self, meta: torch.Tensor, seg_slot, seg_pos0) -> torch.Tensor:
+        """meta: this step's tokens, positions and slots, int32 [3, batch], in pinned memory that stays as it is
+        until the copy made here has run."""
+        self.meta.copy_(meta, non_blocking=True)
         self.calls += 1
         if self.graph is None:
             if self.calls < 2:          # the first step of a batch size runs as it is; a size that comes again is captured
-                return r.model.forward(self._context(seg_slot, seg_pos0), r._view, self.logit_rows, self.batch)
+                return self.model.forward(self._context(seg_slot, seg_pos0), self.view, self.logit_rows, self.batch)
             # Capturing records the launches without running them, so this step runs once more below, by replay.
+            # No garbage collection meanwhile: freeing device memory or another graph inside a capture aborts.
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                self.logits = r.model.forward(self._context(seg_slot, seg_pos0), r._view, self.logit_rows, self.batch)
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):
+                    self.logits = self.model.forward(self._context(seg_slot, seg_pos0), self.view, self.logit_rows, self.batch)
+            finally:
+                if collecting:
+                    gc.enable()
             self.graph = graph
         self.graph.replay()
         return self.logits

@@ -108,3 +108,28 @@ def test_changing_first_token_changes_logits(case):
     toks[0] = (toks[0] + 1) % CONFIGS[name]["vocab_size"]
     got = replay(folder, "float32", traces.whole({rid: toks}), PAGE_SIZE[name], 4096)
     assert relative_error(got[(rid, len(toks) - 1)], want["float32"][rid][len(toks) - 1]) > 1e-3
+
+
+def test_a_runner_with_captured_steps_is_freed_without_the_cycle_collector(case):
+    """A runner and its captured graphs form no reference cycle: dropping the runner frees them at once, not at a
+    moment of the cycle collector's choosing (which may fall inside another capture, where freeing aborts)."""
+    import gc
+    import weakref
+    from geneinfer_amd.engine import Runner, StepEntry, load_model
+    name, folder, requests, _ = case
+    model = load_model(folder, "bfloat16", "cuda:0")
+    gc.collect()
+    gc.disable()
+    try:
+        runner = Runner(model, page_size=PAGE_SIZE[name], max_tokens=256, max_requests=2, max_rows=64)
+        runner.open("a")
+        runner.step([StepEntry("a", [1, 2, 3], (2,))])
+        for t in (4, 5, 6):                                   # the second one-token step of a batch size is captured
+            runner.step([StepEntry("a", [t], (0,))])
+        assert runner.use_graphs and runner._graphs[1].graph is not None
+        graph_ref, runner_ref = weakref.ref(runner._graphs[1]), weakref.ref(runner)
+        torch.cuda.synchronize()
+        del runner
+        assert runner_ref() is None and graph_ref() is None
+    finally:
+        gc.enable()
