@@ -217,3 +217,28 @@ def test_windowed_groups_are_planned_per_group():
     eng.run_until_idle()
     assert eng.result(j).error == "" and len(eng.result(j).generated_tokens) == 25
     assert runner.cache.free_pages() == [10, 10]
+
+
+def test_step_uploads_ring_on_the_cpu():
+    """The ring that carries a step's int32 data: pieces are snapshots, start at 16-byte multiples, keep their
+    values while later steps fill other buffers, and what exceeds the ring is copied the ordinary way."""
+    import numpy as np
+    from geneinfer_amd.engine.runner import _StepUploads
+    ring = _StepUploads("cpu", capacity=32)
+    kept = []
+    for step in range(2 * _StepUploads.DEPTH):
+        ring.begin_step()
+        a = np.arange(5, dtype=np.int32) + 100 * step
+        piece = ring.put(a)
+        a[:] = -1                                             # the caller may reuse its array at once
+        second = ring.put(np.full((2, 3), step, dtype=np.int64))
+        staged = ring.stage([step, step + 1])
+        assert piece.tolist() == [100 * step + i for i in range(5)] and second.tolist() == [step] * 6 and staged.tolist() == [step, step + 1]
+        assert piece.dtype == second.dtype == staged.dtype == torch.int32
+        assert ring.used % 4 == 0 and piece.data_ptr() % 16 == second.data_ptr() % 16
+        big = ring.put(np.arange(100, dtype=np.int32))        # more than the ring holds
+        assert big.tolist() == list(range(100))
+        ring.end_step()
+        kept.append((step, piece))
+        for s, p in kept[-(_StepUploads.DEPTH - 1):]:         # the pieces of the last steps are still what they were
+            assert p.tolist() == [100 * s + i for i in range(5)]
