@@ -269,24 +269,33 @@ def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, w
 class AttentionPlan:
     """How a step's rows are shared between the two bfloat16 attention kernels: requests that bring
     one row go to the decode kernel, portions of prompts are cut into tiles of up to 128 rows for
-    the prompt kernel.  Made once per step and used by every layer."""
+    the prompt kernel.  Short portions go to the decode kernel too, row by row (every row attends
+    over its own prefix, which the cache holds by then): a tile's workgroup walks the whole context
+    in sequence, however few its rows, while the decode kernel cuts each row's context into pieces
+    for the whole chip (break-even near 90 rows at the Llama-3.2-1B shape; above SHORT_TOTAL rows
+    in all, the rows' repeated reading of the context costs more than the tiles' sequence).
+    Made once per step and used by every layer."""
     TILE = int(__import__("os").environ.get("GI_ATTENTION_TILE", "128"))      # rows of a prompt tile: 64 or 128
+    SHORT, SHORT_TOTAL = 64, 64          # portions of up to SHORT rows count as short; they go row by row while they sum to at most SHORT_TOTAL
 
     @classmethod
     def all_decode(cls, n_rows, max_context, device):
         """Every row is a request's single new row (what a captured decode step uses: nothing in it depends on the step)."""
         plan = cls.__new__(cls)
-        plan.n_decode, plan.n_tiles, plan.max_decode_context = n_rows, 0, max_context
+        plan.n_decode, plan.n_tiles, plan.max_decode_context, plan.single_rows = n_rows, 0, max_context, True
         plan.decode_rows = None                                  # rows 0 .. n_rows-1
         plan.tiles = torch.empty(0, dtype=torch.int32, device=device)
         return plan
 
     def __init__(self, seg_start, seg_len, seg_pos0, seg_slot, device, to_device=None):
         dec, tiles, self.max_decode_context = [], [], 0
+        short_rows = sum(n for n in seg_len if 1 < n <= self.SHORT)
+        row_by_row = self.SHORT if short_rows <= self.SHORT_TOTAL else 1
+        self.single_rows = all(n == 1 for n in seg_len)          # every row is a request's only new row
         for start, n, pos0, slot in zip(seg_start, seg_len, seg_pos0, seg_slot):
-            if n == 1:
-                dec.append(start)
-                self.max_decode_context = max(self.max_decode_context, pos0 + 1)
+            if n <= row_by_row:
+                dec.extend(range(start, start + n))
+                self.max_decode_context = max(self.max_decode_context, pos0 + n)
             else:
                 for off in range(0, n, self.TILE):
                     tiles.append((start + off, min(self.TILE, n - off), pos0 + off, slot))
@@ -393,7 +402,7 @@ def attention_from_products(q, k, v, cos, sin, cache, out, ctx, table, n_heads, 
     if not (cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.dtype == torch.float32):
         return False
     plan = _plan_of(ctx)
-    if plan.n_tiles or not plan.n_decode or not attention_bf16_supports(hd, cache.shape[3], False):
+    if plan.n_tiles or not plan.single_rows or not attention_bf16_supports(hd, cache.shape[3], False):      # rows of one portion need each other's keys in the cache
         return False
     if plan.n_decode > FUSED_DECODE_MAX_ROWS:
         return False

@@ -219,16 +219,26 @@ ATT_CASES = [  # n_heads, n_kv, hd, page_size, window
 ]
 
 
+SEGMENTS = {
+    # request 0: rows at positions 150..299 (a portion on top of 150 cached positions); request 1: its last row;
+    # request 2: its only row; request 3: rows 0..76 (a whole prompt); request 4: its last row
+    "long portions": [(0, 150, 150), (1, 130, 1), (2, 0, 1), (3, 0, 77), (4, 529, 1)],
+    # short portions, 60 rows in all: the matrix-core path takes them row by row through the decode kernel
+    "short portions": [(0, 250, 50), (1, 130, 1), (2, 0, 1), (3, 70, 7), (4, 527, 3)],
+    # short portions that sum to more than 64 rows stay tiles
+    "many short portions": [(0, 240, 60), (1, 130, 1), (3, 47, 30), (4, 490, 40)],
+}
+
+
 @pytest.mark.parametrize("n_heads,n_kv,hd,ps,window", ATT_CASES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_attention_over_pages(n_heads, n_kv, hd, ps, window, dtype):
+@pytest.mark.parametrize("portions", list(SEGMENTS))
+def test_attention_over_pages(n_heads, n_kv, hd, ps, window, dtype, portions):
     """Portions of prompts on top of an existing cache, beside single decoded rows, on scrambled pages."""
     from geneinfer_amd.parts import StepContext
     contexts = [300, 131, 1, 77, 530]
     cache, table, dense = build_paged(contexts, n_kv, hd, ps, dtype, seed=hd + n_heads)
-    # request 0: rows at positions 150..299 (a portion on top of 150 cached positions); request 1: its last row;
-    # request 2: its only row; request 3: rows 0..76 (a whole prompt); request 4: its last row
-    segs = [(0, 150, 150), (1, 130, 1), (2, 0, 1), (3, 0, 77), (4, 529, 1)]
+    segs = SEGMENTS[portions]
     rows, seg_start, seg_len, seg_pos0, seg_slot = [], [], [], [], []
     for slot, pos0, n in segs:
         seg_start.append(len(rows)); seg_len.append(n); seg_pos0.append(pos0); seg_slot.append(slot + 1)
