@@ -39,7 +39,8 @@ template <int HD, int NW>
 __global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
                                                                   bf16_t* __restrict__ out, const int4* __restrict__ tiles,
                                                                   const int* __restrict__ table, int table_stride, long page_stride,
-                                                                  int page_size, int n_heads, int n_kv, int window, float scale) {
+                                                                  int page_size, int n_heads, int n_kv, int window, float scale,
+                                                                  int n_splits, const int* __restrict__ tile_first, float* __restrict__ part) {
     constexpr int NT = 64 * NW;                 // threads; the tile has 32 * NW query rows
     constexpr int K_STRIDE = HD + 8;            // bf16 elements; 16-byte reads of 32 rows hit distinct banks
     constexpr int V_STRIDE = KV_TILE + 4;       // 8-byte reads of 32 rows hit distinct banks
@@ -49,7 +50,10 @@ __global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t*
     __shared__ __attribute__((aligned(16))) bf16_t Ks[KV_TILE * K_STRIDE];
     __shared__ __attribute__((aligned(16))) bf16_t Vs[HD * V_STRIDE];
 
-    const int4 tile = tiles[gridDim.x - 1 - blockIdx.x];     // later tiles of a prompt see more keys: they start first
+    // With few tiles the keys of a tile are shared out over n_splits workgroups (grid x = tiles * splits); each writes
+    // an unnormalised partial result {m, l, O} per row, as the decode kernel's splits do, for the same combine kernel.
+    const int tile_index = gridDim.x / n_splits - 1 - blockIdx.x / n_splits, split = blockIdx.x % n_splits;
+    const int4 tile = tiles[tile_index];                     // later tiles of a prompt see more keys: they start first
     const int row0 = tile.x, n_rows = tile.y, pos0 = tile.z, slot = tile.w;
     const int head = blockIdx.y, g = head / (n_heads / n_kv);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -82,6 +86,10 @@ __global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t*
     const int last_pos = pos0 + n_rows - 1;
     const int first_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
     const long v_plane = (long)n_kv * page_size * HD;
+    // this workgroup's share of the key tiles [first_lo, last_pos]: whole tiles of 64, the same number for every split
+    const int range_first = first_lo & ~(KV_TILE - 1);
+    const int per_split = ((last_pos - range_first) / KV_TILE + n_splits) / n_splits * KV_TILE;
+    const int kv_first = range_first + split * per_split, my_last = min(last_pos, kv_first + per_split - 1);
 
     // A tile of 64 key positions travels global memory -> registers -> LDS; the next tile's loads are
     // issued before the products of this one, and the page numbers they need one tile earlier still,
@@ -96,8 +104,8 @@ __global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t*
         for (int i = 0; i < CHUNKS; ++i) {
             const int e = tid + NT * i;
             const int kv_k = kv0 + e / (HD / 8), kv_v = kv0 + (e / HD) * 8;
-            k_page[i] = kv_k <= last_pos ? tab[page_index(kv_k)] : -1;
-            v_page[i] = kv_v <= last_pos ? tab[page_index(kv_v)] : -1;
+            k_page[i] = kv_k <= my_last ? tab[page_index(kv_k)] : -1;
+            v_page[i] = kv_v <= my_last ? tab[page_index(kv_v)] : -1;
         }
     };
     auto fetch = [&](int kv0) {                 // with the pages that fetch_pages(kv0) brought
@@ -125,15 +133,14 @@ __global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t*
         }
     };
 
-    const int kv_first = first_lo & ~(KV_TILE - 1);
     fetch_pages(kv_first);
     fetch(kv_first);
     fetch_pages(kv_first + KV_TILE);            // beyond the last position: no lookups
-    for (int kv0 = kv_first; kv0 <= last_pos; kv0 += KV_TILE) {
+    for (int kv0 = kv_first; kv0 <= my_last; kv0 += KV_TILE) {
         __syncthreads();                        // the previous tile has been read by everyone
         stash();
         __syncthreads();
-        if (kv0 + KV_TILE <= last_pos) {
+        if (kv0 + KV_TILE <= my_last) {
             fetch(kv0 + KV_TILE);
             fetch_pages(kv0 + 2 * KV_TILE);
         }
@@ -198,6 +205,18 @@ __global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t*
         }
     }
     if (!row_ok) return;
+    if (n_splits > 1) {                                       // part[row of the split tiles][head][split] = {m, l, O[HD]}
+        float* dst = part + (((size_t)(tile_first[tile_index] + my_row) * n_heads + head) * n_splits + split) * (HD + 2);
+        if (hf == 0) {
+            dst[0] = m;
+            dst[1] = l;
+        }
+#pragma unroll
+        for (int i = 0; i < DT; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) dst[2 + 32 * i + 8 * (v / 4) + 4 * hf + (v & 3)] = o[i][v];
+        return;
+    }
     const float inv = 1.0f / l;
     bf16_t* orow = out + ((size_t)(row0 + my_row) * n_heads + head) * HD;
 #pragma unroll
@@ -542,29 +561,42 @@ GI_API int gi_attention_bf16_supports(int hd, int page_size, int prompt) {
     return hd == 32 || hd == 64 || hd == 96 || hd == 128 || hd == 256;
 }
 
-// tiles hold at most `rows_per_tile` rows each (64 or 128).
+// tiles hold at most `rows_per_tile` rows each (64 or 128).  n_splits > 1: every tile's keys are shared out over that
+// many workgroups; `tile_first[i]` is the number of rows in the tiles before tile i, `rows` lists the tiles' rows in
+// that order (n_rows of them), `part` has room for n_rows * n_heads * n_splits * (hd + 2) floats.
 GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out, const int* tiles, int n_tiles, int rows_per_tile,
                                     const int* table, int table_stride, long page_stride, int page_size, int n_heads, int n_kv, int hd,
-                                    int window, float scale, hipStream_t stream) {
+                                    int window, float scale, int n_splits, const int* tile_first, const int* rows, int n_rows, float* part,
+                                    long part_floats, hipStream_t stream) {
     GI_REQUIRE(rows_per_tile == 64 || rows_per_tile == 128, "attention_prompt: tiles of %d rows are not supported (64 or 128)", rows_per_tile);
     GI_REQUIRE(n_tiles > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_prompt: bad counts (%d tiles, %d heads, %d kv heads)",
                n_tiles, n_heads, n_kv);
     GI_REQUIRE(gi_attention_bf16_supports(hd, page_size, 1), "attention_prompt: head size %d with page size %d is not supported", hd, page_size);
     GI_REQUIRE(page_stride >= 2L * n_kv * page_size * hd && page_stride % 8 == 0, "attention_prompt: bad page stride %ld", page_stride);
     GI_REQUIRE(n_heads <= 65535, "attention_prompt: too many heads");
-    dim3 grid(n_tiles, n_heads);
+    GI_REQUIRE(n_splits >= 1 && n_splits <= MAX_SPLITS, "attention_prompt: the number of splits %d is outside 1..%d", n_splits, MAX_SPLITS);
+    GI_REQUIRE(n_splits == 1 || (tile_first && rows && part && n_rows > 0 && part_floats >= (long)n_rows * n_heads * n_splits * (hd + 2)),
+               "attention_prompt: splitting needs the tiles' row offsets, their rows and scratch for the partial results");
+    dim3 grid(n_tiles * n_splits, n_heads);
 #define GO(HD)                                                                                                                          \
     do {                                                                                                                                \
         if (rows_per_tile == 64)                                                                                                        \
             attention_prompt_kernel<HD, 2><<<grid, 128, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
-                                                                     table_stride, page_stride, page_size, n_heads, n_kv, window, scale); \
+                                                                     table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits,  \
+                                                                     tile_first, part);                                                 \
         else                                                                                                                            \
             attention_prompt_kernel<HD, 4><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
-                                                                     table_stride, page_stride, page_size, n_heads, n_kv, window, scale); \
+                                                                     table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits,  \
+                                                                     tile_first, part);                                                 \
     } while (0)
     if (hd == 32) GO(32); else if (hd == 64) GO(64); else if (hd == 96) GO(96); else GO(128);
 #undef GO
     GI_CHECK_LAUNCH("attention_prompt");
+    if (n_splits > 1) {
+        dim3 cgrid(n_rows, n_heads);
+        attention_decode_combine_kernel<<<cgrid, 64, 0, stream>>>(part, (bf16_t*)out, rows, n_heads, hd, n_splits);
+        GI_CHECK_LAUNCH("attention_prompt (combine)");
+    }
     return 0;
 }
 

@@ -32,7 +32,7 @@ _SIGNATURES = {
                            c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
     "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
-                                 c_float, c_void_p],
+                                 c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p],
     "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_int, c_int, c_void_p],
@@ -285,6 +285,7 @@ class AttentionPlan:
         plan.n_decode, plan.n_tiles, plan.max_decode_context, plan.single_rows = n_rows, 0, max_context, True
         plan.decode_rows = None                                  # rows 0 .. n_rows-1
         plan.tiles = torch.empty(0, dtype=torch.int32, device=device)
+        plan.n_tile_rows, plan.max_tile_context, plan.tile_first, plan.tile_rows = 0, 0, None, None
         return plan
 
     def __init__(self, seg_start, seg_len, seg_pos0, seg_slot, device, to_device=None):
@@ -300,14 +301,32 @@ class AttentionPlan:
                 for off in range(0, n, self.TILE):
                     tiles.append((start + off, min(self.TILE, n - off), pos0 + off, slot))
         self.n_decode, self.n_tiles = len(dec), len(tiles)
+        self.n_tile_rows = sum(t[1] for t in tiles)
+        self.max_tile_context = max((t[2] + t[1] for t in tiles), default=0)
         put = to_device if to_device is not None else (lambda values: torch.tensor(values, dtype=torch.int32).to(device))
         flat_tiles = [v for t in tiles for v in t]
         self.decode_rows = put(dec) if dec and tiles else None      # no prompt rows: the decode rows are all rows, in order
         self.tiles = put(flat_tiles) if tiles else torch.empty(0, dtype=torch.int32, device=device)      # read 16 bytes at a time: its own piece
+        # for sharing a tile's keys out over workgroups: rows before each tile, and the tiles' rows in order
+        firsts, count = [], 0
+        for t in tiles:
+            firsts.append(count)
+            count += t[1]
+        self.tile_first = put(firsts) if tiles else None
+        self.tile_rows = put([r for t in tiles for r in range(t[0], t[0] + t[1])]) if tiles else None
 
 
 def attention_bf16_supports(hd, page_size, prompt: bool) -> bool:
     return bool(lib().gi_attention_bf16_supports(hd, page_size, 1 if prompt else 0))
+
+
+def prompt_attention_splits(n_tiles, n_heads, span, target_groups=512):
+    """Workgroups a tile's keys are shared out over: none while the tiles alone fill the chip (two workgroups a
+    compute unit) or the context is short; every share keeps at least 256 keys."""
+    groups = n_tiles * n_heads
+    if groups >= target_groups // 2:
+        return 1
+    return max(1, min(-(-target_groups // groups), span // 256, 64))
 
 
 def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096):
@@ -360,8 +379,12 @@ def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, 
             if not (t is None or (t.dtype == torch.float32 and t.shape == (n, hd // 2) and t.is_contiguous())):
                 raise KernelError("attention: cos/sin must be float32 [n, hd/2]")
     if plan.n_tiles:
+        n_splits = prompt_attention_splits(plan.n_tiles, n_heads, plan.max_tile_context if not window else min(plan.max_tile_context, window + plan.TILE))
+        n_part = plan.n_tile_rows * n_heads * n_splits * (hd + 2) if n_splits > 1 else 0
+        part = torch.empty(n_part, dtype=torch.float32, device=out.device) if n_part else None
         _call("gi_attention_prompt_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles, plan.TILE,
-              table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, _stream())
+              table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits,
+              _ptr(plan.tile_first), _ptr(plan.tile_rows), plan.n_tile_rows, _ptr(part), n_part, _stream())
     if plan.n_decode:
         span = plan.max_decode_context if not window else min(plan.max_decode_context, window + 31)
         n_splits, n_waves = decode_attention_shape(plan.n_decode, n_heads, n_kv, hd, span, target_waves)

@@ -258,6 +258,32 @@ def test_attention_over_pages(n_heads, n_kv, hd, ps, window, dtype, portions):
     assert torch.equal(torch.nan_to_num(cache, nan=-1.0), torch.nan_to_num(before, nan=-1.0)), "attention wrote into the cache"
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd,ps,window", [(4, 2, 64, 16, None), (3, 1, 32, 16, None), (8, 8, 128, 32, None), (6, 2, 96, 16, 700), (4, 4, 64, 16, 450)])
+def test_few_prompt_tiles_over_a_long_context_share_their_keys_out(n_heads, n_kv, hd, ps, window):
+    """Two portions on top of long cached contexts: few tiles, so each tile's keys go to several workgroups and a combine
+    kernel; among the keys one far one is scaled so that a lost share would show."""
+    from geneinfer_amd.parts import StepContext
+    o = ops()
+    contexts = [1500, 730, 40]
+    cache, table, dense = build_paged(contexts, n_kv, hd, ps, torch.bfloat16, seed=hd + n_heads + 7, scale_one=(333, 3.0))
+    segs = [(0, 1400, 100), (1, 600, 130), (2, 39, 1)]
+    rows, seg_start, seg_len, seg_pos0, seg_slot = [], [], [], [], []
+    for slot, pos0, n in segs:
+        seg_start.append(len(rows)); seg_len.append(n); seg_pos0.append(pos0); seg_slot.append(slot + 1)
+        rows += [(slot, pos0 + i) for i in range(n)]
+    T = len(rows)
+    q = randn(T, n_heads * hd, dtype=torch.bfloat16, seed=3)
+    pos = torch.tensor([p for _, p in rows], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([s_ + 1 for s_, _ in rows], dtype=torch.int32, device=DEV)
+    ctx = StepContext(n_rows=T, dtype=torch.bfloat16, device=torch.device(DEV), tokens=pos, row_pos=pos, row_slot=slots, seg_slot=seg_slot,
+                      seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0)
+    assert o.prompt_attention_splits(3, n_heads, 1500 if not window else window + 128) > 1
+    out = torch.full((T, n_heads * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    o.attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window)
+    want = plain_attention_rows(q, dense, rows, n_heads, n_kv, hd, window)
+    assert rel(out, want) < 8e-3, rel(out, want)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_finds_one_far_key(dtype):
     """Among 700 keys one is scaled so that its score stands out: the output must be its value."""
