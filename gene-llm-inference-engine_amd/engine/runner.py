@@ -193,9 +193,15 @@ class Runner:
         graph reads tokens, positions and slots from fixed device buffers that are filled before
         every replay; nothing else in it depends on the step."""
         batch = meta.shape[1]
-        g = self._graphs.get(batch)
+        # The attention kernel's cut of the context into pieces is fixed at capture, for the longest context the graph
+        # is to serve well: one graph per batch size and power-of-two bracket of the step's longest context.
+        longest, bracket = max(seg_pos0) + 1, 1024
+        while bracket < longest:
+            bracket *= 2
+        bracket = min(bracket, self.max_positions)
+        g = self._graphs.get((batch, bracket))
         if g is None:
-            g = self._graphs[batch] = _DecodeGraph(self.model, self._view, self.max_positions, batch)
+            g = self._graphs[(batch, bracket)] = _DecodeGraph(self.model, self._view, bracket, batch)
         return g.run(meta, seg_slot, seg_pos0)
 
 
@@ -255,13 +261,13 @@ class _DecodeGraph:
     its graphs must not form a reference cycle, or they would be freed by the cycle collector at a moment of its
     choosing, possibly while another graph is being captured, which the HIP runtime answers by aborting."""
 
-    def __init__(self, model: DecoderModel, view, max_positions: int, batch: int):
+    def __init__(self, model: DecoderModel, view, longest_context: int, batch: int):
         from ..kernels.ops import AttentionPlan
         self.model, self.view, self.batch = model, view, batch
         dev = model.device
         self.meta = torch.zeros((3, batch), dtype=torch.int32, device=dev)
         self.logit_rows = torch.arange(batch, dtype=torch.int32, device=dev)
-        self.plan = AttentionPlan.all_decode(batch, max_positions, dev)
+        self.plan = AttentionPlan.all_decode(batch, longest_context, dev)
         self.graph = None
         self.logits = None
         self.calls = 0

@@ -126,8 +126,10 @@ def test_a_runner_with_captured_steps_is_freed_without_the_cycle_collector(case)
         runner.step([StepEntry("a", [1, 2, 3], (2,))])
         for t in (4, 5, 6):                                   # the second one-token step of a batch size is captured
             runner.step([StepEntry("a", [t], (0,))])
-        assert runner.use_graphs and runner._graphs[1].graph is not None
-        graph_ref, runner_ref = weakref.ref(runner._graphs[1]), weakref.ref(runner)
+        (graph,) = runner._graphs.values()
+        assert runner.use_graphs and graph.graph is not None
+        graph_ref, runner_ref = weakref.ref(graph), weakref.ref(runner)
+        del graph
         torch.cuda.synchronize()
         del runner
         assert runner_ref() is None and graph_ref() is None
