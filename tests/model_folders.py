@@ -25,8 +25,13 @@ TINY_B = dict(hidden_size=96, intermediate_size=160, num_hidden_layers=3, num_at
 TINY_C = dict(hidden_size=80, intermediate_size=112, num_hidden_layers=1, num_attention_heads=6, num_key_value_heads=3,
               head_dim=48, vocab_size=301, rope_theta=25000.0, rope_scaling=None, rms_norm_eps=3e-5,
               tie_word_embeddings=False, max_position_embeddings=256)
-PAGE_SIZE = {"A": 4, "B": 8, "C": 16}
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# A fourth whose head size and page size the matrix-core attention kernels take (A, B and C run the exact attention
+# kernels in both dtypes: pages of 4 and 8 positions, heads of 48 channels), with prompts long enough for several tiles.
+TINY_D = dict(hidden_size=128, intermediate_size=208, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+              head_dim=64, vocab_size=515, rope_theta=1000000.0, rope_scaling=None, rms_norm_eps=2e-5,
+              tie_word_embeddings=False, max_position_embeddings=2048)
+PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
 def full_config(sizes: dict) -> dict:

@@ -19,7 +19,7 @@ def test_only_required_keys_get_the_reference_defaults():
     assert c.attn_dim == 64 and c.kv_dim == 64
 
 
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_every_size_comes_from_the_file(name):
     sizes = CONFIGS[name]
     c = parse_config(full_config(sizes))

@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 # of a plain model that rounds to bfloat16 where the engine stores bfloat16 (see
 # `assert_within_bfloat16_noise`).
 TOLERANCE = {"float32": 2e-5}
-LENGTHS = {"A": [5, 11, 17, 70, 45], "B": [1, 9, 33, 40, 75, 51], "C": [3, 66, 37, 50]}
+LENGTHS = {"A": [5, 11, 17, 70, 45], "B": [1, 9, 33, 40, 75, 51], "C": [3, 66, 37, 50], "D": [150, 300, 37, 90, 700]}
 
 
 def make_requests(name, seed=5):
@@ -25,7 +25,7 @@ def make_requests(name, seed=5):
     return {f"r{i}": [rng.randrange(vocab) for _ in range(n)] for i, n in enumerate(LENGTHS[name])}
 
 
-@pytest.fixture(scope="module", params=["A", "B", "C"])
+@pytest.fixture(scope="module", params=["A", "B", "C", "D"])
 def case(request, tmp_path_factory):
     name = request.param
     folder = tmp_path_factory.mktemp(f"tiny{name}")
