@@ -2,3 +2,4 @@
 from .needs import PagedKvNeed, StateNeed
 from .pages import OutOfPages, PageError, PagePool
 from .manager import CacheError, CacheManager, PageGroup
+from .prefix import PrefixIndex

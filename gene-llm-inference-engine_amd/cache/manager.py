@@ -21,6 +21,7 @@ import torch
 
 from .needs import PagedKvNeed, StateNeed
 from .pages import OutOfPages, PagePool
+from .prefix import PrefixIndex
 
 
 class CacheError(RuntimeError):
@@ -54,6 +55,15 @@ class PageGroup:
             i = int(self.n_held[slot])
             self.table_host[slot, i] = self.pool.allocate()
             self.n_held[slot] = i + 1
+        self.dirty.add(slot)
+
+    def adopt(self, slot: int, pages: Sequence[int]) -> None:
+        """The first pages of a request that has none yet: full pages another request computed (the caller has
+        retained them for this request)."""
+        if int(self.n_held[slot]) != 0:
+            raise CacheError("only a request without pages can adopt shared ones")
+        self.table_host[slot, :len(pages)] = np.asarray(pages, dtype=np.int32)
+        self.n_held[slot] = len(pages)
         self.dirty.add(slot)
 
     def drop_behind_window(self, slot: int, length: int) -> None:
@@ -124,6 +134,7 @@ class CacheManager:
                     self.states[i] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
             elif need is not None:
                 raise CacheError(f"run-order entry {i} has an unknown cache need {need!r}")
+        self._state_needed = any(isinstance(need, StateNeed) for need in needs)
         for need, entries in by_need.items():
             g = PageGroup(need, entries, n_pages, page_size, max_requests, max_positions, dtype, device, allocate_storage)
             for li, e in enumerate(entries):
@@ -135,19 +146,47 @@ class CacheManager:
         self._free_slots = list(range(max_requests - 1, -1, -1))
         self._slot: Dict[Hashable, int] = {}
         self._length: Dict[Hashable, int] = {}
+        self.prefix: Optional[PrefixIndex] = None
+
+    def enable_prefix_sharing(self) -> bool:
+        """Lets requests share the pages of equal prompt prefixes (`self.prefix`).  Possible when one group of
+        pages without a window holds all of a request's past: with a window, pages of a prefix are given back
+        while it is still shared; with fixed-size state, the state after the prefix would have to be kept too."""
+        if self.prefix is None and len(self.groups) == 1 and self.groups[0].need.window is None and not self._state_needed:
+            self.prefix = PrefixIndex(self.groups[0].pool, self.page_size)
+        return self.prefix is not None
 
     # ------------------------------------------------------------------------------ requests
-    def open(self, request: Hashable) -> int:
+    def open(self, request: Hashable, shared_pages: Sequence[int] = ()) -> int:
+        """shared_pages: full pages of an equal prompt prefix, retained for this request by `self.prefix.match`;
+        the request starts with their positions in place."""
         if request in self._slot:
             raise CacheError(f"request {request!r} is already open")
         if not self._free_slots:
             raise CacheError(f"all {self.max_requests} request slots are in use")
+        if shared_pages and self.prefix is None:
+            raise CacheError("pages can be shared only after enable_prefix_sharing()")
+        if len(shared_pages) * self.page_size > self.max_positions:
+            raise CacheError("more shared pages than a request may hold")
         slot = self._free_slots.pop()
         self._slot[request] = slot
-        self._length[request] = 0
+        self._length[request] = len(shared_pages) * self.page_size
         for s in self.states.values():
             s[slot].zero_()
+        if shared_pages:
+            self.groups[0].adopt(slot, shared_pages)
         return slot
+
+    def pages_of(self, request: Hashable) -> List[int]:
+        """The request's page table in the first group (what the prefix index names pages by)."""
+        return self.groups[0].held_pages(self.slot(request))
+
+    def evictable_pages(self) -> int:
+        return self.prefix.evictable() if self.prefix is not None else 0
+
+    def evict(self, count: int) -> int:
+        """Gives back up to `count` pages that only the prefix index still holds; returns how many."""
+        return self.prefix.evict(count) if self.prefix is not None and count > 0 else 0
 
     def close(self, request: Hashable) -> None:
         slot = self.slot(request)
@@ -266,23 +305,27 @@ class CacheManager:
         return self.states[entry]
 
     def check_consistency(self) -> None:
-        """Every page is either free or held by exactly one open request (no sharing is used)."""
+        """Every page is free, or held by the requests and the prefix index that its reference count says;
+        without prefix sharing a page has at most one holder."""
         for gi, g in enumerate(self.groups):
-            held: Dict[int, Hashable] = {}
+            holders: Dict[int, List[Hashable]] = {}
             for request, slot in self._slot.items():
                 for p in g.held_pages(slot):
                     if p < 0:
                         raise CacheError(f"group {gi}: request {request!r} holds no page at a live place")
-                    if p in held:
-                        raise CacheError(f"group {gi}: page {p} is held by {held[p]!r} and {request!r}")
-                    held[p] = request
+                    holders.setdefault(p, []).append(request)
+                    if len(holders[p]) > 1 and (self.prefix is None or gi != 0):
+                        raise CacheError(f"group {gi}: page {p} is held by {holders[p][0]!r} and {request!r}")
+            indexed = set(self.prefix._entry) if self.prefix is not None and gi == 0 else set()
+            in_use = set(holders) | indexed
             free = set(g.pool._free)
             if len(free) != len(g.pool._free):
                 raise CacheError(f"group {gi}: a page is twice in the free stack")
-            if free & set(held):
-                raise CacheError(f"group {gi}: pages {sorted(free & set(held))} are free and held")
-            if len(free) + len(held) != g.pool.n_pages:
-                raise CacheError(f"group {gi}: {g.pool.n_pages - len(free) - len(held)} pages are lost")
+            if free & in_use:
+                raise CacheError(f"group {gi}: pages {sorted(free & in_use)} are free and held")
+            if len(free) + len(in_use) != g.pool.n_pages:
+                raise CacheError(f"group {gi}: {g.pool.n_pages - len(free) - len(in_use)} pages are lost")
             for p in range(g.pool.n_pages):
-                if g.pool.ref_count(p) != (1 if p in held else 0):
-                    raise CacheError(f"group {gi}: page {p} has reference count {g.pool.ref_count(p)}")
+                expected = len(holders.get(p, ())) + (1 if p in indexed else 0)
+                if g.pool.ref_count(p) != expected:
+                    raise CacheError(f"group {gi}: page {p} has reference count {g.pool.ref_count(p)}, {expected} holders")

@@ -79,8 +79,9 @@ class Runner:
         self._uploads = _StepUploads(model.device, min(8 * self.max_rows + 1024, 1 << 18))       # at most 1 MiB a buffer; what is larger is copied the ordinary way
 
     # -------------------------------------------------------------------------------- requests
-    def open(self, request: Hashable) -> None:
-        self.cache.open(request)
+    def open(self, request: Hashable, shared_pages: Sequence[int] = ()) -> None:
+        """shared_pages: full pages of an equal prompt prefix (`CacheManager.open`)."""
+        self.cache.open(request, shared_pages)
 
     def close(self, request: Hashable) -> None:
         self.cache.close(request)

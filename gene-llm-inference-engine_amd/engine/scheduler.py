@@ -12,6 +12,11 @@ Policy, as the reference's engine (src/runtime/engine.cpp:64-205):
     it goes to the front of the waiting queue and is later fed again from its first token,
     prompt and generated tokens alike, with its sampler's state kept, so that it continues as if
     nothing had happened.
+  * prefix sharing (on unless the configuration or the model's cache rules it out): a request that starts with
+    tokens an earlier request has processed takes that request's full pages and is fed from there (at least its
+    last token is always fed: it produces the logits).  Pages only the prefix index still holds count as free when
+    rows are planned and are given back before the step that needs them.  A preempted request is closed like any
+    other, so what it had computed usually serves it again when it returns.
   * only the row of a request's last known token returns logits; the request's own sampler draws
     the next token from them.  A sampled end token finishes the request (it stays the last
     generated token); so does reaching `max_positions` (prompt plus generated tokens).
@@ -34,6 +39,7 @@ class EngineConfig:
     max_running: int = 8        # requests that hold cache memory and take part in steps at the same time
     step_rows: int = 0          # rows per step; 0 = the runner's max_rows
     prefill_chunk: int = 0      # most prompt tokens one request adds to a step; 0 = no limit besides step_rows
+    prefix_cache: bool = True   # requests with equal first tokens share the pages of that prefix
 
 
 @dataclass
@@ -53,6 +59,7 @@ class EngineResult:
     stopped_by_end_token: bool = False
     error: str = ""
     preemptions: int = 0
+    cached_tokens: int = 0      # positions taken from shared pages instead of being computed (all admissions)
     first_pass: int = -1
     first_token_pass: int = -1
     last_pass: int = -1
@@ -67,6 +74,9 @@ class EngineStats:
     max_rows_in_pass: int = 0
     max_chunk: int = 0
     max_running_seen: int = 0
+    prefix_tokens: int = 0      # positions served by shared pages
+    prefix_hits: int = 0        # admissions that found at least one shared page
+    evicted_pages: int = 0
 
 
 class _Job:
@@ -74,6 +84,7 @@ class _Job:
         self.id, self.request, self.sampler, self.steps = jid, request, sampler, steps
         self.tokens: List[int] = [int(t) for t in request.prompt]      # prompt followed by generated tokens
         self.fed = 0                                                     # tokens[0:fed] are in the cache
+        self.indexed_upto = 0                                            # ... and tokens[0:indexed_upto] known to the prefix index
         self.result = EngineResult(id=jid, prompt_tokens=list(self.tokens))
         self.key = ("job", jid)
 
@@ -88,8 +99,9 @@ class Engine:
         if cfg.step_rows < 0 or cfg.prefill_chunk < 0:
             raise ValueError("Engine: step_rows and prefill_chunk must be >= 0")
         step_rows = cfg.step_rows if 0 < cfg.step_rows <= runner.max_rows else runner.max_rows
-        self.cfg = EngineConfig(min(cfg.max_running, runner.cache.max_requests), step_rows, cfg.prefill_chunk or step_rows)
+        self.cfg = EngineConfig(min(cfg.max_running, runner.cache.max_requests), step_rows, cfg.prefill_chunk or step_rows, cfg.prefix_cache)
         self.runner = runner
+        self.prefix = runner.cache.prefix if cfg.prefix_cache and runner.cache.enable_prefix_sharing() else None
         self.end_tokens = set(int(t) for t in end_tokens)
         self.jobs: List[_Job] = []
         self.waiting: Deque[_Job] = deque()
@@ -128,8 +140,17 @@ class Engine:
     def _admit(self) -> None:
         while self.waiting and len(self.running) < self.cfg.max_running:
             job = self.waiting.popleft()
-            self.runner.open(job.key)
-            job.fed = 0
+            shared = []
+            if self.prefix is not None:
+                # at least one token must still be fed (it produces the logits), and the position limit must leave a row
+                usable = min(len(job.tokens) - 1, job.steps - 1)
+                shared = self.prefix.match(job.tokens, usable) if usable > 0 else []
+            self.runner.open(job.key, shared)
+            job.fed = job.indexed_upto = len(shared) * self.runner.cache.page_size
+            if shared:
+                job.result.cached_tokens += job.fed
+                self.stats.prefix_tokens += job.fed
+                self.stats.prefix_hits += 1
             self.running.append(job)
         self.stats.max_running_seen = max(self.stats.max_running_seen, len(self.running))
 
@@ -151,6 +172,8 @@ class Engine:
         Empty if not even one row fits in the free pages."""
         cache = self.runner.cache
         free = cache.free_pages()
+        if self.prefix is not None:
+            free[0] += cache.evictable_pages()         # pages only the prefix index holds can be given back
         budget = self.cfg.step_rows
         taken = []
         for phase in (0, 1):
@@ -188,6 +211,10 @@ class Engine:
             entries.append(StepEntry(job.key, job.tokens[job.fed:job.fed + n], (n - 1,) if last else ()))
             if last:
                 wanting.append(job)
+        if self.prefix is not None:                  # make room: the plan counted pages that the prefix index still holds
+            cache = self.runner.cache
+            needed = sum(cache.pages_needed(job.key, n)[0] for job, n in taken)
+            self.stats.evicted_pages += cache.evict(needed - cache.free_pages()[0])
         logits = self.runner.step(entries)
         st = self.stats
         st.passes += 1
@@ -203,6 +230,9 @@ class Engine:
             if job.result.first_pass < 0:
                 job.result.first_pass = st.passes
             job.fed += n
+            if self.prefix is not None and job.fed // self.prefix.page_size > job.indexed_upto // self.prefix.page_size:
+                self.prefix.insert(job.tokens, job.fed, self.runner.cache.pages_of(job.key))      # the pages that became full
+                job.indexed_upto = job.fed
             if job.id in next_token:
                 nxt = next_token[job.id]
                 st.logits_rows += 1

@@ -227,3 +227,96 @@ def test_one_position_for_each_is_the_same_as_the_general_path(seed):
             assert (ga.table_host == gb.table_host).all() and ga.pool.free_count == gb.pool.free_count
         assert all(a.length(r) == b.length(r) for r in live)
         b.check_consistency()
+
+
+# ------------------------------------------------------------------------------- prefix sharing
+def test_prefix_index_matches_true_prefixes_of_full_pages_only():                 # src/model/prefix_cache.h:1-11
+    from geneinfer_amd.cache import PagePool, PrefixIndex
+    pool = PagePool(12)
+    index = PrefixIndex(pool, page_size=4)
+    tokens = list(range(100, 114))                                                # 3 full pages and 2 tokens
+    pages = [pool.allocate() for _ in range(4)]
+    assert index.insert(tokens, 14, pages) == 3 and len(index) == 3                # the partly filled page is not named
+    assert [pool.ref_count(p) for p in pages] == [2, 2, 2, 1]
+    assert index.insert(tokens, 14, pages) == 0                                    # known links are followed, not named again
+    found = index.match(tokens, 14)
+    assert found == pages[:3] and [pool.ref_count(p) for p in pages[:3]] == [3, 3, 3]      # retained for the caller
+    for p in found:
+        pool.release(p)
+    assert index.match(tokens, 11) == pages[:2] and index.match(tokens, 3) == []   # the limit counts whole pages
+    for p in pages[:2]:
+        pool.release(p)
+    other = tokens[:4] + [7, 7, 7, 7] + tokens[8:]                                 # equal first page, then another, then an equal third
+    assert index.match(other, 14) == pages[:1]                                     # the third page is no prefix of this
+    pool.release(pages[0])
+    assert index.match(tokens[4:], 10) == []                                       # the same tokens elsewhere in a prompt do not match
+    # another request computed the same first page itself, then went on differently: its copy is not named, its second page is
+    own = [pool.allocate() for _ in range(2)]
+    assert index.insert(other, 8, own) == 1 and own[0] not in index and own[1] in index
+    assert index.match(other, 8) == [pages[0], own[1]]
+
+
+def test_prefix_index_gives_back_least_recently_used_leaves_that_nobody_uses():    # src/model/prefix_cache.cpp:60-97
+    from geneinfer_amd.cache import PagePool, PrefixIndex
+    pool = PagePool(10)
+    index = PrefixIndex(pool, page_size=2)
+    a = [pool.allocate() for _ in range(3)]
+    b = [pool.allocate() for _ in range(2)]
+    index.insert([1, 1, 2, 2, 3, 3], 6, a)
+    index.insert([9, 9, 8, 8], 4, b)
+    assert index.evictable() == 0 and index.evict(5) == 0                          # everything is still used by its request
+    for p in a + b:
+        pool.release(p)                                                            # the requests end
+    assert index.evictable() == 5 and pool.free_count == 5
+    held = index.match([1, 1, 2, 2], 4)                                            # a request uses a's first two pages (and touches them)
+    assert held == a[:2] and index.evictable() == 3
+    assert index.evict(1) == 1 and a[2] not in index and b[1] in index             # a's leaf was used before b's
+    assert index.evict(10) == 2 and len(index) == 2 and pool.free_count == 8       # b's leaf, then b's root; the used pages stay
+    assert [pool.ref_count(p) for p in held] == [2, 2]
+    for p in held:
+        pool.release(p)
+    index.clear()
+    assert pool.free_count == 10 and len(index) == 0
+
+
+def test_prefix_index_forgets_a_used_leaf_to_reach_an_unused_page_above():
+    from geneinfer_amd.cache import PagePool, PrefixIndex
+    pool = PagePool(4)
+    index = PrefixIndex(pool, page_size=1)
+    chain = [pool.allocate() for _ in range(3)]
+    index.insert([5, 6, 7], 3, chain)
+    pool.release(chain[0]); pool.release(chain[1])                                 # only the last page is still used by someone
+    assert index.evictable() == 2
+    assert index.evict(2) == 2 and len(index) == 0                                 # the used leaf is forgotten, then the two above go
+    assert pool.ref_count(chain[2]) == 1 and pool.free_count == 3
+
+
+def test_requests_open_on_shared_pages():
+    m = manager([FULL], n_pages=8, page_size=4, max_requests=3, max_positions=32)
+    assert m.enable_prefix_sharing() and m.prefix is not None
+    m.open("a")
+    m.reserve([("a", 10)]); m.advance("a", 10)
+    tokens = list(range(10))
+    assert m.prefix.insert(tokens, 10, m.pages_of("a")) == 2
+    shared = m.prefix.match(tokens + [77], 10)
+    m.open("b", shared)
+    assert m.length("b") == 8 and m.pages_of("b") == m.pages_of("a")[:2]
+    m.check_consistency()
+    m.reserve([("b", 3)]); m.advance("b", 3)
+    assert m.pages_of("b")[2] not in m.pages_of("a")                              # what b writes goes to a page of its own
+    m.close("a")
+    m.check_consistency()
+    assert m.free_pages() == [8 - 3] and m.evictable_pages() == 0                  # a's third page is free, the shared two serve b
+    m.close("b")
+    assert m.free_pages() == [6] and m.evictable_pages() == 2 and m.evict(5) == 2 and m.free_pages() == [8]
+    m.check_consistency()
+    with pytest.raises(CacheError, match="already open|shared"):
+        m2 = manager([FULL], n_pages=4, page_size=4, max_requests=2, max_positions=16)
+        m2.open("x", [0])
+
+
+def test_prefix_sharing_needs_one_group_without_window_or_state():
+    assert not manager([FULL, WINDOW], n_pages=8, page_size=4, max_requests=2, max_positions=32).enable_prefix_sharing()
+    assert not manager([WINDOW], n_pages=8, page_size=4, max_requests=2, max_positions=32).enable_prefix_sharing()
+    from geneinfer_amd.cache import StateNeed
+    assert not manager([FULL, StateNeed((3,), torch.float32)], n_pages=8, page_size=4, max_requests=2, max_positions=32).enable_prefix_sharing()

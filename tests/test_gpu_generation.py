@@ -87,9 +87,47 @@ def test_scheduler_gives_each_request_what_it_gets_alone(folders, name, temperat
             r = eng.result(jid)
             assert r.finished and r.error == "" and r.generated_tokens == want, (max_tokens, jid, r.preemptions)
         llm.runner.cache.check_consistency()
+        if eng.prefix is not None:
+            eng.prefix.clear()
         assert llm.runner.cache.free_pages() == [max_tokens // ps]
         preempted += eng.stats.preemptions
     assert preempted > 0, "no pool was tight enough to preempt"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_requests_with_an_equal_beginning_share_its_pages(folders, dtype):
+    """Requests that begin alike take the pages an earlier one computed: fewer rows are fed, and every request still
+    ends with the tokens it gets alone (bit for bit in 32-bit, where the keys of a position never depend on the batch)."""
+    import geneinfer_amd as gi
+    from geneinfer_amd.engine import EngineConfig, EngineRequest
+    from geneinfer_amd.sampling import SamplerConfig
+    name, new = "B", 10
+    system = prompts_for(name, [70], seed=31)[0]
+    tails = prompts_for(name, [5, 1, 12, 30], seed=32)
+    prompts = [system + t for t in tails] + [system[:40], tails[3] + system]
+    def run(prefix_cache, max_tokens):
+        llm = gi.LLM(folders[name], dtype=dtype, page_size=16, max_tokens=max_tokens, max_running=3, max_rows=64)
+        eng = llm.engine(EngineConfig(max_running=3, step_rows=48, prefix_cache=prefix_cache))
+        ids = [eng.submit(EngineRequest(prompts[0], len(prompts[0]) + new - 1, SamplerConfig(0.0)))]
+        eng.run_until_idle()                                         # the first one has finished when the others arrive
+        ids += [eng.submit(EngineRequest(p, len(p) + new - 1, SamplerConfig(0.0))) for p in prompts[1:]]
+        eng.run_until_idle()
+        llm.runner.cache.check_consistency()
+        return eng, [eng.result(j) for j in ids]
+    plain_eng, plain = run(False, 1024)
+    for max_tokens in (1024, 192):                                   # roomy; and so tight that named pages must be given back
+        eng, shared = run(True, max_tokens)
+        assert eng.prefix is not None and eng.stats.prefix_hits >= 4 and eng.stats.prefix_tokens >= 3 * 64 + 32
+        assert eng.stats.rows <= plain_eng.stats.rows - (3 * 64 + 32) + 64 * eng.stats.preemptions
+        for a, b in zip(shared, plain):
+            assert a.finished and a.error == ""
+            if dtype == "float32":
+                assert a.generated_tokens == b.generated_tokens
+            else:                                                    # the first token at least, where the plain model is clear about it
+                assert len(a.generated_tokens) == len(b.generated_tokens)
+        assert sum(r.cached_tokens for r in shared) == eng.stats.prefix_tokens
+        if max_tokens == 192:
+            assert eng.stats.evicted_pages > 0 or eng.stats.preemptions > 0
 
 
 def test_scheduler_in_bfloat16_runs_mixed_batches(folders):

@@ -26,10 +26,11 @@ class FakeRunner:
         self.model = SimpleNamespace(spec=SimpleNamespace(vocab_size=VOCAB))
         self.max_rows, self.max_positions = max_rows, max_positions
         self.fed, self.log = {}, []
+        self.page_size, self.on_page = page_size, {}          # what each page of the first group holds, place by place
 
-    def open(self, r):
-        self.cache.open(r)
-        self.fed[r] = []
+    def open(self, r, shared_pages=()):
+        self.cache.open(r, shared_pages)
+        self.fed[r] = [self.on_page[(int(p), i)] for p in shared_pages for i in range(self.page_size)]      # what the shared pages hold
 
     def close(self, r):
         self.cache.close(r)
@@ -45,6 +46,11 @@ class FakeRunner:
         for e in entries:
             assert len(self.fed[e.request]) == self.cache.length(e.request)
             for i, t in enumerate(e.tokens):
+                at = len(self.fed[e.request])
+                page = self.cache.pages_of(e.request)[at // self.page_size - int(self.cache.groups[0].first_live[self.cache.slot(e.request)])]
+                assert self.cache.groups[0].pool.ref_count(page) == 1 or (self.cache.prefix is not None and page in self.cache.prefix and
+                                                                          self.cache.groups[0].pool.ref_count(page) == 2 and False), "a shared page is written"
+                self.on_page[(page, at % self.page_size)] = int(t)
                 self.fed[e.request].append(int(t))
                 if i in e.want:
                     seed = int.from_bytes(hashlib.sha256(str(self.fed[e.request]).encode()).digest()[:8], "little")
@@ -53,6 +59,15 @@ class FakeRunner:
         self.log.append([(e.request, len(e.tokens), tuple(e.want)) for e in entries])
         self.cache.check_consistency()
         return torch.from_numpy(np.stack(rows)) if rows else None
+
+
+def pages_when_forgotten(runner):
+    """Free pages per group once the prefix index has let go of what it keeps."""
+    runner.cache.check_consistency()
+    if runner.cache.prefix is not None:
+        assert runner.cache.prefix.evictable() == len(runner.cache.prefix)       # nobody else holds them
+        runner.cache.prefix.clear()
+    return runner.cache.free_pages()
 
 
 def host_sample_row(row, sampler):
@@ -87,17 +102,27 @@ END = {7, 31}                                     # about one token in 25 ends a
     (64, 4, 0, 0), (64, 1, 0, 0), (64, 6, 1, 0), (64, 3, 3, 1), (40, 4, 8, 5), (30, 4, 64, 16), (26, 5, 8, 0), (25, 3, 3, 5),
     (25, 6, 64, 0), (48, 2, 5, 16), (24, 8, 0, 0), (24, 4, 8, 3),
 ])
-def test_every_request_gets_the_tokens_it_gets_alone(n_pages, max_running, step_rows, chunk):      # src/runtime/engine.h:8-9, tools/engine_check_main.cpp:179-211
+@pytest.mark.parametrize("prefix_cache", [False, True])
+def test_every_request_gets_the_tokens_it_gets_alone(n_pages, max_running, step_rows, chunk, prefix_cache):      # src/runtime/engine.h:8-9, tools/engine_check_main.cpp:179-211
     rng = random.Random(n_pages * 100 + max_running)
     requests = make_requests(rng, 9)
+    if prefix_cache:                                                   # some requests start like others, by one page and more
+        requests[3] = (requests[2][0][:9] + requests[3][0], *requests[3][1:])
+        requests[6] = (requests[2][0] + requests[6][0], 0, requests[6][2])
+        requests[7] = (list(requests[6][0]), 0, requests[7][2])
     runner = FakeRunner(n_pages=n_pages, max_requests=8, max_rows=64)
-    eng = Engine(runner, EngineConfig(max_running, step_rows, chunk), END, sample=host_sample)
+    eng = Engine(runner, EngineConfig(max_running, step_rows, chunk, prefix_cache), END, sample=host_sample)
+    assert (eng.prefix is not None) == prefix_cache
     ids = [eng.submit(EngineRequest(p, limit, cfg)) for p, limit, cfg in requests[:5]]
     for _ in range(3):                                                 # the rest arrive while the first are running
         eng.step()
     ids += [eng.submit(EngineRequest(p, limit, cfg)) for p, limit, cfg in requests[5:]]
     eng.run_until_idle()
     assert eng.idle() and not runner.cache.open_requests()
+    runner.cache.check_consistency()
+    if prefix_cache:                                                   # what is not free is what the prefix index keeps
+        assert runner.cache.free_pages() == [n_pages - len(eng.prefix)] and eng.prefix.evictable() == len(eng.prefix)
+        eng.prefix.clear()
     assert runner.cache.free_pages() == [n_pages]                      # nothing leaked
     for jid, (prompt, limit, cfg) in zip(ids, requests):
         res = eng.result(jid)
@@ -112,7 +137,10 @@ def test_every_request_gets_the_tokens_it_gets_alone(n_pages, max_running, step_
     st = eng.stats
     assert st.passes == len(runner.log) and st.rows == sum(n for e in runner.log for _, n, _ in e)
     assert st.max_rows_in_pass <= rows_limit and st.max_running_seen <= max_running
-    print(f"pages {n_pages}: {st.passes} passes, {st.preemptions} preemptions")
+    assert st.prefix_tokens == sum(eng.result(j).cached_tokens for j in ids) and (st.prefix_hits > 0) == (st.prefix_tokens > 0)
+    assert prefix_cache or st.prefix_tokens == 0
+    print(f"pages {n_pages}: {st.passes} passes, {st.preemptions} preemptions, {st.prefix_hits} prefix hits ({st.prefix_tokens} positions), "
+          f"{st.evicted_pages} pages evicted")
     test_every_request_gets_the_tokens_it_gets_alone.preemptions += st.preemptions
 
 
@@ -160,7 +188,7 @@ def test_portions_shrink_to_the_free_pages_and_the_youngest_is_preempted():
     assert eng.stats.preemptions >= 1 and eng.result(y).preemptions >= 1 and eng.result(x).preemptions == 0      # the youngest goes
     for jid, prompt, limit in ((x, [1] * 10, 24), (y, [2] * 18, 22)):
         assert eng.result(jid).generated_tokens == alone(prompt, limit, SamplerConfig(0.0), ())[0]
-    assert runner.cache.free_pages() == [6]
+    assert pages_when_forgotten(runner) == [6]
 
 
 def test_a_lone_request_that_cannot_fit_fails_with_the_reference_message():        # src/runtime/engine.cpp:157-163
@@ -170,7 +198,7 @@ def test_a_lone_request_that_cannot_fit_fails_with_the_reference_message():     
     eng.run_until_idle()
     r = eng.result(big)
     assert r.finished and r.error == POOL_TOO_SMALL and len(r.generated_tokens) == 12 - 8 + 1
-    assert runner.cache.free_pages() == [3]
+    assert runner.cache.free_pages()[0] + runner.cache.evictable_pages() == 3
     small = eng.submit(EngineRequest([3] * 5, 9, SamplerConfig(0.0)))              # the engine goes on afterwards
     eng.run_until_idle()
     assert eng.result(small).error == "" and len(eng.result(small).generated_tokens) == 5
@@ -217,6 +245,51 @@ def test_windowed_groups_are_planned_per_group():
     eng.run_until_idle()
     assert eng.result(j).error == "" and len(eng.result(j).generated_tokens) == 25
     assert runner.cache.free_pages() == [10, 10]
+
+
+def test_requests_with_an_equal_beginning_share_its_pages():                       # src/runtime/engine.cpp:64-98
+    runner = FakeRunner(page_size=4, n_pages=32, max_rows=64)
+    eng = Engine(runner, EngineConfig(max_running=1), sample=host_sample)          # one after the other
+    system = [rng_token for rng_token in range(10, 23)]                            # 13 tokens: 3 full pages and one more
+    prompts = [system + [1, 2], system + [3], system[:8], system[:9], [9] + system]
+    limits = [20, 0, 9, 0, 0]
+    ids = [eng.submit(EngineRequest(p, lim, SamplerConfig(0.0))) for p, lim in zip(prompts, limits)]
+    eng.run_until_idle()
+    cached = [eng.result(j).cached_tokens for j in ids]
+    # nothing yet; 3 pages; at least the last token is fed (7 usable tokens: 1 page) and so is the row the limit of 9 leaves;
+    # 2 pages of the 8 usable tokens; another first token: no prefix
+    assert cached == [0, 12, 4, 8, 0]
+    for j, p, lim in zip(ids, prompts, limits):
+        assert eng.result(j).generated_tokens == alone(p, lim, SamplerConfig(0.0), ())[0]
+    for j, p in zip(ids, prompts):                                                 # what was cached was not fed again
+        rows = sum(n for e in runner.log for r, n, _ in e if r == ("job", j))
+        new_prompt_rows = min(len(p), eng.jobs[j].steps) - eng.result(j).cached_tokens
+        assert new_prompt_rows <= rows <= new_prompt_rows + len(eng.result(j).generated_tokens)
+    assert eng.stats.prefix_hits == 3 and eng.stats.prefix_tokens == 24
+    assert pages_when_forgotten(runner) == [32]
+
+
+def test_pages_only_the_prefix_index_holds_are_given_back_before_anyone_is_preempted():
+    runner = FakeRunner(page_size=4, n_pages=8, max_rows=64)                       # 32 positions
+    eng = Engine(runner, EngineConfig(max_running=2), sample=host_sample)
+    a = eng.submit(EngineRequest(list(range(1, 17)), 20, SamplerConfig(0.0)))      # fills 5 pages, 4 of them stay named
+    eng.run_until_idle()
+    assert len(eng.prefix) == 5 and runner.cache.free_pages() == [3]
+    b = eng.submit(EngineRequest(list(range(30, 48)), 30, SamplerConfig(0.0)))     # needs 8 pages in the end
+    eng.run_until_idle()
+    assert eng.result(b).error == "" and eng.stats.preemptions == 0 and eng.stats.evicted_pages == 5
+    assert eng.result(b).generated_tokens == alone(list(range(30, 48)), 30, SamplerConfig(0.0), ())[0]
+    assert pages_when_forgotten(runner) == [8]
+
+
+def test_prefix_sharing_can_be_switched_off_and_is_off_where_the_cache_cannot_share():
+    eng = Engine(FakeRunner(), EngineConfig(prefix_cache=False), sample=host_sample)
+    assert eng.prefix is None
+    j = eng.submit(EngineRequest([1] * 9, 12, SamplerConfig(0.0)))
+    k = eng.submit(EngineRequest([1] * 9, 12, SamplerConfig(0.0)))
+    eng.run_until_idle()
+    assert eng.result(k).cached_tokens == 0 and eng.result(j).generated_tokens == eng.result(k).generated_tokens
+    assert Engine(FakeRunner(windows=True), sample=host_sample).prefix is None     # a windowed group gives pages back early
 
 
 def test_step_uploads_ring_on_the_cpu():
