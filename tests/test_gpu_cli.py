@@ -54,3 +54,34 @@ def test_make_random_model_writes_a_loadable_folder(tmp_path):
     assert r.returncode == 0, r.stderr
     logits = PlainLlama(tmp_path / "m").logits([1, 2, 3])
     assert logits.shape == (3, 301) and torch.isfinite(logits).all()
+
+
+@pytest.mark.gpu
+def test_gi_serve_bench_levels_generate_what_each_request_generates_alone(tmp_path):
+    """In 32-bit the tokens do not depend on who else runs.  Requests admitted together find nothing in an
+    empty index (the pages are named once they are full); with --warm-cache the unmeasured run has left every
+    prompt's full pages (block size 8, 50 prompt tokens of which the last is always computed: 6 pages)."""
+    write_model(tmp_path / "m", CONFIGS["B"], seed=4)
+    exe = str(ROOT / "bin" / "gi_serve_bench")
+    common = [exe, "--model", str(tmp_path / "m"), "--concurrency", "1,4", "--prompt-tokens", "50", "--decode-tokens", "12", "--runs", "1",
+              "--weights", "f32", "--block-size", "8", "--shared-prefix", "40"]
+    r = subprocess.run(common, capture_output=True, text=True, timeout=170)
+    assert r.returncode == 0, r.stdout + r.stderr
+    rows = [line.split() for line in r.stdout.splitlines() if line[:1].isdigit()]
+    assert [int(row[0]) for row in rows] == [1, 4] and all("identical" in " ".join(row) for row in rows)
+    assert int(rows[0][6]) == 0 and int(rows[1][6]) == 0                        # cached positions of the measured run
+    warm = subprocess.run(common + ["--warm-cache"], capture_output=True, text=True, timeout=170)
+    assert warm.returncode == 0, warm.stdout + warm.stderr
+    rows = [line.split() for line in warm.stdout.splitlines() if line[:1].isdigit()]
+    assert int(rows[0][6]) == 48 and int(rows[1][6]) == 4 * 48
+    off = subprocess.run(common + ["--no-prefix-cache"], capture_output=True, text=True, timeout=170)
+    assert off.returncode == 0 and all(int(line.split()[6]) == 0 for line in off.stdout.splitlines() if line[:1].isdigit())
+
+
+def test_gi_serve_bench_usage_errors():
+    exe = str(ROOT / "bin" / "gi_serve_bench")
+    for args, msg in (([], "--model is required"), (["--model", "x", "--concurrency", "0"], "--concurrency needs positive integers"),
+                      (["--model", "x", "--weights", "int8"], "--weights must be native or f32"), (["--model", "x", "--runs"], "missing value for --runs"),
+                      (["--model", "x", "--max-seq-len", "8"], "--max-seq-len is shorter"), (["--model", "x", "--what"], "unknown option --what")):
+        r = subprocess.run([exe, *args], capture_output=True, text=True, timeout=60)
+        assert r.returncode == 2 and msg in r.stderr and "usage: gi_serve_bench" in r.stderr
