@@ -93,6 +93,43 @@ class PageGroup:
     def held_pages(self, slot: int) -> List[int]:
         return [int(p) for p in self.table_host[slot, int(self.first_live[slot]):int(self.n_held[slot])]]
 
+    def can_rewind_to(self, slot: int, length: int) -> bool:
+        """Whether the pages the row at position `length` sees are still held (a window may have given them back)."""
+        if self.need.window is None or length == 0:
+            return True
+        return int(self.first_live[slot]) <= max(0, length - self.need.window + 1) // self.page_size
+
+    def pages_freed_by_rewind(self, slot: int, length: int) -> int:
+        first = max(-(-length // self.page_size), int(self.first_live[slot]))
+        return sum(1 for i in range(first, int(self.n_held[slot])) if self.pool.ref_count(int(self.table_host[slot, i])) == 1)
+
+    def shared_page_at(self, slot: int, length: int) -> bool:
+        """Whether position `length` falls inside a held page that someone else holds too: it must be copied
+        before the request writes there again."""
+        i = length // self.page_size
+        return length % self.page_size != 0 and i < int(self.n_held[slot]) and self.pool.ref_count(int(self.table_host[slot, i])) > 1
+
+    def rewind(self, slot: int, length: int) -> None:
+        """Gives back the pages that hold only positions from `length` on, last first (the reference's truncate,
+        src/model/kv_cache.cpp:100-109), and makes the page that `length` falls into the request's own
+        (its make_writable, src/model/kv_cache.cpp:116-141: a copy of the whole page, every layer)."""
+        if length == 0:
+            self.release_all(slot)
+            return
+        keep = max(-(-length // self.page_size), int(self.first_live[slot]))
+        for i in range(int(self.n_held[slot]) - 1, keep - 1, -1):
+            self.pool.release(int(self.table_host[slot, i]))
+            self.table_host[slot, i] = -1
+        self.n_held[slot] = min(int(self.n_held[slot]), keep)
+        if self.shared_page_at(slot, length):
+            i = length // self.page_size
+            old, new = int(self.table_host[slot, i]), self.pool.allocate()
+            if self.storage is not None:
+                self.storage[:, new].copy_(self.storage[:, old])
+            self.pool.release(old)
+            self.table_host[slot, i] = new
+        self.dirty.add(slot)
+
     def sync(self, upload=None) -> None:
         if self.table_dev is None or not self.dirty:
             self.dirty.clear()
@@ -287,6 +324,29 @@ class CacheManager:
         self._length[request] = new_length
         for g in self.groups:
             g.drop_behind_window(slot, new_length)
+
+    def truncate(self, request: Hashable, length: int) -> None:
+        """Rewind: the request keeps its first `length` positions and its next token goes to position `length`.
+        Pages beyond are given back; a page that `length` falls into and that others hold too (a shared prefix,
+        the prefix index) is copied first, so that what they see never changes.  Refused, with nothing changed,
+        where the past cannot be restored: fixed-size state, or pages that a window has given back.
+        Behaviour as the reference's rewind (src/model/transformer.cpp:545-552, src/model/kv_cache.cpp:100-141)."""
+        slot, old = self.slot(request), self._length[request]
+        if not 0 <= length <= old:
+            raise CacheError(f"request {request!r} holds {old} positions; it cannot be cut to {length}")
+        if length == old:
+            return
+        if self._state_needed:
+            raise CacheError("a request with fixed-size state cannot be rewound: the state of earlier positions is gone")
+        for g in self.groups:
+            if not g.can_rewind_to(slot, length):
+                raise CacheError(f"request {request!r} cannot be rewound to {length}: a window of {g.need.window} has given those pages back")
+        for g in self.groups:
+            if g.shared_page_at(slot, length) and g.pool.free_count + g.pages_freed_by_rewind(slot, length) < 1:
+                raise OutOfPages("no free page to copy a shared page into")
+        for g in self.groups:
+            g.rewind(slot, length)
+        self._length[request] = length
 
     def sync(self, upload=None) -> None:
         """Brings the device copies of changed page tables up to date.  `upload(int32 array) -> device tensor`

@@ -86,6 +86,10 @@ class Runner:
     def close(self, request: Hashable) -> None:
         self.cache.close(request)
 
+    def truncate(self, request: Hashable, length: int) -> None:
+        """Rewind: the request's next token goes to position `length` (`CacheManager.truncate`)."""
+        self.cache.truncate(request, length)
+
     def is_open(self, request: Hashable) -> bool:
         return self.cache.is_open(request)
 

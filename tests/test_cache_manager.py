@@ -159,6 +159,14 @@ def test_random_orders_of_requests_keep_the_books(seed):
             rid = rng.choice(list(live))
             m.close(rid)
             del live[rid]
+        elif action < 0.4 and live:                                            # a rewind, where the cache can do one
+            rid = rng.choice(list(live))
+            to = rng.randint(0, live[rid])
+            try:
+                m.truncate(rid, to)
+                live[rid] = to
+            except CacheError as e:
+                assert "window" in str(e) and len(needs) == 3 and m.length(rid) == live[rid]
         elif live:
             batch = rng.sample(list(live), rng.randint(1, len(live)))
             adds = [(rid, rng.randint(1, 7)) for rid in batch if live[rid] < 33]
@@ -320,3 +328,89 @@ def test_prefix_sharing_needs_one_group_without_window_or_state():
     assert not manager([WINDOW], n_pages=8, page_size=4, max_requests=2, max_positions=32).enable_prefix_sharing()
     from geneinfer_amd.cache import StateNeed
     assert not manager([FULL, StateNeed((3,), torch.float32)], n_pages=8, page_size=4, max_requests=2, max_positions=32).enable_prefix_sharing()
+
+
+def test_rewind_gives_pages_back_and_goes_on_from_there():                        # src/model/kv_cache.cpp:100-109
+    m = manager([FULL], n_pages=6, page_size=4)
+    m.open("a")
+    m.reserve([("a", 14)]); m.advance("a", 14)                                    # pages 0..3
+    pages = m.pages_of("a")
+    m.truncate("a", 14)                                                           # nothing to do
+    assert m.pages_of("a") == pages
+    m.truncate("a", 6)
+    assert m.length("a") == 6 and m.pages_of("a") == pages[:2] and m.free_pages() == [4]
+    m.check_consistency()
+    m.reserve([("a", 3)]); m.advance("a", 3)                                      # positions 6, 7 in the kept page, 8 in a new one
+    assert m.pages_of("a") == pages[:2] + [pages[2]]                              # the page freed last comes back first
+    m.truncate("a", 8)                                                            # exactly at a page's edge: the page after it goes
+    assert m.pages_of("a") == pages[:2]
+    m.truncate("a", 0)
+    assert m.length("a") == 0 and m.pages_of("a") == [] and m.free_pages() == [6]
+    m.reserve([("a", 1)]); m.advance("a", 1)
+    m.check_consistency()
+    with pytest.raises(CacheError, match="cannot be cut"):
+        m.truncate("a", 2)
+    with pytest.raises(CacheError, match="cannot be cut"):
+        m.truncate("a", -1)
+    with pytest.raises(CacheError, match="not open"):
+        m.truncate("b", 0)
+
+
+def test_rewind_into_a_shared_page_copies_it_first():                             # src/model/kv_cache.cpp:116-141
+    m = CacheManager([FULL, FULL], [None, None], page_size=4, n_pages=5, max_requests=3, max_positions=32, dtype=torch.float32)
+    assert m.enable_prefix_sharing()
+    g = m.groups[0]
+    m.open("a")
+    m.reserve([("a", 8)]); m.advance("a", 8)
+    first, second = m.pages_of("a")
+    g.storage[:, second] = torch.arange(g.storage[:, second].numel(), dtype=torch.float32).reshape(g.storage[:, second].shape)
+    tokens = list(range(8))
+    m.prefix.insert(tokens, 8, m.pages_of("a"))
+    m.open("b", m.prefix.match(tokens + [9], 8))                                  # b shares both pages
+    m.truncate("b", 6)                                                            # b will write position 6: inside the second page
+    mine = m.pages_of("b")
+    assert mine[0] == first and mine[1] != second and m.pages_of("a") == [first, second]
+    assert torch.equal(g.storage[:, mine[1]], g.storage[:, second])               # every layer, keys and values
+    m.check_consistency()
+    g.storage[:, mine[1], :, :, 2:] = -1.0                                        # what b writes from position 6 on
+    assert (g.storage[:, second] >= 0).all()                                      # a and the index still see their own
+    m.truncate("b", 5)                                                            # its own page now: no second copy
+    assert m.pages_of("b") == mine
+    m.truncate("b", 4)                                                            # at the edge: the copy goes, the shared first page stays
+    assert m.pages_of("b") == [first] and m.free_pages() == [3]
+    # no page to copy into: refused with nothing changed
+    m.open("c")
+    m.reserve([("c", 9)]); m.advance("c", 9)                                      # the 3 free pages
+    with pytest.raises(OutOfPages):
+        m.truncate("b", 2)
+    assert m.length("b") == 4 and m.pages_of("b") == [first]
+    m.close("c")
+    m.truncate("b", 2)                                                            # the first page is shared as well
+    assert m.pages_of("b")[0] != first and m.length("b") == 2
+    m.check_consistency()
+    for r in ("a", "b"):
+        m.close(r)
+    m.prefix.clear()
+    m.check_consistency()
+    assert m.free_pages() == [5]
+
+
+def test_rewind_is_refused_where_the_past_is_gone():
+    m = manager([WINDOW], n_pages=6, page_size=4)                                 # window 10
+    m.open("a")
+    for _ in range(30):
+        m.reserve([("a", 1)]); m.advance("a", 1)                                  # the next row sees 21..: pages 0..4 were given back
+    assert int(m.groups[0].first_live[m.slot("a")]) == 5
+    before = (m.pages_of("a"), m.free_pages())
+    with pytest.raises(CacheError, match="window of 10"):
+        m.truncate("a", 20)                                                       # would need positions 11..19
+    assert (m.pages_of("a"), m.free_pages(), m.length("a")) == (*before, 30)
+    m.truncate("a", 29)                                                           # sees 20..28: page 5 on, all held
+    assert m.length("a") == 29
+    m.truncate("a", 0)                                                            # a fresh start needs nothing
+    assert m.free_pages() == [6] and int(m.groups[0].first_live[m.slot("a")]) == 0
+    s = manager([FULL, StateNeed((3,))])
+    s.open("a")
+    s.reserve([("a", 5)]); s.advance("a", 5)
+    with pytest.raises(CacheError, match="fixed-size state"):
+        s.truncate("a", 2)

@@ -110,6 +110,56 @@ def test_changing_first_token_changes_logits(case):
     assert relative_error(got[(rid, len(toks) - 1)], want["float32"][rid][len(toks) - 1]) > 1e-3
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_rewind_and_go_another_way(case, dtype):
+    """A request is cut back (inside a page, at a page's edge, to nothing) and fed other tokens: the logits are
+    those of the sequence as it now stands.  One rewind falls into a page that a second request shares; that
+    request's later logits do not change."""
+    from geneinfer_amd.engine import Runner, StepEntry, load_model
+    name, folder, requests, _ = case
+    ps, vocab = PAGE_SIZE[name], CONFIGS[name]["vocab_size"]
+    rng = random.Random(77)
+    base = [rng.randrange(vocab) for _ in range(3 * ps + 3)]
+    plain, rounded = PlainLlama(folder), PlainLlama(folder, storage=torch.bfloat16)
+    model = load_model(folder, dtype, "cuda:0")
+    runner = Runner(model, page_size=ps, max_tokens=16 * ps, max_requests=2, max_rows=4096)
+    assert runner.cache.enable_prefix_sharing()
+    runner.open("a")
+    runner.step([StepEntry("a", base, ())])
+    runner.cache.prefix.insert(base, len(base), runner.cache.pages_of("a"))
+    runner.open("b", runner.cache.prefix.match(base, len(base) - 1))          # b shares a's three full pages
+    assert runner.length("b") == 3 * ps
+    got, exact, near = {}, {}, {}
+    def feed(rid, history, tokens):
+        rows = runner.step([StepEntry(rid, tokens, tuple(range(len(tokens))))]).cpu()
+        now = history + tokens
+        e, r = plain.logits(now), rounded.logits(now)
+        for i, row in enumerate(rows):
+            key = (rid, len(got))
+            got[key], exact[key], near[key] = row, e[len(history) + i], r[len(history) + i]
+        return now
+    seq_b = feed("b", base[:3 * ps], base[3 * ps:3 * ps + 2])
+    seq_a = list(base)
+    for cut in (2 * ps + 3, 2 * ps, ps - 1, 0):                                 # the first falls into a page that b shares
+        runner.truncate("a", cut)
+        assert runner.length("a") == cut
+        other = [rng.randrange(vocab) for _ in range(ps + 2)]
+        seq_a = feed("a", seq_a[:cut], other[:1])                               # one token through the decode path
+        seq_a = feed("a", seq_a, other[1:])                                     # then a portion
+        runner.cache.check_consistency()
+    assert set(runner.cache.pages_of("a")).isdisjoint(runner.cache.pages_of("b")[:3])
+    feed("b", seq_b, base[3 * ps + 2:])                                         # b still reads the pages as a first wrote them
+    if dtype == "float32":
+        worst = max(relative_error(row, exact[key]) for key, row in got.items())
+        assert worst < TOLERANCE["float32"], f"worst relative error {worst:.3e}"
+    else:
+        assert_within_bfloat16_noise(got, exact.__getitem__, near.__getitem__, f"tiny {name}, rewind")
+    runner.close("a"); runner.close("b")
+    runner.cache.prefix.clear()
+    runner.cache.check_consistency()
+    assert runner.cache.free_pages() == [g.pool.n_pages for g in runner.cache.groups]
+
+
 def test_a_runner_with_captured_steps_is_freed_without_the_cycle_collector(case):
     """A runner and its captured graphs form no reference cycle: dropping the runner frees them at once, not at a
     moment of the cycle collector's choosing (which may fall inside another capture, where freeing aborts)."""
