@@ -26,49 +26,67 @@ constexpr float LOG2E = 1.4426950408889634f;
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // =========================================================================================== prompt
-// Workgroup: 4 waves, a tile of up to 128 consecutive rows of one request (32 per wave), one query
-// head.  Keys and values come in tiles of 64 positions through LDS.  The score product is taken
-// transposed, S^T[kv][q] = K * Q^T, so that each lane owns one query row (column lane%32) and the
-// softmax statistics of a row live in one lane (and its partner lane^32); the output is
-// accumulated transposed as well, O^T[d][q] = V^T * P^T.
+// Workgroup: PAIR row tiles of one request (up to 32 * NW consecutive rows each), one query head.
+// 32 rows belong to two waves: each takes one half (32 positions) of every tile of 64 keys and
+// keeps its own running maximum, sum and output, which meet in LDS at the end.  That way a row's
+// walk over the keys, a chain of dependent steps (products, maximum, exponentials, products),
+// is shared by two waves that fill each other's waits.
+// With PAIR = 2 a late tile of a prompt shares its workgroup with an early one: the two walk the
+// keys together from the first position on, the early tile's waves stop where their rows end, and
+// every workgroup of a prompt has about the same number of keys to visit (tile i sees i + 1 tiles
+// of keys; a workgroup per tile would leave the chip waiting for the last ones).
+// Keys and values come in tiles of 64 positions through LDS, staged once for all waves.  The
+// score product is taken transposed, S^T[kv][q] = K * Q^T, so that each lane owns one query row
+// (column lane%32) and the softmax statistics of a row live in one lane (and its partner lane^32);
+// the output is accumulated transposed as well, O^T[d][q] = V^T * P^T.
 //
-// tiles[i] = {first row in the step, number of rows, position of the first row, request slot}.
+// tiles[i] = {first row in the step, number of rows, position of the first row, request slot};
+// workgroup w takes tiles[PAIR * w .. PAIR * w + PAIR), of one request (a tile of 0 rows fills a pair).
 constexpr int KV_TILE = 64;
 
-template <int HD, int NW>
-__global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
-                                                                  bf16_t* __restrict__ out, const int4* __restrict__ tiles,
-                                                                  const int* __restrict__ table, int table_stride, long page_stride,
-                                                                  int page_size, int n_heads, int n_kv, int window, float scale,
-                                                                  int n_splits, const int* __restrict__ tile_first, float* __restrict__ part) {
-    constexpr int NT = 64 * NW;                 // threads; the tile has 32 * NW query rows
+template <int HD, int NW, int PAIR>
+__global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
+                                                                          bf16_t* __restrict__ out, const int4* __restrict__ tiles,
+                                                                          const int* __restrict__ table, int table_stride, long page_stride,
+                                                                          int page_size, int n_heads, int n_kv, int window, float scale,
+                                                                          int n_splits, const int* __restrict__ tile_first, float* __restrict__ part) {
+    constexpr int NT = 128 * NW * PAIR;         // threads
     constexpr int K_STRIDE = HD + 8;            // bf16 elements; 16-byte reads of 32 rows hit distinct banks
     constexpr int V_STRIDE = KV_TILE + 4;       // 8-byte reads of 32 rows hit distinct banks
     constexpr int QSTEPS = HD / 16, DT = HD / 32;
-    constexpr int CHUNKS = KV_TILE * HD / 8 / NT;           // 16-byte pieces of the keys (and of the values) per thread and tile
-    static_assert(KV_TILE * HD / 8 % NT == 0, "the tile must divide among the threads");
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[KV_TILE * K_STRIDE];
-    __shared__ __attribute__((aligned(16))) bf16_t Vs[HD * V_STRIDE];
+    constexpr int K_PIECES = KV_TILE * HD / 8;              // 16-byte pieces of a tile of keys; the values have as many
+    constexpr int PP = (2 * K_PIECES + NT - 1) / NT;        // pieces per thread and tile
+    constexpr int K_BYTES = KV_TILE * K_STRIDE * 2, V_BYTES = HD * V_STRIDE * 2;
+    constexpr int MERGE_STRIDE = HD + 3;                    // floats per row in the final exchange: {m, l, O[HD]}, odd against bank conflicts
+    static_assert(NW * 32 * MERGE_STRIDE * 4 <= 2 * (K_BYTES + V_BYTES), "the final exchange of one row tile must fit in the key and value tiles' memory");
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * (K_BYTES + V_BYTES)];     // two tiles: one is read while the next is written
+    auto keys_of = [&](int b) { return reinterpret_cast<bf16_t*>(lds + b * (K_BYTES + V_BYTES)); };
+    auto values_of = [&](int b) { return reinterpret_cast<bf16_t*>(lds + b * (K_BYTES + V_BYTES) + K_BYTES); };
 
-    // With few tiles the keys of a tile are shared out over n_splits workgroups (grid x = tiles * splits); each writes
+    // With few tiles the keys are shared out over n_splits workgroups (grid x = groups of tiles * splits); each writes
     // an unnormalised partial result {m, l, O} per row, as the decode kernel's splits do, for the same combine kernel.
-    const int tile_index = gridDim.x / n_splits - 1 - blockIdx.x / n_splits, split = blockIdx.x % n_splits;
-    const int4 tile = tiles[tile_index];                     // later tiles of a prompt see more keys: they start first
-    const int row0 = tile.x, n_rows = tile.y, pos0 = tile.z, slot = tile.w;
-    const int head = blockIdx.y, g = head / (n_heads / n_kv);
+    const int group = gridDim.x / n_splits - 1 - blockIdx.x / n_splits, split = blockIdx.x % n_splits;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int ks = wave & 1;                                    // which half of every key tile
+    const int half = PAIR == 2 ? (wave >> 1) / NW : 0, wv = (wave >> 1) - half * NW;
+    const int4 tile_a = tiles[PAIR * group];
+    const int4 tile_b = PAIR == 2 ? tiles[PAIR * group + PAIR - 1] : int4{0, 0, 0, 0};
+    const int4 tile = half ? tile_b : tile_a;
+    const int row0 = tile.x, n_rows = tile.y, pos0 = tile.z, slot = tile_a.w;
+    const int head = blockIdx.y, g = head / (n_heads / n_kv);
     const int col = lane & 31, hf = lane >> 5;
     const int* tab = table + (size_t)slot * table_stride;
 
-    const int my_row = wave * 32 + col;                         // this lane's query row within the tile
+    const int my_row = wv * 32 + col;                           // this lane's query row within its tile
     const bool row_ok = my_row < n_rows;
     const int my_pos = row_ok ? pos0 + my_row : -1;
     const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
-    const int wave_last = pos0 + min(n_rows, wave * 32 + 32) - 1;       // the last position this wave's rows see
-    const bool wave_ok = wave * 32 < n_rows;
-    const bool wave_full = wave * 32 + 32 <= n_rows;
-    const int wave_first = wave_full ? pos0 + wave * 32 : -1;           // keys up to here are seen by every row of the wave (none if rows are missing)
+    const int wave_last = pos0 + min(n_rows, wv * 32 + 32) - 1;         // the last position this wave's rows see
+    const bool wave_ok = wv * 32 < n_rows;
+    const bool wave_full = wv * 32 + 32 <= n_rows;
+    const int wave_first = wave_full ? pos0 + wv * 32 : -1;             // keys up to here are seen by every row of the wave (none if rows are missing)
     const int wave_lo_max = window > 0 ? max(0, wave_last - window + 1) : 0;      // ... and keys from here on
+    const int wave_lo_min = window > 0 ? max(0, pos0 + wv * 32 - window + 1) : 0; // no row of the wave sees a key before this one
     const float scale2 = scale * LOG2E;
 
     bf16x8 qreg[QSTEPS];
@@ -81,83 +99,129 @@ __global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t*
     floatx16 o[DT];
 #pragma unroll
     for (int i = 0; i < DT; ++i) o[i] = floatx16{};
-    float m = -INFINITY, l = 0.f;
+    float m = -INFINITY, l = 0.f;               // l: this lane's share of the sum (its partner lane^32 holds the rest)
 
-    const int last_pos = pos0 + n_rows - 1;
-    const int first_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+    // the keys the workgroup walks: from the first one any of its rows sees to the last
+    auto lowest = [&](const int4 t) { return (window > 0 && t.z - window + 1 > 0) ? t.z - window + 1 : 0; };
+    int last_pos = tile_a.z + tile_a.y - 1, first_lo = lowest(tile_a);
+    if (PAIR == 2 && tile_b.y > 0) {
+        last_pos = max(last_pos, tile_b.z + tile_b.y - 1);
+        first_lo = min(first_lo, lowest(tile_b));
+    }
     const long v_plane = (long)n_kv * page_size * HD;
     // this workgroup's share of the key tiles [first_lo, last_pos]: whole tiles of 64, the same number for every split
     const int range_first = first_lo & ~(KV_TILE - 1);
     const int per_split = ((last_pos - range_first) / KV_TILE + n_splits) / n_splits * KV_TILE;
     const int kv_first = range_first + split * per_split, my_last = min(last_pos, kv_first + per_split - 1);
 
-    // A tile of 64 key positions travels global memory -> registers -> LDS; the next tile's loads are
-    // issued before the products of this one, and the page numbers they need one tile earlier still,
-    // so that neither the table lookup nor the load itself is waited for.
+    // A tile of 64 key positions travels global memory -> registers -> LDS in 16-byte pieces, keys first, then the
+    // values (stored transposed in the cache: HD rows of positions); a wave takes 64 consecutive pieces at a time.
+    // For head sizes 32, 64 and 128 those 64 pieces lie in one page (they cover 16, 8 or 4 key rows, or 64 value
+    // rows of 8 or 16 positions, and pages hold multiples of 16 positions): the page number, the place in the page
+    // and the address of the page are then the same for the whole wave and worked out by the scalar unit, and a lane
+    // only adds an offset that never changes.  Other head sizes look their pages up lane by lane.
+    constexpr bool ONE_PAGE = HD == 32 || HD == 64 || HD == 128;
     const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
     auto page_index = [&](int kv) { return page_shift >= 0 ? kv >> page_shift : kv / page_size; };
     auto place_of = [&](int kv) { return page_shift >= 0 ? kv & (page_size - 1) : kv % page_size; };
-    uint4 k_reg[CHUNKS], v_reg[CHUNKS];
-    int k_page[CHUNKS], v_page[CHUNKS];
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    __builtin_assume(wave_u >= 0 && wave_u < NT / 64);
+    int kv_off[PP], per_place[PP], in_lds[PP], page[PP];
+    unsigned in_page[PP];                       // elements from the start of the page's keys (or values) at place 0
+    bool has[PP], is_key[PP];
+    constexpr int DEPTH = PP == 1 ? 3 : 2;      // tiles on their way from the cache's memory, in registers (their number is paid in waves per compute unit)
+    uint4 reg[DEPTH][PP];
+#pragma unroll
+    for (int i = 0; i < PP; ++i) {
+        const int e0 = ONE_PAGE ? 64 * (wave_u + (NT / 64) * i) : tid + NT * i, e = ONE_PAGE ? e0 + lane : e0;      // e0: what the lookups go by
+        has[i] = e0 < 2 * K_PIECES;
+        is_key[i] = e0 < K_PIECES;
+        if (is_key[i]) {                                      // keys: 64 rows of HD
+            const int r = e / (HD / 8), c = (e % (HD / 8)) * 8, r0 = e0 / (HD / 8);
+            kv_off[i] = r0;
+            in_page[i] = g * page_size * HD + c + (r - r0) * HD;
+            per_place[i] = HD;
+            in_lds[i] = r * K_STRIDE + c;
+        } else {                                              // values: HD rows of 64 positions, 8 positions a piece
+            const int ev = e - K_PIECES, d = ev % HD, c = (ev / HD) * 8, c0 = ((e0 - K_PIECES) / HD) * 8;
+            kv_off[i] = c0;
+            in_page[i] = (g * HD + d) * page_size + (c - c0);
+            per_place[i] = 1;
+            in_lds[i] = d * V_STRIDE + c;
+        }
+    }
     auto fetch_pages = [&](int kv0) {
 #pragma unroll
-        for (int i = 0; i < CHUNKS; ++i) {
-            const int e = tid + NT * i;
-            const int kv_k = kv0 + e / (HD / 8), kv_v = kv0 + (e / HD) * 8;
-            k_page[i] = kv_k <= my_last ? tab[page_index(kv_k)] : -1;
-            v_page[i] = kv_v <= my_last ? tab[page_index(kv_v)] : -1;
+        for (int i = 0; i < PP; ++i) page[i] = (has[i] && kv0 + kv_off[i] <= my_last) ? tab[page_index(kv0 + kv_off[i])] : -1;
+    };
+    // Positions beyond the last one (or before a window) have no page (-1).  Their loads go to a page the request
+    // does hold instead of being skipped, so that every tile issues the same loads and the count of loads in flight
+    // is known where a tile's registers are waited for; what they bring is finite, and those keys are masked.
+    const int held_page = tab[page_index(max(my_last, 0))];
+    auto fetch = [&](int kv0, uint4* to) {      // with the pages that fetch_pages(kv0) brought
+#pragma unroll
+        for (int i = 0; i < PP; ++i) {
+            if (!has[i]) continue;
+            const int pg = page[i] >= 0 ? page[i] : held_page;
+            const bf16_t* at_place = cache + (long)pg * page_stride + (is_key[i] ? 0 : v_plane) + place_of(kv0 + kv_off[i]) * per_place[i];
+            to[i] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(at_place) + (size_t)(2u * in_page[i]));
         }
     };
-    auto fetch = [&](int kv0) {                 // with the pages that fetch_pages(kv0) brought
+    auto stash = [&](const uint4* from, bf16_t* Ks, bf16_t* Vs) {
 #pragma unroll
-        for (int i = 0; i < CHUNKS; ++i) {
-            const int e = tid + NT * i;
-            {   // keys: 64 rows of HD
-                const int r = e / (HD / 8), c = (e % (HD / 8)) * 8, kv = kv0 + r;
-                k_reg[i] = k_page[i] >= 0 ? load16(cache + (long)k_page[i] * page_stride + ((long)g * page_size + place_of(kv)) * HD + c) : uint4{0, 0, 0, 0};
+        for (int i = 0; i < PP; ++i) {
+            if (!has[i]) continue;
+            if (is_key[i]) {
+                *reinterpret_cast<uint4*>(&Ks[in_lds[i]]) = from[i];
+            } else {
+                uint2* dst = reinterpret_cast<uint2*>(&Vs[in_lds[i]]);
+                dst[0] = uint2{from[i].x, from[i].y};
+                dst[1] = uint2{from[i].z, from[i].w};
             }
-            {   // values, already transposed in the cache: HD rows of 64 positions, 8 positions a piece
-                const int d = e % HD, c = (e / HD) * 8, kv = kv0 + c;
-                v_reg[i] = v_page[i] >= 0 ? load16(cache + (long)v_page[i] * page_stride + v_plane + ((long)g * HD + d) * page_size + place_of(kv)) : uint4{0, 0, 0, 0};
-            }
-        }
-    };
-    auto stash = [&]() {
-#pragma unroll
-        for (int i = 0; i < CHUNKS; ++i) {
-            const int e = tid + NT * i;
-            *reinterpret_cast<uint4*>(&Ks[(e / (HD / 8)) * K_STRIDE + (e % (HD / 8)) * 8]) = k_reg[i];
-            uint2* dst = reinterpret_cast<uint2*>(&Vs[(e % HD) * V_STRIDE + (e / HD) * 8]);
-            dst[0] = uint2{v_reg[i].x, v_reg[i].y};
-            dst[1] = uint2{v_reg[i].z, v_reg[i].w};
         }
     };
 
+    // Tile t of the keys waits in LDS buffer t % 2 while the products of tile t - 1 run.  Its loads were issued
+    // DEPTH tiles earlier (the products of a tile take less time than a load that misses the cache) into register
+    // set t % DEPTH, and the page numbers they need one tile before that.  One barrier a tile: it orders this tile's
+    // reads before the write after next, and the next tile's write before its reads.
     fetch_pages(kv_first);
-    fetch(kv_first);
-    fetch_pages(kv_first + KV_TILE);            // beyond the last position: no lookups
-    for (int kv0 = kv_first; kv0 <= my_last; kv0 += KV_TILE) {
-        __syncthreads();                        // the previous tile has been read by everyone
-        stash();
-        __syncthreads();
-        if (kv0 + KV_TILE <= my_last) {
-            fetch(kv0 + KV_TILE);
-            fetch_pages(kv0 + 2 * KV_TILE);
-        }
-        if (!wave_ok) continue;
+    fetch(kv_first, reg[0]);
+    fetch_pages(kv_first + KV_TILE);            // beyond the last position: no lookups, and no loads then
+    stash(reg[0], keys_of(0), values_of(0));
+    // (the queries are named here so that their loads are waited for once, with the first tile's, and the waits
+    // inside the loop count the tiles' loads only)
 #pragma unroll
-        for (int st = 0; st < KV_TILE / 32; ++st) {
-            const int kv_base = kv0 + 32 * st;
-            if (kv_base > wave_last) break;                               // beyond every row of this wave
+    for (int k = 0; k < QSTEPS; ++k) asm volatile("" ::"v"(qreg[k]));
+#pragma unroll
+    for (int d = 1; d <= DEPTH; ++d) {
+        fetch(kv_first + d * KV_TILE, reg[d % DEPTH]);
+        fetch_pages(kv_first + (d + 1) * KV_TILE);
+    }
+    barrier_lds();
+    int buf = 0, kv0 = kv_first;
+    while (kv0 <= my_last) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d, kv0 += KV_TILE, buf ^= 1) {      // the tile in LDS is number d (mod DEPTH), the next one sits in set (d + 1) % DEPTH
+        if (kv0 > my_last) break;
+        // (also for the last tiles, where nothing more is to come: a tile without loads would leave the number of
+        // loads in flight unknown to the compiler, which then waits for all of them)
+        stash(reg[(d + 1) % DEPTH], keys_of(buf ^ 1), values_of(buf ^ 1));
+        fetch(kv0 + (1 + DEPTH) * KV_TILE, reg[(d + 1) % DEPTH]);
+        fetch_pages(kv0 + (2 + DEPTH) * KV_TILE);
+        const int kv_base = kv0 + 32 * ks;                              // this wave's half of the tile
+        if (wave_ok && kv_base <= wave_last && kv_base + 32 > wave_lo_min) {      // else: no row of this wave sees a key of it
+            const bf16_t* Ks = keys_of(buf);
+            const bf16_t* Vs = values_of(buf);
             floatx16 s = floatx16{};
 #pragma unroll
-            for (int ks = 0; ks < QSTEPS; ++ks) {
-                const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(&Ks[(32 * st + col) * K_STRIDE + 16 * ks + 8 * hf]));
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[ks], s, 0, 0, 0);
+            for (int k = 0; k < QSTEPS; ++k) {
+                const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(&Ks[(32 * ks + col) * K_STRIDE + 16 * k + 8 * hf]));
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[k], s, 0, 0, 0);
             }
             // element v of s: key position kv_base + 8*(v/4) + 4*hf + v%4, query row `col`.  Scores are kept
             // in units of log2 e (scale2 = scale * log2 e), so that e^(s - m) is one exp2.
-            const bool inside = kv_base + 31 <= wave_first && kv_base >= wave_lo_max;     // every key of the tile is seen by every row of the wave
+            const bool inside = kv_base + 31 <= wave_first && kv_base >= wave_lo_max;     // every key here is seen by every row of the wave
             float mx = -INFINITY;
             if (inside) {
 #pragma unroll
@@ -179,7 +243,6 @@ __global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t*
                 s[v] = exp2_fast(fmaf(s[v], scale2, -m_use));
                 sum += s[v];
             }
-            sum += __shfl_xor(sum, 32, 64);
             if (__any(m_new != m)) {                                      // some row's maximum rose: rescale what was gathered so far
                 const float corr = exp2_fast(m - m_use);
                 l *= corr;
@@ -194,19 +257,52 @@ __global__ __launch_bounds__(64 * NW) void attention_prompt_kernel(const bf16_t*
             for (int t = 0; t < 2; ++t) {                                 // two groups of 16 key positions
                 const uint4 pb = {pack2(s[8 * t], s[8 * t + 1]), pack2(s[8 * t + 2], s[8 * t + 3]), pack2(s[8 * t + 4], s[8 * t + 5]),
                                   pack2(s[8 * t + 6], s[8 * t + 7])};
-                // slot e of this lane is key position 32*st + 16*t + 8*(e/4) + 4*hf + e%4 of the tile
+                // slot e of this lane is key position 32*ks + 16*t + 8*(e/4) + 4*hf + e%4 of the tile
 #pragma unroll
                 for (int i = 0; i < DT; ++i) {
-                    const bf16_t* vrow = &Vs[(32 * i + col) * V_STRIDE + 32 * st + 16 * t + 4 * hf];
+                    const bf16_t* vrow = &Vs[(32 * i + col) * V_STRIDE + 32 * ks + 16 * t + 4 * hf];
                     const uint2 lo = *reinterpret_cast<const uint2*>(vrow), hi = *reinterpret_cast<const uint2*>(vrow + 8);
                     o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(uint4{lo.x, lo.y, hi.x, hi.y}), as_bf16x8(pb), o[i], 0, 0, 0);
                 }
             }
         }
+        barrier_lds();                          // not __syncthreads(): the loads of the tiles to come stay in flight
+      }
     }
-    if (!row_ok) return;
+    l += __shfl_xor(l, 32, 64);                                // both lanes of a row used the same maxima: their sums add up
+
+    // The two waves of 32 rows meet: the wave of the second key halves leaves {m, l, O} in LDS (the key tiles are
+    // done with), the other one adds it to its own and writes the rows out.  One row tile at a time.
+    float* xch = reinterpret_cast<float*>(lds) + (size_t)(wv * 32 + col) * MERGE_STRIDE;
+#pragma unroll
+    for (int pass = 0; pass < PAIR; ++pass) {
+        if (pass > 0) __syncthreads();
+        if (half == pass && ks == 1 && row_ok) {
+            if (hf == 0) {
+                xch[0] = m;
+                xch[1] = l;
+            }
+#pragma unroll
+            for (int i = 0; i < DT; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) xch[2 + 32 * i + 8 * (v / 4) + 4 * hf + (v & 3)] = o[i][v];
+        }
+        __syncthreads();
+        if (half == pass && ks == 0 && row_ok) {
+            const float m1 = xch[0], l1 = xch[1];
+            const float m_all = fmaxf(m, m1);
+            const float w0 = (m == -INFINITY) ? 0.f : exp2_fast(m - m_all), w1 = (m1 == -INFINITY) ? 0.f : exp2_fast(m1 - m_all);
+            l = l * w0 + l1 * w1;
+            m = m_all;
+#pragma unroll
+            for (int i = 0; i < DT; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o[i][v] = o[i][v] * w0 + xch[2 + 32 * i + 8 * (v / 4) + 4 * hf + (v & 3)] * w1;
+        }
+    }
+    if (!row_ok || ks != 0) return;
     if (n_splits > 1) {                                       // part[row of the split tiles][head][split] = {m, l, O[HD]}
-        float* dst = part + (((size_t)(tile_first[tile_index] + my_row) * n_heads + head) * n_splits + split) * (HD + 2);
+        float* dst = part + (((size_t)(tile_first[PAIR * group + half] + my_row) * n_heads + head) * n_splits + split) * (HD + 2);
         if (hf == 0) {
             dst[0] = m;
             dst[1] = l;
@@ -561,10 +657,12 @@ GI_API int gi_attention_bf16_supports(int hd, int page_size, int prompt) {
     return hd == 32 || hd == 64 || hd == 96 || hd == 128 || hd == 256;
 }
 
-// tiles hold at most `rows_per_tile` rows each (64 or 128).  n_splits > 1: every tile's keys are shared out over that
-// many workgroups; `tile_first[i]` is the number of rows in the tiles before tile i, `rows` lists the tiles' rows in
-// that order (n_rows of them), `part` has room for n_rows * n_heads * n_splits * (hd + 2) floats.
-GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out, const int* tiles, int n_tiles, int rows_per_tile,
+// tiles hold at most `rows_per_tile` rows each (64 or 128).  `paired` != 0: tiles 2w and 2w + 1 belong to one request
+// and share workgroup w (a late tile of a prompt beside an early one; a tile of 0 rows fills a pair).  n_splits > 1:
+// the keys of a workgroup's tiles are shared out over that many workgroups; `tile_first[i]` is the number of rows in
+// the tiles before tile i, `rows` lists the tiles' rows in that order (n_rows of them), `part` has room for
+// n_rows * n_heads * n_splits * (hd + 2) floats.
+GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out, const int* tiles, int n_tiles, int rows_per_tile, int paired,
                                     const int* table, int table_stride, long page_stride, int page_size, int n_heads, int n_kv, int hd,
                                     int window, float scale, int n_splits, const int* tile_first, const int* rows, int n_rows, float* part,
                                     long part_floats, hipStream_t stream) {
@@ -577,20 +675,23 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
     GI_REQUIRE(n_splits >= 1 && n_splits <= MAX_SPLITS, "attention_prompt: the number of splits %d is outside 1..%d", n_splits, MAX_SPLITS);
     GI_REQUIRE(n_splits == 1 || (tile_first && rows && part && n_rows > 0 && part_floats >= (long)n_rows * n_heads * n_splits * (hd + 2)),
                "attention_prompt: splitting needs the tiles' row offsets, their rows and scratch for the partial results");
-    dim3 grid(n_tiles * n_splits, n_heads);
+    GI_REQUIRE(!paired || n_tiles % 2 == 0, "attention_prompt: %d tiles cannot go in pairs", n_tiles);
+    // Two tiles share a workgroup of 1024 threads up to head size 64; larger heads need more registers than such a
+    // workgroup leaves a thread, and take the same list tile by tile (a filling tile of 0 rows then does nothing).
+    const bool pairs = paired && hd <= 64;
+    dim3 grid((pairs ? n_tiles / 2 : n_tiles) * n_splits, n_heads);
+#define GO_(HD, NW, PAIR)                                                                                                               \
+    attention_prompt_kernel<HD, NW, PAIR><<<grid, 128 * NW * PAIR, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, \
+                                                                                table, table_stride, page_stride, page_size, n_heads, n_kv, window, \
+                                                                                scale, n_splits, tile_first, part)
 #define GO(HD)                                                                                                                          \
     do {                                                                                                                                \
-        if (rows_per_tile == 64)                                                                                                        \
-            attention_prompt_kernel<HD, 2><<<grid, 128, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
-                                                                     table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits,  \
-                                                                     tile_first, part);                                                 \
-        else                                                                                                                            \
-            attention_prompt_kernel<HD, 4><<<grid, 256, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
-                                                                     table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits,  \
-                                                                     tile_first, part);                                                 \
+        if (rows_per_tile == 64) { if (pairs) GO_(HD, 2, (HD <= 64 ? 2 : 1)); else GO_(HD, 2, 1); }                                     \
+        else { if (pairs) GO_(HD, 4, (HD <= 64 ? 2 : 1)); else GO_(HD, 4, 1); }                                                         \
     } while (0)
     if (hd == 32) GO(32); else if (hd == 64) GO(64); else if (hd == 96) GO(96); else GO(128);
 #undef GO
+#undef GO_
     GI_CHECK_LAUNCH("attention_prompt");
     if (n_splits > 1) {
         dim3 cgrid(n_rows, n_heads);

@@ -44,6 +44,11 @@ __device__ __forceinline__ float load_f32(const bf16_t* p, size_t i) { return bf
 __device__ __forceinline__ void store_f32(float* p, size_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void store_f32(bf16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
 
+// A workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads() also waits for every load
+// from global memory the wave has in flight, which undoes a prefetch into registers; use this one where the
+// barrier orders LDS reads and writes and nothing else.
+__device__ __forceinline__ void barrier_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Butterfly reductions over the 64 lanes of a wave: every lane ends with the same value, and the
 // order of the additions is fixed by the lane numbers alone.
 __device__ __forceinline__ float wave_sum(float v) {

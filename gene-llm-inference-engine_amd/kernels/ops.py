@@ -31,7 +31,7 @@ _SIGNATURES = {
     "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
                            c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
-    "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
+    "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p],
     "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
@@ -276,6 +276,7 @@ class AttentionPlan:
     in all, the rows' repeated reading of the context costs more than the tiles' sequence).
     Made once per step and used by every layer."""
     TILE = int(__import__("os").environ.get("GI_ATTENTION_TILE", "128"))      # rows of a prompt tile: 64 or 128
+    PAIRS = True                         # a portion's late tiles share workgroups with its early ones
     SHORT, SHORT_TOTAL = 64, 64          # portions of up to SHORT rows count as short; they go row by row while they sum to at most SHORT_TOTAL
 
     @classmethod
@@ -285,11 +286,11 @@ class AttentionPlan:
         plan.n_decode, plan.n_tiles, plan.max_decode_context, plan.single_rows = n_rows, 0, max_context, True
         plan.decode_rows = None                                  # rows 0 .. n_rows-1
         plan.tiles = torch.empty(0, dtype=torch.int32, device=device)
-        plan.n_tile_rows, plan.max_tile_context, plan.tile_first, plan.tile_rows = 0, 0, None, None
+        plan.n_tile_rows, plan.max_tile_context, plan.tile_first, plan.tile_rows, plan.paired = 0, 0, None, None, False
         return plan
 
     def __init__(self, seg_start, seg_len, seg_pos0, seg_slot, device, to_device=None):
-        dec, tiles, self.max_decode_context = [], [], 0
+        dec, tiles, portions, self.max_decode_context = [], [], [], 0
         short_rows = sum(n for n in seg_len if 1 < n <= self.SHORT)
         row_by_row = self.SHORT if short_rows <= self.SHORT_TOTAL else 1
         self.single_rows = all(n == 1 for n in seg_len)          # every row is a request's only new row
@@ -298,8 +299,18 @@ class AttentionPlan:
                 dec.extend(range(start, start + n))
                 self.max_decode_context = max(self.max_decode_context, pos0 + n)
             else:
-                for off in range(0, n, self.TILE):
-                    tiles.append((start + off, min(self.TILE, n - off), pos0 + off, slot))
+                portions.append([(start + off, min(self.TILE, n - off), pos0 + off, slot) for off in range(0, n, self.TILE)])
+        # Tile i of a portion sees the keys of the tiles before it: the last tile goes with the first, the last but
+        # one with the second, ... so that every pair has about the same number of keys to visit and reads them once
+        # for both (a tile of no rows fills the middle pair of an odd number).  Without a portion of two tiles, no pairs.
+        self.paired = self.PAIRS and any(len(p) > 1 for p in portions)
+        for p in portions:
+            if not self.paired:
+                tiles.extend(p)
+                continue
+            for i in range((len(p) + 1) // 2):
+                late, early = p[len(p) - 1 - i], p[i]
+                tiles.extend((late, early if early is not late else (late[0], 0, late[2], late[3])))
         self.n_decode, self.n_tiles = len(dec), len(tiles)
         self.n_tile_rows = sum(t[1] for t in tiles)
         self.max_tile_context = max((t[2] + t[1] for t in tiles), default=0)
@@ -320,10 +331,10 @@ def attention_bf16_supports(hd, page_size, prompt: bool) -> bool:
     return bool(lib().gi_attention_bf16_supports(hd, page_size, 1 if prompt else 0))
 
 
-def prompt_attention_splits(n_tiles, n_heads, span, target_groups=512):
-    """Workgroups a tile's keys are shared out over: none while the tiles alone fill the chip (two workgroups a
-    compute unit) or the context is short; every share keeps at least 256 keys."""
-    groups = n_tiles * n_heads
+def prompt_attention_splits(n_groups, n_heads, span, target_groups=512):
+    """Workgroups the keys of a tile (or pair of tiles) are shared out over: none while the tiles alone fill the chip
+    (two workgroups a compute unit) or the context is short; every share keeps at least 256 keys."""
+    groups = n_groups * n_heads
     if groups >= target_groups // 2:
         return 1
     return max(1, min(-(-target_groups // groups), span // 256, 64))
@@ -379,11 +390,13 @@ def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, 
             if not (t is None or (t.dtype == torch.float32 and t.shape == (n, hd // 2) and t.is_contiguous())):
                 raise KernelError("attention: cos/sin must be float32 [n, hd/2]")
     if plan.n_tiles:
-        n_splits = prompt_attention_splits(plan.n_tiles, n_heads, plan.max_tile_context if not window else min(plan.max_tile_context, window + plan.TILE))
+        n_splits = prompt_attention_splits(plan.n_tiles // 2 if plan.paired else plan.n_tiles, n_heads,
+                                           plan.max_tile_context if not window else min(plan.max_tile_context, window + plan.TILE),
+                                           target_groups=256 if plan.paired else 512)      # a pair's workgroup has twice the waves
         n_part = plan.n_tile_rows * n_heads * n_splits * (hd + 2) if n_splits > 1 else 0
         part = torch.empty(n_part, dtype=torch.float32, device=out.device) if n_part else None
         _call("gi_attention_prompt_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles, plan.TILE,
-              table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits,
+              1 if plan.paired else 0, table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits,
               _ptr(plan.tile_first), _ptr(plan.tile_rows), plan.n_tile_rows, _ptr(part), n_part, _stream())
     if plan.n_decode:
         span = plan.max_decode_context if not window else min(plan.max_decode_context, window + 31)

@@ -85,3 +85,30 @@ def test_gi_serve_bench_usage_errors():
                       (["--model", "x", "--max-seq-len", "8"], "--max-seq-len is shorter"), (["--model", "x", "--what"], "unknown option --what")):
         r = subprocess.run([exe, *args], capture_output=True, text=True, timeout=60)
         assert r.returncode == 2 and msg in r.stderr and "usage: gi_serve_bench" in r.stderr
+
+
+@pytest.mark.gpu
+def test_gi_bench_reports_one_request(tmp_path):
+    write_model(tmp_path / "m", CONFIGS["A"], seed=2)
+    report = tmp_path / "report.json"
+    r = subprocess.run([str(ROOT / "bin" / "gi_bench"), "--model", str(tmp_path / "m"), "--prompt-tokens", "20", "--decode-tokens", "9", "--runs", "2",
+                        "--label", "tiny", "--json", str(report), "--block-size", "4"], capture_output=True, text=True, timeout=170)
+    assert r.returncode == 0, r.stderr
+    assert "workload: 20 prompt + 9 decode positions, 2 measured runs (+1 warmup)" in r.stdout and "| tiny |" in r.stdout
+    j = json.loads(report.read_text())
+    assert j["prompt_tokens"] == 20 and j["decode_tokens"] == 9 and j["label"] == "tiny" and j["bf16_weights"] is True
+    assert j["prefill_tokens_per_s"] > 0 and j["decode_ms_min"] <= j["decode_ms_median"] <= j["decode_ms_p95"] <= j["decode_ms_max"]
+    cfg = CONFIGS["A"]
+    kv_dim = cfg["num_key_value_heads"] * (cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_attention_heads"])
+    assert j["cache_bytes_per_token"] == cfg["num_hidden_layers"] * 2 * kv_dim * 2 * (20 + 9 // 2)
+    clamped = subprocess.run([str(ROOT / "bin" / "gi_bench"), "--model", str(tmp_path / "m"), "--prompt-tokens", "500", "--decode-tokens", "40", "--runs", "1",
+                              "--max-seq-len", "32", "--weights", "f32", "--sequential-prefill"], capture_output=True, text=True, timeout=170)
+    assert clamped.returncode == 0 and "workload: 31 prompt + 1 decode positions" in clamped.stdout, clamped.stdout + clamped.stderr
+
+
+def test_gi_bench_usage_errors():
+    exe = str(ROOT / "bin" / "gi_bench")
+    for args, msg in (([], "--model is required"), (["--model", "x", "--runs", "0"], "must be positive"),
+                      (["--model", "x", "--weights", "int8"], "--weights must be native or f32"), (["--model", "x", "--isa", "avx2"], "unknown option --isa")):
+        r = subprocess.run([exe, *args], capture_output=True, text=True, timeout=60)
+        assert r.returncode == 2 and msg in r.stderr and "usage: gi_bench" in r.stderr

@@ -227,6 +227,8 @@ SEGMENTS = {
     "short portions": [(0, 250, 50), (1, 130, 1), (2, 0, 1), (3, 70, 7), (4, 527, 3)],
     # short portions that sum to more than 64 rows stay tiles
     "many short portions": [(0, 240, 60), (1, 130, 1), (3, 47, 30), (4, 490, 40)],
+    # portions of several tiles: a late tile shares its workgroup with an early one (3 tiles: the middle one alone; 4: two pairs)
+    "several tiles": [(0, 0, 300), (1, 130, 1), (4, 100, 430)],
 }
 
 
