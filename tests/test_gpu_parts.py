@@ -145,6 +145,10 @@ def toy_model(tmp_path_factory):
     _, weights = read_model_folder(folder)
     rng = random.Random(4)
     requests = {f"t{i}": [rng.randrange(cfg.vocab_size) for _ in range(n)] for i, n in enumerate([40, 9, 63, 21, 34])}
+    # the routed feed-forward is exercised: every expert is some row's choice, and no choice hangs on the last digits
+    top2 = torch.cat([torch.topk(toy.router_logits(cfg, weights, toks), 2, dim=-1).values for toks in requests.values()])
+    chosen = torch.cat([toy.router_logits(cfg, weights, toks).argmax(-1) for toks in requests.values()])
+    assert set(chosen.tolist()) == set(range(cfg.num_experts)) and float((top2[:, 0] - top2[:, 1]).min()) > 1e-4
     return cfg, folder, weights, requests
 
 
@@ -160,8 +164,8 @@ def test_toy_architecture_under_every_cut(toy_model, dtype, mode):
              "mixed": lambda r: traces.mixed(r, seed=8)}[mode](requests)
     runner = Runner(model, page_size=16 if dtype == "bfloat16" else 4, max_tokens=traces.peak_tokens(steps, 16), max_requests=4)
     groups = runner.cache.groups
-    assert [(g.need.window, g.entries) for g in groups] == [(None, [0, 3]), (cfg.window, [1])]      # entry 4 reads entry 1's pages
-    assert list(runner.cache.states) == [2] and runner.cache.state(2).shape == (4, cfg.hidden_size)
+    assert [(g.need.window, g.entries) for g in groups] == [(None, [1, 4]), (cfg.window, [2])]      # entry 5 reads entry 2's pages
+    assert list(runner.cache.states) == [0, 3] and runner.cache.state(3).shape == (4, cfg.hidden_size)      # both decay mixers
     where, got = traces.wanted_positions(steps), {}
     for s in steps:
         for e in s["entries"]:

@@ -2,9 +2,15 @@
 needs are data: it is registered, built, loaded and stepped through the framework's public
 interfaces without a change to the framework's files.
 
-Layers: 0 full attention, 1 windowed attention, 2 a "decay" mixer with a state of its own
-(s <- decay * s + h per row, out = W s), each followed by SwiGLU.  Run order: 0, 1, 2, then layer
-0 once more (a cache of its own) and layer 1 once more reading the pages of its first run.
+Layers: 0 full attention whose positions are encoded by a toy rule of its own (angles
+pos * step * (k + 1) instead of the rotary frequencies), 1 windowed attention, 2 a "decay" mixer
+with a state of its own (s <- decay * s + h per row, out = W s), each followed by SwiGLU; 3 a
+second decay mixer followed by a feed-forward with routing (a router picks one of three small
+SwiGLU experts per row and scales it by the router's probability of it).  Run order: 3, 0, 1, 2,
+then layer 0 once more (a cache of its own) and layer 1 once more reading the pages of its first
+run.  Layer 3 runs first so that the router sees values computed in 32-bit on both sides of the
+comparison (embedding, norm, decay mixer): in bfloat16 the engine and the plain model then take
+the same expert unless two router logits agree to six digits.
 """
 from __future__ import annotations
 
@@ -16,7 +22,7 @@ import torch
 from geneinfer_amd.cache import StateNeed
 from geneinfer_amd.config import (AttentionSpec, LayerSpec, ModelSpec, RmsNormSpec, RotarySpec, RunEntry, SwiGluSpec,
                                   register_architecture)
-from geneinfer_amd.parts import Mixer, register_mixer
+from geneinfer_amd.parts import FeedForward, Mixer, PositionEncoding, register_feed_forward, register_mixer, register_position_encoding
 from geneinfer_amd.weights import TensorNeed
 from plain_llama import causal_attention, rms_norm, rope_inverse_frequencies, rope_rotate, swiglu
 
@@ -56,6 +62,66 @@ class DecayMixer(Mixer):
 
 
 @dataclass(frozen=True)
+class LinearAnglesSpec:
+    kind: ClassVar[str] = "toy_linear_angles"
+    head_dim: int
+    step: float
+
+
+class LinearAngles(PositionEncoding):
+    """Pair k of a head is turned by pos * step * (k + 1).  What an attention part asks of a position
+    encoding is `prepare(ctx) -> (cos, sin)`, float32 [rows, head_dim / 2]."""
+
+    def prepare(self, ctx):
+        key = ("toy_linear_angles", self.spec)
+        if key not in ctx.memo:
+            k = torch.arange(1, self.spec.head_dim // 2 + 1, dtype=torch.float64, device=ctx.device)
+            angles = ctx.row_pos.double()[:, None] * (self.spec.step * k)[None, :]
+            ctx.memo[key] = (torch.cos(angles).float().contiguous(), torch.sin(angles).float().contiguous())
+        return ctx.memo[key]
+
+
+@dataclass(frozen=True)
+class RoutedSpec:
+    kind: ClassVar[str] = "toy_routed"
+    hidden_size: int
+    intermediate_size: int
+    n_experts: int
+    prefix: str                       # tensors: prefix + "router", prefix + "e{i}.gate" / ".up" / ".down"
+
+
+class RoutedFeedForward(FeedForward):
+    """Per row: the expert with the largest router logit (the lowest index among equals), scaled by its softmax
+    probability.  Everything in 32-bit."""
+
+    def __init__(self, spec, tensors, dtype, device):
+        super().__init__(spec, tensors, dtype, device)
+        self.router = tensors[spec.prefix + "router"].float()
+        self.experts = [tuple(tensors[f"{spec.prefix}e{i}.{n}"].float() for n in ("gate", "up", "down")) for i in range(spec.n_experts)]
+        self.in_dtype = torch.float32
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        d, inter = spec.hidden_size, spec.intermediate_size
+        needs = [TensorNeed(spec.prefix + "router", (spec.n_experts, d))]
+        for i in range(spec.n_experts):
+            needs += [TensorNeed(f"{spec.prefix}e{i}.gate", (inter, d)), TensorNeed(f"{spec.prefix}e{i}.up", (inter, d)),
+                      TensorNeed(f"{spec.prefix}e{i}.down", (d, inter))]
+        return needs
+
+    def forward(self, h, residual, ctx):
+        h = h.float()
+        logits = h @ self.router.T
+        chosen = torch.argmax(logits, dim=-1)                 # the first of equal maxima
+        share = torch.softmax(logits, dim=-1).gather(1, chosen[:, None])
+        for i, (gate, up, down) in enumerate(self.experts):
+            rows = torch.nonzero(chosen == i).flatten()
+            if rows.numel():
+                x = h[rows]
+                residual[rows] += share[rows] * ((torch.nn.functional.silu(x @ gate.T) * (x @ up.T)) @ down.T)
+
+
+@dataclass(frozen=True)
 class ToyConfig:
     hidden_size: int = 48
     intermediate_size: int = 80
@@ -65,6 +131,9 @@ class ToyConfig:
     vocab_size: int = 200
     window: int = 6
     decay: float = 0.7
+    angle_step: float = 0.05
+    num_experts: int = 3
+    expert_intermediate_size: int = 24
     rms_norm_eps: float = 1e-5
     rope_theta: float = 10000.0
     max_position_embeddings: int = 256
@@ -80,16 +149,19 @@ class ToyConfig:
 
     def model_spec(self) -> ModelSpec:
         d, rot = self.hidden_size, RotarySpec(self.head_dim, self.rope_theta, None)
-        def attention(l, window):
+        def attention(l, window, position):
             p = f"layers.{l}.attn."
             return AttentionSpec(d, self.num_attention_heads, self.num_key_value_heads, self.head_dim, p + "q", p + "k", p + "v", p + "o",
-                                 position=rot, window=window)
-        def rest(l, mixer):
+                                 position=position, window=window)
+        def rest(l, mixer, feed_forward=None):
             p = f"layers.{l}."
-            return LayerSpec(mixer=mixer, feed_forward=SwiGluSpec(d, self.intermediate_size, p + "ff.gate", p + "ff.up", p + "ff.down"),
+            feed_forward = feed_forward or SwiGluSpec(d, self.intermediate_size, p + "ff.gate", p + "ff.up", p + "ff.down")
+            return LayerSpec(mixer=mixer, feed_forward=feed_forward,
                              mixer_norm=RmsNormSpec(d, self.rms_norm_eps, p + "norm1"), feed_forward_norm=RmsNormSpec(d, self.rms_norm_eps, p + "norm2"))
-        layers = (rest(0, attention(0, None)), rest(1, attention(1, self.window)), rest(2, DecaySpec(d, self.decay, "layers.2.decay.w")))
-        order = (RunEntry(0), RunEntry(1), RunEntry(2), RunEntry(0), RunEntry(1, cache_of=1))
+        layers = (rest(0, attention(0, None, LinearAnglesSpec(self.head_dim, self.angle_step))), rest(1, attention(1, self.window, rot)),
+                  rest(2, DecaySpec(d, self.decay, "layers.2.decay.w")),
+                  rest(3, DecaySpec(d, self.decay, "layers.3.decay.w"), RoutedSpec(d, self.expert_intermediate_size, self.num_experts, "layers.3.moe.")))
+        order = (RunEntry(3), RunEntry(0), RunEntry(1), RunEntry(2), RunEntry(0), RunEntry(1, cache_of=2))
         return ModelSpec(architecture=self.architecture, vocab_size=self.vocab_size, hidden_size=d, max_positions=self.max_position_embeddings,
                          embedding="embed", final_norm=RmsNormSpec(d, self.rms_norm_eps, "final_norm"), lm_head="head", layers=layers,
                          run_order=order)
@@ -98,7 +170,22 @@ class ToyConfig:
 def register():
     """Idempotent: the registries refuse a second class under a name, not the same class again."""
     register_mixer("toy_decay", DecayMixer)
+    register_feed_forward("toy_routed", RoutedFeedForward)
+    register_position_encoding("toy_linear_angles", LinearAngles)
     register_architecture(ToyConfig.architecture, ToyConfig, model_type="toy_mixed")
+
+
+def router_logits(cfg: ToyConfig, w: dict, tokens, dtype=torch.float64):
+    """What the router of layer 3 (the first to run) sees for a whole sequence, from the plain parts."""
+    w = {k: v.to(dtype) for k, v in w.items()}
+    x = w["embed"][torch.tensor(tokens)]
+    xb = rms_norm(x, w["layers.3.norm1"], cfg.rms_norm_eps)
+    s, outs = torch.zeros(cfg.hidden_size, dtype=dtype), []
+    for t in range(len(tokens)):
+        s = cfg.decay * s + xb[t]
+        outs.append(w["layers.3.decay.w"] @ s)
+    x = x + torch.stack(outs)
+    return rms_norm(x, w["layers.3.norm2"], cfg.rms_norm_eps) @ w["layers.3.moe.router"].T
 
 
 def plain_logits(cfg: ToyConfig, w: dict, tokens, dtype=torch.float64, store=lambda t: t):
@@ -106,20 +193,21 @@ def plain_logits(cfg: ToyConfig, w: dict, tokens, dtype=torch.float64, store=lam
     w = {k: v.to(dtype) for k, v in w.items()}
     T, H, KV, hd = len(tokens), cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     pos = torch.arange(T)
-    inv = rope_inverse_frequencies(hd, cfg.rope_theta)
+    inv_of = {0: cfg.angle_step * torch.arange(1, hd // 2 + 1, dtype=torch.float64), 1: rope_inverse_frequencies(hd, cfg.rope_theta)}
     x = w["embed"][torch.tensor(tokens)]
     spec = cfg.model_spec()
     kept = {}
     for i, entry in enumerate(spec.run_order):
         l, p = entry.layer, f"layers.{entry.layer}."
         xb = rms_norm(x, w[p + "norm1"], cfg.rms_norm_eps)
-        if l == 2:
+        if l >= 2:
             s, outs = torch.zeros(cfg.hidden_size, dtype=dtype), []
             for t in range(T):
                 s = cfg.decay * s + xb[t]
-                outs.append(w["layers.2.decay.w"] @ s)
+                outs.append(w[p + "decay.w"] @ s)
             x = x + torch.stack(outs)
         else:
+            inv = inv_of[l]
             xb = store(xb)
             q = store(rope_rotate((xb @ w[p + "attn.q"].T).reshape(T, H, hd), pos, inv))
             if entry.cache_of is None:
@@ -130,6 +218,14 @@ def plain_logits(cfg: ToyConfig, w: dict, tokens, dtype=torch.float64, store=lam
                 k, v = kept[entry.cache_of]
             att = store(causal_attention(q, k, v, cfg.window if l == 1 else None)).reshape(T, H * hd)
             x = x + att @ w[p + "attn.o"].T
+        if l == 3:                                            # the routed feed-forward: one expert per row, in 32-bit on the device
+            xb = rms_norm(x, w[p + "norm2"], cfg.rms_norm_eps)
+            logits = xb @ w[p + "moe.router"].T
+            for t in range(T):
+                e = int(torch.argmax(logits[t]))
+                share = torch.softmax(logits[t], dim=-1)[e]
+                x[t] = x[t] + share * swiglu(xb[t:t + 1], w[f"{p}moe.e{e}.gate"], w[f"{p}moe.e{e}.up"], w[f"{p}moe.e{e}.down"], lambda v: v)[0]
+            continue
         xb = store(rms_norm(x, w[p + "norm2"], cfg.rms_norm_eps))
         x = x + swiglu(xb, w[p + "ff.gate"], w[p + "ff.up"], w[p + "ff.down"], store)
     return store(rms_norm(x, w["final_norm"], cfg.rms_norm_eps)) @ w["head"].T
