@@ -33,6 +33,7 @@ class DecoderModel:
         self.final_norm = norm_class(spec.final_norm)(spec.final_norm, tensors, dtype, device)
         self.head_in_dtype = activation_dtype_for(self.lm_head, dtype)
         self.run_order = spec.run_order
+        self.trace = None                        # see set_trace
         self.graph_safe = all(getattr(l, "graph_safe", False) for l in self.layers) and getattr(self.final_norm, "graph_safe", False)
 
     # ----------------------------------------------------------------------------- what it needs
@@ -58,8 +59,13 @@ class DecoderModel:
         [n_logit_rows, vocab] of the rows listed in `logit_rows`, or None if there are none."""
         x = torch.empty((ctx.n_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device)
         ops.embed(self.embedding, ctx.tokens, x)
+        trace = self.trace
+        if trace is not None:
+            trace("embedding", -1, x)
         for i, entry in enumerate(self.run_order):
+            ctx.trace = None if trace is None else (lambda tag, rows, i=i: trace(tag, i, rows))
             self.layers[entry.layer].forward(x, ctx, cache.layer_cache(i))
+        ctx.trace = None
         if n_logit_rows == 0:
             return None
         logits = torch.empty((n_logit_rows, self.spec.vocab_size), dtype=torch.float32, device=self.device)
@@ -68,8 +74,18 @@ class DecoderModel:
         else:
             picked = torch.empty((n_logit_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device)
             normed = self.final_norm(ops.gather_rows(x, logit_rows, picked), self.head_in_dtype)
+        if trace is not None:
+            trace("final_norm", -1, normed if torch.is_tensor(normed) else self.final_norm(ops.gather_rows(x, logit_rows, torch.empty(
+                (n_logit_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device)), torch.float32))
         linear(normed, self.lm_head, logits)
         return logits
+
+    def set_trace(self, trace) -> None:
+        """Debugging, as the reference's Model::set_trace (src/model/model.h): `trace(tag, run-order entry or -1, rows)` is
+        called with the step's residual stream after the embedding ("embedding"), after each half of every block
+        ("attn_out", "ffn_out") and with the normed rows that the logits are taken from ("final_norm").  While a trace is
+        set no step is replayed from a captured graph."""
+        self.trace = trace
 
 
 def load_model(folder, dtype="bfloat16", device="cuda:0") -> DecoderModel:

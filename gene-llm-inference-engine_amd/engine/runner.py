@@ -126,7 +126,7 @@ class Runner:
         """Runs the batch; returns float32 logits [wanted, vocab] on the device in the order of the
         entries and of each entry's `want`, or None if nothing was wanted.  The tensor is valid
         until the next step."""
-        if self.use_graphs and all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries) and entries:
+        if self.use_graphs and self.model.trace is None and all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries) and entries:
             return self._step_of_single_tokens(entries)
         n_rows = self._validate(entries)
         self.cache.reserve([(e.request, len(e.tokens)) for e in entries])       # OutOfPages: nothing changed

@@ -44,6 +44,7 @@ class StepContext:
     seg_pos0: List[int]                      # position of the first row
     memo: Dict[Any, Any] = field(default_factory=dict)     # per-step tables shared by layers (rotary cos/sin)
     upload: Optional[Callable[[np.ndarray], torch.Tensor]] = None      # the runner's way of bringing int32 step data to the device
+    trace: Optional[Callable[[str, torch.Tensor], None]] = None        # debugging: a block reports (tag, residual stream [T, hidden]) after each of its two halves
 
     def to_device(self, values) -> torch.Tensor:
         """int32 data made on the host for this step (row lists, tile lists) as a device tensor, valid during the step."""

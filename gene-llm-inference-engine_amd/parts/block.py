@@ -40,7 +40,11 @@ class PreNormBlock:
 
     def forward(self, x, ctx, cache):
         self.mixer.forward(self._normed(self.mixer_norm, self.mixer, x, ctx), x, ctx, cache)
+        if ctx.trace is not None:
+            ctx.trace("attn_out", x)
         self.feed_forward.forward(self._normed(self.feed_forward_norm, self.feed_forward, x, ctx), x, ctx)
+        if ctx.trace is not None:
+            ctx.trace("ffn_out", x)
 
 
 register_block("prenorm", PreNormBlock)

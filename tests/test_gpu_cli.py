@@ -112,3 +112,48 @@ def test_gi_bench_usage_errors():
                       (["--model", "x", "--weights", "int8"], "--weights must be native or f32"), (["--model", "x", "--isa", "avx2"], "unknown option --isa")):
         r = subprocess.run([exe, *args], capture_output=True, text=True, timeout=60)
         assert r.returncode == 2 and msg in r.stderr and "usage: gi_bench" in r.stderr
+
+
+@pytest.mark.gpu
+def test_gi_forward_dumps_logits_and_the_last_position_layer_by_layer(tmp_path):
+    import numpy as np
+    from plain_llama import read_model_folder
+    name = "B"
+    write_model(tmp_path / "m", CONFIGS[name], seed=6)
+    cfg, vocab, hidden = CONFIGS[name], CONFIGS[name]["vocab_size"], CONFIGS[name]["hidden_size"]
+    tokens = [3, 14, 15, 92, 65, 35, 89, 79, 32, 38, 46, 26, 43, 38, 32, 79, 50, 28, 84, 19]
+    exe = str(ROOT / "bin" / "gi_forward")
+    ids = [str(t) for t in tokens]
+    r = subprocess.run([exe, str(tmp_path / "m"), str(tmp_path / "one"), "--weights", "f32", "--block-size", "4", *ids], capture_output=True, text=True, timeout=170)
+    assert r.returncode == 0 and f"positions={len(tokens)} vocab={vocab} avg_ms_per_token=" in r.stdout, r.stdout + r.stderr
+    logits = torch.from_numpy(np.fromfile(tmp_path / "one" / "logits.f32", dtype="<f4")).reshape(len(tokens), vocab)
+    want = PlainLlama(tmp_path / "m").logits(tokens)
+    assert float((logits.double() - want).abs().max() / want.abs().max()) < 2e-5
+    _, weights = read_model_folder(tmp_path / "m")
+    embedding = torch.from_numpy(np.fromfile(tmp_path / "one" / "embedding.f32", dtype="<f4"))
+    assert torch.equal(embedding, weights["model.embed_tokens.weight"][tokens[-1]].float())       # of the last position
+    files = sorted(p.name for p in (tmp_path / "one").glob("layer*.f32"))
+    assert files == sorted(f"layer{i:02d}_{tag}.f32" for i in range(cfg["num_hidden_layers"]) for tag in ("attn_out", "ffn_out"))
+    assert all((tmp_path / "one" / f).stat().st_size == 4 * hidden for f in files)
+    final = torch.from_numpy(np.fromfile(tmp_path / "one" / "final_norm.f32", dtype="<f4"))
+    head = weights.get("lm_head.weight", weights["model.embed_tokens.weight"]).float()
+    assert float((head @ final - logits[-1]).abs().max() / logits[-1].abs().max()) < 1e-5            # what the logits are taken from
+    # a portion on top of single tokens, cut by --max-batch, after a decoy sequence that is rewound: the same rows, bit for bit
+    r = subprocess.run([exe, str(tmp_path / "m"), str(tmp_path / "two"), "--weights", "f32", "--block-size", "4", "--prefill", "12", "--head", "5",
+                        "--max-batch", "4", "--decoy", *ids], capture_output=True, text=True, timeout=170)
+    assert r.returncode == 0, r.stderr
+    rows = torch.from_numpy(np.fromfile(tmp_path / "two" / "logits.f32", dtype="<f4")).reshape(-1, vocab)
+    assert rows.shape[0] == len(tokens) - 11 and torch.equal(rows, logits[11:])
+    assert not list((tmp_path / "two").glob("layer*.f32")) and not (tmp_path / "two" / "embedding.f32").exists()
+    native = subprocess.run([exe, str(tmp_path / "m"), str(tmp_path / "three"), "--prefill", "20", *ids], capture_output=True, text=True, timeout=170)
+    assert native.returncode == 0 and (tmp_path / "three" / "logits.f32").stat().st_size == 4 * vocab
+
+
+def test_gi_forward_usage_and_errors(tmp_path):
+    exe = str(ROOT / "bin" / "gi_forward")
+    r = subprocess.run([exe, "x"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 2 and "usage: gi_forward" in r.stderr
+    for args, msg in ((["x", str(tmp_path / "o")], "no token ids given"), (["x", str(tmp_path / "o"), "--prefill", "3", "--head", "3", "1", "2", "3"], "--head must be smaller"),
+                      (["x", str(tmp_path / "o"), "--prefill", "9", "1", "2"], "--prefill must be between"), (["x", str(tmp_path / "o"), "--prefill"], "--prefill needs a value")):
+        r = subprocess.run([exe, *args, *([] if "1" in args or "--prefill" == args[-1] else ["--max-seq-len", "8"])], capture_output=True, text=True, timeout=60)
+        assert r.returncode == 1 and msg in r.stderr, r.stderr
