@@ -275,7 +275,8 @@ class AttentionPlan:
     for the whole chip (break-even near 90 rows at the Llama-3.2-1B shape; above SHORT_TOTAL rows
     in all, the rows' repeated reading of the context costs more than the tiles' sequence).
     Made once per step and used by every layer."""
-    TILE = int(__import__("os").environ.get("GI_ATTENTION_TILE", "128"))      # rows of a prompt tile: 64 or 128
+    TILE = int(__import__("os").environ.get("GI_ATTENTION_TILE", "0"))        # rows of a prompt tile, 64 or 128; 0: by the step's size
+    SMALL_STEP = 768                     # up to this many tiled rows in a step, tiles of 64 rows fill the chip better (measured at 32 heads)
     PAIRS = True                         # a portion's late tiles share workgroups with its early ones
     SHORT, SHORT_TOTAL = 64, 64          # portions of up to SHORT rows count as short; they go row by row while they sum to at most SHORT_TOTAL
 
@@ -286,7 +287,7 @@ class AttentionPlan:
         plan.n_decode, plan.n_tiles, plan.max_decode_context, plan.single_rows = n_rows, 0, max_context, True
         plan.decode_rows = None                                  # rows 0 .. n_rows-1
         plan.tiles = torch.empty(0, dtype=torch.int32, device=device)
-        plan.n_tile_rows, plan.max_tile_context, plan.tile_first, plan.tile_rows, plan.paired = 0, 0, None, None, False
+        plan.n_tile_rows, plan.max_tile_context, plan.tile_first, plan.tile_rows, plan.paired, plan.tile = 0, 0, None, None, False, 128
         return plan
 
     def __init__(self, seg_start, seg_len, seg_pos0, seg_slot, device, to_device=None):
@@ -294,12 +295,13 @@ class AttentionPlan:
         short_rows = sum(n for n in seg_len if 1 < n <= self.SHORT)
         row_by_row = self.SHORT if short_rows <= self.SHORT_TOTAL else 1
         self.single_rows = all(n == 1 for n in seg_len)          # every row is a request's only new row
+        self.tile = self.TILE or (64 if sum(n for n in seg_len if n > row_by_row) <= self.SMALL_STEP else 128)
         for start, n, pos0, slot in zip(seg_start, seg_len, seg_pos0, seg_slot):
             if n <= row_by_row:
                 dec.extend(range(start, start + n))
                 self.max_decode_context = max(self.max_decode_context, pos0 + n)
             else:
-                portions.append([(start + off, min(self.TILE, n - off), pos0 + off, slot) for off in range(0, n, self.TILE)])
+                portions.append([(start + off, min(self.tile, n - off), pos0 + off, slot) for off in range(0, n, self.tile)])
         # Tile i of a portion sees the keys of the tiles before it: the last tile goes with the first, the last but
         # one with the second, ... so that every pair has about the same number of keys to visit and reads them once
         # for both (a tile of no rows fills the middle pair of an odd number).  Without a portion of two tiles, no pairs.
@@ -329,6 +331,9 @@ class AttentionPlan:
 
 def attention_bf16_supports(hd, page_size, prompt: bool) -> bool:
     return bool(lib().gi_attention_bf16_supports(hd, page_size, 1 if prompt else 0))
+
+
+PAIRED_TARGET_GROUPS = 256
 
 
 def prompt_attention_splits(n_groups, n_heads, span, target_groups=512):
@@ -391,11 +396,11 @@ def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, 
                 raise KernelError("attention: cos/sin must be float32 [n, hd/2]")
     if plan.n_tiles:
         n_splits = prompt_attention_splits(plan.n_tiles // 2 if plan.paired else plan.n_tiles, n_heads,
-                                           plan.max_tile_context if not window else min(plan.max_tile_context, window + plan.TILE),
-                                           target_groups=256 if plan.paired else 512)      # a pair's workgroup has twice the waves
+                                           plan.max_tile_context if not window else min(plan.max_tile_context, window + plan.tile),
+                                           target_groups=PAIRED_TARGET_GROUPS if plan.paired else 512)      # a pair's workgroup has twice the waves
         n_part = plan.n_tile_rows * n_heads * n_splits * (hd + 2) if n_splits > 1 else 0
         part = torch.empty(n_part, dtype=torch.float32, device=out.device) if n_part else None
-        _call("gi_attention_prompt_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles, plan.TILE,
+        _call("gi_attention_prompt_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), plan.tiles.data_ptr(), plan.n_tiles, plan.tile,
               1 if plan.paired else 0, table.data_ptr(), table.stride(0), cache.stride(0), page_size, n_heads, n_kv, hd, window, scale, n_splits,
               _ptr(plan.tile_first), _ptr(plan.tile_rows), plan.n_tile_rows, _ptr(part), n_part, _stream())
     if plan.n_decode:

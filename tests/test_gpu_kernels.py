@@ -234,10 +234,12 @@ SEGMENTS = {
 
 @pytest.mark.parametrize("n_heads,n_kv,hd,ps,window", ATT_CASES)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("portions", list(SEGMENTS))
-def test_attention_over_pages(n_heads, n_kv, hd, ps, window, dtype, portions):
-    """Portions of prompts on top of an existing cache, beside single decoded rows, on scrambled pages."""
+@pytest.mark.parametrize("portions,tile", [(name, 0) for name in SEGMENTS] + [("long portions", 128), ("several tiles", 128)])
+def test_attention_over_pages(n_heads, n_kv, hd, ps, window, dtype, portions, tile, monkeypatch):
+    """Portions of prompts on top of an existing cache, beside single decoded rows, on scrambled pages.
+    tile: rows of a prompt tile (0: as the step's size decides, which is 64 for steps as small as these)."""
     from geneinfer_amd.parts import StepContext
+    monkeypatch.setattr(ops().AttentionPlan, "TILE", tile)
     contexts = [300, 131, 1, 77, 530]
     cache, table, dense = build_paged(contexts, n_kv, hd, ps, dtype, seed=hd + n_heads)
     segs = SEGMENTS[portions]
