@@ -60,6 +60,83 @@ __global__ __launch_bounds__(256) void gemm_exact_kernel(const TA* __restrict__ 
     }
 }
 
+// The same product for at most FEW_ROWS rows of 32-bit activations (decoding): one lane per output column walks its
+// weight row alone, so that a product with a handful of rows is spread over N lanes instead of N / 64 workgroups.
+// Every output is the same chain of fused multiply-adds over ascending k as in the kernel above: the bits do not
+// depend on which of the two kernels a row met.  A lane reads 16 bytes of its own row at a time (the rows of a
+// wave's lanes are K elements apart, so a cache line a lane has touched serves its next loads); the activations
+// are the same for all lanes.
+constexpr int FEW_ROWS = 4;
+
+template <typename TW> struct Sixteen;                      // 16 bytes of a weight row, widened
+template <> struct Sixteen<float> {
+    static constexpr int N = 4;
+    static __device__ __forceinline__ void load(const float* p, float (&w)[4]) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    }
+};
+template <> struct Sixteen<bf16_t> {
+    static constexpr int N = 8;
+    static __device__ __forceinline__ void load(const bf16_t* p, float (&w)[8]) {
+        const uint4 v = *reinterpret_cast<const uint4*>(p);
+        const uint32_t u[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            w[2 * i] = __uint_as_float(u[i] << 16);
+            w[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+        }
+    }
+};
+
+template <typename TW, bool ACCUMULATE, int MR>
+__global__ __launch_bounds__(64) void gemm_exact_few_rows_kernel(const float* __restrict__ A, const TW* __restrict__ W, float* __restrict__ C, int M,
+                                                                 int N, int K, long lda, long ldw, long ldc) {
+    constexpr int PIECE = Sixteen<TW>::N, AHEAD = 32;        // elements per load; loads in flight per lane (512 bytes: four cache lines of its row)
+    const int n = blockIdx.x * 64 + threadIdx.x;
+    const TW* wrow = W + (size_t)min(n, N - 1) * ldw;
+    float acc[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = 0.f;
+    const int k_whole = K - K % (PIECE * AHEAD);
+    for (int k0 = 0; k0 < k_whole; k0 += PIECE * AHEAD) {
+        float w[AHEAD][PIECE];
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) Sixteen<TW>::load(wrow + k0 + u * PIECE, w[u]);
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u)
+#pragma unroll
+            for (int j = 0; j < PIECE; ++j)
+#pragma unroll
+                for (int m = 0; m < MR; ++m)
+                    if (m < M) acc[m] = fmaf(A[(size_t)m * lda + k0 + u * PIECE + j], w[u][j], acc[m]);
+    }
+    for (int k = k_whole; k < K; ++k) {
+        const float w = load_f32(wrow, (size_t)k);
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+            if (m < M) acc[m] = fmaf(A[(size_t)m * lda + k], w, acc[m]);
+    }
+    if (n >= N) return;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        if (m >= M) break;
+        const size_t o = (size_t)m * ldc + n;
+        C[o] = ACCUMULATE ? C[o] + acc[m] : acc[m];
+    }
+}
+
+template <typename TW>
+int launch_few_rows(const void* A, const void* W, void* C, int accumulate, int M, int N, int K, long lda, long ldw, long ldc, hipStream_t stream) {
+    const unsigned blocks = (unsigned)((N + 63) / 64);
+#define FEW(ACC, MR) gemm_exact_few_rows_kernel<TW, ACC, MR><<<blocks, 64, 0, stream>>>((const float*)A, (const TW*)W, (float*)C, M, N, K, lda, ldw, ldc)
+    if (M == 1) { if (accumulate) FEW(true, 1); else FEW(false, 1); }
+    else if (M == 2) { if (accumulate) FEW(true, 2); else FEW(false, 2); }
+    else { if (accumulate) FEW(true, FEW_ROWS); else FEW(false, FEW_ROWS); }
+#undef FEW
+    return 0;
+}
+
 template <typename TA, typename TW>
 int launch(const void* A, const void* W, void* C, int c_dtype, int accumulate, int M, int N, int K, long lda, long ldw, long ldc,
            hipStream_t stream) {
@@ -81,6 +158,15 @@ GI_API int gi_gemm_exact(const void* A, int a_dtype, const void* W, int w_dtype,
     GI_REQUIRE(lda >= K && ldw >= K && ldc >= N, "gemm_exact: leading dimensions (%ld, %ld, %ld) too small for K %d, N %d", lda, ldw, ldc, K, N);
     GI_REQUIRE((M + BM - 1) / BM <= 65535, "gemm_exact: M %d is too large", M);
     int rc;
+    // a few rows of 32-bit activations into a 32-bit result: a lane per output column (the loads need 16-byte pieces of the weight rows)
+    const long w_piece = w_dtype == GI_F32 ? 4 : 8;
+    if (M <= FEW_ROWS && a_dtype == GI_F32 && c_dtype == GI_F32 && (w_dtype == GI_F32 || w_dtype == GI_BF16) && ldw % w_piece == 0 &&
+        ((uintptr_t)W & 15) == 0) {
+        rc = w_dtype == GI_F32 ? launch_few_rows<float>(A, W, C, accumulate, M, N, K, lda, ldw, ldc, stream)
+                               : launch_few_rows<bf16_t>(A, W, C, accumulate, M, N, K, lda, ldw, ldc, stream);
+        GI_CHECK_LAUNCH("gemm_exact (few rows)");
+        return rc;
+    }
     if (a_dtype == GI_F32 && w_dtype == GI_F32) rc = launch<float, float>(A, W, C, c_dtype, accumulate, M, N, K, lda, ldw, ldc, stream);
     else if (a_dtype == GI_F32 && w_dtype == GI_BF16) rc = launch<float, bf16_t>(A, W, C, c_dtype, accumulate, M, N, K, lda, ldw, ldc, stream);
     else if (a_dtype == GI_BF16 && w_dtype == GI_BF16) rc = launch<bf16_t, bf16_t>(A, W, C, c_dtype, accumulate, M, N, K, lda, ldw, ldc, stream);

@@ -40,14 +40,21 @@ def test_gemm_exact(m, n, k, dtypes):
     assert rel(out[:, :n], 2 * want) < 2e-6 and not torch.equal(before, out[:, :n])
 
 
-def test_gemm_exact_rows_alone_have_the_same_bits():
-    a, w = randn(37, 200, seed=3), randn(90, 200, seed=4)
+@pytest.mark.parametrize("w_dtype,k", [(torch.float32, 200), (torch.float32, 203), (torch.bfloat16, 264), (torch.bfloat16, 520)])
+def test_gemm_exact_rows_alone_have_the_same_bits(w_dtype, k):
+    """One to four rows take the kernel with a lane per output column, more rows the tiled one; k = 203 leaves a tail
+    beside the 16-byte loads, 264 and 520 pieces of 8 beside whole groups of 64."""
+    a, w = randn(37, k, seed=3), randn(90, -(-k // 8) * 8, dtype=w_dtype, seed=4)[:, :k]      # the row stride stays a multiple of the 16-byte piece
     full = torch.empty(37, 90, device=DEV)
     ops().gemm_exact(a, w, full)
-    for i in (0, 17, 36):
-        one = torch.empty(1, 90, device=DEV)
-        ops().gemm_exact(a[i:i + 1], w, one)
-        assert torch.equal(one[0], full[i])
+    for first, rows in ((0, 1), (17, 1), (36, 1), (5, 2), (9, 3), (30, 4)):
+        few = torch.empty(rows, 90, device=DEV)
+        ops().gemm_exact(a[first:first + rows], w, few)
+        assert torch.equal(few, full[first:first + rows])
+        ops().gemm_exact(a[first:first + rows], w, few, accumulate=True)
+        both = full[first:first + rows].clone()
+        ops().gemm_exact(a[first:first + rows].repeat(17, 1)[:rows + 13], w, (wide := torch.cat([both, torch.zeros(13, 90, device=DEV)])), accumulate=True)
+        assert torch.equal(few, wide[:rows])                                # adding onto what is there, the same in both kernels
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 16, 8), (1, 2048, 2048), (3, 100, 136), (8, 130, 264), (16, 64, 128), (17, 1000, 520),
