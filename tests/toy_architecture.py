@@ -2,9 +2,11 @@
 needs are data: it is registered, built, loaded and stepped through the framework's public
 interfaces without a change to the framework's files.
 
-Layers: 0 full attention whose positions are encoded by a toy rule of its own (angles
+Layers (pre-norm blocks with RMS norms unless said otherwise): 0 full attention whose positions are encoded by a toy rule of its own (angles
 pos * step * (k + 1) instead of the rotary frequencies), 1 windowed attention, 2 a "decay" mixer
-with a state of its own (s <- decay * s + h per row, out = W s), each followed by SwiGLU; 3 a
+with a state of its own (s <- decay * s + h per row, out = W s), each followed by SwiGLU, layer 2
+in a block arrangement of its own (mixer and feed-forward both read one norm of the block's input, a
+norm that also removes the mean, and both add onto the residual stream); 3 a
 second decay mixer followed by a feed-forward with routing (a router picks one of three small
 SwiGLU experts per row and scales it by the router's probability of it).  Run order: 3, 0, 1, 2,
 then layer 0 once more (a cache of its own) and layer 1 once more reading the pages of its first
@@ -22,7 +24,8 @@ import torch
 from geneinfer_amd.cache import StateNeed
 from geneinfer_amd.config import (AttentionSpec, LayerSpec, ModelSpec, RmsNormSpec, RotarySpec, RunEntry, SwiGluSpec,
                                   register_architecture)
-from geneinfer_amd.parts import FeedForward, Mixer, PositionEncoding, register_feed_forward, register_mixer, register_position_encoding
+from geneinfer_amd.parts import (FeedForward, Mixer, Norm, PositionEncoding, feed_forward_class, mixer_class, norm_class, register_block,
+                                 register_feed_forward, register_mixer, register_norm, register_position_encoding)
 from geneinfer_amd.weights import TensorNeed
 from plain_llama import causal_attention, rms_norm, rope_inverse_frequencies, rope_rotate, swiglu
 
@@ -59,6 +62,58 @@ class DecayMixer(Mixer):
                 s = self.spec.decay * s + h[i].float()
                 residual[i] += self.w @ s
             cache.state[slot] = s
+
+
+@dataclass(frozen=True)
+class CenteredNormSpec:
+    kind: ClassVar[str] = "toy_centered_norm"
+    size: int
+    eps: float
+    weight: str
+
+
+class CenteredNorm(Norm):
+    """w * (x - mean(x)) / sqrt(var(x) + eps), in 32-bit; the result is stored as the consumer asks."""
+
+    def __init__(self, spec, tensors, dtype, device):
+        super().__init__(spec, tensors, dtype, device)
+        self.weight = tensors[spec.weight].float()
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        return [TensorNeed(spec.weight, (spec.size,), "norm")]
+
+    def __call__(self, x, out_dtype, rows=None):
+        x = x if rows is None else x[rows.long()]
+        centered = x - x.mean(dim=-1, keepdim=True)
+        return (self.weight * centered * torch.rsqrt(centered.square().mean(dim=-1, keepdim=True) + self.spec.eps)).to(out_dtype)
+
+
+class ParallelBlock:
+    """x += mixer(norm(x)) + feed_forward(norm(x)): one norm, read by both halves.  What the model asks of a block:
+    `tensor_needs(layer_spec)`, `cache_need(layer_spec)`, `forward(x, ctx, cache)`, `graph_safe`."""
+    graph_safe = False
+
+    def __init__(self, spec, tensors, dtype, device):
+        self.spec = spec
+        self.mixer_norm = self.feed_forward_norm = norm_class(spec.mixer_norm)(spec.mixer_norm, tensors, dtype, device)
+        self.mixer = mixer_class(spec.mixer)(spec.mixer, tensors, dtype, device)
+        self.feed_forward = feed_forward_class(spec.feed_forward)(spec.feed_forward, tensors, dtype, device)
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        return (norm_class(spec.mixer_norm).tensor_needs(spec.mixer_norm) + mixer_class(spec.mixer).tensor_needs(spec.mixer) +
+                feed_forward_class(spec.feed_forward).tensor_needs(spec.feed_forward))
+
+    @classmethod
+    def cache_need(cls, spec):
+        return mixer_class(spec.mixer).cache_need(spec.mixer)
+
+    def forward(self, x, ctx, cache):
+        for_mixer = self.mixer_norm(x, getattr(self.mixer, "in_dtype", ctx.dtype))
+        for_feed_forward = self.mixer_norm(x, getattr(self.feed_forward, "in_dtype", ctx.dtype))       # before the mixer changes x
+        self.mixer.forward(for_mixer, x, ctx, cache)
+        self.feed_forward.forward(for_feed_forward, x, ctx)
 
 
 @dataclass(frozen=True)
@@ -153,13 +208,16 @@ class ToyConfig:
             p = f"layers.{l}.attn."
             return AttentionSpec(d, self.num_attention_heads, self.num_key_value_heads, self.head_dim, p + "q", p + "k", p + "v", p + "o",
                                  position=position, window=window)
-        def rest(l, mixer, feed_forward=None):
+        def rest(l, mixer, feed_forward=None, parallel=False):
             p = f"layers.{l}."
             feed_forward = feed_forward or SwiGluSpec(d, self.intermediate_size, p + "ff.gate", p + "ff.up", p + "ff.down")
+            if parallel:
+                norm = CenteredNormSpec(d, self.rms_norm_eps, p + "norm1")
+                return LayerSpec(mixer=mixer, feed_forward=feed_forward, mixer_norm=norm, feed_forward_norm=norm, block="toy_parallel")
             return LayerSpec(mixer=mixer, feed_forward=feed_forward,
                              mixer_norm=RmsNormSpec(d, self.rms_norm_eps, p + "norm1"), feed_forward_norm=RmsNormSpec(d, self.rms_norm_eps, p + "norm2"))
         layers = (rest(0, attention(0, None, LinearAnglesSpec(self.head_dim, self.angle_step))), rest(1, attention(1, self.window, rot)),
-                  rest(2, DecaySpec(d, self.decay, "layers.2.decay.w")),
+                  rest(2, DecaySpec(d, self.decay, "layers.2.decay.w"), parallel=True),
                   rest(3, DecaySpec(d, self.decay, "layers.3.decay.w"), RoutedSpec(d, self.expert_intermediate_size, self.num_experts, "layers.3.moe.")))
         order = (RunEntry(3), RunEntry(0), RunEntry(1), RunEntry(2), RunEntry(0), RunEntry(1, cache_of=2))
         return ModelSpec(architecture=self.architecture, vocab_size=self.vocab_size, hidden_size=d, max_positions=self.max_position_embeddings,
@@ -172,6 +230,8 @@ def register():
     register_mixer("toy_decay", DecayMixer)
     register_feed_forward("toy_routed", RoutedFeedForward)
     register_position_encoding("toy_linear_angles", LinearAngles)
+    register_norm("toy_centered_norm", CenteredNorm)
+    register_block("toy_parallel", ParallelBlock)
     register_architecture(ToyConfig.architecture, ToyConfig, model_type="toy_mixed")
 
 
@@ -199,6 +259,15 @@ def plain_logits(cfg: ToyConfig, w: dict, tokens, dtype=torch.float64, store=lam
     kept = {}
     for i, entry in enumerate(spec.run_order):
         l, p = entry.layer, f"layers.{entry.layer}."
+        if l == 2:                                            # the parallel block: one centered norm feeds both halves
+            c = x - x.mean(dim=-1, keepdim=True)
+            xb = w[p + "norm1"] * c * torch.rsqrt(c.square().mean(dim=-1, keepdim=True) + cfg.rms_norm_eps)
+            s, outs = torch.zeros(cfg.hidden_size, dtype=dtype), []
+            for t in range(T):
+                s = cfg.decay * s + xb[t]
+                outs.append(w[p + "decay.w"] @ s)
+            x = x + torch.stack(outs) + swiglu(store(xb), w[p + "ff.gate"], w[p + "ff.up"], w[p + "ff.down"], store)
+            continue
         xb = rms_norm(x, w[p + "norm1"], cfg.rms_norm_eps)
         if l >= 2:
             s, outs = torch.zeros(cfg.hidden_size, dtype=dtype), []
