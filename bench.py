@@ -43,7 +43,7 @@ def main() -> int:
 
     import torch
     from geneinfer_amd.config import LlamaConfig
-    from geneinfer_amd.engine import Runner, StepEntry, random_model
+    from geneinfer_amd.engine import Engine, EngineConfig, EngineRequest, Runner, StepEntry, random_model
     from geneinfer_amd.sampling import Sampler, SamplerConfig, sample_rows
 
     sizes = dict(LLAMA_1B)
@@ -57,7 +57,7 @@ def main() -> int:
     gen = torch.Generator().manual_seed(1)
 
     def make_runner(batch):
-        per_request = -(-(PROMPT + NEW_TOKENS + args.steps + args.warmup) // 64) * 64
+        per_request = -(-(PROMPT + NEW_TOKENS + args.steps + args.warmup + 2 * batch + 8) // 64) * 64
         return Runner(model, page_size=PAGE, max_tokens=batch * per_request, max_requests=batch, max_rows=max(PROMPT, batch),
                       max_positions=CONTEXT)
 
@@ -67,26 +67,30 @@ def main() -> int:
         return runner.step([StepEntry(rid, toks, (PROMPT - 1,))])
 
     def decode(batch, steps, warmup):
-        """Greedy decoding of `batch` requests after their prompts; returns (seconds for `steps` steps, context at the middle)."""
+        """Greedy decoding of `batch` requests after their prompts, through the scheduler (what serving runs); returns
+        (seconds for `steps` decode steps, mean context at the middle of them)."""
         runner = make_runner(batch)
-        samplers = [Sampler(SamplerConfig(temperature=0.0), vocab) for _ in range(batch)]
-        tokens = [sample_rows(prefill(runner, r), [samplers[r]])[0] for r in range(batch)]
-
-        def one():
-            nonlocal tokens
-            logits = runner.step([StepEntry(r, [tokens[r]], (0,)) for r in range(batch)])
-            tokens = sample_rows(logits, samplers)
-
+        engine = Engine(runner, EngineConfig(max_running=batch, prefix_cache=False))
+        limit = min(CONTEXT, PROMPT + NEW_TOKENS + steps + warmup + 2 * batch)
+        for r in range(batch):
+            engine.submit(EngineRequest(torch.randint(0, vocab, (PROMPT,), generator=gen).tolist(), limit, SamplerConfig(temperature=0.0)))
+        decoding = 0
+        while decoding < 2:                                  # the prompts, in steps of up to max_rows rows, until steps hold decode rows only
+            rows = engine.stats.rows
+            assert engine.step()
+            decoding = decoding + 1 if engine.stats.rows - rows == batch and engine.stats.passes > batch else 0
         for _ in range(warmup):
-            one()
+            engine.step()
         torch.cuda.synchronize()
+        context = sum(runner.length(job.key) for job in engine.running) / batch + steps / 2
+        passes = engine.stats.passes
         t0 = time.perf_counter()
         for _ in range(steps):
-            one()
+            engine.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        context = PROMPT + warmup + steps // 2
-        del runner
+        assert engine.stats.passes - passes == steps and len(engine.running) == batch, "a timed step was not a decode step of the whole batch"
+        del engine, runner
         torch.cuda.empty_cache()
         return dt, context
 

@@ -159,7 +159,23 @@ class Runner:
         return logits
 
     # --------------------------------------------------------------------------- captured decode
-    def _step_of_single_tokens(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    @property
+    def can_step_from_device(self) -> bool:
+        """Whether `step_from_device` is served: by the captured decode step."""
+        return bool(self.use_graphs) and self.model.trace is None
+
+    def step_from_device(self, requests: Sequence[Hashable], tokens: torch.Tensor) -> torch.Tensor:
+        """A decode step whose tokens are still on the device: request i brings `tokens[i]` (int32, typically what the
+        sampler made of the previous step's logits and nobody has waited for yet) and wants its logits.  The caller
+        can so put the next step in the queue before the host knows the last one's tokens.  The tokens are not
+        checked against the vocabulary (a sampler makes none outside it); everything else is `step`'s."""
+        if not self.can_step_from_device:
+            raise StepError("tokens on the device are taken by the captured decode step only")
+        if not (tokens.dtype == torch.int32 and tokens.shape == (len(requests),) and tokens.device == torch.device(self.model.device)):
+            raise StepError("step_from_device: tokens must be int32 [requests] on the model's device")
+        return self._step_of_single_tokens([StepEntry(r, [0], (0,)) for r in requests], tokens)
+
+    def _step_of_single_tokens(self, entries: Sequence[StepEntry], tokens_on_device: Optional[torch.Tensor] = None) -> torch.Tensor:
         """The decode step: every request brings one token and wants its logits.  The same checks and the
         same bookkeeping as the general path, done over whole lists at once (this path runs once per
         generated token of every request, so its host time counts)."""
@@ -186,13 +202,13 @@ class Runner:
         self._uploads.begin_step()
         cache.sync(self._uploads.put)
         meta = self._uploads.stage(np.array([tokens, lengths, slots], dtype=np.int32)).view(3, n)
-        logits = self._decode_step(meta, slots, lengths)
+        logits = self._decode_step(meta, slots, lengths, tokens_on_device)
         self._uploads.end_step()
         cache.advance_one_each(requests, slots, lengths)
         self.steps_run += 1
         return logits
 
-    def _decode_step(self, meta: torch.Tensor, seg_slot, seg_pos0) -> torch.Tensor:
+    def _decode_step(self, meta: torch.Tensor, seg_slot, seg_pos0, tokens_on_device=None) -> torch.Tensor:
         """A step in which every request brings one token and wants its logits runs as a replay of a
         HIP graph captured once per batch size: the launches of the whole pass cost one call.  The
         graph reads tokens, positions and slots from fixed device buffers that are filled before
@@ -207,7 +223,7 @@ class Runner:
         g = self._graphs.get((batch, bracket))
         if g is None:
             g = self._graphs[(batch, bracket)] = _DecodeGraph(self.model, self._view, bracket, batch)
-        return g.run(meta, seg_slot, seg_pos0)
+        return g.run(meta, seg_slot, seg_pos0, tokens_on_device)
 
 
 class _StepUploads:
@@ -284,10 +300,12 @@ class _DecodeGraph:
         ctx.memo["attention_plan"] = self.plan
         return ctx
 
-    def run(self, meta: torch.Tensor, seg_slot, seg_pos0) -> torch.Tensor:
+    def run(self, meta: torch.Tensor, seg_slot, seg_pos0, tokens_on_device=None) -> torch.Tensor:
         """meta: this step's tokens, positions and slots, int32 [3, batch], in pinned memory that stays as it is
-        until the copy made here has run."""
+        until the copy made here has run.  tokens_on_device: the tokens, if the host does not know them yet."""
         self.meta.copy_(meta, non_blocking=True)
+        if tokens_on_device is not None:
+            self.meta[0].copy_(tokens_on_device, non_blocking=True)
         self.calls += 1
         if self.graph is None:
             if self.calls < 2:          # the first step of a batch size runs as it is; a size that comes again is captured

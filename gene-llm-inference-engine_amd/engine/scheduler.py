@@ -20,6 +20,12 @@ Policy, as the reference's engine (src/runtime/engine.cpp:64-205):
   * only the row of a request's last known token returns logits; the request's own sampler draws
     the next token from them.  A sampled end token finishes the request (it stays the last
     generated token); so does reaching `max_positions` (prompt plus generated tokens).
+  * decoding ahead (on where the runner can take a step's tokens from the device): while every running request
+    decodes and no other can be admitted, the next step is put in the queue before the host has read the tokens of the
+    last one (they go from the sampling kernel straight into the next step), so the device does not wait for the
+    host between steps.  A request that turns out to have ended (an end token) has one row too many computed, which
+    nobody sees; ends by length are known beforehand.  Admission, portions of prompts, filtered sampling and a
+    shortage of pages all fall back to steps whose tokens are read before the next one is planned.
 Each request gets the tokens it would get alone through `generate()` with the same seed.
 """
 from __future__ import annotations
@@ -28,7 +34,8 @@ from collections import deque
 from dataclasses import dataclass, field
 from typing import Callable, Deque, Iterable, List, Optional, Sequence
 
-from ..sampling import Sampler, SamplerConfig, sample_rows
+from ..cache.pages import OutOfPages
+from ..sampling import Sampler, SamplerConfig, sample_rows, sample_rows_on_device
 from .runner import Runner, StepEntry
 
 POOL_TOO_SMALL = "the KV pool is too small for this request"
@@ -40,6 +47,7 @@ class EngineConfig:
     step_rows: int = 0          # rows per step; 0 = the runner's max_rows
     prefill_chunk: int = 0      # most prompt tokens one request adds to a step; 0 = no limit besides step_rows
     prefix_cache: bool = True   # requests with equal first tokens share the pages of that prefix
+    decode_ahead: bool = True   # queue the next decode step before the host has read the last one's tokens
 
 
 @dataclass
@@ -89,6 +97,13 @@ class _Job:
         self.key = ("job", jid)
 
 
+class _Flight:
+    """A decode step in the queue whose tokens the host has not read yet."""
+
+    def __init__(self, taken, tokens, host, ready, pass_no):
+        self.taken, self.tokens, self.host, self.ready, self.pass_no = taken, tokens, host, ready, pass_no      # taken: [(job, rows)]
+
+
 class Engine:
     def __init__(self, runner: Runner, config: Optional[EngineConfig] = None, end_tokens: Iterable[int] = (), sample=sample_rows):
         """`sample(logits, samplers) -> tokens` draws one token per row of logits with that row's sampler."""
@@ -99,7 +114,8 @@ class Engine:
         if cfg.step_rows < 0 or cfg.prefill_chunk < 0:
             raise ValueError("Engine: step_rows and prefill_chunk must be >= 0")
         step_rows = cfg.step_rows if 0 < cfg.step_rows <= runner.max_rows else runner.max_rows
-        self.cfg = EngineConfig(min(cfg.max_running, runner.cache.max_requests), step_rows, cfg.prefill_chunk or step_rows, cfg.prefix_cache)
+        self.cfg = EngineConfig(min(cfg.max_running, runner.cache.max_requests), step_rows, cfg.prefill_chunk or step_rows, cfg.prefix_cache,
+                                cfg.decode_ahead)
         self.runner = runner
         self.prefix = runner.cache.prefix if cfg.prefix_cache and runner.cache.enable_prefix_sharing() else None
         self.end_tokens = set(int(t) for t in end_tokens)
@@ -107,6 +123,13 @@ class Engine:
         self.waiting: Deque[_Job] = deque()
         self.running: List[_Job] = []                                    # in admission order
         self.stats = EngineStats()
+        # decoding ahead: the step in the queue, and two pinned buffers its tokens come back through in turn
+        self._flight: Optional[_Flight] = None
+        self._landing_strips, self._strip = None, 0
+        if cfg.decode_ahead and sample is sample_rows and hasattr(runner, "step_from_device"):
+            import torch
+            if torch.device(runner.model.device).type == "cuda":
+                self._landing_strips = [torch.empty(self.cfg.max_running, dtype=torch.int32, pin_memory=True) for _ in range(2)]
 
     # ----------------------------------------------------------------------------- interface
     def submit(self, request: EngineRequest) -> int:
@@ -125,7 +148,7 @@ class Engine:
         return job.id
 
     def idle(self) -> bool:
-        return not self.waiting and not self.running
+        return not self.waiting and not self.running and self._flight is None
 
     def result(self, jid: int) -> EngineResult:
         if not 0 <= jid < len(self.jobs):
@@ -154,8 +177,8 @@ class Engine:
             self.running.append(job)
         self.stats.max_running_seen = max(self.stats.max_running_seen, len(self.running))
 
-    def _finish(self, job: _Job, error: str = "") -> None:
-        job.result.finished, job.result.error, job.result.last_pass = True, error, self.stats.passes
+    def _finish(self, job: _Job, error: str = "", pass_no: Optional[int] = None) -> None:
+        job.result.finished, job.result.error, job.result.last_pass = True, error, self.stats.passes if pass_no is None else pass_no
         self.runner.close(job.key)
         self.running.remove(job)
 
@@ -193,6 +216,8 @@ class Engine:
 
     def step(self) -> bool:
         """Runs one step.  False (and nothing done) if no request waits or runs."""
+        if self._flight is not None:
+            return self._step_behind_a_flight()
         self._admit()
         if not self.running:
             return False
@@ -216,6 +241,21 @@ class Engine:
             needed = sum(cache.pages_needed(job.key, n)[0] for job, n in taken)
             self.stats.evicted_pages += cache.evict(needed - cache.free_pages()[0])
         logits = self.runner.step(entries)
+        self._count_pass(taken)
+
+        if self._landing_strips is not None and len(wanting) == len(taken) == len(self.running) and self.runner.can_step_from_device:
+            # every running request decodes: its token may stay on the device for the next step
+            tokens = sample_rows_on_device(logits, [j.sampler for j in wanting])
+            if tokens is not None:
+                self._flight = self._take_off(taken, tokens)
+                return True
+        sampled = self._sample(logits, [j.sampler for j in wanting]) if wanting else []
+        next_token = {j.id: t for j, t in zip(wanting, sampled)}
+        for job in [job for job, n in taken if self._after_rows(job, n, next_token.get(job.id), self.stats.passes)]:
+            self._finish(job)
+        return True
+
+    def _count_pass(self, taken) -> None:
         st = self.stats
         st.passes += 1
         n_rows = sum(n for _, n in taken)
@@ -223,31 +263,67 @@ class Engine:
         st.max_rows_in_pass = max(st.max_rows_in_pass, n_rows)
         st.max_chunk = max(st.max_chunk, max(n for _, n in taken))
 
-        sampled = self._sample(logits, [j.sampler for j in wanting]) if wanting else []
-        next_token = {j.id: t for j, t in zip(wanting, sampled)}
-        done = []
-        for job, n in taken:
-            if job.result.first_pass < 0:
-                job.result.first_pass = st.passes
-            job.fed += n
-            if self.prefix is not None and job.fed // self.prefix.page_size > job.indexed_upto // self.prefix.page_size:
-                self.prefix.insert(job.tokens, job.fed, self.runner.cache.pages_of(job.key))      # the pages that became full
-                job.indexed_upto = job.fed
-            if job.id in next_token:
-                nxt = next_token[job.id]
-                st.logits_rows += 1
-                job.result.generated_tokens.append(nxt)
-                job.tokens.append(nxt)
-                if job.result.first_token_pass < 0:
-                    job.result.first_token_pass = st.passes
-                if nxt in self.end_tokens:
-                    job.result.stopped_by_end_token = True
-                    done.append(job)
-                    continue
-                if job.request.on_token is not None:
-                    job.request.on_token(nxt)
-            if job.fed >= job.steps:
-                done.append(job)
-        for job in done:
-            self._finish(job)
+    def _after_rows(self, job: _Job, n: int, nxt: Optional[int], pass_no: int) -> bool:
+        """The job's books after `n` of its rows have run (and `nxt` was drawn from the last one's logits, if it
+        was the job's last known token).  True if the job is finished."""
+        st = self.stats
+        if job.result.first_pass < 0:
+            job.result.first_pass = pass_no
+        job.fed += n
+        if self.prefix is not None and job.fed // self.prefix.page_size > job.indexed_upto // self.prefix.page_size:
+            self.prefix.insert(job.tokens, job.fed, self.runner.cache.pages_of(job.key))      # the pages that became full
+            job.indexed_upto = job.fed
+        if nxt is not None:
+            st.logits_rows += 1
+            job.result.generated_tokens.append(nxt)
+            job.tokens.append(nxt)
+            if job.result.first_token_pass < 0:
+                job.result.first_token_pass = pass_no
+            if nxt in self.end_tokens:
+                job.result.stopped_by_end_token = True
+                return True
+            if job.request.on_token is not None:
+                job.request.on_token(nxt)
+        return job.fed >= job.steps
+
+    # ------------------------------------------------------------------------------ decoding ahead
+    def _take_off(self, taken, tokens) -> _Flight:
+        """The step's tokens (one per job of `taken`, in its order) start their way to the host, and nobody waits
+        here; the step counts as in flight."""
+        import torch
+        host = self._landing_strips[self._strip][:len(taken)]
+        self._strip ^= 1
+        host.copy_(tokens, non_blocking=True)
+        ready = torch.cuda.Event()
+        ready.record()
+        return _Flight(list(taken), tokens, host, ready, self.stats.passes)
+
+    def _step_behind_a_flight(self) -> bool:
+        """With a decode step in flight: the next one is queued with that step's tokens where they are, if the same
+        requests go on for certain; then the flight's tokens are read and the requests' books brought up to date."""
+        flight, ahead = self._flight, None
+        jobs = [job for job, _ in flight.taken]
+        goes_on = (len(jobs) == len(self.running) and not any(j.result.finished for j in jobs)          # nobody of it ended last time,
+                   and all(j.fed + n < j.steps for j, n in flight.taken)                                # nobody ends by length now,
+                   and (not self.waiting or len(self.running) >= self.cfg.max_running)                  # and nobody else could join
+                   and self.runner.can_step_from_device)
+        if goes_on:
+            try:
+                if self.prefix is not None:
+                    cache = self.runner.cache
+                    needed = sum(cache.pages_needed(j.key, 1)[0] for j in jobs)
+                    self.stats.evicted_pages += cache.evict(needed - cache.free_pages()[0])
+                logits = self.runner.step_from_device([j.key for j in jobs], flight.tokens)
+            except OutOfPages:                       # nothing has changed: the step after the landing sorts it out
+                logits = None
+            if logits is not None:
+                self._count_pass([(j, 1) for j in jobs])
+                ahead = self._take_off([(j, 1) for j in jobs], sample_rows_on_device(logits, [j.sampler for j in jobs]))
+        flight.ready.synchronize()
+        sampled = flight.host.tolist()
+        finished = [job for (job, n), nxt in zip(flight.taken, sampled)
+                    if not job.result.finished and self._after_rows(job, n, nxt, flight.pass_no)]
+        for job in finished:                         # (a finished request's row in the step ahead is nobody's)
+            self._finish(job, pass_no=flight.pass_no)
+        self._flight = ahead
         return True

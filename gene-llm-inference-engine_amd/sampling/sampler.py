@@ -116,6 +116,23 @@ class Sampler:
         return sample_rows(logits.reshape(1, -1), [self])[0]
 
 
+def sample_rows_on_device(logits: torch.Tensor, samplers: Sequence[Sampler]):
+    """The tokens of `sample_rows`, left on the device (int32 [n]) without waiting for them, when every
+    sampler is greedy or every one samples the plain softmax (each then draws its uniform number now);
+    None, with nothing drawn, when a row needs the host (top-k, top-p) or the kinds are mixed."""
+    n, vocab = logits.shape
+    if n != len(samplers):
+        raise ValueError(f"{n} rows of logits for {len(samplers)} samplers")
+    kinds = {s.kind for s in samplers}
+    out = torch.empty(n, dtype=torch.int32, device=logits.device)
+    if kinds == {"greedy"}:
+        return ops.argmax(logits, out)
+    if kinds == {"plain"}:
+        both = torch.tensor([[s.temperature for s in samplers], [s.stream.next_uniform() for s in samplers]], dtype=torch.float32).to(logits.device)
+        return ops.sample_temperature(logits, both[0], both[1], out)
+    return None
+
+
 def sample_rows(logits: torch.Tensor, samplers: Sequence[Sampler]) -> List[int]:
     """Row i of `logits` (float32 [n, vocab], on the device) is sampled with samplers[i].
     A sampler draws one uniform number per call unless it is greedy."""

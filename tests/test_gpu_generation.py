@@ -94,6 +94,49 @@ def test_scheduler_gives_each_request_what_it_gets_alone(folders, name, temperat
     assert preempted > 0, "no pool was tight enough to preempt"
 
 
+@pytest.mark.parametrize("temperature", [0.0, 0.8])
+def test_decoding_ahead_changes_no_token(folders, temperature):
+    """The scheduler queues a decode step before it has read the tokens of the last one.  With end tokens that cut
+    requests short at different times (a row too many is then computed for them), with requests that wait for a free
+    place and with a pool so small that pages run out, every request ends as it does when every step's tokens are read
+    first, and as it does alone; and steps were in fact queued ahead."""
+    import geneinfer_amd as gi
+    from geneinfer_amd.engine import EngineConfig, EngineRequest
+    from geneinfer_amd.sampling import SamplerConfig
+    name, new, ps = "B", 40, PAGE_SIZE["B"]
+    prompts = prompts_for(name, [7, 19, 3, 30, 12, 5], seed=77)
+    roomy = gi.LLM(folders[name], dtype="float32", page_size=ps, max_tokens=512, max_running=1)
+    free_run = [roomy.generate(p, steps=len(p) + new - 1, temperature=temperature, seed=3 + i).generated_tokens for i, p in enumerate(prompts)]
+    end_tokens = {free_run[0][9], free_run[1][23], free_run[3][4]}                  # three requests stop early, at different steps
+    roomy.end_tokens = sorted(end_tokens)
+    alone = [roomy.generate(p, steps=len(p) + new - 1, temperature=temperature, seed=3 + i) for i, p in enumerate(prompts)]
+    assert sum(a.stopped_by_end_token for a in alone) >= 3 and any(not a.stopped_by_end_token for a in alone)
+    outcomes = {}
+    for ahead in (True, False):
+        for max_tokens, max_running in ((1024, 4), (1024, 6), (80, 4)):
+            llm = gi.LLM(folders[name], dtype="float32", page_size=ps, max_tokens=max_tokens, max_running=max_running, max_rows=64,
+                         end_tokens=sorted(end_tokens))
+            eng = llm.engine(EngineConfig(max_running=max_running, decode_ahead=ahead))
+            assert (eng._landing_strips is not None) == ahead
+            flights = 0
+            ids = [eng.submit(EngineRequest(p, len(p) + new - 1, SamplerConfig(temperature, seed=3 + i))) for i, p in enumerate(prompts)]
+            while eng.step():
+                flights += eng._flight is not None
+            assert eng.idle()
+            results = [eng.result(j) for j in ids]
+            for r, a in zip(results, alone):
+                assert r.finished and r.error == "" and r.generated_tokens == a.generated_tokens and r.stopped_by_end_token == a.stopped_by_end_token
+            llm.runner.cache.check_consistency()
+            if eng.prefix is not None:
+                eng.prefix.clear()
+            assert llm.runner.cache.free_pages() == [max_tokens // ps]
+            assert (flights > 10) == ahead
+            outcomes[(ahead, max_tokens, max_running)] = eng.stats
+    assert outcomes[(True, 80, 4)].preemptions > 0 and outcomes[(False, 80, 4)].preemptions > 0, "the small pool never ran out"
+    # a row too many for each request that an end token stopped while a step was queued ahead, nothing else
+    assert 0 <= outcomes[(True, 1024, 6)].rows - outcomes[(False, 1024, 6)].rows <= sum(a.stopped_by_end_token for a in alone)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_requests_with_an_equal_beginning_share_its_pages(folders, dtype):
     """Requests that begin alike take the pages an earlier one computed: fewer rows are fed, and every request still
