@@ -31,6 +31,7 @@ class StepEntry:
     request: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = field(default_factory=tuple)      # places among `tokens` whose logits are asked for
+    at: Optional[int] = None                                # where the caller believes its first token goes; None: wherever the cache says
 
 
 class _CacheView:
@@ -115,7 +116,16 @@ class Runner:
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise StepError(f"request {e.request!r} wants logits at place {w} of {len(e.tokens)} tokens")
-            if self.cache.length(e.request) + len(e.tokens) > self.max_positions:
+            held = self.cache.length(e.request)
+            if e.at is not None and int(e.at) != held:
+                # The positions are the cache's own.  A caller that names one is checked against it, in the order of
+                # the reference's forward_rows (src/model/transformer.cpp:298-307): the range first, then the gap.  An earlier position is no silent rewind here: `truncate` is a call of its own.
+                if int(e.at) < 0 or int(e.at) + len(e.tokens) > self.max_positions:
+                    raise StepError(f"positions {int(e.at)} .. {int(e.at) + len(e.tokens) - 1} of request {e.request!r} exceed the context length {self.max_positions}")
+                if int(e.at) > held:
+                    raise StepError(f"a portion of request {e.request!r} at position {int(e.at)} leaves a gap: the cache holds {held} positions")
+                raise StepError(f"a portion of request {e.request!r} at position {int(e.at)} lies under the {held} positions the cache holds; rewind first")
+            if held + len(e.tokens) > self.max_positions:
                 raise StepError(f"request {e.request!r} would pass the position limit {self.max_positions}")
             n_rows += len(e.tokens)
         if n_rows > self.max_rows:
@@ -126,7 +136,7 @@ class Runner:
         """Runs the batch; returns float32 logits [wanted, vocab] on the device in the order of the
         entries and of each entry's `want`, or None if nothing was wanted.  The tensor is valid
         until the next step."""
-        if self.use_graphs and self.model.trace is None and all(len(e.tokens) == 1 and tuple(e.want) == (0,) for e in entries) and entries:
+        if self.use_graphs and self.model.trace is None and all(len(e.tokens) == 1 and tuple(e.want) == (0,) and e.at is None for e in entries) and entries:
             return self._step_of_single_tokens(entries)
         n_rows = self._validate(entries)
         self.cache.reserve([(e.request, len(e.tokens)) for e in entries])       # OutOfPages: nothing changed

@@ -145,6 +145,20 @@ def test_gi_forward_dumps_logits_and_the_last_position_layer_by_layer(tmp_path):
     rows = torch.from_numpy(np.fromfile(tmp_path / "two" / "logits.f32", dtype="<f4")).reshape(-1, vocab)
     assert rows.shape[0] == len(tokens) - 11 and torch.equal(rows, logits[11:])
     assert not list((tmp_path / "two").glob("layer*.f32")) and not (tmp_path / "two" / "embedding.f32").exists()
+    # --traced: the whole sequence as portions with the trace on: the last position's activations are those of the token-by-token run
+    r = subprocess.run([exe, str(tmp_path / "m"), str(tmp_path / "four"), "--weights", "f32", "--block-size", "4", "--prefill", "20", "--max-batch", "7",
+                        "--traced", *ids], capture_output=True, text=True, timeout=170)
+    assert r.returncode == 0, r.stderr
+    assert np.array_equal(np.fromfile(tmp_path / "four" / "logits.f32", dtype="<f4"), logits[-1].numpy())
+    for f in files + ["embedding.f32", "final_norm.f32"]:
+        assert np.array_equal(np.fromfile(tmp_path / "four" / f, dtype="<f4"), np.fromfile(tmp_path / "one" / f, dtype="<f4")), f
+    # --pos-shift: a portion anywhere but where the cache ends is refused with a clean error (tests/verify_batch.py:128-139,
+    # tests/verify_device.py:233-235 of the reference ask the same of it)
+    for extra, msg in ((["--prefill", "3", "--head", "1", "--pos-shift", "1"], "leaves a gap"),
+                       (["--max-seq-len", "20", "--prefill", "20", "--pos-shift", "1"], "exceed the context length 20"),
+                       (["--prefill", "4", "--head", "2", "--pos-shift", "-1"], "lies under")):
+        r = subprocess.run([exe, str(tmp_path / "m"), str(tmp_path / "five"), "--weights", "f32", *extra, *ids], capture_output=True, text=True, timeout=170)
+        assert r.returncode == 1 and msg in r.stderr, (extra, r.stderr)
     native = subprocess.run([exe, str(tmp_path / "m"), str(tmp_path / "three"), "--prefill", "20", *ids], capture_output=True, text=True, timeout=170)
     assert native.returncode == 0 and (tmp_path / "three" / "logits.f32").stat().st_size == 4 * vocab
 

@@ -241,9 +241,18 @@ def test_step_refuses_bad_batches_and_changes_nothing(folders):
     for bad, msg in (([], "at least one entry"), ([StepEntry("zz", [1])], "not open"), ([StepEntry("a", [])], "no tokens"),
                      ([StepEntry("a", [256])], "outside the vocabulary"), ([StepEntry("a", [1], (1,))], "wants logits at place 1"),
                      ([StepEntry("a", [1]), StepEntry("a", [2])], "twice"), ([StepEntry("a", [1] * 10)], "position limit 12"),
-                     ([StepEntry("a", [1] * 8), StepEntry("b", [1] * 9)], "max_rows")):
+                     ([StepEntry("a", [1] * 8), StepEntry("b", [1] * 9)], "max_rows"),
+                     # a caller that names the position of its first token is held to what the cache holds
+                     ([StepEntry("a", [1], (0,), at=4)], "leaves a gap: the cache holds 3"), ([StepEntry("a", [1, 2], at=2)], "lies under the 3 positions"),
+                     ([StepEntry("a", [1], at=-1)], "exceed the context length 12"), ([StepEntry("b", [1] * 4, at=9)], "exceed the context length 12"),
+                     ([StepEntry("b", [1], (0,), at=1)], "leaves a gap: the cache holds 0")):
         with pytest.raises(StepError, match=msg):
             runner.step(bad)
+    assert runner.length("a") == 3 and runner.length("b") == 0
+    named = runner.step([StepEntry("b", [9], (0,), at=0)])             # the right position changes nothing
+    runner.truncate("b", 0)
+    assert torch.equal(named, runner.step([StepEntry("b", [9], (0,))]))
+    runner.truncate("b", 0)
     with pytest.raises(OutOfPages):                                   # 4 pages in all: a holds 1 and needs 2 more, b needs 2
         runner.step([StepEntry("a", [5] * 8, ()), StepEntry("b", [5] * 8, ())])
     assert runner.length("a") == 3 and runner.length("b") == 0 and runner.cache.free_pages() == [3]
