@@ -11,9 +11,13 @@ most positions of prompt plus generated tokens, temperature 0 is greedy, top_k 0
 from __future__ import annotations
 
 import json
+import time
 from pathlib import Path
 from typing import Iterable, List, Optional, Sequence
 
+import torch
+
+from .kernels import ops
 from .engine import Engine, EngineConfig, EngineRequest, Runner, generate, load_model, random_model
 from .sampling import Sampler, SamplerConfig
 
@@ -52,6 +56,21 @@ class LLM:
         max_tokens = max_tokens or max_running * min(context, 65536)
         self.runner = Runner(self.model, page_size=page_size, max_tokens=max_tokens, max_requests=max_running,
                              max_rows=max_rows, max_positions=context)
+
+    def set_profiling(self, on: bool) -> None:
+        """Per-kernel timing of everything this process steps from now on (`kernels.ops.KernelProfile`): the device
+        is waited for around every kernel and no step is replayed from a captured graph, so the run is slower
+        than an unobserved one.  `profile_report` gives the table; switching off forgets it."""
+        self._profile = ops.set_profiling(on)
+        self._profile_from = (self.runner.rows_run, self.runner.steps_run, time.perf_counter())
+
+    def profile_report(self) -> str:
+        """Empty if nothing was measured (the reference's `profile_report`, src/model/model.h:43-44)."""
+        if getattr(self, "_profile", None) is None:
+            return ""
+        torch.cuda.synchronize()
+        rows, steps, since = self._profile_from
+        return self._profile.report(self.runner.rows_run - rows, self.runner.steps_run - steps, time.perf_counter() - since)
 
     def generate(self, prompt_ids: Sequence[int], steps: int = 0, temperature: float = 0.8, top_k: int = 0, top_p: float = 1.0,
                  seed: int = 1, on_token=None):

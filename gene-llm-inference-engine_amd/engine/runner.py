@@ -18,6 +18,7 @@ import numpy as np
 import torch
 
 from ..cache import CacheManager
+from ..kernels import ops
 from ..parts import LayerCache, StepContext
 from .model import DecoderModel
 
@@ -75,6 +76,7 @@ class Runner:
                                   max_positions=self.max_positions, dtype=model.dtype, device=model.device)
         self._view = _CacheView(self.cache, needs, reads_from)
         self.steps_run = 0
+        self.rows_run = 0
         self.use_graphs = bool(use_graphs) and model.graph_safe
         self._graphs = {}
         self._uploads = _StepUploads(model.device, min(8 * self.max_rows + 1024, 1 << 18))       # at most 1 MiB a buffer; what is larger is copied the ordinary way
@@ -136,7 +138,7 @@ class Runner:
         """Runs the batch; returns float32 logits [wanted, vocab] on the device in the order of the
         entries and of each entry's `want`, or None if nothing was wanted.  The tensor is valid
         until the next step."""
-        if self.use_graphs and self.model.trace is None and all(len(e.tokens) == 1 and tuple(e.want) == (0,) and e.at is None for e in entries) and entries:
+        if self.can_step_from_device and all(len(e.tokens) == 1 and tuple(e.want) == (0,) and e.at is None for e in entries) and entries:
             return self._step_of_single_tokens(entries)
         n_rows = self._validate(entries)
         self.cache.reserve([(e.request, len(e.tokens)) for e in entries])       # OutOfPages: nothing changed
@@ -166,13 +168,15 @@ class Runner:
         for e in entries:
             self.cache.advance(e.request, len(e.tokens))
         self.steps_run += 1
+        self.rows_run += n_rows
         return logits
 
     # --------------------------------------------------------------------------- captured decode
     @property
     def can_step_from_device(self) -> bool:
-        """Whether `step_from_device` is served: by the captured decode step."""
-        return bool(self.use_graphs) and self.model.trace is None
+        """Whether `step_from_device` is served: by the captured decode step, which nobody may be watching from the
+        inside (a trace of the layers, a timing of the kernels)."""
+        return bool(self.use_graphs) and self.model.trace is None and not ops.profiling()
 
     def step_from_device(self, requests: Sequence[Hashable], tokens: torch.Tensor) -> torch.Tensor:
         """A decode step whose tokens are still on the device: request i brings `tokens[i]` (int32, typically what the
@@ -216,6 +220,7 @@ class Runner:
         self._uploads.end_step()
         cache.advance_one_each(requests, slots, lengths)
         self.steps_run += 1
+        self.rows_run += n
         return logits
 
     def _decode_step(self, meta: torch.Tensor, seg_slot, seg_pos0, tokens_on_device=None) -> torch.Tensor:

@@ -7,6 +7,8 @@ from __future__ import annotations
 import ctypes
 from ctypes import c_float, c_int, c_long, c_void_p
 
+from typing import Optional
+
 import torch
 
 from . import library
@@ -68,8 +70,69 @@ def _call(name, *args):
     fn = _FUNCTIONS.get(name)
     if fn is None:
         fn = _FUNCTIONS[name] = getattr(lib(), name)
+    if _profile is not None:
+        return _profile.timed(name, fn, args)
     if fn(*args) != 0:
         raise KernelError(lib().gi_last_error().decode())
+
+
+class KernelProfile:
+    """Time per kernel entry point, with the device waited for before and after every call (so the times add up, and
+    a step takes longer than it does unobserved).  What the reference's device model reports with --profile
+    (src/gpu/gpu_transformer.cpp:178-224), by entry point and weight shape instead of a fixed list of sections.
+    Matrix products are kept apart by the weight's shape, which tells the projections from one another, and count the
+    weight bytes they read."""
+
+    def __init__(self):
+        self.seconds, self.calls, self.weight_bytes = {}, {}, {}
+        self.note = None                        # (label suffix, weight bytes) of the product about to be launched
+
+    def timed(self, name, fn, args):
+        import time
+        label, nbytes = name[3:], 0
+        if self.note is not None:
+            label, nbytes = f"{label} {self.note[0]}", self.note[1]
+            self.note = None
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        rc = fn(*args)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if rc != 0:
+            raise KernelError(lib().gi_last_error().decode())
+        self.seconds[label] = self.seconds.get(label, 0.0) + dt
+        self.calls[label] = self.calls.get(label, 0) + 1
+        self.weight_bytes[label] = self.weight_bytes.get(label, 0) + nbytes
+
+    def report(self, positions: int, steps: int, wall_seconds: float) -> str:
+        if not self.seconds or positions <= 0:
+            return ""
+        inside = sum(self.seconds.values())
+        lines = [f"device profile: {positions} positions in {steps} steps, {wall_seconds * 1e3 / positions:.3f} ms per position "
+                 "(the device waits before and after every kernel)",
+                 f"  {'kernel':<34} {'calls':>8} {'ms/position':>12} {'share':>7} {'weights GB/s':>13}"]
+        for label in sorted(self.seconds, key=self.seconds.get, reverse=True):
+            sec, nbytes = self.seconds[label], self.weight_bytes[label]
+            rate = f"{nbytes / sec / 1e9:.1f}" if nbytes and sec > 0 else ""
+            lines.append(f"  {label:<34} {self.calls[label]:>8} {sec * 1e3 / positions:>12.4f} {100 * sec / wall_seconds:>6.1f}% {rate:>13}")
+        rest = max(wall_seconds - inside, 0.0)
+        lines.append(f"  {'host work, uploads, downloads':<34} {'':>8} {rest * 1e3 / positions:>12.4f} {100 * rest / wall_seconds:>6.1f}%")
+        return "\n".join(lines) + "\n"
+
+
+_profile: Optional[KernelProfile] = None
+
+
+def set_profiling(on: bool) -> Optional[KernelProfile]:
+    """Switches the per-kernel timing on (a fresh KernelProfile, which is returned) or off.  While it is on, steps are
+    not replayed from captured graphs: a replay has no kernel boundaries to wait at."""
+    global _profile
+    _profile = KernelProfile() if on else None
+    return _profile
+
+
+def profiling() -> bool:
+    return _profile is not None
 
 
 # The current stream's handle, asked for at every launch (it changes under graph capture).  torch's
@@ -245,6 +308,8 @@ def gemm_exact(a, w, out, accumulate=False):
         raise KernelError(f"gemm: out is {tuple(out.shape)}, ({m}, {n}) is needed")
     if not (a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1):
         raise KernelError("gemm: operands need unit inner stride")
+    if _profile is not None:
+        _profile.note = (f"{n}x{k}", n * k * w.element_size())
     _call("gi_gemm_exact", a.data_ptr(), _code(a, "gemm: a"), w.data_ptr(), _code(w, "gemm: w"), out.data_ptr(), _code(out, "gemm: out"),
           1 if accumulate else 0, m, n, k, a.stride(0), w.stride(0), out.stride(0), _stream())
     return out
@@ -475,6 +540,8 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False):
         raise KernelError("gemm_bf16: operands must be bfloat16 with K and row strides multiples of 8, 16-byte aligned")
     n_scratch = lib().gi_gemm_bf16_scratch_floats(m, n, k)           # partial sums where k is split over workgroups
     scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device) if n_scratch else None
+    if _profile is not None:
+        _profile.note = (f"{n}x{k}{' gated' if gated else ''}", n * k * w.element_size())
     _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,
           m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _stream())
     return out

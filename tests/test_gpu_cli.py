@@ -31,8 +31,9 @@ def test_gi_generate_greedy_dumps_the_plain_tokens(tmp_path):
                             "--no-echo", "--quiet"], capture_output=True, text=True, timeout=170)
     assert quiet.returncode == 0 and len(quiet.stdout.split()) == 4 and "prompt:" not in quiet.stderr and "gpu:" not in quiet.stderr
     again = subprocess.run([str(ROOT / "bin" / "gi_generate"), "--model", str(tmp_path / "m"), "--prompt-ids", "1,2,3", "--steps", "6", "--seed", "5",
-                            "--no-echo", "--quiet"], capture_output=True, text=True, timeout=170)
-    assert again.stdout == quiet.stdout                                         # the same seed, the same tokens
+                            "--no-echo", "--quiet", "--profile"], capture_output=True, text=True, timeout=170)
+    assert again.stdout == quiet.stdout                                         # the same seed, the same tokens, watched or not
+    assert "device profile: 6 positions in 5 steps" in again.stderr and "gemm_bf16" in again.stderr and "weights GB/s" in again.stderr
 
 
 def test_gi_generate_usage_errors(tmp_path):
@@ -74,7 +75,8 @@ def test_gi_serve_bench_levels_generate_what_each_request_generates_alone(tmp_pa
     assert warm.returncode == 0, warm.stdout + warm.stderr
     rows = [line.split() for line in warm.stdout.splitlines() if line[:1].isdigit()]
     assert int(rows[0][6]) == 48 and int(rows[1][6]) == 4 * 48
-    off = subprocess.run(common + ["--no-prefix-cache"], capture_output=True, text=True, timeout=170)
+    off = subprocess.run(common + ["--no-prefix-cache", "--profile"], capture_output=True, text=True, timeout=170)
+    assert "device profile: " in off.stdout and "gemm_exact" in off.stdout
     assert off.returncode == 0 and all(int(line.split()[6]) == 0 for line in off.stdout.splitlines() if line[:1].isdigit())
 
 
@@ -92,8 +94,9 @@ def test_gi_bench_reports_one_request(tmp_path):
     write_model(tmp_path / "m", CONFIGS["A"], seed=2)
     report = tmp_path / "report.json"
     r = subprocess.run([str(ROOT / "bin" / "gi_bench"), "--model", str(tmp_path / "m"), "--prompt-tokens", "20", "--decode-tokens", "9", "--runs", "2",
-                        "--label", "tiny", "--json", str(report), "--block-size", "4"], capture_output=True, text=True, timeout=170)
+                        "--label", "tiny", "--json", str(report), "--block-size", "4", "--profile"], capture_output=True, text=True, timeout=170)
     assert r.returncode == 0, r.stderr
+    assert "device profile: 29 positions in 10 steps" in r.stdout                # one more run, the watched one, after the measured two
     assert "workload: 20 prompt + 9 decode positions, 2 measured runs (+1 warmup)" in r.stdout and "| tiny |" in r.stdout
     j = json.loads(report.read_text())
     assert j["prompt_tokens"] == 20 and j["decode_tokens"] == 9 and j["label"] == "tiny" and j["bf16_weights"] is True

@@ -38,6 +38,46 @@ def test_greedy_generation_through_the_entry_point(folders):
     assert llm.runner.cache.free_pages() == [16]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_profiling_times_every_kernel_and_changes_no_token(folders, dtype):
+    """With the per-kernel timing on, no step is replayed from a graph and every kernel is waited for; the tokens are
+    those of the unobserved run, the report names the kernels with their counts, and the products say whose weights
+    they read.  Switched off, decoding is replayed from graphs again."""
+    import geneinfer_amd as gi
+    from geneinfer_amd.kernels import ops
+    cfg = CONFIGS["B"]
+    llm = gi.LLM(folders["B"], dtype=dtype, page_size=PAGE_SIZE["B"], max_tokens=128, max_running=2)
+    prompt = prompts_for("B", [9])[0]
+    assert llm.profile_report() == ""
+    plain_run = llm.generate(prompt, steps=len(prompt) + 5, temperature=0.0).generated_tokens
+    graphs = len(llm.runner._graphs)
+    assert graphs >= 1 and llm.runner.can_step_from_device
+    try:
+        llm.set_profiling(True)
+        assert not llm.runner.can_step_from_device
+        steps_before = llm.runner.steps_run
+        assert llm.generate(prompt, steps=len(prompt) + 5, temperature=0.0).generated_tokens == plain_run
+        report = llm.profile_report()
+    finally:
+        llm.set_profiling(False)
+    steps = llm.runner.steps_run - steps_before
+    assert steps == 7 and f"device profile: {len(prompt) + 5} positions in 7 steps" in report      # the prompt but its last token, then one by one
+    rows = {line[2:36].strip(): line[36:].split() for line in report.splitlines()[2:]}
+    layers, hidden, inter = cfg["num_hidden_layers"], cfg["hidden_size"], cfg["intermediate_size"]
+    product = "gemm_exact" if dtype == "float32" else "gemm_bf16"
+    down = f"{product} {hidden}x{inter}"
+    assert down in rows and int(rows[down][0]) == layers * steps and float(rows[down][-1]) > 0        # calls; weights GB/s
+    assert f"{product} {cfg['vocab_size']}x{hidden}" in rows
+    assert int(rows[f"{product} {cfg['vocab_size']}x{hidden}"][0]) == steps - 1                          # the head: not for the prompt, whose logits nobody wants
+    assert any(k.startswith("attention") for k in rows) and any(k.startswith("rmsnorm") for k in rows) and "embed" in rows
+    assert "host work, uploads, downloads" in rows
+    shares = [float(v[-1 if len(v) == 3 else -2].rstrip("%")) for k, v in rows.items() if k != "host work, uploads, downloads"]
+    assert 0 < sum(shares) <= 100.5
+    assert llm.runner.can_step_from_device and not ops.profiling()
+    assert llm.generate(prompt, steps=len(prompt) + 5, temperature=0.0).generated_tokens == plain_run
+    assert len(llm.runner._graphs) == graphs and llm.profile_report() == ""
+
+
 def test_temperature_sampling_follows_the_seeded_stream(folders):
     """Tiny B: temperature 0.8 with a seeded generator; every draw is re-derived from the plain
     logits and the plain sampler with the same uniform numbers."""
