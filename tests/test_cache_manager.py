@@ -191,7 +191,7 @@ def test_random_orders_of_requests_keep_the_books(seed):
         m.close(rid)
     m.check_consistency()
     assert all(f == g.pool.n_pages for f, g in zip(m.free_pages(), m.groups))
-    assert refused > 0 or seed % 2 == 0 or True
+    assert refused > 0                                                         # the pool did run out: the refusals above were exercised
 
 
 @pytest.mark.parametrize("seed", range(4))
