@@ -184,6 +184,7 @@ class CacheManager:
         self._slot: Dict[Hashable, int] = {}
         self._length: Dict[Hashable, int] = {}
         self.prefix: Optional[PrefixIndex] = None
+        self.evicted_pages = 0                       # pages taken back from the prefix index so far
 
     def enable_prefix_sharing(self) -> bool:
         """Lets requests share the pages of equal prompt prefixes (`self.prefix`).  Possible when one group of
@@ -223,7 +224,25 @@ class CacheManager:
 
     def evict(self, count: int) -> int:
         """Gives back up to `count` pages that only the prefix index still holds; returns how many."""
-        return self.prefix.evict(count) if self.prefix is not None and count > 0 else 0
+        freed = self.prefix.evict(count) if self.prefix is not None and count > 0 else 0
+        self.evicted_pages += freed
+        return freed
+
+    def available_pages(self) -> List[int]:
+        """Per group: free pages plus the pages that only the prefix index still holds, which a reservation takes back
+        when it needs them.  Whoever reserves (a scheduler's step, a lone `generate`, a replay) gets them, whether or
+        not it was the one that filled the index."""
+        out = self.free_pages()
+        if self.prefix is not None:
+            out[0] += self.prefix.evictable()
+        return out
+
+    def _make_room(self, need: Sequence[int]) -> bool:
+        """True if every group has `need[g]` free pages, after index-only pages were taken back where that helps."""
+        if self.prefix is not None and need[0] > self.groups[0].pool.free_count and need[0] <= self.groups[0].pool.free_count + self.prefix.evictable():
+            if all(n <= g.pool.free_count for n, g in zip(need[1:], self.groups[1:])):
+                self.evict(need[0] - self.groups[0].pool.free_count)
+        return all(n <= g.pool.free_count for n, g in zip(need, self.groups))
 
     def close(self, request: Hashable) -> None:
         slot = self.slot(request)
@@ -261,12 +280,15 @@ class CacheManager:
     def free_pages(self) -> List[int]:
         return [g.pool.free_count for g in self.groups]
 
-    def fits(self, additions: Sequence[Tuple[Hashable, int]]) -> bool:
+    def _pages_for(self, additions: Sequence[Tuple[Hashable, int]]) -> List[int]:
         need = [0] * len(self.groups)
         for request, n_new in additions:
             for gi, n in enumerate(self.pages_needed(request, n_new)):
                 need[gi] += n
-        return all(n <= g.pool.free_count for n, g in zip(need, self.groups))
+        return need
+
+    def fits(self, additions: Sequence[Tuple[Hashable, int]]) -> bool:
+        return all(n <= a for n, a in zip(self._pages_for(additions), self.available_pages()))
 
     def reserve(self, additions: Sequence[Tuple[Hashable, int]]) -> None:
         """Pages for n_new more positions of every named request, or `OutOfPages` with nothing changed."""
@@ -279,7 +301,7 @@ class CacheManager:
                 raise CacheError("a reservation must add at least one position")
             if self.length(request) + n_new > self.max_positions:
                 raise CacheError(f"request {request!r} would reach position {self._length[request] + n_new}, beyond the limit {self.max_positions}")
-        if not self.fits(additions):
+        if not self._make_room(self._pages_for(additions)):
             raise OutOfPages(f"not enough free pages (free per group: {self.free_pages()})")
         for request, n_new in additions:
             slot, length = self._slot[request], self._length[request]
@@ -293,13 +315,13 @@ class CacheManager:
         slot_arr, next_len = np.asarray(slots, dtype=np.int64), np.asarray(lengths, dtype=np.int64) + 1
         if int(next_len.max()) > self.max_positions:
             raise CacheError(f"a request would pass the position limit {self.max_positions}")
-        growing = []
+        growing, counts = [], []
         for g in self.groups:
             need = (next_len + g.page_size - 1) // g.page_size > g.n_held[slot_arr]
-            count = int(need.sum())
-            if count > g.pool.free_count:
-                raise OutOfPages(f"not enough free pages (free per group: {self.free_pages()})")
-            growing.append(np.nonzero(need)[0] if count else ())
+            counts.append(int(need.sum()))
+            growing.append(np.nonzero(need)[0] if counts[-1] else ())
+        if any(counts) and not self._make_room(counts):
+            raise OutOfPages(f"not enough free pages (free per group: {self.free_pages()})")
         for g, idx in zip(self.groups, growing):
             for i in idx:
                 g.grow(slots[i], int(next_len[i]))
@@ -342,7 +364,7 @@ class CacheManager:
             if not g.can_rewind_to(slot, length):
                 raise CacheError(f"request {request!r} cannot be rewound to {length}: a window of {g.need.window} has given those pages back")
         for g in self.groups:
-            if g.shared_page_at(slot, length) and g.pool.free_count + g.pages_freed_by_rewind(slot, length) < 1:
+            if g.shared_page_at(slot, length) and g.pool.free_count + g.pages_freed_by_rewind(slot, length) < 1 and self.evict(1) < 1:
                 raise OutOfPages("no free page to copy a shared page into")
         for g in self.groups:
             g.rewind(slot, length)
@@ -376,7 +398,7 @@ class CacheManager:
                     holders.setdefault(p, []).append(request)
                     if len(holders[p]) > 1 and (self.prefix is None or gi != 0):
                         raise CacheError(f"group {gi}: page {p} is held by {holders[p][0]!r} and {request!r}")
-            indexed = set(self.prefix._entry) if self.prefix is not None and gi == 0 else set()
+            indexed = set(self.prefix.pages()) if self.prefix is not None and gi == 0 else set()
             in_use = set(holders) | indexed
             free = set(g.pool._free)
             if len(free) != len(g.pool._free):

@@ -24,6 +24,7 @@ class PagePool:
         self.n_pages = int(n_pages)
         self._free: List[int] = list(range(self.n_pages - 1, -1, -1))    # a stack; its top is the end
         self._refs = [0] * self.n_pages
+        self.on_change = None            # called with (page, new reference count) after every retain and release
 
     @property
     def free_count(self) -> int:
@@ -49,6 +50,8 @@ class PagePool:
         if self._refs[page] == 0:
             raise PageError(f"page {page} is free and cannot be retained")
         self._refs[page] += 1
+        if self.on_change is not None:
+            self.on_change(page, self._refs[page])
 
     def release(self, page: int) -> None:
         self._check(page)
@@ -57,3 +60,5 @@ class PagePool:
         self._refs[page] -= 1
         if self._refs[page] == 0:
             self._free.append(page)
+        if self.on_change is not None:
+            self.on_change(page, self._refs[page])

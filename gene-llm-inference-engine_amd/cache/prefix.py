@@ -1,131 +1,184 @@
-"""Sharing of the pages of prompt prefixes that were computed before.
+"""Sharing of the pages of prompt beginnings that were computed before.
 
-The keys and values of a position depend only on the tokens up to it, so a request that starts
-with tokens an earlier request has processed can use that request's pages instead of computing
-them again.  The index knows *full* pages only: an entry says "after the chain of pages that
-ends in page P, the page that holds these `page_size` tokens is page B".  A lookup walks a
-prompt page by page from the root, so only a true prefix matches; the tokens are compared
-themselves, not their hashes.  The index holds one reference to every page it names; requests
-that use a page hold their own.  Pages that only the index references can be given back when
-memory runs short, least recently used leaf first.
+The keys and values of a position depend only on the tokens up to it, so a request that begins
+with tokens an earlier request has processed can read that request's pages instead of computing
+them again.  This index is a tree of *full* pages: the children of a node are the pages that
+followed it in some request, found by the `page_size` tokens they hold (the tokens themselves, not
+a hash of them); the children of the root are first pages.  A lookup walks a prompt down from the
+root, so only a true beginning matches.
 
-Behaviour as the reference's prefix cache (src/model/prefix_cache.h:1-11,
-src/model/prefix_cache.cpp:11-97).
+The index holds one reference to every page it names, requests hold their own.  It learns of every
+change of a named page's reference count through the pool's `on_change` hook, and so knows at all
+times how many pages nobody but itself holds (`evictable()`, constant time) and which of them are
+leaves: those wait in a heap ordered by last use, and `evict(k)` pops them, least recently used
+first, in O(k log n).  Heap entries are not removed when a page is used again or gains a child;
+they are recognised as stale when popped (the node's stamp has moved on).
+
+What it does is what the reference's prefix cache does (src/model/prefix_cache.h:1-11): full pages
+only, one reference per named page, `match` retains for the caller, leaves nobody uses go first.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
-from typing import Dict, List, Sequence, Tuple
+import heapq
+from typing import Dict, List, Optional, Sequence, Tuple
 
 from .pages import PagePool
 
-ROOT = -1
 
+class _Node:
+    __slots__ = ("page", "tokens", "parent", "children", "stamp", "only_mine")
 
-@dataclass
-class _Entry:
-    parent: int                 # the page before this one in the chain, ROOT for a prompt's first page
-    tokens: Tuple[int, ...]
-    tick: int                   # last use
-    children: int = 0
+    def __init__(self, page: int, tokens: Tuple[int, ...], parent: Optional["_Node"], stamp: int):
+        self.page, self.tokens, self.parent = page, tokens, parent
+        self.children: Dict[Tuple[int, ...], "_Node"] = {}
+        self.stamp = stamp                  # time of last use; also tells a fresh heap entry from a stale one
+        self.only_mine = False              # the index's reference is the page's only one
 
 
 class PrefixIndex:
     def __init__(self, pool: PagePool, page_size: int):
         self.pool, self.page_size = pool, int(page_size)
-        self._page_of: Dict[Tuple[int, Tuple[int, ...]], int] = {}      # (parent page, tokens) -> page
-        self._entry: Dict[int, _Entry] = {}                              # by page
+        self._first: Dict[Tuple[int, ...], _Node] = {}       # the root's children
+        self._by_page: Dict[int, _Node] = {}
+        self._only_mine = 0                                   # named pages whose reference count is 1
+        self._idle_leaves: List[Tuple[int, int]] = []         # heap of (stamp, page): leaves nobody else holds, and stale entries
         self._clock = 0
+        pool.on_change = self._references_changed
 
     def __len__(self) -> int:
-        return len(self._entry)
+        return len(self._by_page)
 
     def __contains__(self, page: int) -> bool:
-        return page in self._entry
+        return page in self._by_page
 
-    def _touch(self, page: int) -> None:
+    def pages(self):
+        """The pages the index names (and holds a reference to)."""
+        return self._by_page.keys()
+
+    # ------------------------------------------------------------------------- bookkeeping
+    def _references_changed(self, page: int, count: int) -> None:
+        node = self._by_page.get(page)
+        if node is None:
+            return
+        alone = count == 1
+        if alone != node.only_mine:
+            node.only_mine = alone
+            self._only_mine += 1 if alone else -1
+            if alone:
+                self._offer(node)
+
+    def _offer(self, node: _Node) -> None:
+        if node.only_mine and not node.children:
+            heapq.heappush(self._idle_leaves, (node.stamp, node.page))
+
+    def _touch(self, node: _Node) -> None:
         self._clock += 1
-        self._entry[page].tick = self._clock
+        node.stamp = self._clock
+        self._offer(node)                   # its older entry is stale now
 
+    def _children_of(self, node: Optional[_Node]) -> Dict[Tuple[int, ...], _Node]:
+        return self._first if node is None else node.children
+
+    # ----------------------------------------------------------------------------- lookups
     def match(self, tokens: Sequence[int], limit: int) -> List[int]:
-        """The longest known chain of full pages that is a prefix of tokens[:limit].  Every page returned
+        """The longest known chain of full pages that is a beginning of tokens[:limit].  Every page returned
         is retained once for the caller (who hands them to a request, or releases them)."""
-        ps, parent, found = self.page_size, ROOT, []
+        ps, node, found = self.page_size, None, []
         for i in range(min(limit, len(tokens)) // ps):
-            page = self._page_of.get((parent, tuple(int(t) for t in tokens[i * ps:(i + 1) * ps])))
-            if page is None:
+            nxt = self._children_of(node).get(tuple(tokens[i * ps:(i + 1) * ps]))
+            if nxt is None:
                 break
-            self.pool.retain(page)
-            self._touch(page)
-            found.append(page)
-            parent = page
+            self.pool.retain(nxt.page)
+            self._touch(nxt)
+            found.append(nxt.page)
+            node = nxt
         return found
 
     def insert(self, tokens: Sequence[int], n_tokens: int, pages: Sequence[int]) -> int:
-        """The first n_tokens positions of a request hold `tokens` in `pages` (its page table): its full
-        pages become the known pages of their chain links, unless a link is known already (then the known
-        page is followed, whatever the request's own copy).  Returns how many pages were newly named."""
-        ps, parent, added = self.page_size, ROOT, 0
+        """The first n_tokens positions of a request hold `tokens` in `pages` (its page table): its full pages
+        are named, each under the page before it, unless that place is taken already (then the page that has
+        it is followed, whatever the request's own copy).  Returns how many pages were newly named."""
+        ps, node, added = self.page_size, None, 0
         for i in range(min(n_tokens // ps, len(pages))):
-            key = (parent, tuple(int(t) for t in tokens[i * ps:(i + 1) * ps]))
-            known = self._page_of.get(key)
+            key = tuple(tokens[i * ps:(i + 1) * ps])
+            known = self._children_of(node).get(key)
             if known is not None:
                 self._touch(known)
-                parent = known
+                node = known
                 continue
             page = int(pages[i])
-            if page in self._entry:             # a page is never named twice (a consistent caller never gets here)
+            if page in self._by_page:       # a page has one place in the tree
                 break
-            self.pool.retain(page)
             self._clock += 1
-            self._entry[page] = _Entry(parent, key[1], self._clock)
-            self._page_of[key] = page
-            if parent != ROOT:
-                self._entry[parent].children += 1
-            parent = page
+            new = _Node(page, key, node, self._clock)
+            self._by_page[page] = new
+            self._children_of(node)[key] = new
+            self.pool.retain(page)          # (the hook sees a named page with at least two holders: nothing to count)
+            node = new
             added += 1
         return added
 
-    def _forget(self, page: int) -> None:
-        e = self._entry.pop(page)
-        del self._page_of[(e.parent, e.tokens)]
-        if e.parent != ROOT:
-            self._entry[e.parent].children -= 1
-        self.pool.release(page)
-
+    # ---------------------------------------------------------------------------- giving back
     def evictable(self) -> int:
-        """Pages `evict` could give back right now: those only the index references."""
-        return sum(1 for page in self._entry if self.pool.ref_count(page) == 1)
+        """Pages nobody but the index holds: what `evict` can give back."""
+        return self._only_mine
+
+    def _forget(self, node: _Node) -> None:
+        del self._by_page[node.page]
+        del self._children_of(node.parent)[node.tokens]
+        if node.only_mine:
+            self._only_mine -= 1
+        self.pool.release(node.page)
+        if node.parent is not None:
+            self._offer(node.parent)        # it may have become a leaf nobody uses
+
+    def _next_idle_leaf(self) -> Optional[_Node]:
+        while self._idle_leaves:
+            stamp, page = heapq.heappop(self._idle_leaves)
+            node = self._by_page.get(page)
+            if node is not None and node.stamp == stamp and node.only_mine and not node.children:
+                return node
+        return None
+
+    def _uncover(self) -> bool:
+        """No leaf can be given back, yet some page further up is held by the index alone (a request computed its
+        own copy of that page and went on from the index's).  Below the least recently used such page, the leaves
+        that requests still use are forgotten (the requests keep their pages; nothing is freed), and again until what
+        is left below it are pages of the index alone, whose leaves `evict` can then give back."""
+        buried = [n for n in self._by_page.values() if n.only_mine]
+        if not buried:
+            return False
+        top = min(buried, key=lambda n: n.stamp)
+        order, stack = [], list(top.children.values())
+        while stack:                        # the pages below `top`, every page before the pages under it
+            n = stack.pop()
+            order.append(n)
+            stack.extend(n.children.values())
+        for n in reversed(order):           # ... and now every page after the pages under it
+            if not n.children and not n.only_mine:
+                self._forget(n)
+        return True
 
     def evict(self, count: int) -> int:
-        """Gives back up to `count` pages nobody else uses, least recently used leaves first; returns how
-        many.  A page only the index holds may sit above a leaf a request still uses: then that leaf is
-        forgotten (the request keeps its page), which frees nothing yet but uncovers the page above."""
+        """Gives back up to `count` pages that nobody else holds, least recently used leaves first; returns how
+        many were given back."""
         freed = 0
         while freed < count:
-            victim, victim_frees = None, False
-            for page, e in self._entry.items():
-                if e.children:
-                    continue
-                frees = self.pool.ref_count(page) == 1
-                if not frees:
-                    above, a = False, e.parent
-                    while a != ROOT and not above:
-                        above = self.pool.ref_count(a) == 1
-                        a = self._entry[a].parent
-                    if not above:
-                        continue
-                if victim is None or (frees and not victim_frees) or (frees == victim_frees and e.tick < self._entry[victim].tick):
-                    victim, victim_frees = page, frees
-            if victim is None:
-                break
-            self._forget(victim)
-            freed += 1 if victim_frees else 0
+            node = self._next_idle_leaf()
+            if node is None:
+                if self._only_mine == 0 or not self._uncover():
+                    break
+                continue
+            self._forget(node)
+            freed += 1
         return freed
 
     def clear(self) -> None:
         """Forgets everything (pages that requests use stay with them)."""
-        for page in list(self._entry):
+        pages = list(self._by_page)
+        self._by_page.clear()
+        self._first.clear()
+        self._idle_leaves.clear()
+        self._only_mine = 0
+        for page in pages:
             self.pool.release(page)
-        self._entry.clear()
-        self._page_of.clear()

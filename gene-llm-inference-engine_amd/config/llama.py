@@ -12,12 +12,10 @@ import json
 from dataclasses import dataclass, asdict
 from typing import Optional
 
+from .errors import ConfigError
+from .registry import register_architecture
 from .spec import (AttentionSpec, LayerSpec, Llama3Scaling, ModelSpec, RmsNormSpec, RotarySpec,
                    RunEntry, SwiGluSpec)
-
-
-class ConfigError(ValueError):
-    """config.json cannot be run by this engine; the message names the key."""
 
 
 _MAX_INT = 100_000_000   # src/loader/hf_checkpoint.cpp:31
@@ -200,3 +198,6 @@ class LlamaConfig:
             lm_head=embedding if self.tie_word_embeddings else "lm_head.weight",
             layers=tuple(layers), run_order=tuple(RunEntry(l) for l in range(self.num_hidden_layers)),
             ignorable_tensors=tuple(ignorable))
+
+
+register_architecture(LlamaConfig.architecture, LlamaConfig, model_type=LlamaConfig.model_type)

@@ -3,7 +3,8 @@
 config.json names its architecture in `architectures[0]` (for instance "LlamaForCausalLM");
 files without that key are matched by `model_type`.  The reference has no registry: one class
 serves its two model types through a flag (src/loader/hf_checkpoint.cpp:96-111).  Here every
-architecture registers a configuration class with `from_dict(dict)` and `model_spec()`.
+architecture registers a configuration class with `from_dict(dict)` and `model_spec()`, from its
+own module; this one names none of them.
 """
 from __future__ import annotations
 
@@ -11,7 +12,7 @@ import json
 from pathlib import Path
 from typing import Dict
 
-from .llama import ConfigError, LlamaConfig
+from .errors import ConfigError
 
 _BY_ARCHITECTURE: Dict[str, type] = {}
 _BY_MODEL_TYPE: Dict[str, str] = {}
@@ -59,5 +60,3 @@ def read_config(folder):
         raise ConfigError(f"config.json: {e}") from None
     return parse_config(cfg)
 
-
-register_architecture(LlamaConfig.architecture, LlamaConfig, model_type=LlamaConfig.model_type)

@@ -69,6 +69,20 @@ class SwiGluSpec:
 
 
 @dataclass(frozen=True)
+class ScaleSpec:
+    """Rows multiplied by a constant (for instance a token table that is stored unscaled)."""
+    kind: ClassVar[str] = "scale"
+    factor: float
+
+
+@dataclass(frozen=True)
+class SoftCapSpec:
+    """x <- cap * tanh(x / cap): values kept within (-cap, cap)."""
+    kind: ClassVar[str] = "softcap"
+    cap: float
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One layer: which parts, and in which arrangement (`block`) they are wired."""
     mixer: Any
@@ -99,6 +113,8 @@ class ModelSpec:
     layers: Tuple[LayerSpec, ...]
     run_order: Tuple[RunEntry, ...]
     ignorable_tensors: Tuple[str, ...] = field(default=())   # regular expressions of names a file may hold unused
+    after_embedding: Tuple[Any, ...] = field(default=())     # row-transform specs applied, in order, to the rows of the token table
+    after_head: Tuple[Any, ...] = field(default=())          # ... and to the logits
 
     def __post_init__(self):
         for i, e in enumerate(self.run_order):

@@ -253,3 +253,26 @@ GI_API int gi_gather_rows(const float* x, const int* rows, float* out, int n_out
     GI_CHECK_LAUNCH("gather_rows");
     return 0;
 }
+
+// ------------------------------------------------------------------------------- row transforms
+// In place over float32 rows [n_rows, dim] with row stride `stride`: x <- x * factor, or x <- cap * tanh(x / cap).
+template <bool CAP>
+__global__ void rows_in_place_kernel(float* __restrict__ x, int dim, long stride, float c) {
+    float* row = x + (size_t)blockIdx.x * stride;
+    for (int d = blockIdx.y * blockDim.x + threadIdx.x; d < dim; d += gridDim.y * blockDim.x) row[d] = CAP ? c * tanhf(row[d] / c) : row[d] * c;
+}
+
+GI_API int gi_scale_rows(float* x, int n_rows, int dim, long stride, float factor, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && dim > 0 && stride >= dim, "scale_rows: bad sizes (rows %d, dim %d, stride %ld)", n_rows, dim, stride);
+    rows_in_place_kernel<false><<<dim3(n_rows, min(64, (dim + 1023) / 1024)), 256, 0, stream>>>(x, dim, stride, factor);
+    GI_CHECK_LAUNCH("scale_rows");
+    return 0;
+}
+
+GI_API int gi_softcap_rows(float* x, int n_rows, int dim, long stride, float cap, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && dim > 0 && stride >= dim, "softcap_rows: bad sizes (rows %d, dim %d, stride %ld)", n_rows, dim, stride);
+    GI_REQUIRE(cap > 0.f, "softcap_rows: the cap %g must be positive", (double)cap);
+    rows_in_place_kernel<true><<<dim3(n_rows, min(64, (dim + 1023) / 1024)), 256, 0, stream>>>(x, dim, stride, cap);
+    GI_CHECK_LAUNCH("softcap_rows");
+    return 0;
+}

@@ -466,15 +466,6 @@ int epilogue_of(int c_dtype, int accumulate) {
 
 }  // namespace
 
-// Number of k-splits the skinny kernel would use, so that the caller can size the scratch
-// (splits * M * N floats).  Enough workgroups to cover the chip, each with at least 256 of k.
-// Tuning knob: 0 lets the entry point choose the tile height of the tiled kernel, 64 or 128 forces it.
-static int g_force_bm = 0, g_piped = 1;
-GI_API void gi_gemm_bf16_set_tile(int bm) { g_force_bm = bm; }
-// Tuning knob: 0 sends large products to the register-staged tiled kernel instead of the LDS-ring kernel.
-GI_API void gi_gemm_bf16_set_piped(int on) { g_piped = on; }
-
-
 // Number of k-splits of the skinny kernel for a product with 17..64 rows, so that the caller can size
 // the scratch (splits * M * N floats); 0: the output is wide enough to fill the chip without a split,
 // no scratch is needed.  Enough workgroups to cover the chip, each with at least one block of k.
@@ -580,7 +571,7 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     }
 
     GI_REQUIRE((M + 63) / 64 <= 65535, "gemm_bf16: M %d is too large", M);
-    if (K % PK == 0 && N >= 128 && g_piped) {
+    if (K % PK == 0 && N >= 128) {
 #define PIPED(BM_, BN_, WM_, WN_, ST_, EPI_, OUT_, LDC_, SPLITS_, KPS_, SLAB_)                                                          \
     do {                                                                                                                                \
         constexpr int bytes = ST_ * (BM_ + BN_) * 128;                                                                                  \
@@ -623,7 +614,7 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
         return 0;
     }
 #define TILED(BM_, EPI_) gemm_bf16_tiled_kernel<BM_, EPI_><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
-    if (g_force_bm == 64 || (g_force_bm == 0 && (long)((M + 127) / 128) * ((N + BN - 1) / BN) < 512)) {   // few tiles: smaller ones fill more of the chip
+    if ((long)((M + 127) / 128) * ((N + BN - 1) / BN) < 512) {   // few tiles: smaller ones fill more of the chip
         dim3 grid((N + BN - 1) / BN, (M + 63) / 64);
         if (epi == EPI_STORE_F32) TILED(64, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(64, EPI_ADD_F32);
         else if (epi == EPI_STORE_BF16) TILED(64, EPI_STORE_BF16); else TILED(64, EPI_GATED_BF16);

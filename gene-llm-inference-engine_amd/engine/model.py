@@ -9,7 +9,7 @@ import torch
 
 from ..config import ModelSpec, read_config
 from ..kernels import ops
-from ..parts import LayerCache, StepContext, block_class, linear, model_tensor_needs, norm_class
+from ..parts import LayerCache, StepContext, block_class, linear, model_tensor_needs, norm_class, row_transform_class, weight_bytes
 from ..parts.linear import activation_dtype_for
 from ..weights import load_tensors, random_tensors
 
@@ -32,9 +32,11 @@ class DecoderModel:
         self.layers = [block_class(l.block)(l, tensors, dtype, device) for l in spec.layers]
         self.final_norm = norm_class(spec.final_norm)(spec.final_norm, tensors, dtype, device)
         self.head_in_dtype = activation_dtype_for(self.lm_head, dtype)
+        self.after_embedding = [row_transform_class(t)(t, tensors, dtype, device) for t in spec.after_embedding]
+        self.after_head = [row_transform_class(t)(t, tensors, dtype, device) for t in spec.after_head]
         self.run_order = spec.run_order
         self.trace = None                        # see set_trace
-        self.graph_safe = all(getattr(l, "graph_safe", False) for l in self.layers) and getattr(self.final_norm, "graph_safe", False)
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in (*self.layers, self.final_norm, *self.after_embedding, *self.after_head))
 
     # ----------------------------------------------------------------------------- what it needs
     def cache_needs(self):
@@ -43,15 +45,10 @@ class DecoderModel:
         return needs, [e.cache_of for e in self.run_order]
 
     def weight_bytes_read_per_step(self) -> int:
-        """Bytes of weights one step reads when it uses every matrix once (the token table is read by row)."""
-        seen, total = set(), 0
-        for block, entry in ((self.layers[e.layer], e) for e in self.run_order):
-            for part in (block.mixer, block.feed_forward, block.mixer_norm, block.feed_forward_norm):
-                for t in vars(part).values():
-                    if isinstance(t, torch.Tensor) and t.dtype in (torch.bfloat16, torch.float32):
-                        total += t.numel() * t.element_size()
-        total += self.lm_head.numel() * self.lm_head.element_size() + self.final_norm.weight.numel() * self.final_norm.weight.element_size()
-        return total
+        """Bytes of weights one step reads when it uses every matrix once: what every part of the run order holds (a
+        layer named twice is read twice), the final norm and the head; the token table is read by row and not counted."""
+        return (sum(weight_bytes(self.layers[e.layer]) for e in self.run_order) + weight_bytes(self.final_norm) + weight_bytes(self.lm_head)
+                + weight_bytes(self.after_embedding) + weight_bytes(self.after_head))
 
     # ------------------------------------------------------------------------------- the pass
     def forward(self, ctx: StepContext, cache, logit_rows: Optional[torch.Tensor], n_logit_rows: int):
@@ -59,6 +56,8 @@ class DecoderModel:
         [n_logit_rows, vocab] of the rows listed in `logit_rows`, or None if there are none."""
         x = torch.empty((ctx.n_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device)
         ops.embed(self.embedding, ctx.tokens, x)
+        for transform in self.after_embedding:
+            transform(x)
         trace = self.trace
         if trace is not None:
             trace("embedding", -1, x)
@@ -78,6 +77,8 @@ class DecoderModel:
             trace("final_norm", -1, normed if torch.is_tensor(normed) else self.final_norm(ops.gather_rows(x, logit_rows, torch.empty(
                 (n_logit_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device)), torch.float32))
         linear(normed, self.lm_head, logits)
+        for transform in self.after_head:
+            transform(logits)
         return logits
 
     def set_trace(self, trace) -> None:

@@ -163,13 +163,29 @@ class Runner:
         ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
                           row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0,
                           upload=self._uploads.put)
-        logits = self.model.forward(ctx, self._view, rows_dev, len(logit_rows))
+        logits = self._forward(ctx, rows_dev, len(logit_rows))
         self._uploads.end_step()
         for e in entries:
             self.cache.advance(e.request, len(e.tokens))
         self.steps_run += 1
         self.rows_run += n_rows
         return logits
+
+    def _forward(self, ctx: StepContext, rows_dev, n_logit_rows: int):
+        """The pass.  Fixed-size state is committed only by a pass that succeeds: parts write their state slots as they
+        go, so the slots of the step's requests are kept aside first and put back if the pass raises (the requests'
+        lengths have not moved yet, and pages reserved for the step stay with their requests for the next try)."""
+        states = self.cache.states
+        if not states:
+            return self.model.forward(ctx, self._view, rows_dev, n_logit_rows)
+        slots = torch.tensor(sorted(set(ctx.seg_slot)), dtype=torch.int64, device=self.model.device)
+        kept = {entry: state.index_select(0, slots) for entry, state in states.items()}
+        try:
+            return self.model.forward(ctx, self._view, rows_dev, n_logit_rows)
+        except BaseException:
+            for entry, state in states.items():
+                state.index_copy_(0, slots, kept[entry])
+            raise
 
     # --------------------------------------------------------------------------- captured decode
     @property

@@ -14,9 +14,11 @@ Policy, as the reference's engine (src/runtime/engine.cpp:64-205):
     nothing had happened.
   * prefix sharing (on unless the configuration or the model's cache rules it out): a request that starts with
     tokens an earlier request has processed takes that request's full pages and is fed from there (at least its
-    last token is always fed: it produces the logits).  Pages only the prefix index still holds count as free when
-    rows are planned and are given back before the step that needs them.  A preempted request is closed like any
-    other, so what it had computed usually serves it again when it returns.
+    last token is always fed: it produces the logits).  The index of such pages belongs to the cache manager and
+    outlives the scheduler that filled it; pages only the index still holds count as free when rows are planned,
+    and any reservation that needs them takes them back (this scheduler's, another one's on the same runner, a lone
+    `generate`).  A preempted request is closed like any other, so what it had computed usually serves it again
+    when it returns.
   * only the row of a request's last known token returns logits; the request's own sampler draws
     the next token from them.  A sampled end token finishes the request (it stays the last
     generated token); so does reaching `max_positions` (prompt plus generated tokens).
@@ -123,6 +125,7 @@ class Engine:
         self.waiting: Deque[_Job] = deque()
         self.running: List[_Job] = []                                    # in admission order
         self.stats = EngineStats()
+        self._evicted_before = runner.cache.evicted_pages
         # decoding ahead: the step in the queue, and two pinned buffers its tokens come back through in turn
         self._flight: Optional[_Flight] = None
         self._landing_strips, self._strip = None, 0
@@ -194,9 +197,7 @@ class Engine:
         """The rows of the next step: [(job, n_rows)] in step order, decoding requests first.
         Empty if not even one row fits in the free pages."""
         cache = self.runner.cache
-        free = cache.free_pages()
-        if self.prefix is not None:
-            free[0] += cache.evictable_pages()         # pages only the prefix index holds can be given back
+        free = cache.available_pages()             # pages only the prefix index holds are taken back by the step's reservation
         budget = self.cfg.step_rows
         taken = []
         for phase in (0, 1):
@@ -236,10 +237,6 @@ class Engine:
             entries.append(StepEntry(job.key, job.tokens[job.fed:job.fed + n], (n - 1,) if last else ()))
             if last:
                 wanting.append(job)
-        if self.prefix is not None:                  # make room: the plan counted pages that the prefix index still holds
-            cache = self.runner.cache
-            needed = sum(cache.pages_needed(job.key, n)[0] for job, n in taken)
-            self.stats.evicted_pages += cache.evict(needed - cache.free_pages()[0])
         logits = self.runner.step(entries)
         self._count_pass(taken)
 
@@ -258,6 +255,7 @@ class Engine:
     def _count_pass(self, taken) -> None:
         st = self.stats
         st.passes += 1
+        st.evicted_pages = self.runner.cache.evicted_pages - self._evicted_before
         n_rows = sum(n for _, n in taken)
         st.rows += n_rows
         st.max_rows_in_pass = max(st.max_rows_in_pass, n_rows)
@@ -309,10 +307,6 @@ class Engine:
                    and self.runner.can_step_from_device)
         if goes_on:
             try:
-                if self.prefix is not None:
-                    cache = self.runner.cache
-                    needed = sum(cache.pages_needed(j.key, 1)[0] for j in jobs)
-                    self.stats.evicted_pages += cache.evict(needed - cache.free_pages()[0])
                 logits = self.runner.step_from_device([j.key for j in jobs], flight.tokens)
             except OutOfPages:                       # nothing has changed: the step after the landing sorts it out
                 logits = None

@@ -29,6 +29,8 @@ _SIGNATURES = {
                       c_int, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_silu_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "gi_gather_rows": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "gi_scale_rows": [c_void_p, c_int, c_int, c_long, c_float, c_void_p],
+    "gi_softcap_rows": [c_void_p, c_int, c_int, c_long, c_float, c_void_p],
     "gi_gemm_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
                            c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
@@ -297,6 +299,24 @@ def gather_rows(x, rows, out):
     return out
 
 
+def _rows_in_place(name, x, c):
+    _dev(x)
+    if not (x.dim() == 2 and x.dtype == torch.float32 and x.stride(1) == 1):
+        raise KernelError(f"{name}: x must be float32 [n, dim] with unit inner stride")
+    _call("gi_" + name, x.data_ptr(), x.shape[0], x.shape[1], x.stride(0), float(c), _stream())
+    return x
+
+
+def scale_rows(x, factor):
+    """x *= factor, in place."""
+    return _rows_in_place("scale_rows", x, factor)
+
+
+def softcap_rows(x, cap):
+    """x = cap * tanh(x / cap), in place."""
+    return _rows_in_place("softcap_rows", x, cap)
+
+
 def gemm_exact(a, w, out, accumulate=False):
     """out (=|+=) a @ w.T in 32-bit arithmetic with one summation order for every batch size."""
     _dev(a, w, out)
@@ -340,7 +360,6 @@ class AttentionPlan:
     for the whole chip (break-even near 90 rows at the Llama-3.2-1B shape; above SHORT_TOTAL rows
     in all, the rows' repeated reading of the context costs more than the tiles' sequence).
     Made once per step and used by every layer."""
-    TILE = int(__import__("os").environ.get("GI_ATTENTION_TILE", "0"))        # rows of a prompt tile, 64 or 128; 0: by the step's size
     SMALL_STEP = 768                     # up to this many tiled rows in a step, tiles of 64 rows fill the chip better (measured at 32 heads)
     PAIRS = True                         # a portion's late tiles share workgroups with its early ones
     SHORT, SHORT_TOTAL = 64, 64          # portions of up to SHORT rows count as short; they go row by row while they sum to at most SHORT_TOTAL
@@ -360,7 +379,7 @@ class AttentionPlan:
         short_rows = sum(n for n in seg_len if 1 < n <= self.SHORT)
         row_by_row = self.SHORT if short_rows <= self.SHORT_TOTAL else 1
         self.single_rows = all(n == 1 for n in seg_len)          # every row is a request's only new row
-        self.tile = self.TILE or (64 if sum(n for n in seg_len if n > row_by_row) <= self.SMALL_STEP else 128)
+        self.tile = 64 if sum(n for n in seg_len if n > row_by_row) <= self.SMALL_STEP else 128        # rows of a prompt tile
         for start, n, pos0, slot in zip(seg_start, seg_len, seg_pos0, seg_slot):
             if n <= row_by_row:
                 dec.extend(range(start, start + n))

@@ -1,8 +1,9 @@
 """Parts of a layer (mixer, feed-forward, norm, position encoding, block) and their registries."""
-from .base import (FeedForward, LayerCache, Mixer, Norm, Part, PositionEncoding, StepContext, block_class,
+from .base import (FeedForward, LayerCache, Mixer, Norm, Part, PositionEncoding, RowTransform, StepContext, block_class,
                    feed_forward_class, mixer_class, norm_class, position_class, register_block, register_feed_forward,
-                   register_mixer, register_norm, register_position_encoding)
-from . import norm, rope, attention, mlp, block          # registers the built-in kinds
+                   register_mixer, register_norm, register_position_encoding, register_row_transform, row_transform_class,
+                   weight_bytes, weight_tensors)
+from . import norm, rope, attention, mlp, block, transform          # registers the built-in kinds
 from .linear import linear
 from ..weights.loader import TensorNeed
 

@@ -3,7 +3,12 @@
 Order of operations as the reference's pass (src/gpu/gpu_transformer.cpp:390-409): q, k, v
 products; rotation of q and k; all new keys and values are written to their pages; then every
 row attends over its request's pages up to its own position; output product added onto the
-residual.  The three input products run as one with the stacked matrix [q; k; v]."""
+residual.  The three input products run as one with the stacked matrix [q; k; v].
+
+The position encoding is a part of its own (`spec.position`).  One that turns the pairs
+(i, i + head_dim/2) of whole heads hands over its cosines and sines, and the kernel that writes the
+pages (or, for a few decoded rows, the attention kernel itself) applies them; any other encoding
+changes q and k in place with its own kernels first, and the pages are then written unrotated."""
 from __future__ import annotations
 
 import torch
@@ -16,7 +21,6 @@ from .linear import activation_dtype_for, linear
 
 
 class Attention(Mixer):
-    graph_safe = True
     accepts_deferred_norm = True      # its input goes into `linear` only
 
     def __init__(self, spec, tensors, dtype, device):
@@ -30,6 +34,7 @@ class Attention(Mixer):
         self.position = None if s.position is None else position_class(s.position)(s.position, tensors, dtype, device)
         self.in_dtype = activation_dtype_for(self.w_qkv, dtype)
         self.att_dtype = activation_dtype_for(self.w_o, dtype)
+        self.graph_safe = self.position is None or bool(getattr(self.position, "graph_safe", False))
 
     @classmethod
     def tensor_needs(cls, spec):
@@ -43,7 +48,8 @@ class Attention(Mixer):
 
     def forward(self, h, residual, ctx, cache):
         s, T = self.spec, ctx.n_rows
-        cos, sin = self.position.prepare(ctx) if self.position is not None else (None, None)
+        tables = self.position.half_split_tables(ctx) if self.position is not None else None
+        cos, sin = tables if tables is not None else (None, None)
         att = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
         if cache.writes:
             qkv = torch.empty((T, self.a_dim + 2 * self.kv_dim), dtype=torch.float32, device=ctx.device)
@@ -52,6 +58,8 @@ class Attention(Mixer):
         else:                       # the pages are another layer's: only the queries are made
             q, k, v = torch.empty((T, self.a_dim), dtype=torch.float32, device=ctx.device), None, None
             linear(h, self.w_qkv[:self.a_dim], q)
+        if self.position is not None and tables is None:          # an encoding with kernels of its own: q and k are turned in place
+            self.position.apply(q, k, ctx, s.n_heads, s.n_kv_heads, s.head_dim)
         # a step of single decoded rows: one kernel rotates, writes the pages and attends
         if not ops.attention_from_products(q, k, v, cos, sin, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, s.window):
             q_rot = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)

@@ -9,7 +9,10 @@ manager).
 Kinds of parts and what each must provide:
 
 * norm:              `tensor_needs(spec)`, `__call__(x_f32[T, size], out_dtype) -> [T, size]`
-* position encoding: `prepare(ctx) -> tables` (made once per step and kept in ctx.memo)
+* position encoding: `apply(q, k, ctx, ...)` turns the float32 queries and keys of a step's rows in place, with
+                     kernels of its own; or `half_split_tables(ctx) -> (cos, sin)` if it is a rotation of the pairs
+                     (i, i + head_dim/2) of whole heads, which the attention kernels apply themselves
+* row transform:     `__call__(x_f32[T, n])` changes rows in place (after the embedding, or on the logits)
 * mixer:             `tensor_needs(spec)`, `cache_need(spec)`, `forward(h, residual, ctx, cache)`
 * feed-forward:      `tensor_needs(spec)`, `forward(h, residual, ctx)`
 * block:             `forward(x, ctx, cache)` wiring norms, mixer and feed-forward around the
@@ -90,6 +93,9 @@ class Part:
 
 
 class Mixer(Part):
+    """A mixer with a `StateNeed` takes the rows of a request in order, reads `cache.state[slot]` at the first and may
+    write it as it goes: the step function puts the slots of a step's requests back as they were if the pass raises."""
+
     @classmethod
     def cache_need(cls, spec):
         """A `PagedKvNeed`, a `StateNeed` or None."""
@@ -110,11 +116,64 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    def prepare(self, ctx: StepContext):
+    """How positions enter a mixer's queries and keys.  A mixer asks `half_split_tables` first: an encoding that
+    turns the pairs (i, i + head_dim/2) of every whole head by an angle per (row, pair) answers with the angles'
+    cosines and sines, and the kernels that write the cache and attend apply them on the way (nothing is launched
+    for the rotation).  Every other encoding (another pairing, a part of the head only, something that is no
+    rotation) answers None and gets `apply` called with the rows' float32 queries and keys, which it changes in
+    place with kernels of its own before they are stored and attended over."""
+
+    def half_split_tables(self, ctx: StepContext):
+        """(cos, sin), float32 [rows, head_dim/2] each, made once per step (kept in ctx.memo), or None."""
+        return None
+
+    def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], ctx: StepContext, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
+        """q: float32 [rows, n_heads*head_dim], k: float32 [rows, n_kv_heads*head_dim] or None (the keys are another
+        entry's); both may be column ranges of a wider tensor (unit inner stride, any row stride)."""
+        raise NotImplementedError(f"{type(self).__name__} gives neither half-split tables nor an apply step")
+
+
+class RowTransform(Part):
+    """An elementwise change of float32 rows in place: what a model may ask for between the token table and the
+    first layer, and on the logits."""
+
+    def __call__(self, x: torch.Tensor) -> None:
         raise NotImplementedError
 
 
-_REGISTRIES: Dict[str, Dict[str, type]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}}
+def weight_tensors(obj, _seen=None):
+    """The floating-point tensors that `obj` (a part, a block, a list of them) holds, each object visited once:
+    what a step reads of it when it uses every weight once.  A part whose step reads other tensors than it holds
+    (experts of which only some run) says which in a method `weights_read_per_step()`."""
+    seen = _seen if _seen is not None else set()
+    if id(obj) in seen:
+        return
+    seen.add(id(obj))
+    if torch.is_tensor(obj):
+        if obj.dtype in (torch.bfloat16, torch.float32, torch.float16):
+            yield obj
+    elif isinstance(obj, (list, tuple)):
+        for v in obj:
+            yield from weight_tensors(v, seen)
+    elif isinstance(obj, dict):
+        for v in obj.values():
+            yield from weight_tensors(v, seen)
+    elif callable(getattr(obj, "weights_read_per_step", None)):
+        yield from weight_tensors(list(obj.weights_read_per_step()), seen)
+    elif isinstance(obj, Part) or callable(getattr(obj, "forward", None)):
+        for v in vars(obj).values():
+            yield from weight_tensors(v, seen)
+
+
+def weight_bytes(obj) -> int:
+    """Bytes of `weight_tensors(obj)`, memory that several of them name counted once."""
+    by_address: Dict[int, int] = {}
+    for t in weight_tensors(obj):
+        by_address[t.data_ptr()] = max(by_address.get(t.data_ptr(), 0), t.numel() * t.element_size())
+    return sum(by_address.values())
+
+
+_REGISTRIES: Dict[str, Dict[str, type]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}, "row_transform": {}}
 
 
 def _register(family: str, kind: str, cls: type) -> None:
@@ -136,6 +195,7 @@ def register_feed_forward(kind, cls): _register("feed_forward", kind, cls)
 def register_norm(kind, cls): _register("norm", kind, cls)
 def register_position_encoding(kind, cls): _register("position", kind, cls)
 def register_block(kind, cls): _register("block", kind, cls)
+def register_row_transform(kind, cls): _register("row_transform", kind, cls)
 
 
 def mixer_class(spec): return _lookup("mixer", spec.kind)
@@ -143,3 +203,4 @@ def feed_forward_class(spec): return _lookup("feed_forward", spec.kind)
 def norm_class(spec): return _lookup("norm", spec.kind)
 def position_class(spec): return _lookup("position", spec.kind)
 def block_class(kind: str): return _lookup("block", kind)
+def row_transform_class(spec): return _lookup("row_transform", spec.kind)

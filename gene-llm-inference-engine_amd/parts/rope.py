@@ -44,7 +44,7 @@ class RotaryHalfSplit(PositionEncoding):
         self.half = spec.head_dim // 2
         self.inv_freq = torch.tensor(inverse_frequencies(spec.head_dim, spec.theta, spec.scaling), dtype=torch.float64, device=device)
 
-    def prepare(self, ctx):
+    def half_split_tables(self, ctx):
         """(cos, sin), float32 [T, head_dim/2], for the rows of this step."""
         key = ("rotary", self.spec)
         if key not in ctx.memo:

@@ -414,3 +414,55 @@ def test_rewind_is_refused_where_the_past_is_gone():
     s.reserve([("a", 5)]); s.advance("a", 5)
     with pytest.raises(CacheError, match="fixed-size state"):
         s.truncate("a", 2)
+
+
+def test_prefix_index_counts_hold_under_random_use():
+    """Random requests over a small alphabet (so that beginnings repeat) open on matched pages, fill pages, name them, end;
+    now and then pages are taken back.  At every point the index's constant-time count equals a recount, every page it
+    names has a place under its parent, `evict(k)` gives back min(k, evictable) pages, and at the end nothing is lost."""
+    import random
+    from geneinfer_amd.cache import PagePool, PrefixIndex
+    rng = random.Random(3)
+    pool = PagePool(40)
+    index = PrefixIndex(pool, page_size=2)
+    live = {}                                                                      # request -> (tokens, pages it holds)
+    for turn in range(600):
+        roll = rng.random()
+        if roll < 0.45 and len(live) < 5:
+            tokens = [rng.randrange(3) for _ in range(rng.choice([2, 4, 5, 8, 12]))]
+            pages = index.match(tokens, len(tokens) - 1)
+            need = -(-len(tokens) // 2) - len(pages)
+            if need > pool.free_count:
+                short, could = need - pool.free_count, recount(index, pool)
+                assert index.evict(short) == min(short, could)
+            if need > pool.free_count:
+                for p in pages:
+                    pool.release(p)
+                continue
+            pages += [pool.allocate() for _ in range(need)]
+            index.insert(tokens, len(tokens), pages)
+            live[turn] = (tokens, pages)
+        elif roll < 0.85 and live:
+            _, pages = live.pop(rng.choice(list(live)))
+            for p in reversed(pages):
+                pool.release(p)
+        else:
+            k, before, could = rng.randint(1, 6), pool.free_count, recount(index, pool)
+            assert index.evict(k) == min(k, could) == pool.free_count - before
+        assert index.evictable() == recount(index, pool)
+        assert pool.free_count + len(set(p for _, pages in live.values() for p in pages) | set(index.pages())) == pool.n_pages
+        for page in index.pages():
+            node = index._by_page[page]
+            assert index._children_of(node.parent)[node.tokens] is node and pool.ref_count(page) >= 1
+    for _, pages in live.values():
+        for p in pages:
+            pool.release(p)
+    assert index.evictable() == len(index)
+    named, free = len(index), pool.free_count
+    assert index.evict(named // 2) == named // 2 and pool.free_count == free + named // 2
+    index.clear()
+    assert pool.free_count == pool.n_pages and len(index) == 0
+
+
+def recount(index, pool):
+    return sum(1 for page in index.pages() if pool.ref_count(page) == 1)

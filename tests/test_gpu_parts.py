@@ -51,11 +51,11 @@ def test_rotary_part_tables_are_shared_within_a_step():
     spec = RotarySpec(32, 500000.0, Llama3Scaling(4.0, 1.0, 4.0, 32))
     part = position_class(spec)(spec, {}, torch.float32, DEV)
     ctx = step_context([(0, 35, 4), (1, 0, 1)], torch.float32)
-    cos, sin = part.prepare(ctx)
+    cos, sin = part.half_split_tables(ctx)
     inv = rope_inverse_frequencies(32, 500000.0, dict(factor=4.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=32))
     ang = ctx.row_pos.cpu().double()[:, None] * inv[None, :]
     assert (cos.cpu().double() - ang.cos()).abs().max() < 1e-7 and (sin.cpu().double() - ang.sin()).abs().max() < 1e-7
-    again = position_class(spec)(spec, {}, torch.float32, DEV).prepare(ctx)
+    again = position_class(spec)(spec, {}, torch.float32, DEV).half_split_tables(ctx)
     assert again[0] is cos                                            # a second layer with the same spec reuses the step's tables
 
 
@@ -134,17 +134,26 @@ def test_registries_refuse_unknown_kinds_and_double_registration():
 
 
 # ------------------------------------------------------------------------------------ toy model
-@pytest.fixture(scope="module")
-def toy_model(tmp_path_factory):
+# Two toy configurations that differ in every size and constant.  The second has heads of 32 channels, which the
+# matrix-core attention kernels take in bfloat16 with pages of 16 positions: its windowed layer then feeds those
+# kernels page tables with entries that the window has given back.
+TOYS = {"small": (toy.ToyConfig(), [40, 9, 63, 21, 34], 5),
+        "wide": (toy.ToyConfig(hidden_size=64, intermediate_size=96, num_attention_heads=4, num_key_value_heads=2, head_dim=32, vocab_size=173,
+                               window=20, decay=0.6, angle_step=0.03, rotary_dim=20, embedding_scale=0.8, logit_cap=5.0, num_experts=2,
+                               expert_intermediate_size=40, rms_norm_eps=3e-6, max_position_embeddings=320), [40, 9, 150, 21, 100], 6)}
+
+
+@pytest.fixture(scope="module", params=list(TOYS))
+def toy_model(request, tmp_path_factory):
     from geneinfer_amd.weights import write_random_model
     toy.register()
     toy.register()                                                    # registering the same classes again is harmless
-    cfg = toy.ToyConfig()
+    cfg, lengths, seed = TOYS[request.param]
     folder = tmp_path_factory.mktemp("toy")
-    write_random_model(folder, cfg, seed=5, dtype="bfloat16", std=0.2)
+    write_random_model(folder, cfg, seed=seed, dtype="bfloat16", std=0.2)
     _, weights = read_model_folder(folder)
     rng = random.Random(4)
-    requests = {f"t{i}": [rng.randrange(cfg.vocab_size) for _ in range(n)] for i, n in enumerate([40, 9, 63, 21, 34])}
+    requests = {f"t{i}": [rng.randrange(cfg.vocab_size) for _ in range(n)] for i, n in enumerate(lengths)}
     # the routed feed-forward is exercised: every expert is some row's choice, and no choice hangs on the last digits
     top2 = torch.cat([torch.topk(toy.router_logits(cfg, weights, toks), 2, dim=-1).values for toks in requests.values()])
     chosen = torch.cat([toy.router_logits(cfg, weights, toks).argmax(-1) for toks in requests.values()])
@@ -153,20 +162,29 @@ def toy_model(tmp_path_factory):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("mode", ["whole", "tail_singly", "portions", "mixed"])
+@pytest.mark.parametrize("mode", ["whole", "tail_singly", "portions", "long_portions", "mixed"])
 def test_toy_architecture_under_every_cut(toy_model, dtype, mode):
     from geneinfer_amd.cache import PagedKvNeed, StateNeed
     from geneinfer_amd.engine import Runner, StepEntry, load_model
+    from geneinfer_amd.parts import weight_bytes
     cfg, folder, weights, requests = toy_model
     model = load_model(folder, dtype, DEV)                            # config.json names the toy architecture; nothing else does
     assert type(model.config) is toy.ToyConfig
+    # portions of 40, 110, ... rows: a portion long enough for the tiled prompt kernel begins behind pages the window gave back
     steps = {"whole": traces.whole, "tail_singly": lambda r: traces.tail_singly(r, 32), "portions": traces.portions,
-             "mixed": lambda r: traces.mixed(r, seed=8)}[mode](requests)
+             "long_portions": lambda r: traces.portions(r, sizes=(40, 110, 70)), "mixed": lambda r: traces.mixed(r, seed=8)}[mode](requests)
     runner = Runner(model, page_size=16 if dtype == "bfloat16" else 4, max_tokens=traces.peak_tokens(steps, 16), max_requests=4)
     groups = runner.cache.groups
     assert [(g.need.window, g.entries) for g in groups] == [(None, [1, 4]), (cfg.window, [2])]      # entry 5 reads entry 2's pages
     assert list(runner.cache.states) == [0, 3] and runner.cache.state(3).shape == (4, cfg.hidden_size)      # both decay mixers
+    # what a step reads of the weights is asked of the parts, whatever a block calls them: every tensor of the file but the
+    # token table, the two attention layers that run twice counted twice
+    by_layer = lambda l: sum(4 * t.numel() for n, t in weights.items() if n.startswith(f"layers.{l}."))
+    in_float32 = sum(by_layer(l) for l in (3, 0, 1, 2, 0, 1)) + 4 * weights["final_norm"].numel() + 4 * weights["head"].numel()
+    read = model.weight_bytes_read_per_step()
+    assert read == in_float32 if dtype == "float32" else in_float32 // 2 <= read < in_float32
     where, got = traces.wanted_positions(steps), {}
+    gave_back = 0
     for s in steps:
         for e in s["entries"]:
             if not runner.is_open(e["id"]):
@@ -174,11 +192,13 @@ def test_toy_architecture_under_every_cut(toy_model, dtype, mode):
         logits = runner.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
         for row, key in zip(logits.cpu(), where[s["step"]]):
             got[key] = row
+        gave_back += sum(int(groups[1].first_live[runner.cache.slot(r)]) > 0 for r in runner.cache.open_requests())
         for rid in s["end"]:
             runner.close(rid)
         runner.cache.check_consistency()
         held = [sum(len(g.held_pages(runner.cache.slot(r))) for r in runner.cache.open_requests()) for g in groups]
         assert held[1] <= len(runner.cache.open_requests()) * (2 + (cfg.window + 8) // runner.page_size + 1)     # windowed pages are given back
+    assert gave_back > 0, "no request ever ran with pages that its window had given back"
     assert runner.cache.free_pages() == [g.pool.n_pages for g in groups]
     exact = {rid: toy.plain_logits(cfg, weights, toks) for rid, toks in requests.items()}
     if dtype == "float32":
@@ -188,3 +208,28 @@ def test_toy_architecture_under_every_cut(toy_model, dtype, mode):
         rounded = {rid: toy.plain_logits(cfg, weights, toks, store=lambda t: t.to(torch.bfloat16).double()) for rid, toks in requests.items()}
         assert_within_bfloat16_noise(got, lambda k: exact[k[0]][k[1]], lambda k: rounded[k[0]][k[1]], mode)
     assert runner.use_graphs is False                                 # the toy mixer reads host-side step data: no step of this model is captured
+
+
+def test_a_pass_that_raises_leaves_state_and_lengths_as_they_were(toy_model):
+    """The second decay mixer of the run order fails once, after the first one has written its state: the step raises, the
+    state slots and the request's length are what they were, and the same step then gives the logits of an undisturbed run."""
+    from geneinfer_amd.engine import Runner, StepEntry, load_model
+    cfg, folder, weights, requests = toy_model
+    toks = requests["t0"]
+    model = load_model(folder, "float32", DEV)
+    runner = Runner(model, page_size=4, max_tokens=256, max_requests=2)
+    runner.open("a")
+    runner.step([StepEntry("a", toks[:7], ())])
+    before = {e: s.clone() for e, s in runner.cache.states.items()}
+    late = model.layers[2].mixer                                      # runs after layer 3's mixer (run-order entry 0)
+    def failing(h, residual, ctx, cache):
+        raise RuntimeError("no luck")
+    late.forward = failing
+    with pytest.raises(RuntimeError, match="no luck"):
+        runner.step([StepEntry("a", toks[7:12], (4,))])
+    del late.forward
+    assert runner.length("a") == 7 and all(torch.equal(s, before[e]) for e, s in runner.cache.states.items())
+    got = runner.step([StepEntry("a", toks[7:12], (4,))])[0].cpu()
+    assert relative_error(got, toy.plain_logits(cfg, weights, toks[:12])[11]) < 2e-5
+    runner.close("a")
+    runner.cache.check_consistency()

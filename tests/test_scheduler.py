@@ -315,3 +315,45 @@ def test_step_uploads_ring_on_the_cpu():
         kept.append((step, piece))
         for s, p in kept[-(_StepUploads.DEPTH - 1):]:         # the pieces of the last steps are still what they were
             assert p.tolist() == [100 * s + i for i in range(5)]
+
+
+def test_pages_the_prefix_index_keeps_serve_whoever_reserves_next():
+    """The index belongs to the cache manager and outlives the scheduler that filled it: on a pool that only fits after
+    index-only pages are taken back, a lone `generate`, a scheduler without prefix sharing and a bare reservation all
+    run, and none of them finds the pool too small."""
+    runner = FakeRunner(page_size=4, n_pages=8, max_requests=2, max_positions=32)
+    filler = Engine(runner, EngineConfig(max_running=1, prefix_cache=True), sample=host_sample)
+    prompt = list(range(1, 27))
+    filler.submit(EngineRequest(prompt, 28, SamplerConfig(temperature=0.0)))
+    filler.run_until_idle()
+    cache = runner.cache
+    assert cache.prefix is not None and cache.evictable_pages() == 7 and cache.free_pages() == [1]      # 28 positions: 7 full pages stay named
+    # a lone request through the single-request loop
+    other = [40 + i % 9 for i in range(20)]
+    got = generate(runner, Sampler(SamplerConfig(temperature=0.0), VOCAB), other, 24, sample=host_sample_row)
+    assert got.generated_tokens == alone(other, 24, SamplerConfig(temperature=0.0), ())[0]
+    assert cache.evicted_pages >= 5
+    # refill the index, then a scheduler that does not share prefixes
+    filler.submit(EngineRequest(prompt, 28, SamplerConfig(temperature=0.0)))
+    filler.run_until_idle()
+    assert cache.free_pages()[0] + cache.evictable_pages() == 8 and cache.evictable_pages() >= 6
+    plain = Engine(runner, EngineConfig(max_running=1, prefix_cache=False), sample=host_sample)
+    jid = plain.submit(EngineRequest(other, 24, SamplerConfig(temperature=0.0)))
+    plain.run_until_idle()
+    assert plain.result(jid).error == "" and plain.result(jid).generated_tokens == got.generated_tokens
+    assert plain.stats.evicted_pages > 0
+    # and a bare reservation
+    filler.submit(EngineRequest(prompt, 28, SamplerConfig(temperature=0.0)))
+    filler.run_until_idle()
+    runner.open("bare")
+    runner.open("second")
+    assert cache.fits([("bare", 26)]) and not cache.fits([("bare", 26), ("second", 5)])
+    cache.reserve([("bare", 26)])
+    cache.advance("bare", 26)
+    cache.check_consistency()
+    with pytest.raises(OutOfPages):
+        cache.reserve([("second", 5)])
+    cache.reserve([("second", 4)])
+    runner.close("bare")
+    runner.close("second")
+    assert pages_when_forgotten(runner) == [8]

@@ -2,8 +2,11 @@
 needs are data: it is registered, built, loaded and stepped through the framework's public
 interfaces without a change to the framework's files.
 
-Layers (pre-norm blocks with RMS norms unless said otherwise): 0 full attention whose positions are encoded by a toy rule of its own (angles
-pos * step * (k + 1) instead of the rotary frequencies), 1 windowed attention, 2 a "decay" mixer
+Layers (pre-norm blocks with RMS norms unless said otherwise): 0 full attention whose positions are encoded by a
+rule and a pairing of its own (neighbouring channels (2i, 2i+1) of the first `rotary_dim` channels of a head are
+turned by pos * step * (i + 1), the rest of the head is left alone: the encoding applies itself to q and k),
+1 windowed attention with half-split pairs but angles of its own (pos * step * (k + 1): the encoding hands the
+attention kernels its cosines and sines), 2 a "decay" mixer
 with a state of its own (s <- decay * s + h per row, out = W s), each followed by SwiGLU, layer 2
 in a block arrangement of its own (mixer and feed-forward both read one norm of the block's input, a
 norm that also removes the mean, and both add onto the residual stream); 3 a
@@ -12,7 +15,8 @@ SwiGLU experts per row and scales it by the router's probability of it).  Run or
 then layer 0 once more (a cache of its own) and layer 1 once more reading the pages of its first
 run.  Layer 3 runs first so that the router sees values computed in 32-bit on both sides of the
 comparison (embedding, norm, decay mixer): in bfloat16 the engine and the plain model then take
-the same expert unless two router logits agree to six digits.
+the same expert unless two router logits agree to six digits.  The rows of the token table are scaled by a
+constant before the first layer and the logits are capped softly (the model's two row-transform places).
 """
 from __future__ import annotations
 
@@ -22,12 +26,12 @@ from typing import ClassVar
 import torch
 
 from geneinfer_amd.cache import StateNeed
-from geneinfer_amd.config import (AttentionSpec, LayerSpec, ModelSpec, RmsNormSpec, RotarySpec, RunEntry, SwiGluSpec,
+from geneinfer_amd.config import (AttentionSpec, LayerSpec, ModelSpec, RmsNormSpec, RunEntry, ScaleSpec, SoftCapSpec, SwiGluSpec,
                                   register_architecture)
 from geneinfer_amd.parts import (FeedForward, Mixer, Norm, PositionEncoding, feed_forward_class, mixer_class, norm_class, register_block,
                                  register_feed_forward, register_mixer, register_norm, register_position_encoding)
 from geneinfer_amd.weights import TensorNeed
-from plain_llama import causal_attention, rms_norm, rope_inverse_frequencies, rope_rotate, swiglu
+from plain_llama import causal_attention, rms_norm, rope_rotate, swiglu
 
 
 @dataclass(frozen=True)
@@ -96,7 +100,7 @@ class ParallelBlock:
 
     def __init__(self, spec, tensors, dtype, device):
         self.spec = spec
-        self.mixer_norm = self.feed_forward_norm = norm_class(spec.mixer_norm)(spec.mixer_norm, tensors, dtype, device)
+        self.mixer_norm = norm_class(spec.mixer_norm)(spec.mixer_norm, tensors, dtype, device)
         self.mixer = mixer_class(spec.mixer)(spec.mixer, tensors, dtype, device)
         self.feed_forward = feed_forward_class(spec.feed_forward)(spec.feed_forward, tensors, dtype, device)
 
@@ -124,16 +128,58 @@ class LinearAnglesSpec:
 
 
 class LinearAngles(PositionEncoding):
-    """Pair k of a head is turned by pos * step * (k + 1).  What an attention part asks of a position
-    encoding is `prepare(ctx) -> (cos, sin)`, float32 [rows, head_dim / 2]."""
+    """Pair (k, k + head_dim/2) of a head is turned by pos * step * (k + 1): a rotation of half-split pairs over the
+    whole head, so the attention kernels apply it themselves from `half_split_tables(ctx) -> (cos, sin)`, float32
+    [rows, head_dim / 2]."""
+    graph_safe = True                                         # everything step-dependent is read on the device
 
-    def prepare(self, ctx):
+    def half_split_tables(self, ctx):
         key = ("toy_linear_angles", self.spec)
         if key not in ctx.memo:
             k = torch.arange(1, self.spec.head_dim // 2 + 1, dtype=torch.float64, device=ctx.device)
             angles = ctx.row_pos.double()[:, None] * (self.spec.step * k)[None, :]
             ctx.memo[key] = (torch.cos(angles).float().contiguous(), torch.sin(angles).float().contiguous())
         return ctx.memo[key]
+
+
+@dataclass(frozen=True)
+class NeighbourPairsSpec:
+    kind: ClassVar[str] = "toy_neighbour_pairs"
+    head_dim: int
+    rotary_dim: int                   # the first so many channels of a head are turned, in pairs (2i, 2i + 1)
+    step: float
+
+
+class NeighbourPairs(PositionEncoding):
+    """Another pairing, and only a part of the head: no half-split tables, so the attention part calls `apply` with
+    the rows' float32 queries and keys (column ranges of the stacked product) and stores them as they come back."""
+    graph_safe = True
+
+    def apply(self, q, k, ctx, n_heads, n_kv_heads, head_dim):
+        assert head_dim == self.spec.head_dim and q.dtype == torch.float32 and q.shape == (ctx.n_rows, n_heads * head_dim)
+        half = self.spec.rotary_dim // 2
+        i = torch.arange(1, half + 1, dtype=torch.float64, device=ctx.device)
+        angles = ctx.row_pos.double()[:, None] * (self.spec.step * i)[None, :]
+        cos, sin = torch.cos(angles).float()[:, None, :], torch.sin(angles).float()[:, None, :]
+        for x, heads in ((q, n_heads), (k, n_kv_heads)):
+            if x is None:
+                continue
+            v = x.unflatten(1, (heads, head_dim))                 # a view: x may be a column range of a wider tensor
+            a, b = v[..., 0:2 * half:2].clone(), v[..., 1:2 * half:2].clone()
+            v[..., 0:2 * half:2] = a * cos - b * sin
+            v[..., 1:2 * half:2] = a * sin + b * cos
+
+
+def turn_neighbour_pairs(x, positions, rotary_dim, step):
+    """The plain statement of NeighbourPairs for a whole sequence; x is [T, heads, head_dim]."""
+    half = rotary_dim // 2
+    angles = positions.double()[:, None] * (step * torch.arange(1, half + 1, dtype=torch.float64))[None, :]
+    cos, sin = torch.cos(angles).to(x.dtype)[:, None, :], torch.sin(angles).to(x.dtype)[:, None, :]
+    out = x.clone()
+    a, b = x[..., 0:2 * half:2], x[..., 1:2 * half:2]
+    out[..., 0:2 * half:2] = a * cos - b * sin
+    out[..., 1:2 * half:2] = a * sin + b * cos
+    return out
 
 
 @dataclass(frozen=True)
@@ -187,10 +233,12 @@ class ToyConfig:
     window: int = 6
     decay: float = 0.7
     angle_step: float = 0.05
+    rotary_dim: int = 12
+    embedding_scale: float = 1.5
+    logit_cap: float = 3.0
     num_experts: int = 3
     expert_intermediate_size: int = 24
     rms_norm_eps: float = 1e-5
-    rope_theta: float = 10000.0
     max_position_embeddings: int = 256
 
     architecture = "ToyMixedForCausalLM"
@@ -203,7 +251,7 @@ class ToyConfig:
         return {"architectures": [self.architecture], "model_type": "toy_mixed", **{k: getattr(self, k) for k in self.__dataclass_fields__}}
 
     def model_spec(self) -> ModelSpec:
-        d, rot = self.hidden_size, RotarySpec(self.head_dim, self.rope_theta, None)
+        d = self.hidden_size
         def attention(l, window, position):
             p = f"layers.{l}.attn."
             return AttentionSpec(d, self.num_attention_heads, self.num_key_value_heads, self.head_dim, p + "q", p + "k", p + "v", p + "o",
@@ -216,13 +264,14 @@ class ToyConfig:
                 return LayerSpec(mixer=mixer, feed_forward=feed_forward, mixer_norm=norm, feed_forward_norm=norm, block="toy_parallel")
             return LayerSpec(mixer=mixer, feed_forward=feed_forward,
                              mixer_norm=RmsNormSpec(d, self.rms_norm_eps, p + "norm1"), feed_forward_norm=RmsNormSpec(d, self.rms_norm_eps, p + "norm2"))
-        layers = (rest(0, attention(0, None, LinearAnglesSpec(self.head_dim, self.angle_step))), rest(1, attention(1, self.window, rot)),
+        layers = (rest(0, attention(0, None, NeighbourPairsSpec(self.head_dim, self.rotary_dim, self.angle_step))),
+                  rest(1, attention(1, self.window, LinearAnglesSpec(self.head_dim, self.angle_step))),
                   rest(2, DecaySpec(d, self.decay, "layers.2.decay.w"), parallel=True),
                   rest(3, DecaySpec(d, self.decay, "layers.3.decay.w"), RoutedSpec(d, self.expert_intermediate_size, self.num_experts, "layers.3.moe.")))
         order = (RunEntry(3), RunEntry(0), RunEntry(1), RunEntry(2), RunEntry(0), RunEntry(1, cache_of=2))
         return ModelSpec(architecture=self.architecture, vocab_size=self.vocab_size, hidden_size=d, max_positions=self.max_position_embeddings,
                          embedding="embed", final_norm=RmsNormSpec(d, self.rms_norm_eps, "final_norm"), lm_head="head", layers=layers,
-                         run_order=order)
+                         run_order=order, after_embedding=(ScaleSpec(self.embedding_scale),), after_head=(SoftCapSpec(self.logit_cap),))
 
 
 def register():
@@ -230,6 +279,7 @@ def register():
     register_mixer("toy_decay", DecayMixer)
     register_feed_forward("toy_routed", RoutedFeedForward)
     register_position_encoding("toy_linear_angles", LinearAngles)
+    register_position_encoding("toy_neighbour_pairs", NeighbourPairs)
     register_norm("toy_centered_norm", CenteredNorm)
     register_block("toy_parallel", ParallelBlock)
     register_architecture(ToyConfig.architecture, ToyConfig, model_type="toy_mixed")
@@ -238,7 +288,7 @@ def register():
 def router_logits(cfg: ToyConfig, w: dict, tokens, dtype=torch.float64):
     """What the router of layer 3 (the first to run) sees for a whole sequence, from the plain parts."""
     w = {k: v.to(dtype) for k, v in w.items()}
-    x = w["embed"][torch.tensor(tokens)]
+    x = w["embed"][torch.tensor(tokens)] * cfg.embedding_scale
     xb = rms_norm(x, w["layers.3.norm1"], cfg.rms_norm_eps)
     s, outs = torch.zeros(cfg.hidden_size, dtype=dtype), []
     for t in range(len(tokens)):
@@ -253,8 +303,9 @@ def plain_logits(cfg: ToyConfig, w: dict, tokens, dtype=torch.float64, store=lam
     w = {k: v.to(dtype) for k, v in w.items()}
     T, H, KV, hd = len(tokens), cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
     pos = torch.arange(T)
-    inv_of = {0: cfg.angle_step * torch.arange(1, hd // 2 + 1, dtype=torch.float64), 1: rope_inverse_frequencies(hd, cfg.rope_theta)}
-    x = w["embed"][torch.tensor(tokens)]
+    linear_angles = cfg.angle_step * torch.arange(1, hd // 2 + 1, dtype=torch.float64)
+    turn = {0: lambda v: turn_neighbour_pairs(v, pos, cfg.rotary_dim, cfg.angle_step), 1: lambda v: rope_rotate(v, pos, linear_angles)}
+    x = w["embed"][torch.tensor(tokens)] * cfg.embedding_scale
     spec = cfg.model_spec()
     kept = {}
     for i, entry in enumerate(spec.run_order):
@@ -276,11 +327,10 @@ def plain_logits(cfg: ToyConfig, w: dict, tokens, dtype=torch.float64, store=lam
                 outs.append(w[p + "decay.w"] @ s)
             x = x + torch.stack(outs)
         else:
-            inv = inv_of[l]
             xb = store(xb)
-            q = store(rope_rotate((xb @ w[p + "attn.q"].T).reshape(T, H, hd), pos, inv))
+            q = store(turn[l]((xb @ w[p + "attn.q"].T).reshape(T, H, hd)))
             if entry.cache_of is None:
-                k = store(rope_rotate((xb @ w[p + "attn.k"].T).reshape(T, KV, hd), pos, inv))
+                k = store(turn[l]((xb @ w[p + "attn.k"].T).reshape(T, KV, hd)))
                 v = store((xb @ w[p + "attn.v"].T).reshape(T, KV, hd))
                 kept[i] = (k, v)
             else:
@@ -297,4 +347,5 @@ def plain_logits(cfg: ToyConfig, w: dict, tokens, dtype=torch.float64, store=lam
             continue
         xb = store(rms_norm(x, w[p + "norm2"], cfg.rms_norm_eps))
         x = x + swiglu(xb, w[p + "ff.gate"], w[p + "ff.up"], w[p + "ff.down"], store)
-    return store(rms_norm(x, w["final_norm"], cfg.rms_norm_eps)) @ w["head"].T
+    logits = store(rms_norm(x, w["final_norm"], cfg.rms_norm_eps)) @ w["head"].T
+    return cfg.logit_cap * torch.tanh(logits / cfg.logit_cap)
