@@ -360,6 +360,7 @@ class AttentionPlan:
     for the whole chip (break-even near 90 rows at the Llama-3.2-1B shape; above SHORT_TOTAL rows
     in all, the rows' repeated reading of the context costs more than the tiles' sequence).
     Made once per step and used by every layer."""
+    TILE = 0                             # rows of a prompt tile, 64 or 128; 0: by the step's size
     SMALL_STEP = 768                     # up to this many tiled rows in a step, tiles of 64 rows fill the chip better (measured at 32 heads)
     PAIRS = True                         # a portion's late tiles share workgroups with its early ones
     SHORT, SHORT_TOTAL = 64, 64          # portions of up to SHORT rows count as short; they go row by row while they sum to at most SHORT_TOTAL
@@ -379,7 +380,7 @@ class AttentionPlan:
         short_rows = sum(n for n in seg_len if 1 < n <= self.SHORT)
         row_by_row = self.SHORT if short_rows <= self.SHORT_TOTAL else 1
         self.single_rows = all(n == 1 for n in seg_len)          # every row is a request's only new row
-        self.tile = 64 if sum(n for n in seg_len if n > row_by_row) <= self.SMALL_STEP else 128        # rows of a prompt tile
+        self.tile = self.TILE or (64 if sum(n for n in seg_len if n > row_by_row) <= self.SMALL_STEP else 128)
         for start, n, pos0, slot in zip(seg_start, seg_len, seg_pos0, seg_slot):
             if n <= row_by_row:
                 dec.extend(range(start, start + n))
