@@ -6,6 +6,9 @@
 // token if rounding lets none win.  (The 64-bit sums are taken in a tree, not one by one: the draw
 // can differ from the reference's only where r falls within rounding of a boundary.)
 #include "common.h"
+#include "geneinfer_no_alloc.h"
+
+#include <mutex>
 
 namespace {
 
@@ -178,5 +181,58 @@ GI_API int gi_sample_temperature(const float* logits, const float* temperature, 
     GI_CHECK_LAUNCH("sample_temperature (sums)");
     sample_pick_kernel<<<n_rows, 256, 0, stream>>>(logits, temperature, uniform, part_m, part_s, out, vocab, stride, n_chunks);
     GI_CHECK_LAUNCH("sample_temperature (pick)");
+    return 0;
+}
+
+// ------------------------------------------------------------------ arg max without a scratch argument
+// The partial results of gi_argmax's first stage live in a static array in device memory instead of memory the caller
+// brings.  In host code the array's name is only a handle for hipGetSymbolAddress: every GPU holds its own copy at its
+// own address, which is asked for once per device and kept; kernels, and anything else on the host that needs the
+// memory, get that address.
+static __device__ __align__(256) unsigned char scratch[GI_NO_ALLOC_ARGMAX_MAX_PARTS * (sizeof(float) + sizeof(int))];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+void* g_scratch_of_device[MAX_DEVICES] = {};
+std::mutex g_scratch_mutex;
+
+// This GPU's copy of `scratch` (the current device's), or nullptr with the error recorded.
+void* scratch_of_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        gi_fail("no_alloc: no current HIP device (or more than %d devices)", MAX_DEVICES);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_of_device[dev] == nullptr) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            gi_fail("no_alloc: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_of_device[dev] = ptr;
+    }
+    return g_scratch_of_device[dev];
+}
+}  // namespace
+
+GI_API int gi_no_alloc_prepare(void) { return scratch_of_current_device() != nullptr ? 0 : -1; }
+
+GI_API int gi_argmax_no_alloc(const float* logits, int* out, int n_rows, int vocab, long stride, hipStream_t stream) {
+    GI_REQUIRE(logits != nullptr && out != nullptr, "argmax_no_alloc: logits and out must be given");
+    GI_REQUIRE(n_rows > 0 && n_rows <= 65535 && vocab > 0 && stride >= vocab, "argmax_no_alloc: bad sizes (rows %d, vocab %d, stride %ld)", n_rows, vocab, stride);
+    const int n_chunks = gi_argmax_chunks(vocab);
+    GI_REQUIRE((long)n_rows * n_chunks <= GI_NO_ALLOC_ARGMAX_MAX_PARTS,
+               "argmax_no_alloc: %d rows x %d runs of %d logits need %ld partial results, the static scratch holds %d; use gi_argmax with scratch of your own",
+               n_rows, n_chunks, CHUNK, (long)n_rows * n_chunks, GI_NO_ALLOC_ARGMAX_MAX_PARTS);
+    unsigned char* ptr = (unsigned char*)scratch_of_current_device();
+    if (ptr == nullptr) return -1;
+    float* part_v = (float*)ptr;
+    int* part_i = (int*)(ptr + (size_t)GI_NO_ALLOC_ARGMAX_MAX_PARTS * sizeof(float));
+    argmax_chunks_kernel<<<dim3(n_chunks, n_rows), 256, 0, stream>>>(logits, part_v, part_i, vocab, stride, n_chunks);
+    GI_CHECK_LAUNCH("argmax_no_alloc (chunks)");
+    argmax_final_kernel<<<n_rows, 64, 0, stream>>>(part_v, part_i, out, n_chunks);
+    GI_CHECK_LAUNCH("argmax_no_alloc (final)");
     return 0;
 }
