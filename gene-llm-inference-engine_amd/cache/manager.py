@@ -39,23 +39,31 @@ class PageGroup:
         self.table_host = np.full((max_requests, self.table_width), -1, dtype=np.int32)
         self.first_live = np.zeros(max_requests, dtype=np.int64)     # pages below this index were given back (windows)
         self.n_held = np.zeros(max_requests, dtype=np.int64)         # table entries in use, counted from 0
-        self.dirty: set = set()
+        self.dirty: set = set()                      # slots whose table row on the device is out of date
+        self.dirty_from = np.zeros(max_requests, dtype=np.int64)     # ... from this entry on,
+        self.on_device = np.zeros(max_requests, dtype=np.int64)      # ... and how many entries of the row the device copy may hold (the rest is -1 there)
         self.storage = None
         self.table_dev = None
         if allocate_storage:
             self.storage = torch.zeros((len(entries), n_pages, 2, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
             self.table_dev = torch.full((max_requests, self.table_width), -1, dtype=torch.int32, device=device)
 
+    def _changed(self, slot: int, first_entry: int) -> None:
+        self.dirty_from[slot] = min(int(self.dirty_from[slot]), first_entry) if slot in self.dirty else first_entry
+        self.dirty.add(slot)
+
     def pages_for(self, slot: int, new_length: int) -> int:
         """Pages to allocate so that positions below new_length have one."""
         return max(0, -(-new_length // self.page_size) - int(self.n_held[slot]))
 
     def grow(self, slot: int, new_length: int) -> None:
+        first = int(self.n_held[slot])
         for _ in range(self.pages_for(slot, new_length)):
             i = int(self.n_held[slot])
             self.table_host[slot, i] = self.pool.allocate()
             self.n_held[slot] = i + 1
-        self.dirty.add(slot)
+        if int(self.n_held[slot]) > first:
+            self._changed(slot, first)
 
     def adopt(self, slot: int, pages: Sequence[int]) -> None:
         """The first pages of a request that has none yet: full pages another request computed (the caller has
@@ -64,7 +72,7 @@ class PageGroup:
             raise CacheError("only a request without pages can adopt shared ones")
         self.table_host[slot, :len(pages)] = np.asarray(pages, dtype=np.int32)
         self.n_held[slot] = len(pages)
-        self.dirty.add(slot)
+        self._changed(slot, 0)
 
     def drop_behind_window(self, slot: int, length: int) -> None:
         """After `length` positions the next row is at position `length`; it sees keys from
@@ -72,12 +80,13 @@ class PageGroup:
         if self.need.window is None:
             return
         keep_from = (length - self.need.window + 1) // self.page_size       # first page still visible
-        i = int(self.first_live[slot])
+        first = i = int(self.first_live[slot])
         while i < min(keep_from, int(self.n_held[slot])):
             self.pool.release(int(self.table_host[slot, i]))
             self.table_host[slot, i] = -1
             i += 1
-            self.dirty.add(slot)
+        if i > first:
+            self._changed(slot, first)
         self.first_live[slot] = max(int(self.first_live[slot]), i)
 
     def release_all(self, slot: int) -> None:
@@ -85,10 +94,10 @@ class PageGroup:
         # first page is then the next one handed out
         for i in range(int(self.n_held[slot]) - 1, int(self.first_live[slot]) - 1, -1):
             self.pool.release(int(self.table_host[slot, i]))
-        self.table_host[slot, :] = -1
+        self.table_host[slot, :int(self.n_held[slot])] = -1
         self.first_live[slot] = 0
         self.n_held[slot] = 0
-        self.dirty.add(slot)
+        self._changed(slot, 0)
 
     def held_pages(self, slot: int) -> List[int]:
         return [int(p) for p in self.table_host[slot, int(self.first_live[slot]):int(self.n_held[slot])]]
@@ -128,22 +137,30 @@ class PageGroup:
                 self.storage[:, new].copy_(self.storage[:, old])
             self.pool.release(old)
             self.table_host[slot, i] = new
-        self.dirty.add(slot)
+        self._changed(slot, min(keep, length // self.page_size))
 
     def sync(self, upload=None) -> None:
+        """Brings the device's copy of the changed rows up to date.  Only the columns that changed go over: from the
+        first changed entry of any dirty row to the last entry that a dirty row holds or held on the device (a request
+        that crosses into a new page sends one column, not its whole row of max_positions / page_size entries)."""
         if self.table_dev is None or not self.dirty:
             self.dirty.clear()
             return
         rows = sorted(self.dirty)
         self.dirty.clear()
+        lo = int(self.dirty_from[rows].min())
+        hi = int(max(self.n_held[rows].max(), self.on_device[rows].max()))
+        self.on_device[rows] = self.n_held[rows]
+        if hi <= lo:
+            return
+        block = self.table_host[rows, lo:hi]
         if upload is not None:                 # int32 array -> device tensor without waiting for the device
             idx = upload(np.asarray(rows, dtype=np.int32))
-            data = upload(self.table_host[rows]).view(len(rows), self.table_host.shape[1])
-            self.table_dev.index_copy_(0, idx.long(), data)
+            data = upload(block).view(len(rows), hi - lo)
+            self.table_dev[:, lo:hi].index_copy_(0, idx.long(), data)
             return
         idx = torch.tensor(rows, dtype=torch.int64)
-        data = torch.from_numpy(self.table_host[rows])
-        self.table_dev.index_copy_(0, idx.to(self.table_dev.device), data.to(self.table_dev.device))
+        self.table_dev[:, lo:hi].index_copy_(0, idx.to(self.table_dev.device), torch.from_numpy(np.ascontiguousarray(block)).to(self.table_dev.device))
 
 
 class CacheManager:

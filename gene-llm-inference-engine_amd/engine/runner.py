@@ -62,10 +62,13 @@ class Runner:
     max_positions longest request; defaults to the model's limit
     use_graphs   replay decode steps (one token per request, all logits wanted) from captured HIP graphs,
                  if every part of the model allows it (`graph_safe`)
+    max_graphs   most captured graphs kept (one per batch size and bracket of the longest context); the one used
+                 longest ago goes when another is needed.  All graphs take their memory from one pool, so what they
+                 hold is what the largest of them needs (a pass's activations and its logits), not the sum.
     """
 
     def __init__(self, model: DecoderModel, *, page_size: int = 16, max_tokens: int = 4096, max_requests: int = 8,
-                 max_rows: int = 4096, max_positions: Optional[int] = None, use_graphs: bool = True):
+                 max_rows: int = 4096, max_positions: Optional[int] = None, use_graphs: bool = True, max_graphs: int = 16):
         self.model = model
         self.page_size = int(page_size)
         self.max_rows = int(max_rows)
@@ -79,6 +82,8 @@ class Runner:
         self.rows_run = 0
         self.use_graphs = bool(use_graphs) and model.graph_safe
         self._graphs = {}
+        self.max_graphs = max(1, int(max_graphs))
+        self._graph_pool = None
         self._uploads = _StepUploads(model.device, min(8 * self.max_rows + 1024, 1 << 18))       # at most 1 MiB a buffer; what is larger is copied the ordinary way
 
     # -------------------------------------------------------------------------------- requests
@@ -253,7 +258,12 @@ class Runner:
         bracket = min(bracket, self.max_positions)
         g = self._graphs.get((batch, bracket))
         if g is None:
-            g = self._graphs[(batch, bracket)] = _DecodeGraph(self.model, self._view, bracket, batch)
+            if len(self._graphs) >= self.max_graphs:         # (never during a capture: a graph may not be freed inside one)
+                del self._graphs[min(self._graphs, key=lambda k: self._graphs[k].last_used)]
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            g = self._graphs[(batch, bracket)] = _DecodeGraph(self.model, self._view, bracket, batch, self._graph_pool)
+        g.last_used = self.steps_run
         return g.run(meta, seg_slot, seg_pos0, tokens_on_device)
 
 
@@ -309,13 +319,14 @@ class _StepUploads:
 
 
 class _DecodeGraph:
-    """The captured pass of one batch size.  It holds the model and the cache view, not the runner: a runner and
+    """The captured pass of one batch size.  The logits a replay returns lie in the graphs' common pool: they are the
+    caller's until the next step, whichever graph that step replays.  It holds the model and the cache view, not the runner: a runner and
     its graphs must not form a reference cycle, or they would be freed by the cycle collector at a moment of its
     choosing, possibly while another graph is being captured, which the HIP runtime answers by aborting."""
 
-    def __init__(self, model: DecoderModel, view, longest_context: int, batch: int):
+    def __init__(self, model: DecoderModel, view, longest_context: int, batch: int, pool=None):
         from ..kernels.ops import AttentionPlan
-        self.model, self.view, self.batch = model, view, batch
+        self.model, self.view, self.batch, self.pool, self.last_used = model, view, batch, pool, 0
         dev = model.device
         self.meta = torch.zeros((3, batch), dtype=torch.int32, device=dev)
         self.logit_rows = torch.arange(batch, dtype=torch.int32, device=dev)
@@ -348,7 +359,7 @@ class _DecodeGraph:
             collecting = gc.isenabled()
             gc.disable()
             try:
-                with torch.cuda.graph(graph):
+                with torch.cuda.graph(graph, pool=self.pool):
                     self.logits = self.model.forward(self._context(seg_slot, seg_pos0), self.view, self.logit_rows, self.batch)
             finally:
                 if collecting:

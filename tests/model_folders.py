@@ -30,6 +30,13 @@ TINY_C = dict(hidden_size=80, intermediate_size=112, num_hidden_layers=1, num_at
 TINY_D = dict(hidden_size=128, intermediate_size=208, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
               head_dim=64, vocab_size=515, rope_theta=1000000.0, rope_scaling=None, rms_norm_eps=2e-5,
               tie_word_embeddings=False, max_position_embeddings=2048)
+# The layer shape of Llama 3.2 1B, which the benchmark runs, with 2 of its 16 layers: every product, the attention and the
+# head at their real sizes (the plain model needs a few seconds for it; weights N(0, 0.02) keep scores and logits of order one).
+LLAMA_1B_SHAPE = dict(hidden_size=2048, intermediate_size=8192, num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8,
+                      head_dim=64, vocab_size=128256, rope_theta=500000.0,
+                      rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                        original_max_position_embeddings=8192),
+                      rms_norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=4096)
 PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16}
 CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
@@ -85,7 +92,9 @@ def write_safetensors_by_hand(path, tensors: dict, shuffle_seed=None, header_pad
         blobs.append(raw)
     text = json.dumps(header).encode() + b" " * header_pad
     with open(path, "wb") as f:
-        f.write(struct.pack("<Q", len(text)) + text + b"".join(blobs))
+        f.write(struct.pack("<Q", len(text)) + text)
+        for raw in blobs:
+            f.write(raw)
 
 
 def write_model(folder, sizes: dict, seed: int = 0, dtype=torch.bfloat16, norm_dtype=None, std: float = 0.2, weights=None):

@@ -166,6 +166,19 @@ class PlainLlama:
         head = self.w["model.embed_tokens.weight"] if self.tied else self.w["lm_head.weight"]
         return x @ head.T
 
+    def logits_at(self, tokens, positions):
+        """The rows `positions` of `logits(tokens)`, with the head applied to those rows only."""
+        x = self.store(rms_norm(self.hidden_states(tokens)[torch.tensor(list(positions))], self.w["model.norm.weight"], self.eps))
+        head = self.w["model.embed_tokens.weight"] if self.tied else self.w["lm_head.weight"]
+        return x @ head.T
+
+    def with_storage(self, storage):
+        """The same model (the weights are shared, not read again) rounding to `storage` where the engine stores it."""
+        other = PlainLlama.__new__(PlainLlama)
+        other.__dict__.update(self.__dict__)
+        other.store = (lambda t: t.to(storage).to(self.dtype)) if storage is not None else (lambda t: t)
+        return other
+
     def greedy(self, prompt, n_new):
         """Greedy continuation, recomputing the whole sequence for every new token."""
         toks = list(prompt)

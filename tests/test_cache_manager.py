@@ -466,3 +466,54 @@ def test_prefix_index_counts_hold_under_random_use():
 
 def recount(index, pool):
     return sum(1 for page in index.pages() if pool.ref_count(page) == 1)
+
+
+def test_the_device_copy_of_the_tables_follows_under_random_use_with_few_columns_sent():
+    """Requests open, grow by portions and single positions, are cut back, slide a window and end, with a sync now and
+    then (not after every change): after each sync the device's tables equal the host's, and a request that only
+    crossed into a new page sent one column, not its row."""
+    rng = random.Random(11)
+    m = CacheManager([FULL, WINDOW], [None, None], page_size=4, n_pages=60, max_requests=4, max_positions=120, dtype=torch.float32, device="cpu")
+    sent = []
+    def upload(values):
+        sent.append(values.size)
+        return torch.from_numpy(values.copy().reshape(-1))
+    live = []
+    for turn in range(500):
+        roll = rng.random()
+        if roll < 0.15 and len(live) < 4:
+            live.append(f"r{turn}")
+            m.open(live[-1])
+        elif roll < 0.75 and live:
+            r = rng.choice(live)
+            n = rng.choice([1, 1, 1, 2, 7, 19])
+            if m.length(r) + n <= 120 and m.fits([(r, n)]):
+                m.reserve([(r, n)]); m.advance(r, n)
+        elif roll < 0.85 and live:
+            r = rng.choice(live)
+            try:
+                m.truncate(r, rng.randrange(m.length(r) + 1))
+            except CacheError:
+                pass                                                              # behind the window: refused
+        elif roll < 0.93 and live:
+            m.close(live.pop(rng.randrange(len(live))))
+        if rng.random() < 0.6:
+            m.sync(upload if rng.random() < 0.5 else None)
+            for g in m.groups:
+                assert (g.table_dev.numpy() == g.table_host).all(), turn
+    m.check_consistency()
+    # one request alone, position by position: a new page sends the row's number and one entry (with a window, also
+    # the entries between the page given back and the new one), never the row of 30 entries
+    for r in live:
+        m.close(r)
+    m.sync(upload)
+    m.open("solo")
+    m.reserve([("solo", 50)]); m.advance("solo", 50)
+    m.sync(upload)
+    del sent[:]
+    for _ in range(8):
+        m.reserve([("solo", 1)]); m.advance("solo", 1)
+        m.sync(upload)
+    assert sent and max(sent) <= 5 and sent.count(1) >= len(sent) // 2, sent
+    for g in m.groups:
+        assert (g.table_dev.numpy() == g.table_host).all()

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(scope="module")
 def folders(tmp_path_factory):
     out = {}
-    for name in ("A", "B"):
+    for name in ("A", "B", "D"):
         out[name] = tmp_path_factory.mktemp(f"gen{name}")
         write_model(out[name], CONFIGS[name], seed=40 + ord(name))
     return out
@@ -182,7 +182,7 @@ def test_requests_with_an_equal_beginning_share_its_pages(folders, dtype):
     """Requests that begin alike take the pages an earlier one computed: fewer rows are fed, and every request still
     ends with the tokens it gets alone (bit for bit in 32-bit, where the keys of a position never depend on the batch)."""
     import geneinfer_amd as gi
-    from geneinfer_amd.engine import EngineConfig, EngineRequest
+    from geneinfer_amd.engine import EngineConfig, EngineRequest, StepEntry
     from geneinfer_amd.sampling import SamplerConfig
     name, new = "B", 10
     system = prompts_for(name, [70], seed=31)[0]
@@ -196,35 +196,74 @@ def test_requests_with_an_equal_beginning_share_its_pages(folders, dtype):
         ids += [eng.submit(EngineRequest(p, len(p) + new - 1, SamplerConfig(0.0))) for p in prompts[1:]]
         eng.run_until_idle()
         llm.runner.cache.check_consistency()
-        return eng, [eng.result(j) for j in ids]
-    plain_eng, plain = run(False, 1024)
+        return llm, eng, [eng.result(j) for j in ids]
+    _, plain_eng, plain = run(False, 1024)
+    exact, rounded = PlainLlama(folders[name]), PlainLlama(folders[name], storage=torch.bfloat16)
     for max_tokens in (1024, 192):                                   # roomy; and so tight that named pages must be given back
-        eng, shared = run(True, max_tokens)
+        llm, eng, shared = run(True, max_tokens)
         assert eng.prefix is not None and eng.stats.prefix_hits >= 4 and eng.stats.prefix_tokens >= 3 * 64 + 32
         assert eng.stats.rows <= plain_eng.stats.rows - (3 * 64 + 32) + 64 * eng.stats.preemptions
         for a, b in zip(shared, plain):
-            assert a.finished and a.error == ""
+            assert a.finished and a.error == "" and len(a.generated_tokens) == len(b.generated_tokens)
             if dtype == "float32":
                 assert a.generated_tokens == b.generated_tokens
-            else:                                                    # the first token at least, where the plain model is clear about it
-                assert len(a.generated_tokens) == len(b.generated_tokens)
         assert sum(r.cached_tokens for r in shared) == eng.stats.prefix_tokens
         if max_tokens == 192:
             assert eng.stats.evicted_pages > 0 or eng.stats.preemptions > 0
+            continue
+        # What the shared pages hold, in either precision: every prompt again, opened on the pages the index still names for
+        # it, the rest fed in one step; the logits behind the shared pages are the plain model's for the whole prompt.
+        runner, index, got, want, near = llm.runner, llm.runner.cache.prefix, {}, {}, {}
+        for i, prompt in enumerate(prompts):
+            pages = index.match(prompt, len(prompt) - 1)
+            if i != 5:
+                assert len(pages) >= (2 if i == 4 else 4)            # 70 equal tokens are four full pages of 16, 40 are two
+            runner.open(("again", i), pages)
+            held = runner.length(("again", i))
+            rows = runner.step([StepEntry(("again", i), prompt[held:], tuple(range(len(prompt) - held)))]).cpu()
+            runner.close(("again", i))
+            e, r = exact.logits(prompt), rounded.logits(prompt)
+            for k, row in enumerate(rows):
+                got[(i, held + k)], want[(i, held + k)], near[(i, held + k)] = row, e[held + k], r[held + k]
+        if dtype == "float32":
+            worst = max(relative_error(row, want[key]) for key, row in got.items())
+            assert worst < 2e-5, worst
+        else:
+            assert_within_bfloat16_noise(got, want.__getitem__, near.__getitem__, "rows behind shared pages")
 
 
 def test_scheduler_in_bfloat16_runs_mixed_batches(folders):
+    """Through the scheduler in bfloat16 (portions of prompts beside decoding requests, four at a time): the logits every
+    token is drawn from are the plain model's for the request's tokens so far, within what rounding explains."""
     import geneinfer_amd as gi
+    from geneinfer_amd.engine import Engine, EngineConfig, EngineRequest
+    from geneinfer_amd.sampling import SamplerConfig, sample_rows
     llm = gi.LLM(folders["B"], dtype="bfloat16", page_size=16, max_tokens=512, max_running=4, max_rows=64)
     prompts = prompts_for("B", [1, 9, 33, 40, 12, 70])
-    out = llm.generate_many(prompts, steps=90, temperature=0.0)
+    seen = []                                                         # (sampler, logits row) of every draw
+    def watching(logits, samplers):
+        seen.extend(zip(samplers, logits.cpu()))
+        return sample_rows(logits, samplers)
+    eng = Engine(llm.runner, EngineConfig(max_running=4, step_rows=24), llm.end_tokens, sample=watching)
+    ids = [eng.submit(EngineRequest(p, 90, SamplerConfig(0.0))) for p in prompts]
+    eng.run_until_idle()
+    out = [eng.result(i) for i in ids]
     assert all(r.finished and r.error == "" and len(r.generated_tokens) == 90 - len(p) + 1 for r, p in zip(out, prompts))
-    plain = PlainLlama(folders["B"], storage=torch.bfloat16)
-    for r, p in zip(out, prompts):                                    # the first token is the plain model's, where that is clear-cut
-        row = plain.logits(p)[-1]
-        top = torch.topk(row, 2).values
-        if float(top[0] - top[1]) > 0.3:
-            assert r.generated_tokens[0] == int(torch.argmax(row))
+    assert eng.stats.max_rows_in_pass > 4 and eng.stats.max_running_seen == 4
+    exact, rounded = PlainLlama(folders["B"]), PlainLlama(folders["B"], storage=torch.bfloat16)
+    by_sampler = {}
+    for sampler, row in seen:
+        by_sampler.setdefault(id(sampler), []).append(row)
+    got, want, near = {}, {}, {}
+    for n, (r, p) in enumerate(zip(out, prompts)):
+        rows = by_sampler[id(eng.jobs[ids[n]].sampler)]
+        tokens = p + r.generated_tokens
+        assert len(rows) == len(r.generated_tokens)
+        e, nr = exact.logits(tokens[:-1]), rounded.logits(tokens[:-1])
+        for k, row in enumerate(rows):                                 # draw k saw the logits at position len(p) - 1 + k
+            got[(n, k)], want[(n, k)], near[(n, k)] = row, e[len(p) - 1 + k], nr[len(p) - 1 + k]
+            assert int(torch.argmax(row)) == r.generated_tokens[k]
+    assert_within_bfloat16_noise(got, want.__getitem__, near.__getitem__, "scheduler in bfloat16")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -250,6 +289,44 @@ def test_long_decoding(folders, dtype):
         rounded = PlainLlama(folders["B"], storage=torch.bfloat16).logits(toks)
         assert_within_bfloat16_noise(got, lambda p: exact[p], lambda p: rounded[p], "long decoding")
     assert runner._graphs and all(g.graph is not None for g in runner._graphs.values()), "decode steps did not replay a graph"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_graphs_across_a_context_bracket_and_between_batch_sizes(folders, dtype):
+    """Captured decode steps are kept per (batch size, power-of-two bracket of the longest context from 1024 on), and the
+    bracket fixes how the attention kernel cuts contexts into pieces.  Three requests decode with the longest crossing
+    position 1024 -> 1025 meanwhile (one stays short, far on the other side of the bracket), in steps of three and of two
+    requests by turns, so that four graphs are captured and each is replayed after another one: every logit row is the
+    plain model's.  Then a runner that may keep two graphs only does the same."""
+    from geneinfer_amd.engine import Runner, StepEntry, load_model
+    seqs = dict(zip("abc", prompts_for("D", [1060, 1050, 90], seed=17)))
+    start = {"a": 1000, "b": 990, "c": 30}
+    model = load_model(folders["D"], dtype, "cuda:0")
+    exact, rounded = PlainLlama(folders["D"]), PlainLlama(folders["D"], storage=torch.bfloat16)
+    want = {r: exact.logits(t) for r, t in seqs.items()}
+    near = {r: rounded.logits(t) for r, t in seqs.items()} if dtype == "bfloat16" else None
+    for max_graphs in (16, 2):
+        runner = Runner(model, page_size=16, max_tokens=2304, max_requests=3, max_graphs=max_graphs)
+        for r, t in seqs.items():
+            runner.open(r)
+            runner.step([StepEntry(r, t[:start[r]], ())])
+        got, at = {}, dict(start)
+        for k in range(60):
+            batch = ["a", "b", "c"] if k % 2 == 0 else ["a", "b"]
+            logits = runner.step([StepEntry(r, [seqs[r][at[r]]], (0,)) for r in batch]).cpu()
+            for r, row in zip(batch, logits):
+                got[(r, at[r])] = row
+                at[r] += 1
+        assert at == {"a": 1060, "b": 1050, "c": 60}
+        if max_graphs == 16:
+            assert set(runner._graphs) == {(3, 1024), (2, 1024), (3, 2048), (2, 2048)} and all(g.graph is not None and g.calls >= 4 for g in runner._graphs.values())
+        else:
+            assert len(runner._graphs) == 2
+        if dtype == "float32":
+            worst = max(relative_error(row, want[r][p]) for (r, p), row in got.items())
+            assert worst < 2e-5, worst
+        else:
+            assert_within_bfloat16_noise(got, lambda k: want[k[0]][k[1]], lambda k: near[k[0]][k[1]], f"graphs across brackets, {max_graphs} kept")
 
 
 @pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 1.5e-2)])

@@ -222,7 +222,7 @@ def plain_attention_rows(q, dense, rows, n_heads, n_kv, hd, window):
 
 ATT_CASES = [  # n_heads, n_kv, hd, page_size, window
     (4, 2, 64, 16, None), (3, 1, 32, 16, None), (8, 8, 128, 32, None), (6, 2, 96, 16, None), (4, 4, 64, 16, 40), (32, 8, 64, 16, None),
-    (5, 5, 48, 16, None), (2, 1, 16, 4, 9),
+    (5, 5, 48, 16, None), (2, 1, 16, 4, 9), (4, 2, 256, 16, None),
 ]
 
 

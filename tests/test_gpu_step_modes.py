@@ -72,7 +72,7 @@ _WHOLE = {}
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("mode", ["whole", "tail_singly", "portions", "mixed"])
+@pytest.mark.parametrize("mode", ["whole", "tail_singly", "portions", "mixed", "mixed_long"])
 def test_step_modes(case, dtype, mode):
     name, folder, requests, want = case
     ps = PAGE_SIZE[name]
@@ -82,9 +82,13 @@ def test_step_modes(case, dtype, mode):
         steps = traces.tail_singly(requests, 32)
     elif mode == "portions":
         steps = traces.portions(requests)
-    else:
+    elif mode == "mixed":
         steps = traces.mixed(requests, seed=3)
         assert max(len(s["entries"]) for s in steps) >= 3, "the mixed trace never held three requests in a step"
+    else:                                                        # portions of 70..200 rows: with tiny D, matrix-core tiles beside decoded rows
+        steps = traces.mixed(requests, seed=5, portion=(70, 200), prompt_share=0.8)
+        if name == "D":
+            assert any(max(len(e["tokens"]) for e in s["entries"]) > 64 and min(len(e["tokens"]) for e in s["entries"]) == 1 for s in steps)
     max_tokens = traces.peak_tokens(steps, round_to=ps)          # so few pages that they are used again
     got = replay(folder, dtype, steps, ps, max_tokens)
     assert len(got) == sum(len(t) for t in requests.values())

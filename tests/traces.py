@@ -23,34 +23,34 @@ def whole(requests, want_every=1):
     return steps
 
 
-def tail_singly(requests, tail=32):
+def tail_singly(requests, tail=32, want_every=1):
     """Most of a request in one step, its last `tail` tokens one by one."""
     steps = []
     for rid, toks in requests.items():
         head = max(0, len(toks) - tail)
         if head:
-            steps.append({"step": len(steps), "entries": [_entry(rid, toks, 0, head)], "end": []})
+            steps.append({"step": len(steps), "entries": [_entry(rid, toks, 0, head, want_every)], "end": []})
         for p in range(head, len(toks)):
-            steps.append({"step": len(steps), "entries": [_entry(rid, toks, p, 1)], "end": [rid] if p == len(toks) - 1 else []})
+            steps.append({"step": len(steps), "entries": [_entry(rid, toks, p, 1, want_every)], "end": [rid] if p == len(toks) - 1 else []})
     return steps
 
 
-def portions(requests, sizes=(7, 2, 5, 3, 2, 11, 1, 4)):
+def portions(requests, sizes=(7, 2, 5, 3, 2, 11, 1, 4), want_every=1):
     """Each request alone, cut into portions whose sizes cycle through `sizes` (down to two tokens and one)."""
     steps = []
     for k, (rid, toks) in enumerate(requests.items()):
         p, i = 0, k                      # every request starts elsewhere in the cycle
         while p < len(toks):
             n = min(sizes[i % len(sizes)], len(toks) - p)
-            steps.append({"step": len(steps), "entries": [_entry(rid, toks, p, n)], "end": [rid] if p + n == len(toks) else []})
+            steps.append({"step": len(steps), "entries": [_entry(rid, toks, p, n, want_every)], "end": [rid] if p + n == len(toks) else []})
             p, i = p + n, i + 1
     return steps
 
 
-def mixed(requests, seed=0, max_live=4, prompt_share=0.6):
+def mixed(requests, seed=0, max_live=4, prompt_share=0.6, portion=(2, 9), want_every=1):
     """Up to `max_live` requests at a time.  The first `prompt_share` of a request is fed in portions
-    of 2..9 tokens, the rest one token a step; in every step a random non-empty subset of the
-    live requests takes part; a finished request ends and the next one starts."""
+    of portion[0]..portion[1] tokens (2..9 unless said otherwise), the rest one token a step; in every step a random
+    non-empty subset of the live requests takes part; a finished request ends and the next one starts."""
     rng = random.Random(seed)
     waiting = list(requests.items())
     live, fed, steps = [], {}, []
@@ -64,8 +64,8 @@ def mixed(requests, seed=0, max_live=4, prompt_share=0.6):
         for rid in part:
             toks = requests[rid]
             prompt = max(1, int(len(toks) * prompt_share))
-            n = min(rng.randint(2, 9), prompt - fed[rid]) if fed[rid] < prompt else 1
-            entries.append(_entry(rid, toks, fed[rid], n))
+            n = min(rng.randint(*portion), prompt - fed[rid]) if fed[rid] < prompt else 1
+            entries.append(_entry(rid, toks, fed[rid], n, want_every))
             fed[rid] += n
             if fed[rid] == len(toks):
                 ended.append(rid)
