@@ -179,9 +179,11 @@ def test_sample_temperature_matches_the_inverse_distribution():
 
 
 # ------------------------------------------------------------------------------------- attention
-def build_paged(requests, n_kv, hd, page_size, dtype, seed, scale_one=None):
+def build_paged(requests, n_kv, hd, page_size, dtype, seed, scale_one=None, gone_before=None):
     """Dense keys/values per request, written into a paged cache with scrambled pages and a rim of
-    NaN pages that nothing may touch.  requests: list of context lengths.  Returns cache, table, dense."""
+    NaN pages that nothing may touch.  requests: list of context lengths.  gone_before: per request index, a position;
+    pages that lie wholly before it have been given back (a window has passed them): their table entries are -1 and
+    nothing of them is in the cache.  Returns cache, table, dense."""
     g = torch.Generator().manual_seed(seed)
     n_pages_needed = sum(-(-n // page_size) for n in requests)
     n_pages = n_pages_needed + 3
@@ -197,6 +199,8 @@ def build_paged(requests, n_kv, hd, page_size, dtype, seed, scale_one=None):
             k[scale_one[0]] *= scale_one[1]                    # one far key that must stand out
         dense.append((k, v))
         for i in range(-(-n // page_size)):
+            if gone_before is not None and (i + 1) * page_size <= gone_before.get(slot, 0):
+                continue
             page = perm[nxt]; nxt += 1
             table[slot + 1, i] = page                          # slot 0 of the table stays unused (-1)
             cache[page] = 0
@@ -248,8 +252,12 @@ def test_attention_over_pages(n_heads, n_kv, hd, ps, window, dtype, portions, ti
     from geneinfer_amd.parts import StepContext
     monkeypatch.setattr(ops().AttentionPlan, "TILE", tile)
     contexts = [300, 131, 1, 77, 530]
-    cache, table, dense = build_paged(contexts, n_kv, hd, ps, dtype, seed=hd + n_heads)
     segs = SEGMENTS[portions]
+    # with a window, the pages that no row of the step can see have been given back
+    gone = {slot: max(0, pos0 - window + 1) for slot, pos0, _ in segs} if window else None
+    cache, table, dense = build_paged(contexts, n_kv, hd, ps, dtype, seed=hd + n_heads, gone_before=gone)
+    if window:
+        assert int((table[1:] == -1).sum()) > int((build_paged(contexts, n_kv, hd, ps, dtype, seed=hd + n_heads)[1][1:] == -1).sum())
     rows, seg_start, seg_len, seg_pos0, seg_slot = [], [], [], [], []
     for slot, pos0, n in segs:
         seg_start.append(len(rows)); seg_len.append(n); seg_pos0.append(pos0); seg_slot.append(slot + 1)
@@ -276,8 +284,9 @@ def test_few_prompt_tiles_over_a_long_context_share_their_keys_out(n_heads, n_kv
     from geneinfer_amd.parts import StepContext
     o = ops()
     contexts = [1500, 730, 40]
-    cache, table, dense = build_paged(contexts, n_kv, hd, ps, torch.bfloat16, seed=hd + n_heads + 7, scale_one=(333, 3.0))
     segs = [(0, 1400, 100), (1, 600, 130), (2, 39, 1)]
+    gone = {slot: max(0, pos0 - window + 1) for slot, pos0, _ in segs} if window else None          # what a window has given back
+    cache, table, dense = build_paged(contexts, n_kv, hd, ps, torch.bfloat16, seed=hd + n_heads + 7, scale_one=(333, 3.0), gone_before=gone)
     rows, seg_start, seg_len, seg_pos0, seg_slot = [], [], [], [], []
     for slot, pos0, n in segs:
         seg_start.append(len(rows)); seg_len.append(n); seg_pos0.append(pos0); seg_slot.append(slot + 1)
@@ -324,7 +333,8 @@ def test_decode_attention_from_unrotated_products(n_heads, n_kv, hd, ps, window,
     shape = ops().decode_attention_shape
     monkeypatch.setattr(ops(), "decode_attention_shape", lambda *a, **k: shape(*a[:5], target_waves=target_waves))
     contexts = [300, 131, 1, 77, 530, 16, 17, 1200, 32, 33]           # the new row's position is the last of each
-    cache, table, dense = build_paged(contexts, n_kv, hd, ps, torch.bfloat16, seed=hd + n_heads + 1)
+    gone = {slot: max(0, n - window) for slot, n in enumerate(contexts)} if window else None        # what a window has given back
+    cache, table, dense = build_paged(contexts, n_kv, hd, ps, torch.bfloat16, seed=hd + n_heads + 1, gone_before=gone)
     T = len(contexts)
     pos = torch.tensor([n - 1 for n in contexts], dtype=torch.int32, device=DEV)
     slots = torch.arange(1, T + 1, dtype=torch.int32, device=DEV)
