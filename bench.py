@@ -3,8 +3,14 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one decode step of the whole batch (default batch 8, each request on a 2,048-token
-prompt in a 4,096-token context).  Prints ONE JSON line: decoded tokens a second as `value`, the
-2,048-token prefill, the decode step's HBM roofline fraction, and decode at batch 1 and 64.
+prompt in a 4,096-token context), through the scheduler with its defaults.  After W warm-up steps,
+five windows of exactly K steps each are timed one after the other (5 K + W new tokens a request:
+256 with the defaults, the benchmark's workload); `value` and `ms_per_step` are the median window's,
+`ms_per_step_min` the fastest's.  Prints ONE JSON line: decoded tokens a second, the 2,048-token
+prefill (median of 5), the decode step's roofline fraction against the published HBM peak and
+against the read bandwidth a plain kernel of this library reaches on this chip, the prefill's
+fraction against the published matrix peak and against a bare loop of matrix instructions, and decode
+at batch 1 and 64 (medians of 5 windows as well).
 """
 import argparse
 import json
@@ -30,8 +36,8 @@ PROMPT, NEW_TOKENS, CONTEXT, PAGE = 2048, 256, 4096, 16
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
-    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--steps", type=int, default=48, help="decode steps per timed window (five windows are timed)")
+    ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration has (0 = all); named in the record")
@@ -44,6 +50,7 @@ def main() -> int:
     import torch
     from geneinfer_amd.config import LlamaConfig
     from geneinfer_amd.engine import Engine, EngineConfig, EngineRequest, Runner, StepEntry, random_model
+    from geneinfer_amd.kernels import ops
     from geneinfer_amd.sampling import Sampler, SamplerConfig, sample_rows
 
     sizes = dict(LLAMA_1B)
@@ -56,8 +63,10 @@ def main() -> int:
     vocab = config.vocab_size
     gen = torch.Generator().manual_seed(1)
 
+    WINDOWS = 5
+
     def make_runner(batch):
-        per_request = -(-(PROMPT + NEW_TOKENS + args.steps + args.warmup + 2 * batch + 8) // 64) * 64
+        per_request = -(-(PROMPT + WINDOWS * args.steps + args.warmup + 2 * batch + 8) // 64) * 64
         return Runner(model, page_size=PAGE, max_tokens=batch * per_request, max_requests=batch, max_rows=max(PROMPT, batch),
                       max_positions=CONTEXT)
 
@@ -67,11 +76,12 @@ def main() -> int:
         return runner.step([StepEntry(rid, toks, (PROMPT - 1,))])
 
     def decode(batch, steps, warmup):
-        """Greedy decoding of `batch` requests after their prompts, through the scheduler (what serving runs); returns
-        (seconds for `steps` decode steps, mean context at the middle of them)."""
+        """Greedy decoding of `batch` requests after their prompts, through the scheduler as serving runs it (its
+        defaults: prefix sharing on, decoding ahead); returns [(seconds for `steps` decode steps, mean context at the
+        middle of them)] for WINDOWS windows timed one after the other, sorted by time."""
         runner = make_runner(batch)
-        engine = Engine(runner, EngineConfig(max_running=batch, prefix_cache=False))
-        limit = min(CONTEXT, PROMPT + NEW_TOKENS + steps + warmup + 2 * batch)
+        engine = Engine(runner, EngineConfig(max_running=batch))
+        limit = min(CONTEXT, PROMPT + WINDOWS * steps + warmup + 2 * batch + 4)
         for r in range(batch):
             engine.submit(EngineRequest(torch.randint(0, vocab, (PROMPT,), generator=gen).tolist(), limit, SamplerConfig(temperature=0.0)))
         decoding = 0
@@ -81,18 +91,20 @@ def main() -> int:
             decoding = decoding + 1 if engine.stats.rows - rows == batch and engine.stats.passes > batch else 0
         for _ in range(warmup):
             engine.step()
-        torch.cuda.synchronize()
-        context = sum(runner.length(job.key) for job in engine.running) / batch + steps / 2
-        passes = engine.stats.passes
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            engine.step()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        assert engine.stats.passes - passes == steps and len(engine.running) == batch, "a timed step was not a decode step of the whole batch"
+        windows = []
+        for _ in range(WINDOWS):
+            torch.cuda.synchronize()
+            context = sum(runner.length(job.key) for job in engine.running) / batch + steps / 2
+            passes = engine.stats.passes
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                engine.step()
+            torch.cuda.synchronize()
+            windows.append((time.perf_counter() - t0, context))
+            assert engine.stats.passes - passes == steps and len(engine.running) == batch, "a timed step was not a decode step of the whole batch"
         del engine, runner
         torch.cuda.empty_cache()
-        return dt, context
+        return sorted(windows)
 
     # ---- prefill of one 2,048-token prompt (median of 5 after one warm-up)
     runner = make_runner(1)
@@ -114,8 +126,16 @@ def main() -> int:
     prefill_rec = {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
                    "frac": round(prefill_flops / prefill_s / (PEAK_TFLOPS[args.dtype] * 1e12), 4)}
 
+    # ---- what a plain kernel reads and a bare loop of matrix instructions computes on this chip
+    own_gbs = ops.measured_read_bandwidth("cuda:0")
+    own_tflops = ops.measured_mfma_rate("cuda:0") if args.dtype == "bf16" else None
+    prefill_rec["tflops"] = round(prefill_flops / prefill_s / 1e12, 1)
+    if own_tflops:
+        prefill_rec["own_peak_tflops"], prefill_rec["frac_of_own_peak"] = round(own_tflops, 1), round(prefill_flops / prefill_s / 1e12 / own_tflops, 4)
+
     # ---- decode
-    dt, context = decode(args.batch, args.steps, args.warmup)
+    windows = decode(args.batch, args.steps, args.warmup)
+    dt, context = windows[len(windows) // 2]
     elem = 2 if args.dtype == "bf16" else 4
     weight_bytes = model.weight_bytes_read_per_step()
     kv_bytes = args.batch * context * L * 2 * KV * elem
@@ -123,21 +143,22 @@ def main() -> int:
     points = {}
     if not args.no_points:
         for b in (1, 64):
-            s = max(8, args.steps // 4)
-            d, _ = decode(b, s, 4)
-            points[f"decode_b{b}"] = round(b * s / d, 1)
+            w = decode(b, max(8, args.steps // 2), 8)
+            points[f"decode_b{b}"] = round(b * max(8, args.steps // 2) / w[len(w) // 2][0], 1)
 
     rec = {
         "metric": "decode tok/s at batch 1/8/64 + prefill tok/s at 2,048 tokens, Llama-3.2-1B",
         "value": round(args.batch * args.steps / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(dt / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(dt / args.steps * 1e3, 4), "ms_per_step_min": round(windows[0][0] / args.steps * 1e3, 4), "windows": WINDOWS,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
         "config": {"model": "Llama-3.2-1B shape", "layers": L, "layers_of_config": layers_full, "hidden": D, "heads": H,
                    "kv_heads": config.num_key_value_heads, "head_dim": hd, "intermediate": I, "vocab": V, "global_batch": args.batch,
                    "seq_len": CONTEXT, "prompt_len": PROMPT, "decode_context": context, "page_size": PAGE, "tied_embeddings": True,
                    "rope": "llama3 theta 5e5 factor 32", "parallelism": "single_gpu"},
         "prefill": prefill_rec,
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s", "frac": round(achieved / HBM_GBS, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s", "frac": round(achieved / HBM_GBS, 4),
+                     "own_peak": round(own_gbs, 1), "frac_of_own_peak": round(achieved / own_gbs, 4)},
         "points": points,
     }
     print(json.dumps(rec))

@@ -236,6 +236,11 @@ class CacheManager:
         """The request's page table in the first group (what the prefix index names pages by)."""
         return self.groups[0].held_pages(self.slot(request))
 
+    def page_row(self, request: Hashable):
+        """The same as an array (a view of the table's row: read it now, do not keep it)."""
+        g, slot = self.groups[0], self.slot(request)
+        return g.table_host[slot, int(g.first_live[slot]):int(g.n_held[slot])]
+
     def evictable_pages(self) -> int:
         return self.prefix.evictable() if self.prefix is not None else 0
 

@@ -43,6 +43,7 @@ class PrefixIndex:
         self._only_mine = 0                                   # named pages whose reference count is 1
         self._idle_leaves: List[Tuple[int, int]] = []         # heap of (stamp, page): leaves nobody else holds, and stale entries
         self._clock = 0
+        self.last_walk = None                # where the last insert ended: (node of the last full page it passed, how many it passed)
         pool.on_change = self._references_changed
 
     def __len__(self) -> int:
@@ -94,17 +95,25 @@ class PrefixIndex:
             node = nxt
         return found
 
-    def insert(self, tokens: Sequence[int], n_tokens: int, pages: Sequence[int]) -> int:
+    def insert(self, tokens: Sequence[int], n_tokens: int, pages: Sequence[int], after=None) -> int:
         """The first n_tokens positions of a request hold `tokens` in `pages` (its page table): its full pages
         are named, each under the page before it, unless that place is taken already (then the page that has
-        it is followed, whatever the request's own copy).  Returns how many pages were newly named."""
-        ps, node, added = self.page_size, None, 0
-        for i in range(min(n_tokens // ps, len(pages))):
+        it is followed, whatever the request's own copy).  Returns how many pages were newly named.
+
+        `after`: what `last_walk` was after an earlier insert of the same request (its tokens up to there unchanged):
+        the walk then starts behind the pages that one passed, unless the index has forgotten the last of them
+        meanwhile (then it starts at the root as without it)."""
+        ps, node, added, first = self.page_size, None, 0, 0
+        if after is not None and self._by_page.get(after[0].page) is after[0]:
+            node, first = after
+        self.last_walk = None
+        for i in range(first, min(n_tokens // ps, len(pages))):
             key = tuple(tokens[i * ps:(i + 1) * ps])
             known = self._children_of(node).get(key)
             if known is not None:
                 self._touch(known)
                 node = known
+                self.last_walk = (node, i + 1)
                 continue
             page = int(pages[i])
             if page in self._by_page:       # a page has one place in the tree
@@ -116,6 +125,7 @@ class PrefixIndex:
             self.pool.retain(page)          # (the hook sees a named page with at least two holders: nothing to count)
             node = new
             added += 1
+            self.last_walk = (new, i + 1)
         return added
 
     # ---------------------------------------------------------------------------- giving back

@@ -94,7 +94,8 @@ class _Job:
         self.id, self.request, self.sampler, self.steps = jid, request, sampler, steps
         self.tokens: List[int] = [int(t) for t in request.prompt]      # prompt followed by generated tokens
         self.fed = 0                                                     # tokens[0:fed] are in the cache
-        self.indexed_upto = 0                                            # ... and tokens[0:indexed_upto] known to the prefix index
+        self.indexed_upto = 0                                            # ... and tokens[0:indexed_upto] known to the prefix index,
+        self.indexed_after = None                                        # ... whose walk ended here (`PrefixIndex.last_walk`)
         self.result = EngineResult(id=jid, prompt_tokens=list(self.tokens))
         self.key = ("job", jid)
 
@@ -173,6 +174,7 @@ class Engine:
                 shared = self.prefix.match(job.tokens, usable) if usable > 0 else []
             self.runner.open(job.key, shared)
             job.fed = job.indexed_upto = len(shared) * self.runner.cache.page_size
+            job.indexed_after = None
             if shared:
                 job.result.cached_tokens += job.fed
                 self.stats.prefix_tokens += job.fed
@@ -269,8 +271,9 @@ class Engine:
             job.result.first_pass = pass_no
         job.fed += n
         if self.prefix is not None and job.fed // self.prefix.page_size > job.indexed_upto // self.prefix.page_size:
-            self.prefix.insert(job.tokens, job.fed, self.runner.cache.pages_of(job.key))      # the pages that became full
-            job.indexed_upto = job.fed
+            # the pages that became full; the walk goes on where this job's last one ended, not from the first page
+            self.prefix.insert(job.tokens, job.fed, self.runner.cache.page_row(job.key), after=job.indexed_after)
+            job.indexed_upto, job.indexed_after = job.fed, self.prefix.last_walk
         if nxt is not None:
             st.logits_rows += 1
             job.result.generated_tokens.append(nxt)

@@ -40,6 +40,8 @@ _SIGNATURES = {
     "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_int, c_int, c_void_p],
+    "gi_probe_stream": [c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p],
+    "gi_probe_mfma": [c_int, c_void_p, c_int, c_void_p],
     "gi_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
 }
@@ -61,6 +63,8 @@ def lib():
         l.gi_attention_bf16_supports.restype = c_int
         l.gi_gemm_bf16_scratch_floats.argtypes = [c_int, c_int, c_int]
         l.gi_gemm_bf16_scratch_floats.restype = c_long
+        l.gi_probe_mfma_flops.argtypes = [c_int, c_int]
+        l.gi_probe_mfma_flops.restype = c_long
         _lib = l
     return _lib
 
@@ -603,3 +607,37 @@ def sample_temperature(logits, temperature, uniform, out):
     _call("gi_sample_temperature", logits.data_ptr(), temperature.data_ptr(), uniform.data_ptr(), out.data_ptr(), part_m.data_ptr(),
           part_s.data_ptr(), n, vocab, logits.stride(0), _stream())
     return out
+
+
+# ------------------------------------------------------------------------------------------------ probes
+def _timed_ms(launch, repeats):
+    """Median time of `launch()` over `repeats` runs, by device events, after one run that is not timed."""
+    launch()
+    times = []
+    for _ in range(repeats):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        launch()
+        stop.record()
+        stop.synchronize()
+        times.append(start.elapsed_time(stop))
+    return sorted(times)[len(times) // 2]
+
+
+def measured_read_bandwidth(device="cuda:0", n_bytes: int = 2 << 30, repeats: int = 5, copy: bool = False) -> float:
+    """GB/s at which a plain kernel of this library reads `n_bytes` of device memory (much more than the caches hold);
+    with `copy`, reads and writes them (bytes moved = 2 * n_bytes)."""
+    src = torch.empty(n_bytes // 4, dtype=torch.int32, device=device).fill_(1)
+    dst = torch.empty_like(src) if copy else None
+    n_blocks = 256 * 16
+    sink = torch.empty(n_blocks * 256, dtype=torch.int32, device=device)
+    ms = _timed_ms(lambda: _call("gi_probe_stream", src.data_ptr(), _ptr(dst), n_bytes, sink.data_ptr(), n_blocks, _stream()), repeats)
+    return (2 if copy else 1) * n_bytes / (ms * 1e-3) / 1e9
+
+
+def measured_mfma_rate(device="cuda:0", iters: int = 20000, repeats: int = 5) -> float:
+    """TFLOP/s of a loop of bfloat16 matrix instructions (32x32x16, eight independent sums a wave, eight waves a compute unit)."""
+    n_blocks = 256 * 2
+    sink = torch.empty(n_blocks * 256, dtype=torch.float32, device=device)
+    ms = _timed_ms(lambda: _call("gi_probe_mfma", iters, sink.data_ptr(), n_blocks, _stream()), repeats)
+    return lib().gi_probe_mfma_flops(iters, n_blocks) / (ms * 1e-3) / 1e12

@@ -264,6 +264,36 @@ def test_prefix_index_matches_true_prefixes_of_full_pages_only():               
     assert index.match(other, 8) == [pages[0], own[1]]
 
 
+def test_prefix_index_goes_on_where_a_request_was_inserted_last():
+    """A request that grows is inserted again and again; with the place its last walk ended at, the new walk passes only
+    the new pages.  If that place has been given back and its page named anew under another chain, the walk starts over."""
+    from geneinfer_amd.cache import PagePool, PrefixIndex
+    pool = PagePool(12)
+    index = PrefixIndex(pool, page_size=2)
+    tokens = [1, 1, 2, 2, 3, 3, 4, 4]
+    pages = [pool.allocate() for _ in range(4)]
+    assert index.insert(tokens, 4, pages) == 2
+    place = index.last_walk
+    assert place[1] == 2 and place[0].page == pages[1]
+    lookups = []
+    real = index._children_of
+    index._children_of = lambda node: lookups.append(node) or real(node)
+    assert index.insert(tokens, 8, pages, after=place) == 2 and len(index) == 4
+    assert all(node is not None for node in lookups)                                  # the root was not visited again
+    index._children_of = real
+    assert index.match(tokens, 8) == pages
+    for p in pages * 2:
+        pool.release(p)                                                            # the request and the match let go
+    assert index.evict(4) == 4 and len(index) == 0
+    # the page comes back under other tokens; the stale place is recognised
+    other = [pool.allocate() for _ in range(2)]
+    assert pages[1] in other
+    index.insert([7, 7, 8, 8], 4, other)
+    again = [pool.allocate() for _ in range(4)]
+    assert index.insert(tokens, 8, again, after=place) == 4
+    assert index.match(tokens, 8) == again and index.match([7, 7, 8, 8, 3, 3], 6) == other
+
+
 def test_prefix_index_gives_back_least_recently_used_leaves_that_nobody_uses():    # src/model/prefix_cache.cpp:60-97
     from geneinfer_amd.cache import PagePool, PrefixIndex
     pool = PagePool(10)
