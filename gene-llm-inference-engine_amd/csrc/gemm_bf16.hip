@@ -1,9 +1,12 @@
 // C[m, n] (=|+=) sum_k A[m, k] * W[n, k] with bfloat16 operands on the matrix cores, 32-bit sums.
 //
 // Both operands are row-major with k contiguous, so each lane's operand of a matrix instruction is
-// one 16-byte load of 8 consecutive k.  Four kernels:
+// one 16-byte load of 8 consecutive k.  Five kernels:
 //
-//   piped   prompts (128 rows or more, K a multiple of 64): tiles of 128 x 128 or 256 x 256,
+//   pingpong  large prompt-sized products (a 256 x 256 tile for every compute unit): operands loaded
+//           from global memory straight into two LDS stages; the workgroup's eight waves form two
+//           groups that take turns at reading LDS and at the matrix instructions.
+//   piped   the other products of 128 rows or more (K a multiple of 64): tiles of 128 x 128,
 //           operands loaded from global memory straight into a ring of LDS stages, several
 //           blocks of k in flight; v_mfma_f32_32x32x16_bf16.
 //   tiled   the other shapes above 64 rows: a BM x 128 tile of C per workgroup of 4 waves,
@@ -34,6 +37,12 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 enum Epilogue : int { EPI_STORE_F32 = 0, EPI_ADD_F32 = 1, EPI_STORE_BF16 = 2, EPI_GATED_BF16 = 3 };
 
 __device__ __forceinline__ float silu_gate(float g, float u) { return (g * (1.0f / (1.0f + expf(-g)))) * u; }
+// The same with the hardware's exp2 and reciprocal (each within a unit or two in the last place of 32 bits): for results
+// that are rounded to bfloat16's 8 bits at once.  The exact form above costs some thirty vector instructions a value,
+// which in a prompt-sized product's epilogue is a tenth of the kernel.
+__device__ __forceinline__ float silu_gate_fast(float g, float u) {
+    return (g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f))) * u;
+}
 
 __device__ __forceinline__ uint4 load16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
@@ -242,6 +251,236 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
                     if (m < M && n < N) write_out<EPI>(C, (size_t)m * ldc + n, acc[i][j][v]);
                 }
             }
+}
+
+// --------------------------------------------------------------------------------------- pingpong
+// A 256 x 256 tile and two LDS stages of 64 k, filled straight from global memory like the piped kernel's, with another
+// order of work inside the workgroup.  Its eight waves form two groups of four, and a compute unit's four SIMDs hold
+// one wave of each group.  A group alternates between a phase R in which it reads the operands of a block's 64 k from
+// LDS into registers (and issues loads that refill the stages) and a phase M in which it does nothing but matrix
+// instructions on them; a workgroup barrier ends every phase, and one group runs a barrier behind the other, so at any
+// time one group reads while the other multiplies: on every SIMD the matrix unit always has a wave that has its
+// operands at hand, instead of two waves that read together and then multiply together.
+//
+//   barrier number      0        1        2        3        4
+//   group 0:    R(0)  |  M(0)  |  R(1)  |  M(1)  |  R(2)  | ...
+//   group 1:          |  R(0)  |  M(0)  |  R(1)  |  M(1)  | ...        R(b), M(b): the phases of block b
+//
+// Every wave passes the same number of barriers: group 1's one ahead is matched by one more of group 0 at the end.
+// Who loads which rows of which block when is said where the loads are set up, below.  Measured (cycle stamps per
+// phase): M takes 1,080 clocks for its 32 matrix instructions, R 500 for its 24 reads plus what its 8 loads take to
+// issue, which is what bounds the interval between two barriers (1,700 clocks); a load costs the wave that issues it
+// 23 clocks when nothing else runs and 70 to 140 here, wherever in the two phases it is put.
+template <int BN, int EPI>
+__global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
+                                                                int M, int N, int K, long lda, long ldw, long ldc) {
+    static_assert(BN == 256, "the sharing of the loads below is written for 256 x 256 tiles");
+    constexpr int BM = 256, WAVES = 8, WM = 64, WN = BN / 2, TM = WM / 32, TN = WN / 32;
+    constexpr int ROWS = BM + BN, STAGE_BYTES = ROWS * 128, LOADS = ROWS / 8 / WAVES;      // a wave-wide load fills 8 rows of 128 bytes
+    extern __shared__ __attribute__((aligned(16))) unsigned char ring[];               // 2 * STAGE_BYTES
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), group = wave >> 2;
+    const int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+    // Row `row` of a stage (0 .. 255: rows of A, 256 .. 511: rows of W): where this lane's 16 bytes of it lie, in bytes from the
+    // tile's first row of A or of W at k = 0.  The piece c of a row lies at piece position c ^ ((row >> 1) & 7): see the piped kernel.
+    // A load's address is a scalar base (the tile's first row, advanced by the block's k) plus this offset, so that issuing one
+    // needs no vector instruction: those wait behind a matrix instruction that is under way.
+    const bf16_t* a_tile = A + (size_t)m0 * lda;
+    const bf16_t* w_tile = W + (size_t)n0 * ldw;
+    auto source = [&](int row) -> unsigned {
+        const int c = (lane & 7) ^ ((row >> 1) & 7);
+        return row < BM ? (unsigned)(((size_t)min(row, M - 1 - m0) * lda + 8 * c) * 2) : (unsigned)(((size_t)min(row - BM, N - 1 - n0) * ldw + 8 * c) * 2);
+    };
+    const unsigned ring_base = (unsigned)(size_t)(lds_ptr_t)ring;
+    auto load_rows = [&](unsigned from, int first_row, int block) {                  // 8 rows from `first_row` (the same for the wave) of block `block`
+        const unsigned dst = ring_base + (block & 1) * STAGE_BYTES + first_row * 128;
+        const bf16_t* base = (first_row < BM ? a_tile : w_tile) + block * PK;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(from), "s"(base) : "memory", "m0");
+    };
+    // What a wave loads, 8 loads of 1 KB a block.  The memory pipeline takes such a load every 23 clocks or so, 64 of them a block:
+    // three quarters of the time the block's matrix instructions take; and a wave that issues one is held for as long as the loads
+    // of its workgroup that are ahead of it take, with its next instructions behind it.  So the loads are issued by the group that
+    // reads, behind its reads of LDS (while it would wait for those and then for the other group's matrix instructions anyway), and
+    // they are spread evenly over the block's two barrier intervals.  Which rows can be loaded when follows from who reads them:
+    //   group 0 reads the first 128 rows of A and all of W, in the first interval of a block; group 1 the last 128 rows of A and all of W, in the second.
+    //   group 0, R(b):  the rows of W of block b + 1           (their stage fell free at the barrier before, when group 1 had read block b - 1)
+    //   group 1, R(b):  the first 128 rows of A of block b + 2 (group 0 has just read those of block b) and the last 128 of block b + 1
+    // Every wave waits for its own loads at the end of its M phase; the rows are read two barriers later or more.
+    const int turn = wave & 3;
+    const int first_row = group == 0 ? BM + turn * 64 : turn * 32;                     // of the wave's load 0; group 1's loads 4 .. 7 lie 128 rows further
+    auto row_of = [&](int i) { return first_row + (group == 0 ? 8 * i : 8 * (i & 3) + 128 * (i >> 2)); };
+    unsigned src[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) src[i] = source(row_of(i) + (lane >> 3));
+    const int n_k = K / PK;
+    auto load_one = [&](int i, int block) {                                         // this wave's load i during R(block)
+        const int of_block = group == 0 ? block + 1 : (i < 4 ? block + 2 : block + 1);
+        if (of_block < n_k) load_rows(src[i], row_of(i), of_block);
+    };
+    auto phase_barrier = [&]() {
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = floatx16{};
+
+    // to begin with: all of block 0, and the first 128 rows of A of block 1 (which the R phase before block 0 would have sent for)
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) load_rows(source((wave * LOADS + i) * 8 + (lane >> 3)), (wave * LOADS + i) * 8, 0);
+    if (n_k > 1) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) load_rows(source((wave * 2 + i) * 8 + (lane >> 3)), (wave * 2 + i) * 8, 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    phase_barrier();
+    if (group == 1) phase_barrier();            // group 1 runs one barrier behind group 0's phases
+
+    const int r = lane & 31, swz = (r >> 1) & 7;
+    const unsigned char* a_rows = ring + (wm + r) * 128;
+    const unsigned char* b_rows = ring + (BM + wn + r) * 128;
+    for (int block = 0; block < n_k; ++block) {
+        const int stage_off = (block & 1) * STAGE_BYTES;
+        // ---- R: the operands of the block's 64 k into registers, and behind the reads this wave's loads
+        // (two of the group's waves send their loads first and read then, two the other way round: the memory pipeline is at work
+        // from the start of the interval, and nobody's reads wait behind everybody's loads)
+        bf16x8 a[PK / 16][TM], b[PK / 16][TN];
+        if (turn & 1) {
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i) load_one(i, block);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int step = 0; step < PK / 16; ++step) {
+            const int chunk = ((2 * step + (lane >> 5)) ^ swz) * 16;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) a[step][i] = as_bf16x8(*reinterpret_cast<const uint4*>(a_rows + stage_off + i * 32 * 128 + chunk));
+#pragma unroll
+            for (int j = 0; j < TN; ++j) b[step][j] = as_bf16x8(*reinterpret_cast<const uint4*>(b_rows + stage_off + j * 32 * 128 + chunk));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (!(turn & 1)) {
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i) load_one(i, block);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                          // the reads are done before anyone may refill the stage
+        phase_barrier();
+        // ---- M: nothing but matrix instructions
+#pragma unroll
+        for (int step = 0; step < PK / 16; ++step)
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b[step][j], a[step][i], acc[i][j], 0, 0, 0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                            // what this wave sent for during R has landed
+        phase_barrier();
+    }
+    if (group == 0) phase_barrier();
+    // The weights were the first operand: a lane's 32x32 result holds row (of A) m = lane%32 and, as element v, column
+    // (row of W) n = 8*(v/4) + 4*(lane/32) + v%4, four neighbouring columns at a time.  The results leave through LDS
+    // (the ring is free now: every wave has passed the barrier behind its last read), 128 bytes of 64 rows at a time
+    // in a part of it that is this wave's own, so that every store instruction writes whole cache lines: eight rows of
+    // 128 bytes instead of 32 pieces of 16 or 32 bytes.  Rows lie 144 bytes apart in LDS (16 consecutive rows then
+    // start in 16 different groups of banks, for the 8- and 16-byte writes as for the 16-byte reads).
+    constexpr int STAGE_ROW = 144;
+    unsigned char* mine = ring + wave * (WM * STAGE_ROW);
+    const int frow = lane >> 3, fchunk = lane & 7;                                 // the flush: lane -> (row within 8, 16-byte piece of 128)
+    if constexpr (EPI == EPI_GATED_BF16) {
+        // columns 32b .. 32b+15 are gates, 32b+16 .. 32b+31 the ups of outputs 16b .. 16b+15: element v beside element v + 8.
+        // The wave's WN columns become WN/2 outputs: 2 * WN/2 bytes a row, flushed 64 outputs (128 bytes) at a time.
+        static_assert(WN % 128 == 0, "the gated flush takes 64 outputs at a time");
+#pragma unroll
+        for (int part = 0; part < WN / 128; ++part) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) {
+                    const int j = 4 * part + jj;
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        const uint2 packed = {f32x2_to_bf16x2(silu_gate_fast(acc[i][j][4 * q], acc[i][j][4 * q + 8]), silu_gate_fast(acc[i][j][4 * q + 1], acc[i][j][4 * q + 9])),
+                                              f32x2_to_bf16x2(silu_gate_fast(acc[i][j][4 * q + 2], acc[i][j][4 * q + 10]), silu_gate_fast(acc[i][j][4 * q + 3], acc[i][j][4 * q + 11]))};
+                        *reinterpret_cast<uint2*>(mine + (i * 32 + (lane & 31)) * STAGE_ROW + (jj * 16 + 8 * q + 4 * (lane >> 5)) * 2) = packed;
+                    }
+                }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int it = 0; it < WM / 8; ++it) {
+                const int row = it * 8 + frow, m = m0 + wm + row, c = (n0 + wn) / 2 + part * 64 + fchunk * 8;      // output column
+                const uint4 v = *reinterpret_cast<const uint4*>(mine + row * STAGE_ROW + fchunk * 16);
+                if (m < M && c + 7 < N / 2 && (ldc & 7) == 0) *reinterpret_cast<uint4*>((bf16_t*)C + (size_t)m * ldc + c) = v;
+                else if (m < M) {
+                    const bf16_t* e = reinterpret_cast<const bf16_t*>(&v);
+#pragma unroll
+                    for (int x = 0; x < 8; ++x)
+                        if (c + x < N / 2) ((bf16_t*)C)[(size_t)m * ldc + c + x] = e[x];
+                }
+            }
+        }
+    } else if constexpr (EPI == EPI_STORE_BF16) {
+#pragma unroll
+        for (int part = 0; part < TN / 2; ++part) {                                // 64 columns = 128 bytes a row at a time
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const floatx16& t = acc[i][2 * part + jj];
+                        *reinterpret_cast<uint2*>(mine + (i * 32 + (lane & 31)) * STAGE_ROW + (jj * 32 + 8 * q + 4 * (lane >> 5)) * 2) =
+                            uint2{f32x2_to_bf16x2(t[4 * q], t[4 * q + 1]), f32x2_to_bf16x2(t[4 * q + 2], t[4 * q + 3])};
+                    }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int it = 0; it < WM / 8; ++it) {
+                const int row = it * 8 + frow, m = m0 + wm + row, c = n0 + wn + part * 64 + fchunk * 8;
+                const uint4 v = *reinterpret_cast<const uint4*>(mine + row * STAGE_ROW + fchunk * 16);
+                if (m < M && c + 7 < N && (ldc & 7) == 0) *reinterpret_cast<uint4*>((bf16_t*)C + (size_t)m * ldc + c) = v;
+                else if (m < M) {
+                    const bf16_t* e = reinterpret_cast<const bf16_t*>(&v);
+#pragma unroll
+                    for (int x = 0; x < 8; ++x)
+                        if (c + x < N) ((bf16_t*)C)[(size_t)m * ldc + c + x] = e[x];
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {                                             // 32 columns = 128 bytes a row at a time
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    *reinterpret_cast<float4*>(mine + (i * 32 + (lane & 31)) * STAGE_ROW + (8 * q + 4 * (lane >> 5)) * 4) =
+                        float4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int it = 0; it < WM / 8; ++it) {
+                const int row = it * 8 + frow, m = m0 + wm + row, c = n0 + wn + j * 32 + fchunk * 4;
+                float4 v = *reinterpret_cast<const float4*>(mine + row * STAGE_ROW + fchunk * 16);
+                if (m >= M) continue;
+                float* dst = (float*)C + (size_t)m * ldc + c;
+                if (c + 3 < N && (ldc & 3) == 0 && (((uintptr_t)C) & 15) == 0) {
+                    if constexpr (EPI == EPI_ADD_F32) {
+                        const float4 old = *reinterpret_cast<const float4*>(dst);
+                        v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
+                    }
+                    *reinterpret_cast<float4*>(dst) = v;
+                } else {
+                    const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int x = 0; x < 4; ++x)
+                        if (c + x < N) write_out<EPI>(C, (size_t)m * ldc + c + x, e[x]);
+                }
+            }
+        }
+    }
 }
 
 // ----------------------------------------------------------------------------------------- skinny
@@ -601,12 +840,31 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
             GI_CHECK_LAUNCH("gemm_bf16 (piped, split)");
             return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream);
         }
-        // Measured at 2,048 rows (K = 2048 and 8192): where 256 x 256 tiles still give every compute unit two, they halve
-        // the traffic into LDS; otherwise 128 x 128, two workgroups per unit with two stages each when there are enough
-        // tiles, else one workgroup of eight waves with four stages.
+        // Measured at 2,048 rows (K = 2048 and 8192): where 256 x 256 tiles give every compute unit one or more, they halve
+        // the traffic into LDS and run the two groups of waves out of step (the ping-pong kernel); otherwise 128 x 128, two
+        // workgroups per unit with two stages each when there are enough tiles, else one workgroup of eight waves with four stages.
         const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128), tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-        if (tiles256 >= 512) PIPED_EPI(256, 256, 4, 2, 2);
-        else if (tiles128 > 256) PIPED_EPI(128, 128, 2, 2, 2);
+        if (tiles256 >= 256) {                         // a 256 x 256 tile or more for every compute unit: the ping-pong kernel
+#define PINGPONG(EPI_)                                                                                                                  \
+    do {                                                                                                                                \
+        constexpr int bytes = 2 * 512 * 128;                                                                                            \
+        static bool raised = false;                                                                                                     \
+        if (!raised) {                                                                                                                  \
+            if (hipFuncSetAttribute((const void*)gemm_bf16_pingpong_kernel<256, EPI_>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) \
+                return gi_fail("gemm_bf16: cannot reserve %d bytes of LDS", bytes);                                                     \
+            raised = true;                                                                                                              \
+        }                                                                                                                               \
+        dim3 grid((N + 255) / 256, (M + 255) / 256);                                                                                    \
+        gemm_bf16_pingpong_kernel<256, EPI_><<<grid, 512, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+    } while (0)
+            GI_REQUIRE(lda < (1L << 22) && ldw < (1L << 22), "gemm_bf16: row strides %ld, %ld are too large for the tile-relative addressing", lda, ldw);
+            if (epi == EPI_STORE_F32) PINGPONG(EPI_STORE_F32); else if (epi == EPI_ADD_F32) PINGPONG(EPI_ADD_F32);
+            else if (epi == EPI_STORE_BF16) PINGPONG(EPI_STORE_BF16); else PINGPONG(EPI_GATED_BF16);
+#undef PINGPONG
+            GI_CHECK_LAUNCH("gemm_bf16 (pingpong)");
+            return 0;
+        }
+        if (tiles128 > 256) PIPED_EPI(128, 128, 2, 2, 2);
         else PIPED_EPI(128, 128, 2, 4, 4);
 #undef PIPED_EPI
 #undef PIPED

@@ -62,6 +62,8 @@ def test_gemm_exact_rows_alone_have_the_same_bits(w_dtype, k):
                                    (513, 384, 1024), (2048, 96, 160),
                                    # the LDS-ring kernel: one block of k, edge tiles, each of its three tile choices
                                    (256, 160, 64), (130, 129, 192), (2100, 2200, 192), (4000, 8200, 128),
+                                   # the ping-pong kernel (a 256 x 256 tile or more for every compute unit): one block of k, an odd number of them, edges
+                                   (4100, 4104, 64), (4096, 4100, 320),
                                    # ... and with k shared out over workgroups because the tiles are few
                                    (72, 256, 1024), (300, 2048, 2048), (65, 130, 512),
                                    # wide outputs finished by the skinny kernel itself, from 12 rows and from 5
@@ -79,7 +81,8 @@ def test_gemm_bf16(m, n, k, out_dtype, accumulate):
 
 
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 8), (5, 48, 136), (16, 160, 96), (17, 176, 64), (64, 32, 264), (70, 192, 128), (300, 8192 // 16, 2048 // 8),
-                                       (40, 6144, 264), (13, 6160, 72), (64, 8192, 512), (2048, 1024, 192), (600, 288, 64), (200, 512, 1024)])
+                                       (40, 6144, 264), (13, 6160, 72), (64, 8192, 512), (2048, 1024, 192), (600, 288, 64), (200, 512, 1024),
+                                       (4100, 2064, 128)])
 def test_gemm_bf16_gated(m, inter, k):
     a = randn(m, k, dtype=torch.bfloat16, seed=15)
     gate, up = randn(inter, k, dtype=torch.bfloat16, seed=16, scale=0.3), randn(inter, k, dtype=torch.bfloat16, seed=17, scale=0.3)
@@ -89,6 +92,22 @@ def test_gemm_bf16_gated(m, inter, k):
     want = torch.nn.functional.silu(a.double() @ gate.double().T) * (a.double() @ up.double().T)
     assert rel(out[:, :inter], want) < 6e-3
     assert torch.all(out[:, inter:] == 3.0)
+
+
+@pytest.mark.parametrize("m,n,k", [(4109, 4120, 192), (4096, 4096, 448)])
+def test_gemm_bf16_ping_pong_with_whole_lines(m, n, k):
+    """Outputs whose rows are 16-byte aligned leave the ping-pong kernel in whole cache lines: every epilogue, with edge tiles."""
+    a, w = randn(m, k, dtype=torch.bfloat16, seed=25), randn(n, k, dtype=torch.bfloat16, seed=26, scale=0.3)
+    want = a.double() @ w.double().T
+    for out_dtype, accumulate in ((torch.float32, False), (torch.float32, True), (torch.bfloat16, False)):
+        base = randn(m, n, seed=27).to(out_dtype)
+        out = base.clone()
+        ops().gemm_bf16(a, w, out, accumulate=accumulate)
+        assert rel(out, want + (base.double() if accumulate else 0)) < (1e-5 if out_dtype == torch.float32 else 5e-3), (out_dtype, accumulate)
+    gate, up = w[:n // 2 // 16 * 16], w[n // 2:n // 2 + n // 2 // 16 * 16]
+    out = torch.full((m, gate.shape[0]), 3.0, dtype=torch.bfloat16, device=DEV)
+    ops().gemm_bf16(a, ops().interleave_gate_up(gate.contiguous(), up.contiguous()), out, gated=True)
+    assert rel(out, torch.nn.functional.silu(a.double() @ gate.double().T) * (a.double() @ up.double().T)) < 6e-3
 
 
 def test_gemm_bf16_refuses_what_it_cannot_do():
