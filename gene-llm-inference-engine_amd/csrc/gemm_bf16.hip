@@ -697,6 +697,71 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
     }
 }
 
+// The same for a few more rows of A (MT tiles of 16) and outputs too narrow to fill the chip with strips of 64 weight rows: a workgroup owns 16
+// weight rows and all of k, its 8 waves take interleaved 128-wide blocks of k, and each wave multiplies its weights with MT tiles
+// of 16 activation rows, all straight from global memory into registers (the waves share nothing: every wave reads another part
+// of k; the activations come from L2, as many bytes again for every 16 rows as the strip has weights, which pays up to 32 rows).
+// One launch does the product and its epilogue; the alternative, k shared out over workgroups with partial sums in memory and a
+// second kernel to add them, costs that kernel's launch and as many bytes of partial sums as the output projection has weights.
+template <int MT, int EPI>
+__global__ __launch_bounds__(512) void gemm_bf16_slim_tiles_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
+                                                                  int M, int N, int K, long lda, long ldw, long ldc) {
+    constexpr int SLICES = 8, STEP = SLICES * SK, DEPTH = 2;
+    __shared__ float red[SLICES][MT][64][4];
+    const int tid = threadIdx.x, lane = tid & 63, slice = tid >> 6;
+    const int r = lane & 15, q = lane >> 4;
+    const int n = blockIdx.x * 16 + r;
+    const bool w_ok = n < N;
+    const bf16_t* wrow = W + (size_t)(w_ok ? n : 0) * ldw + 8 * q;
+    const bf16_t* xrow[MT];
+    bool x_ok[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        x_ok[t] = t * 16 + r < M;
+        xrow[t] = A + (size_t)(x_ok[t] ? t * 16 + r : 0) * lda + 8 * q;
+    }
+    floatx4 acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = floatx4{};
+    uint4 w_buf[DEPTH][4], x_buf[DEPTH][MT][4];
+    auto fetch = [&](int k0, uint4* w, uint4 (*x)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const bool in = k0 + 32 * j + 8 * q < K;
+            w[j] = (in && w_ok) ? load16(wrow + k0 + 32 * j) : uint4{0, 0, 0, 0};
+#pragma unroll
+            for (int t = 0; t < MT; ++t) x[t][j] = (in && x_ok[t]) ? load16(xrow[t] + k0 + 32 * j) : uint4{0, 0, 0, 0};
+        }
+    };
+    const int k_first = slice * SK;
+    fetch(k_first, w_buf[0], x_buf[0]);
+    for (int k0 = k_first; k0 < K; k0 += DEPTH * STEP) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {                     // buffer d holds block k0 + d*STEP
+            fetch(k0 + (d + 1) * STEP, w_buf[(d + 1) % DEPTH], x_buf[(d + 1) % DEPTH]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x_buf[d][t][j]), as_bf16x8(w_buf[d][j]), acc[t], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[slice][t][lane][v] = acc[t][v];
+    __syncthreads();
+    // Element v of a lane's result for tile t: activation row 16*t + 4*q + v, weight row r of the strip.
+    for (int e = tid; e < MT * 256; e += 512) {
+        const int t = e >> 8, m = (e >> 4) & 15, c = e & 15;
+        const int src_lane = c + 16 * (m >> 2), v = m & 3, row = 16 * t + m, col = blockIdx.x * 16 + c;
+        float sum = 0.f;
+#pragma unroll
+        for (int s = 0; s < SLICES; ++s) sum += red[s][t][src_lane][v];
+        if (row < M && col < N) write_out<EPI>(C, (size_t)row * ldc + col, sum);
+    }
+}
+
 int epilogue_of(int c_dtype, int accumulate) {
     if (c_dtype == GI_F32) return accumulate ? EPI_ADD_F32 : EPI_STORE_F32;
     if (c_dtype == GI_BF16 && !accumulate) return EPI_STORE_BF16;
@@ -781,6 +846,23 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
         return 0;
     }
 
+    // 17 to 32 rows, a narrow output and a short k: one launch of the slim kernel with two tiles of activation rows.  Measured at
+    // N = 3072 and 2048, K = 2048 against the skinny kernel's partial sums and their second kernel: 9 against 13 us at 17 and 32 rows,
+    // 11 against 13 at 48, 13 against 13 at 64; at K = 8192 (every workgroup reads all the activations: 1 MB at 64 rows) 21 to 43 us
+    // against 16 to 19, so longer k and more rows stay with the skinny kernel.
+    if (M <= 32 && K <= 2048 && epi != EPI_GATED_BF16 && gi_gemm_bf16_skinny_splits(N, K) > 0) {
+        dim3 grid((N + 15) / 16);
+#define SLIM_TILES(MT_)                                                                                                                             \
+    do {                                                                                                                                            \
+        if (epi == EPI_STORE_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+        else if (epi == EPI_ADD_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_ADD_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+        else gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_BF16><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+    } while (0)
+        SLIM_TILES(2);
+#undef SLIM_TILES
+        GI_CHECK_LAUNCH("gemm_bf16 (slim, tiles)");
+        return 0;
+    }
     if (M <= 64) {
         const int splits = gi_gemm_bf16_skinny_splits(N, K), mt = (M + 15) / 16;
 #define SKINNY_MT(EPI_, PARTIAL_)                                                                                                   \

@@ -67,7 +67,9 @@ def test_gemm_exact_rows_alone_have_the_same_bits(w_dtype, k):
                                    # ... and with k shared out over workgroups because the tiles are few
                                    (72, 256, 1024), (300, 2048, 2048), (65, 130, 512),
                                    # wide outputs finished by the skinny kernel itself, from 12 rows and from 5
-                                   (12, 12300, 520), (40, 12300, 264), (5, 65600, 72), (16, 12288, 256)])
+                                   (12, 12300, 520), (40, 12300, 264), (5, 65600, 72), (16, 12288, 256),
+                                   # 17 to 32 rows, narrow outputs, short k: the slim kernel with two tiles of rows
+                                   (32, 2048, 2048), (20, 3072, 2048), (31, 130, 136), (17, 16, 8)])
 @pytest.mark.parametrize("out_dtype,accumulate", [(torch.float32, False), (torch.float32, True), (torch.bfloat16, False)])
 def test_gemm_bf16(m, n, k, out_dtype, accumulate):
     a, w = randn(m, k, dtype=torch.bfloat16, seed=5), randn(n, k, dtype=torch.bfloat16, seed=6)
