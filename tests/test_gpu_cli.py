@@ -36,9 +36,25 @@ def test_gi_generate_greedy_dumps_the_plain_tokens(tmp_path):
     assert "device profile: 6 positions in 5 steps" in again.stderr and "gemm_bf16" in again.stderr and "weights GB/s" in again.stderr
 
 
+@pytest.mark.gpu
+def test_gi_generate_from_a_configuration_alone_draws_the_weights_make_random_model_writes(tmp_path):
+    """--config FILE --random-seed S: no folder; the tokens are those of the folder that make_random_model writes for the same seed."""
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(full_config(CONFIGS["B"])))
+    made = subprocess.run([str(ROOT / "bin" / "make_random_model"), "--config", str(cfg), "--out", str(tmp_path / "m"), "--seed", "4", "--dtype", "float32"],
+                          capture_output=True, text=True, timeout=120)
+    assert made.returncode == 0, made.stderr
+    common = ["--prompt-ids", "5 9 200 31", "--steps", "12", "--temperature", "0", "--weights", "f32", "--no-echo", "--quiet"]
+    a = subprocess.run([str(ROOT / "bin" / "gi_generate"), "--config", str(cfg), "--random-seed", "4", *common], capture_output=True, text=True, timeout=170)
+    b = subprocess.run([str(ROOT / "bin" / "gi_generate"), "--model", str(tmp_path / "m"), *common], capture_output=True, text=True, timeout=170)
+    assert a.returncode == 0 and b.returncode == 0, a.stderr + b.stderr
+    assert len(a.stdout.split()) == 9 and a.stdout == b.stdout
+
+
 def test_gi_generate_usage_errors(tmp_path):
     exe = str(ROOT / "bin" / "gi_generate")
-    for args, msg in (([], "--model is required"), (["--model", "x", "--weights", "int8"], "--weights must be native or f32"),
+    for args, msg in (([], "give --model DIR, or --config FILE"), (["--model", "x", "--config", "y"], "give --model DIR, or --config FILE"),
+                      (["--model", "x", "--weights", "int8"], "--weights must be native or f32"),
                       (["--model", "x", "--frobnicate"], "unknown option --frobnicate"), (["--model"], "missing value for --model"),
                       (["--model", "x", "--steps", "ten"], "invalid integer for --steps"), (["--model", "x", "--device", "cpu"], "only gpu exists")):
         r = subprocess.run([exe, *args], capture_output=True, text=True, timeout=60)
