@@ -63,15 +63,14 @@ def main() -> int:
     vocab = config.vocab_size
     gen = torch.Generator().manual_seed(1)
 
-    WINDOWS = 5
+    WINDOWS, PREFILL_WARMUP = 5, 4
 
     def make_runner(batch):
         per_request = -(-(PROMPT + WINDOWS * args.steps + args.warmup + 2 * batch + 8) // 64) * 64
         return Runner(model, page_size=PAGE, max_tokens=batch * per_request, max_requests=batch, max_rows=max(PROMPT, batch),
                       max_positions=CONTEXT)
 
-    def prefill(runner, rid):
-        toks = torch.randint(0, vocab, (PROMPT,), generator=gen).tolist()
+    def prefill(runner, rid, toks):
         runner.open(rid)
         return runner.step([StepEntry(rid, toks, (PROMPT - 1,))])
 
@@ -106,17 +105,18 @@ def main() -> int:
         torch.cuda.empty_cache()
         return sorted(windows)
 
-    # ---- prefill of one 2,048-token prompt (median of 5 after one warm-up)
+    # ---- prefill of one 2,048-token prompt (median of 5 after PREFILL_WARMUP untimed ones: the first few run some percent slower)
     runner = make_runner(1)
     times = []
-    for i in range(6):
+    for i in range(PREFILL_WARMUP + 5):
+        toks = torch.randint(0, vocab, (PROMPT,), generator=gen).tolist()       # the prompt is there before the clock starts
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        logits = prefill(runner, i)
+        logits = prefill(runner, i, toks)
         int(torch.argmax(logits[0]))           # the first token reaches the host
         times.append(time.perf_counter() - t0)
         runner.close(i)
-    prefill_s = sorted(times[1:])[len(times[1:]) // 2]
+    prefill_s = sorted(times[PREFILL_WARMUP:])[2]
     del runner
     torch.cuda.empty_cache()
     L, D, I, V = config.num_hidden_layers, config.hidden_size, config.intermediate_size, vocab

@@ -155,9 +155,8 @@ class PageGroup:
             return
         block = self.table_host[rows, lo:hi]
         if upload is not None:                 # int32 array -> device tensor without waiting for the device
-            idx = upload(np.asarray(rows, dtype=np.int32))
-            data = upload(block).view(len(rows), hi - lo)
-            self.table_dev[:, lo:hi].index_copy_(0, idx.long(), data)
+            idx, data = upload(np.asarray(rows, dtype=np.int32), block)      # (both in one copy)
+            self.table_dev[:, lo:hi].index_copy_(0, idx.long(), data.view(len(rows), hi - lo))
             return
         idx = torch.tensor(rows, dtype=torch.int64)
         self.table_dev[:, lo:hi].index_copy_(0, idx.to(self.table_dev.device), torch.from_numpy(np.ascontiguousarray(block)).to(self.table_dev.device))
@@ -393,7 +392,7 @@ class CacheManager:
         self._length[request] = length
 
     def sync(self, upload=None) -> None:
-        """Brings the device copies of changed page tables up to date.  `upload(int32 array) -> device tensor`
+        """Brings the device copies of changed page tables up to date.  `upload(int32 arrays...) -> device tensors`
         is the caller's way of copying without waiting for the device (it must take a snapshot at once)."""
         for g in self.groups:
             g.sync(upload)

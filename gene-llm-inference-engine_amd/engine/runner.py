@@ -163,8 +163,11 @@ class Runner:
             row += n
 
         dev = self.model.device
-        meta_dev = self._uploads.put(meta).view(3, n_rows)
-        rows_dev = self._uploads.put(np.asarray(logit_rows, dtype=np.int32)) if logit_rows else None
+        if logit_rows:
+            meta_dev, rows_dev = self._uploads.put(meta, np.asarray(logit_rows, dtype=np.int32))
+        else:
+            meta_dev, rows_dev = self._uploads.put(meta), None
+        meta_dev = meta_dev.view(3, n_rows)
         ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
                           row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0,
                           upload=self._uploads.put)
@@ -288,17 +291,24 @@ class _StepUploads:
         if self.done[self.turn] is not None:
             self.done[self.turn].synchronize()
 
-    def put(self, values: np.ndarray) -> torch.Tensor:
-        flat = np.ascontiguousarray(values, dtype=np.int32).reshape(-1)
-        n = flat.size
-        if self.used + n > self.capacity:                       # more than the ring was made for: an ordinary copy
-            return torch.from_numpy(flat.copy()).to(self.device)
-        a, b = self.used, self.used + n
-        self.used = (b + 3) & ~3                                # pieces start at multiples of 16 bytes
-        self.host[self.turn][a:b] = torch.from_numpy(flat)
-        piece = self.dev[self.turn][a:b]
-        piece.copy_(self.host[self.turn][a:b], non_blocking=True)
-        return piece
+    def put(self, *arrays):
+        """The arrays on the device (int32, flattened): one tensor for one array, a tuple for several, which then
+        go over in one copy."""
+        flats = [np.ascontiguousarray(values, dtype=np.int32).reshape(-1) for values in arrays]
+        first, spans = self.used, []
+        for flat in flats:
+            a = self.used
+            if a + flat.size > self.capacity:                   # more than the ring was made for: ordinary copies
+                self.used = first
+                pieces = tuple(torch.from_numpy(f.copy()).to(self.device) for f in flats)
+                return pieces[0] if len(pieces) == 1 else pieces
+            self.host[self.turn][a:a + flat.size] = torch.from_numpy(flat)
+            spans.append((a, a + flat.size))
+            self.used = (a + flat.size + 3) & ~3                # pieces start at multiples of 16 bytes
+        last = spans[-1][1]
+        self.dev[self.turn][first:last].copy_(self.host[self.turn][first:last], non_blocking=True)
+        pieces = tuple(self.dev[self.turn][a:b] for a, b in spans)
+        return pieces[0] if len(pieces) == 1 else pieces
 
     def stage(self, values: np.ndarray) -> torch.Tensor:
         """The values in this step's pinned buffer only (for a copy the caller makes itself, into its own device memory)."""

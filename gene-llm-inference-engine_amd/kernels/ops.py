@@ -405,17 +405,18 @@ class AttentionPlan:
         self.n_decode, self.n_tiles = len(dec), len(tiles)
         self.n_tile_rows = sum(t[1] for t in tiles)
         self.max_tile_context = max((t[2] + t[1] for t in tiles), default=0)
-        put = to_device if to_device is not None else (lambda values: torch.tensor(values, dtype=torch.int32).to(device))
-        flat_tiles = [v for t in tiles for v in t]
-        self.decode_rows = put(dec) if dec and tiles else None      # no prompt rows: the decode rows are all rows, in order
-        self.tiles = put(flat_tiles) if tiles else torch.empty(0, dtype=torch.int32, device=device)      # read 16 bytes at a time: its own piece
         # for sharing a tile's keys out over workgroups: rows before each tile, and the tiles' rows in order
         firsts, count = [], 0
         for t in tiles:
             firsts.append(count)
             count += t[1]
-        self.tile_first = put(firsts) if tiles else None
-        self.tile_rows = put([r for t in tiles for r in range(t[0], t[0] + t[1])]) if tiles else None
+        put = to_device if to_device is not None else (lambda *lists: tuple(torch.tensor(values, dtype=torch.int32).to(device) for values in lists))
+        self.decode_rows = self.tile_first = self.tile_rows = None      # no prompt rows: the decode rows are all rows, in order
+        self.tiles = torch.empty(0, dtype=torch.int32, device=device)
+        if tiles:                            # (every piece starts at a multiple of 16 bytes: the kernel reads a tile's four numbers at once)
+            self.tiles, self.tile_first, self.tile_rows, *rest = put([v for t in tiles for v in t], firsts, [r for t in tiles for r in range(t[0], t[0] + t[1])],
+                                                                     *([dec] if dec else []))
+            self.decode_rows = rest[0] if rest else None
 
 
 def attention_bf16_supports(hd, page_size, prompt: bool) -> bool:

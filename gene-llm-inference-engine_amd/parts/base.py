@@ -46,15 +46,17 @@ class StepContext:
     seg_len: List[int]                       # number of rows,
     seg_pos0: List[int]                      # position of the first row
     memo: Dict[Any, Any] = field(default_factory=dict)     # per-step tables shared by layers (rotary cos/sin)
-    upload: Optional[Callable[[np.ndarray], torch.Tensor]] = None      # the runner's way of bringing int32 step data to the device
+    upload: Optional[Callable[..., Any]] = None    # the runner's way of bringing int32 step data to the device: upload(a) -> tensor, upload(a, b) -> (tensor, tensor) in one copy
     trace: Optional[Callable[[str, torch.Tensor], None]] = None        # debugging: a block reports (tag, residual stream [T, hidden]) after each of its two halves
 
-    def to_device(self, values) -> torch.Tensor:
-        """int32 data made on the host for this step (row lists, tile lists) as a device tensor, valid during the step."""
-        arr = np.ascontiguousarray(values, dtype=np.int32)
+    def to_device(self, *values):
+        """int32 data made on the host for this step (row lists, tile lists) as device tensors, valid during the step:
+        one tensor for one list, a tuple for several (which the runner sends in one copy)."""
+        arrays = [np.ascontiguousarray(v, dtype=np.int32) for v in values]
         if self.upload is not None:
-            return self.upload(arr)
-        return torch.from_numpy(arr).to(self.device)
+            return self.upload(*arrays)
+        pieces = tuple(torch.from_numpy(a).to(self.device) for a in arrays)
+        return pieces[0] if len(pieces) == 1 else pieces
 
     @property
     def max_seg_len(self) -> int:

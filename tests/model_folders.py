@@ -37,6 +37,13 @@ LLAMA_1B_SHAPE = dict(hidden_size=2048, intermediate_size=8192, num_hidden_layer
                       rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
                                         original_max_position_embeddings=8192),
                       rms_norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=4096)
+# The layer shape of Llama 3.2 3B (24 query heads over 8 key/value heads of 128 channels, hidden 3072) with one layer and a
+# vocabulary cut to a number that is no multiple of anything: heads of 128 channels and widths that are no power of two in one model.
+LLAMA_3B_SHAPE = dict(hidden_size=3072, intermediate_size=8192, num_hidden_layers=1, num_attention_heads=24, num_key_value_heads=8,
+                      head_dim=128, vocab_size=32003, rope_theta=500000.0,
+                      rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                        original_max_position_embeddings=8192),
+                      rms_norm_eps=1e-5, tie_word_embeddings=True, max_position_embeddings=4096)
 PAGE_SIZE = {"A": 4, "B": 8, "C": 16, "D": 16}
 CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 

@@ -505,9 +505,9 @@ def test_the_device_copy_of_the_tables_follows_under_random_use_with_few_columns
     rng = random.Random(11)
     m = CacheManager([FULL, WINDOW], [None, None], page_size=4, n_pages=60, max_requests=4, max_positions=120, dtype=torch.float32, device="cpu")
     sent = []
-    def upload(values):
-        sent.append(values.size)
-        return torch.from_numpy(values.copy().reshape(-1))
+    def upload(rows, block):
+        sent.append(block.size)
+        return torch.from_numpy(rows.copy().reshape(-1)), torch.from_numpy(block.copy().reshape(-1))
     live = []
     for turn in range(500):
         roll = rng.random()

@@ -4,14 +4,16 @@ key/value heads of 64 channels, feed-forward 8192, vocabulary 128256, llama3 sca
 feed-forward product over 2048 of k, the head over 128256 rows, prompt attention over many paired tiles, decode attention
 with split contexts) meet the plain model under every way of cutting the work, in 32-bit and in bfloat16.  Logits are
 compared at every 16th position and at the last of each request.  What tests/verify_forward.py:72-117 does for the
-reference at its sizes."""
+reference at its sizes.  The layer shape of Llama 3.2 3B (hidden 3072, 24 query heads over 8 key/value heads of 128
+channels, one layer, a cut vocabulary) follows in bfloat16 under the cuts that differ most: whole prompts, and long
+portions beside single tokens with pages used again."""
 import random
 
 import pytest
 import torch
 
 import traces
-from model_folders import LLAMA_1B_SHAPE, assert_within_bfloat16_noise, relative_error, write_model
+from model_folders import LLAMA_1B_SHAPE, LLAMA_3B_SHAPE, assert_within_bfloat16_noise, relative_error, write_model
 from plain_llama import PlainLlama
 
 pytestmark = pytest.mark.gpu
@@ -20,12 +22,10 @@ EVERY = 16
 PAGE = 16
 
 
-@pytest.fixture(scope="module")
-def case(tmp_path_factory):
-    folder = tmp_path_factory.mktemp("llama1b_shape")
-    write_model(folder, LLAMA_1B_SHAPE, seed=31, dtype=torch.bfloat16, std=0.02)
+def make_case(folder, sizes, seed):
+    write_model(folder, sizes, seed=seed, dtype=torch.bfloat16, std=0.02)
     rng = random.Random(9)
-    requests = {f"r{i}": [rng.randrange(LLAMA_1B_SHAPE["vocab_size"]) for _ in range(n)] for i, n in enumerate(LENGTHS)}
+    requests = {f"r{i}": [rng.randrange(sizes["vocab_size"]) for _ in range(n)] for i, n in enumerate(LENGTHS)}
     plain = PlainLlama(folder)
     rounded = plain.with_storage(torch.bfloat16)
     want = {"float32": {}, "bfloat16": {}}
@@ -35,6 +35,16 @@ def case(tmp_path_factory):
             for p, row in zip(places, model.logits_at(toks, places)):
                 want[dtype][(rid, p)] = row
     return folder, requests, want, {}
+
+
+@pytest.fixture(scope="module")
+def case(tmp_path_factory):
+    return make_case(tmp_path_factory.mktemp("llama1b_shape"), LLAMA_1B_SHAPE, 31)
+
+
+@pytest.fixture(scope="module")
+def case_3b(tmp_path_factory):
+    return make_case(tmp_path_factory.mktemp("llama3b_shape"), LLAMA_3B_SHAPE, 32)
 
 
 def model_of(case, dtype):
@@ -95,3 +105,14 @@ def test_llama_1b_layer_shape_under_every_cut(case, dtype, mode):
     else:
         mean_e, mean_n = assert_within_bfloat16_noise(got, want["float32"].__getitem__, want["bfloat16"].__getitem__, f"1B shape, {mode}")
         print(f"1B shape bfloat16 {mode}: mean error {mean_e:.2e} (rounding noise {mean_n:.2e}), {len(steps)} steps")
+
+
+@pytest.mark.parametrize("mode", ["whole", "tail_singly", "mixed_long"])
+def test_llama_3b_layer_shape_in_bfloat16(case_3b, mode):
+    folder, requests, want, _ = case_3b
+    steps = MODES[mode](requests)
+    model = model_of(case_3b, "bfloat16")
+    got = replay(model, steps, traces.peak_tokens(steps, round_to=PAGE))
+    assert set(got) == set(want["bfloat16"])
+    mean_e, mean_n = assert_within_bfloat16_noise(got, want["float32"].__getitem__, want["bfloat16"].__getitem__, f"3B shape, {mode}")
+    print(f"3B shape bfloat16 {mode}: mean error {mean_e:.2e} (rounding noise {mean_n:.2e}), {len(steps)} steps")

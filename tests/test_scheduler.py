@@ -311,6 +311,11 @@ def test_step_uploads_ring_on_the_cpu():
         assert ring.used % 4 == 0 and piece.data_ptr() % 16 == second.data_ptr() % 16
         big = ring.put(np.arange(100, dtype=np.int32))        # more than the ring holds
         assert big.tolist() == list(range(100))
+        x, y = ring.put(np.arange(3), np.arange(7) + step)    # several at once: one copy, each piece aligned
+        assert x.tolist() == [0, 1, 2] and y.tolist() == [step + i for i in range(7)] and y.data_ptr() % 16 == x.data_ptr() % 16
+        used = ring.used
+        x, y = ring.put(np.arange(3), np.arange(100))         # ... and when one of them does not fit, nothing of the ring is used
+        assert x.tolist() == [0, 1, 2] and y.tolist() == list(range(100)) and ring.used == used
         ring.end_step()
         kept.append((step, piece))
         for s, p in kept[-(_StepUploads.DEPTH - 1):]:         # the pieces of the last steps are still what they were
