@@ -9,6 +9,11 @@ with a window gives pages back as soon as no later position can see them; a requ
 gives back everything.  Requests also hold a slot in every fixed-size state tensor
 [slot][...], zeroed when the request opens.
 
+Behind the request slots lies one spare slot that no request ever holds, with one page of its own
+in every group, outside the pool, for positions 0 .. page_size-1: rows that only fill a step up to
+a size it was prepared for (a captured decode step) are computed there, at position 0, and touch
+nothing a request can see.
+
 The reference's pool is one group over all layers with per-sequence tables kept on the host
 (src/model/kv_cache.h:4-13, 73-118); groups, windows and state slots have no counterpart there.
 """
@@ -36,7 +41,8 @@ class PageGroup:
         self.page_size = page_size
         self.pool = PagePool(n_pages)
         self.table_width = -(-max_positions // page_size)
-        self.table_host = np.full((max_requests, self.table_width), -1, dtype=np.int32)
+        self.table_host = np.full((max_requests + 1, self.table_width), -1, dtype=np.int32)
+        self.table_host[max_requests, 0] = n_pages                   # the spare slot's page, behind the pool's
         self.first_live = np.zeros(max_requests, dtype=np.int64)     # pages below this index were given back (windows)
         self.n_held = np.zeros(max_requests, dtype=np.int64)         # table entries in use, counted from 0
         self.dirty: set = set()                      # slots whose table row on the device is out of date
@@ -45,8 +51,8 @@ class PageGroup:
         self.storage = None
         self.table_dev = None
         if allocate_storage:
-            self.storage = torch.zeros((len(entries), n_pages, 2, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
-            self.table_dev = torch.full((max_requests, self.table_width), -1, dtype=torch.int32, device=device)
+            self.storage = torch.zeros((len(entries), n_pages + 1, 2, need.n_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
+            self.table_dev = torch.tensor(self.table_host, dtype=torch.int32, device=device)
 
     def _changed(self, slot: int, first_entry: int) -> None:
         self.dirty_from[slot] = min(int(self.dirty_from[slot]), first_entry) if slot in self.dirty else first_entry
@@ -171,6 +177,7 @@ class CacheManager:
         if page_size < 1 or n_pages < 1 or max_requests < 1 or max_positions < 1:
             raise ValueError("page_size, n_pages, max_requests and max_positions must be positive")
         self.page_size, self.max_requests, self.max_positions = int(page_size), int(max_requests), int(max_positions)
+        self.spare_slot = self.max_requests          # a slot of tables and state that no request holds
         self.groups: List[PageGroup] = []
         self._entry_group: Dict[int, Tuple[int, int]] = {}          # entry -> (group index, layer index in group)
         self.states: Dict[int, torch.Tensor] = {}
@@ -184,7 +191,7 @@ class CacheManager:
                 by_need.setdefault(need, []).append(i)
             elif isinstance(need, StateNeed):
                 if allocate_storage:
-                    self.states[i] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
+                    self.states[i] = torch.zeros((max_requests + 1, *need.shape), dtype=need.dtype, device=device)
             elif need is not None:
                 raise CacheError(f"run-order entry {i} has an unknown cache need {need!r}")
         self._state_needed = any(isinstance(need, StateNeed) for need in needs)

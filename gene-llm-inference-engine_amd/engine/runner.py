@@ -68,7 +68,7 @@ class Runner:
     """
 
     def __init__(self, model: DecoderModel, *, page_size: int = 16, max_tokens: int = 4096, max_requests: int = 8,
-                 max_rows: int = 4096, max_positions: Optional[int] = None, use_graphs: bool = True, max_graphs: int = 16):
+                 max_rows: int = 4096, max_positions: Optional[int] = None, use_graphs: bool = True, max_graphs: int = 48):
         self.model = model
         self.page_size = int(page_size)
         self.max_rows = int(max_rows)
@@ -239,10 +239,14 @@ class Runner:
         cache.reserve_one_each(requests, slots, lengths)                        # OutOfPages: nothing changed
         self._uploads.begin_step()
         cache.sync(self._uploads.put)
-        meta = self._uploads.stage(np.array([tokens, lengths, slots], dtype=np.int32)).view(3, n)
-        logits = self._decode_step(meta, slots, lengths, tokens_on_device)
+        # Captured steps exist for some batch sizes only: rows of the spare slot, at position 0, fill the step up to the next of them.
+        fill = captured_batch_size(n, self.max_rows) - n
+        if fill:
+            tokens, lengths, slots = tokens + [0] * fill, lengths + [0] * fill, slots + [cache.spare_slot] * fill
+        meta = self._uploads.stage(np.array([tokens, lengths, slots], dtype=np.int32)).view(3, n + fill)
+        logits = self._decode_step(meta, slots, lengths, tokens_on_device)[:n]
         self._uploads.end_step()
-        cache.advance_one_each(requests, slots, lengths)
+        cache.advance_one_each(requests, slots[:n], lengths[:n])
         self.steps_run += 1
         self.rows_run += n
         return logits
@@ -268,6 +272,16 @@ class Runner:
             g = self._graphs[(batch, bracket)] = _DecodeGraph(self.model, self._view, bracket, batch, self._graph_pool)
         g.last_used = self.steps_run
         return g.run(meta, seg_slot, seg_pos0, tokens_on_device)
+
+
+def captured_batch_size(n: int, most: int) -> int:
+    """The batch size of the captured decode step that serves n rows: every size up to 8, then multiples of 2 up to 16, of 4
+    up to 64, of 8 up to 128 and of 16 beyond, so that a batch that shrinks request by request as they finish, or grows as they are
+    admitted, meets a few dozen graphs instead of one per size (capturing one costs several steps' time); the added rows
+    are at most a fifth of the step and cost next to nothing (one key each).  Never more than `most` rows."""
+    step = 1 if n <= 8 else 2 if n <= 16 else 4 if n <= 64 else 8 if n <= 128 else 16
+    size = -(-n // step) * step
+    return size if size <= most else n
 
 
 class _StepUploads:
@@ -356,8 +370,8 @@ class _DecodeGraph:
         """meta: this step's tokens, positions and slots, int32 [3, batch], in pinned memory that stays as it is
         until the copy made here has run.  tokens_on_device: the tokens, if the host does not know them yet."""
         self.meta.copy_(meta, non_blocking=True)
-        if tokens_on_device is not None:
-            self.meta[0].copy_(tokens_on_device, non_blocking=True)
+        if tokens_on_device is not None:                 # (of the requests' rows; rows that fill the step up come behind them)
+            self.meta[0, :tokens_on_device.shape[0]].copy_(tokens_on_device, non_blocking=True)
         self.calls += 1
         if self.graph is None:
             if self.calls < 2:          # the first step of a batch size runs as it is; a size that comes again is captured

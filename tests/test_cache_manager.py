@@ -134,13 +134,13 @@ def test_limits_and_misuse():
 
 def test_state_slots_are_zeroed_when_a_request_opens():
     m = CacheManager([StateNeed((2, 3)), FULL], [None, None], page_size=4, n_pages=4, max_requests=2, max_positions=16, device="cpu")
-    assert m.state(0).shape == (2, 2, 3)
+    assert m.state(0).shape == (3, 2, 3)                                       # two request slots and the spare one
     s = m.open("a")
     m.state(0)[s] += 5.0
     m.close("a")
     assert m.open("b") == s and float(m.state(0)[s].abs().sum()) == 0.0
     kv, table, window = m.kv(1)
-    assert kv.shape == (4, 2, 2, 4, 16) and table.shape == (2, 4) and window is None
+    assert kv.shape == (5, 2, 2, 4, 16) and table.shape == (3, 4) and window is None      # the pool's pages and request slots, and the spare ones
 
 
 @pytest.mark.parametrize("seed", range(6))
@@ -547,3 +547,37 @@ def test_the_device_copy_of_the_tables_follows_under_random_use_with_few_columns
     assert sent and max(sent) <= 5 and sent.count(1) >= len(sent) // 2, sent
     for g in m.groups:
         assert (g.table_dev.numpy() == g.table_host).all()
+
+
+def test_the_spare_slot_has_a_page_of_its_own_outside_the_pool():
+    """Behind the request slots: one more row of every table and state tensor, whose first entry names a page behind the pool's
+    pages; no request gets that slot or that page, whatever is opened, grown and closed."""
+    m = CacheManager([FULL, WINDOW, StateNeed((3,), torch.float32)], [None, None, None], page_size=4, n_pages=6, max_requests=2, max_positions=24,
+                     dtype=torch.float32, device="cpu")
+    assert m.spare_slot == 2
+    for g in m.groups:
+        assert g.table_host.shape[0] == 3 and g.table_host[2].tolist() == [6] + [-1] * 5 and g.table_dev[2].tolist() == [6] + [-1] * 5
+        assert g.storage.shape[1] == 7 and g.pool.n_pages == 6
+    assert m.states[2].shape == (3, 3)
+    for turn in range(3):
+        for r in ("a", "b"):
+            assert m.open(r) in (0, 1)
+        with pytest.raises(CacheError):
+            m.open("c")
+        m.reserve([("a", 12), ("b", 12)]); m.advance("a", 12); m.advance("b", 12)
+        m.sync()
+        for g in m.groups:
+            assert 6 not in g.table_host[:2] and g.table_host[2].tolist() == [6] + [-1] * 5 and (g.table_dev.numpy() == g.table_host).all()
+        m.check_consistency()
+        m.close("a"); m.close("b")
+    assert m.free_pages() == [6, 6]
+
+
+def test_batch_sizes_of_captured_decode_steps():
+    from geneinfer_amd.engine.runner import captured_batch_size
+    sizes = [captured_batch_size(n, 4096) for n in range(1, 400)]
+    assert sizes[:8] == list(range(1, 9)) and sizes == sorted(sizes)
+    assert all(n <= s <= max(n + 15, n) and s - n < max(1, n // 4) + 1 for n, s in zip(range(1, 400), sizes))
+    assert all(captured_batch_size(s, 4096) == s for s in sizes)                       # a size of the list serves itself
+    assert len(set(sizes[:64])) == 24 and len(set(sizes)) < 60
+    assert captured_batch_size(9, 9) == 9 and captured_batch_size(9, 10) == 10         # never beyond the rows a step may hold

@@ -86,19 +86,42 @@ def test_gi_serve_bench_levels_generate_what_each_request_generates_alone(tmp_pa
     assert r.returncode == 0, r.stdout + r.stderr
     rows = [line.split() for line in r.stdout.splitlines() if line[:1].isdigit()]
     assert [int(row[0]) for row in rows] == [1, 4] and all("identical" in " ".join(row) for row in rows)
-    assert int(rows[0][6]) == 0 and int(rows[1][6]) == 0                        # cached positions of the measured run
+    assert int(rows[0][7]) == 0 and int(rows[1][7]) == 0                        # cached positions of the measured run
     warm = subprocess.run(common + ["--warm-cache"], capture_output=True, text=True, timeout=170)
     assert warm.returncode == 0, warm.stdout + warm.stderr
     rows = [line.split() for line in warm.stdout.splitlines() if line[:1].isdigit()]
-    assert int(rows[0][6]) == 48 and int(rows[1][6]) == 4 * 48
+    assert int(rows[0][7]) == 48 and int(rows[1][7]) == 4 * 48
     off = subprocess.run(common + ["--no-prefix-cache", "--profile"], capture_output=True, text=True, timeout=170)
     assert "device profile: " in off.stdout and "gemm_exact" in off.stdout
-    assert off.returncode == 0 and all(int(line.split()[6]) == 0 for line in off.stdout.splitlines() if line[:1].isdigit())
+    assert off.returncode == 0 and all(int(line.split()[7]) == 0 for line in off.stdout.splitlines() if line[:1].isdigit())
+
+
+@pytest.mark.gpu
+def test_benches_take_a_configuration_alone_and_requests_of_their_own_lengths(tmp_path):
+    """--config FILE: random weights drawn on the device, no folder.  gi_serve_bench with lengths LO:HI and a row budget: in
+    32-bit every request still generates what it generates alone, with steps of at most --step-rows rows."""
+    from model_folders import full_config
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(full_config(CONFIGS["B"])))
+    r = subprocess.run([str(ROOT / "bin" / "gi_serve_bench"), "--config", str(cfg), "--random-seed", "3", "--concurrency", "2,4", "--prompt-tokens", "5:60",
+                        "--decode-tokens", "3:14", "--runs", "1", "--weights", "f32", "--block-size", "8", "--step-rows", "24"],
+                       capture_output=True, text=True, timeout=170)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "prompt 5 to 60 + decode 3 to 14 tokens per request" in r.stdout and "max rows per pass 24" in r.stdout and "random weights (seed 3)" in r.stdout
+    rows = [line.split() for line in r.stdout.splitlines() if line[:1].isdigit()]
+    assert [int(row[0]) for row in rows] == [2, 4] and all("identical" in " ".join(row) for row in rows) and all(float(row[5]) <= 24 for row in rows)
+    quick = subprocess.run([str(ROOT / "bin" / "gi_serve_bench"), "--config", str(cfg), "--concurrency", "3", "--runs", "1", "--no-compare"],
+                           capture_output=True, text=True, timeout=170)
+    assert quick.returncode == 0 and "not compared" in quick.stdout, quick.stdout + quick.stderr
+    one = subprocess.run([str(ROOT / "bin" / "gi_bench"), "--config", str(cfg), "--prompt-tokens", "20", "--decode-tokens", "5", "--runs", "1"],
+                         capture_output=True, text=True, timeout=170)
+    assert one.returncode == 0 and "workload: 20 prompt + 5 decode positions" in one.stdout and "random weights (seed 0)" in one.stdout, one.stdout + one.stderr
 
 
 def test_gi_serve_bench_usage_errors():
     exe = str(ROOT / "bin" / "gi_serve_bench")
-    for args, msg in (([], "--model is required"), (["--model", "x", "--concurrency", "0"], "--concurrency needs positive integers"),
+    for args, msg in (([], "give --model DIR, or --config FILE"), (["--model", "x", "--prompt-tokens", "9:3"], "LO not above HI"),
+                      (["--model", "x", "--config", "y"], "give --model DIR, or --config FILE"), (["--model", "x", "--concurrency", "0"], "--concurrency needs positive integers"),
                       (["--model", "x", "--weights", "int8"], "--weights must be native or f32"), (["--model", "x", "--runs"], "missing value for --runs"),
                       (["--model", "x", "--max-seq-len", "8"], "--max-seq-len is shorter"), (["--model", "x", "--what"], "unknown option --what")):
         r = subprocess.run([exe, *args], capture_output=True, text=True, timeout=60)
@@ -127,7 +150,7 @@ def test_gi_bench_reports_one_request(tmp_path):
 
 def test_gi_bench_usage_errors():
     exe = str(ROOT / "bin" / "gi_bench")
-    for args, msg in (([], "--model is required"), (["--model", "x", "--runs", "0"], "must be positive"),
+    for args, msg in (([], "give --model DIR, or --config FILE"), (["--model", "x", "--runs", "0"], "must be positive"),
                       (["--model", "x", "--weights", "int8"], "--weights must be native or f32"), (["--model", "x", "--isa", "avx2"], "unknown option --isa")):
         r = subprocess.run([exe, *args], capture_output=True, text=True, timeout=60)
         assert r.returncode == 2 and msg in r.stderr and "usage: gi_bench" in r.stderr

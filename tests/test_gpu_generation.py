@@ -329,6 +329,52 @@ def test_decode_graphs_across_a_context_bracket_and_between_batch_sizes(folders,
             assert_within_bfloat16_noise(got, lambda k: want[k[0]][k[1]], lambda k: near[k[0]][k[1]], f"graphs across brackets, {max_graphs} kept")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_filled_up_to_a_captured_batch_size(folders, dtype):
+    """Above 8 requests a decode step runs at the next batch size of a short list, filled up with rows of the spare slot.  Eleven
+    requests decode, finish one after the other down to nine, and go on: the steps of 11 and 12 requests share one graph,
+    those of 9 and 10 another; every logit row is the plain model's (in 32-bit also bit for bit what a runner without graphs
+    gives), and the rows that filled the steps up have touched no request's page: the pool is whole at the end."""
+    from geneinfer_amd.engine import Runner, StepEntry, load_model
+    n_requests, new = 11, 14
+    seqs = {f"r{i}": t for i, t in enumerate(prompts_for("B", [20 + 3 * i for i in range(n_requests)], seed=23))}
+    model = load_model(folders["B"], dtype, "cuda:0")
+    exact, rounded = PlainLlama(folders["B"]), PlainLlama(folders["B"], storage=torch.bfloat16)
+    want = {r: exact.logits(t) for r, t in seqs.items()}
+    near = {r: rounded.logits(t) for r, t in seqs.items()} if dtype == "bfloat16" else None
+    runs = {}
+    for use_graphs in (True, False):
+        runner = Runner(model, page_size=8, max_tokens=n_requests * 64, max_requests=n_requests, use_graphs=use_graphs)
+        start = {r: len(t) - new for r, t in seqs.items()}
+        for r, t in seqs.items():
+            runner.open(r)
+            runner.step([StepEntry(r, t[:start[r]], ())])
+        got, at, live = {}, dict(start), list(seqs)
+        for k in range(new):
+            if k in (5, 9):                            # 11 -> 10 -> 9 requests
+                runner.close(live.pop(3))
+            logits = runner.step([StepEntry(r, [seqs[r][at[r]]], (0,)) for r in live]).cpu()
+            assert logits.shape[0] == len(live)
+            for r, row in zip(live, logits):
+                got[(r, at[r])] = row
+                at[r] += 1
+        if use_graphs:
+            assert set(runner._graphs) == {(12, 1024), (10, 1024)}, set(runner._graphs)
+            assert all(g.graph is not None for g in runner._graphs.values())
+        for r in live:
+            runner.close(r)
+        runner.cache.check_consistency()
+        assert runner.cache.free_pages() == [g.pool.n_pages for g in runner.cache.groups]
+        runs[use_graphs] = got
+    got = runs[True]
+    if dtype == "float32":
+        worst = max(relative_error(row, want[r][p]) for (r, p), row in got.items())
+        assert worst < 2e-5, worst
+        assert all(torch.equal(row, runs[False][key]) for key, row in got.items())
+    else:
+        assert_within_bfloat16_noise(got, lambda k: want[k[0]][k[1]], lambda k: near[k[0]][k[1]], "filled-up decode steps")
+
+
 @pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 1.5e-2)])
 def test_first_tokens_of_a_sequence(folders, dtype, tol):
     """Positions 0, 1, 2: one key, two keys; a prompt of one token; a page edge at position 4."""

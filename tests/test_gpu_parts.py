@@ -176,7 +176,7 @@ def test_toy_architecture_under_every_cut(toy_model, dtype, mode):
     runner = Runner(model, page_size=16 if dtype == "bfloat16" else 4, max_tokens=traces.peak_tokens(steps, 16), max_requests=4)
     groups = runner.cache.groups
     assert [(g.need.window, g.entries) for g in groups] == [(None, [1, 4]), (cfg.window, [2])]      # entry 5 reads entry 2's pages
-    assert list(runner.cache.states) == [0, 3] and runner.cache.state(3).shape == (4, cfg.hidden_size)      # both decay mixers
+    assert list(runner.cache.states) == [0, 3] and runner.cache.state(3).shape == (4 + 1, cfg.hidden_size)      # both decay mixers; four request slots and the spare one
     # what a step reads of the weights is asked of the parts, whatever a block calls them: every tensor of the file but the
     # token table, the two attention layers that run twice counted twice
     by_layer = lambda l: sum(4 * t.numel() for n, t in weights.items() if n.startswith(f"layers.{l}."))
