@@ -601,14 +601,50 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __r
     }
 }
 
-// Adds the k-split partial sums [splits][M][N] in ascending split order and writes the result.
-template <int EPI>
+// Adds the k-split partial sums [splits][M][N] in ascending split order and writes the result.  A thread takes VEC neighbouring
+// columns and asks for its values of up to eight splits at once: the kernel is one round trip to memory, not one per split.
+template <int EPI, int VEC>
 __global__ void skinny_reduce_kernel(const float* __restrict__ P, void* __restrict__ C, int M, int N, int splits, long ldc) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= (size_t)M * N) return;
-    float s = 0.f;
-    for (int sp = 0; sp < splits; ++sp) s += P[(size_t)sp * M * N + i];
-    write_out<EPI>(C, (i / N) * ldc + (i % N), s);
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC, slab = (size_t)M * N;
+    if (i >= slab) return;
+    float s[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) s[v] = 0.f;
+    for (int sp0 = 0; sp0 < splits; sp0 += 8) {
+        float part[8][VEC];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float* src = P + (size_t)min(sp0 + u, splits - 1) * slab + i;
+            if constexpr (VEC == 4) {
+                const float4 x = *reinterpret_cast<const float4*>(src);
+                part[u][0] = x.x; part[u][1] = x.y; part[u][2] = x.z; part[u][3] = x.w;
+            } else {
+                part[u][0] = *src;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (sp0 + u < splits) {
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) s[v] += part[u][v];
+            }
+    }
+    const size_t row = i / N, col = i % N, o = row * ldc + col;      // (VEC divides N: the VEC columns lie in one row)
+    if constexpr (VEC == 4) {                                        // (the host has checked that rows of C start at multiples of 16 bytes)
+        if constexpr (EPI == EPI_STORE_BF16) {
+            uint2 packed;
+            packed.x = (unsigned)f32_to_bf16(s[0]) | ((unsigned)f32_to_bf16(s[1]) << 16);
+            packed.y = (unsigned)f32_to_bf16(s[2]) | ((unsigned)f32_to_bf16(s[3]) << 16);
+            *reinterpret_cast<uint2*>((bf16_t*)C + o) = packed;
+        } else {
+            float4* dst = reinterpret_cast<float4*>((float*)C + o);
+            float4 x = EPI == EPI_ADD_F32 ? *dst : float4{0.f, 0.f, 0.f, 0.f};
+            x.x += s[0]; x.y += s[1]; x.z += s[2]; x.w += s[3];
+            *dst = x;
+        }
+    } else {
+        write_out<EPI>(C, o, s[0]);
+    }
 }
 
 // The same for the gated product: columns 32b .. 32b+15 of the partial sums are gates, 32b+16 .. 32b+31 the ups of
@@ -772,12 +808,14 @@ int epilogue_of(int c_dtype, int accumulate) {
 
 // Number of k-splits of the skinny kernel for a product with 17..64 rows, so that the caller can size
 // the scratch (splits * M * N floats); 0: the output is wide enough to fill the chip without a split,
-// no scratch is needed.  Enough workgroups to cover the chip, each with at least one block of k.
+// no scratch is needed.  Workgroups for three quarters of the chip or more, each with at least one block of k (measured at 33 to
+// 64 rows, product and reduce kernel together: 192 to 384 workgroups with two blocks of k each take 11 us for N = 3072, K = 2048 and
+// 16 us for N = 2048, K = 8192; twice the workgroups with one block each 12.5 and 17.5 us, half of them 13 and 22 us).
 GI_API int gi_gemm_bf16_skinny_splits(int N, int K) {
     const int strips = (N + 63) / 64;
     if (strips >= 192) return 0;
     int splits = 1;
-    while (strips * splits < 384 && K / (splits * 2) >= KB) splits *= 2;
+    while (strips * splits < 192 && K / (splits * 2) >= KB) splits *= 2;
     return splits;
 }
 
@@ -799,11 +837,19 @@ GI_API long gi_gemm_bf16_scratch_floats(int M, int N, int K) {
 }
 
 static int reduce_partials(const float* scratch, void* C, int epi, int M, int N, int splits, long ldc, hipStream_t stream) {
-    const unsigned blocks = (unsigned)(((size_t)M * N + 255) / 256);
-    if (epi == EPI_GATED_BF16) skinny_reduce_gated_kernel<<<(unsigned)(((size_t)M * (N / 2) + 255) / 256), 256, 0, stream>>>(scratch, (bf16_t*)C, M, N, splits, ldc);
-    else if (epi == EPI_STORE_F32) skinny_reduce_kernel<EPI_STORE_F32><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
-    else if (epi == EPI_ADD_F32) skinny_reduce_kernel<EPI_ADD_F32><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
-    else skinny_reduce_kernel<EPI_STORE_BF16><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);
+    if (epi == EPI_GATED_BF16) {
+        skinny_reduce_gated_kernel<<<(unsigned)(((size_t)M * (N / 2) + 255) / 256), 256, 0, stream>>>(scratch, (bf16_t*)C, M, N, splits, ldc);
+    } else {
+#define REDUCE(VEC_)                                                                                                                    \
+    do {                                                                                                                                \
+        const unsigned blocks = (unsigned)(((size_t)M * N / VEC_ + 255) / 256);                                                         \
+        if (epi == EPI_STORE_F32) skinny_reduce_kernel<EPI_STORE_F32, VEC_><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);  \
+        else if (epi == EPI_ADD_F32) skinny_reduce_kernel<EPI_ADD_F32, VEC_><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc); \
+        else skinny_reduce_kernel<EPI_STORE_BF16, VEC_><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);                      \
+    } while (0)
+        if (N % 4 == 0 && ldc % 4 == 0 && ((uintptr_t)scratch & 15) == 0 && ((uintptr_t)C & 15) == 0) REDUCE(4); else REDUCE(1);
+#undef REDUCE
+    }
     GI_CHECK_LAUNCH("gemm_bf16 (reduce)");
     return 0;
 }
