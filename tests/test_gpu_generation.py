@@ -375,6 +375,50 @@ def test_decode_steps_filled_up_to_a_captured_batch_size(folders, dtype):
         assert_within_bfloat16_noise(got, lambda k: want[k[0]][k[1]], lambda k: near[k[0]][k[1]], "filled-up decode steps")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_far_into_a_large_cache(folders, dtype):
+    """A cache of more than 2^31 elements a layer: with the low pages taken, two requests live in pages whose offsets need
+    more than 32 bits (in elements and in bytes), a prompt in portions and single tokens beside it.  Every kernel that
+    touches the cache (rotation and page write, prompt and decode attention, the fused decode step) meets them."""
+    from geneinfer_amd.engine import Runner, StepEntry, load_model
+    model = load_model(folders["D"], dtype, "cuda:0")
+    per_page = 2 * CONFIGS["D"]["num_key_value_heads"] * 16 * 64                    # elements of a page in one layer
+    n_pages = (1 << 31) // per_page + 200
+    runner = Runner(model, page_size=16, max_tokens=16 * n_pages, max_requests=2)
+    pool = runner.cache.groups[0].pool
+    held = [pool.allocate() for _ in range(n_pages - 150)]                          # what is left lies beyond 2^31 elements
+    assert min(pool._free) * per_page > (1 << 31)
+    seqs = dict(zip("ab", prompts_for("D", [700, 330], seed=29)))
+    exact, rounded = PlainLlama(folders["D"]), PlainLlama(folders["D"], storage=torch.bfloat16)
+    want = {r: exact.logits(t) for r, t in seqs.items()}
+    near = {r: rounded.logits(t) for r, t in seqs.items()} if dtype == "bfloat16" else None
+    got = {}
+    def run(entries):
+        logits = runner.step([StepEntry(r, seqs[r][a:b], tuple(range(b - a))) for r, a, b in entries]).cpu()
+        rows = iter(logits)
+        for r, a, b in entries:
+            for p in range(a, b):
+                got[(r, p)] = next(rows)
+    runner.open("a"); runner.open("b")
+    run([("a", 0, 300)])
+    run([("a", 300, 640), ("b", 0, 290)])
+    for k in range(40):                                                             # a: 640..679 singly, b: 290..329 singly, captured from the second step on
+        run([("a", 640 + k, 641 + k), ("b", 290 + k, 291 + k)])
+    run([("a", 680, 700)])
+    assert int(min(runner.cache.page_row("a"))) * per_page > (1 << 31)
+    if dtype == "float32":
+        worst = max(relative_error(row, want[r][p]) for (r, p), row in got.items())
+        assert worst < 2e-5, worst
+    else:
+        assert_within_bfloat16_noise(got, lambda k: want[k[0]][k[1]], lambda k: near[k[0]][k[1]], "pages far into a large cache")
+    runner.close("a"); runner.close("b")
+    for page in held:
+        pool.release(page)
+    runner.cache.check_consistency()
+    del runner
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("dtype,tol", [("float32", 2e-5), ("bfloat16", 1.5e-2)])
 def test_first_tokens_of_a_sequence(folders, dtype, tol):
     """Positions 0, 1, 2: one key, two keys; a prompt of one token; a page edge at position 4."""
