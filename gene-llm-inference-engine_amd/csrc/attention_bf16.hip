@@ -325,6 +325,241 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
         }
 }
 
+// ------------------------------------------------------------------------------------- prompt, wide
+// The same attention for head size 128 with another division of the work: a wave owns 32 rows and takes whole tiles of
+// 64 keys, a workgroup of NW waves owns one row tile, and a compute unit holds two workgroups that do not wait for each
+// other: where the kernel above ties all waves of a compute unit to one barrier per tile, so that they load together and
+// then multiply together, here a wave multiplies while its neighbour on the SIMD, of the other workgroup, loads or
+// exponentiates.  Nothing is merged at the end, a row's statistics stay in its two lanes.  (At head size 64 the exponentials
+// bound either kernel, and the first one's pairs of tiles balance the work better: measured, and left with the first.)
+//
+// Key and value tiles go from the cache straight into LDS (global_load_lds_dwordx4: lane l of a load lands at the load's
+// LDS address + 16 l, whatever it read), two stages: the loads of tile t + 1 are issued at the start of the step that
+// multiplies tile t and waited for at its end, before the barrier.  LDS rows are not padded (a load cannot pad); instead
+// the 16-byte chunk c of a row lies at chunk position c ^ f(row), so that the 16 lanes a clock serves, which read one
+// chunk column of 16 consecutive rows, hit 16 different bank groups: for the keys (rows of 128 channels, 256 bytes)
+// f(r) = r % 16.  The values (transposed in the cache: per channel, a page's positions) lie in LDS as
+// [group of 16 positions][channel][2 chunks of 8 positions], with the two chunks swapped for channels with (d / 8) % 2 = 1.
+// A wave-wide load so covers 4 or 8 key rows or 32 channels of one group of 16 positions, which lie in one page (pages hold
+// multiples of 16): the page's address and the place in it are worked out by the scalar unit, and a lane adds an offset
+// that never changes.
+//
+// The rows of a key tile are taken in another order by the score product: row i of the matrix instruction reads key
+// pi(i) = 16 (i / 16) + 8 ((i / 4) % 2) + 4 ((i / 8) % 2) + i % 4 of its 32, so that the 8 scores a lane holds for the
+// next product's k index are 8 consecutive keys, and the value operand is one 16-byte read (8 positions of a channel).
+template <int HD, int NW>
+__global__ __launch_bounds__(64 * NW, 2) void attention_prompt_wide_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
+                                                                       bf16_t* __restrict__ out, const int4* __restrict__ tiles,
+                                                                       const int* __restrict__ table, int table_stride, long page_stride,
+                                                                       int page_size, int n_heads, int n_kv, int window, float scale,
+                                                                       int n_splits, const int* __restrict__ tile_first, float* __restrict__ part,
+                                                                       int list_order) {
+    static_assert(HD == 128, "the chunk swizzle is made for key rows of 256 bytes");
+    constexpr int QSTEPS = HD / 16, DT = HD / 32;
+    constexpr int K_BYTES = KV_TILE * HD * 2, V_BYTES = HD * KV_TILE * 2, STAGE = K_BYTES + V_BYTES;
+    constexpr int CK = HD / 8;                               // 16-byte chunks of a key row
+    constexpr int K_LOADS = K_BYTES / 1024, V_LOADS = V_BYTES / 1024, LOADS = (K_LOADS + V_LOADS) / NW;      // wave-wide loads of 1 KB: per tile, per wave
+    static_assert((K_LOADS + V_LOADS) % NW == 0 && K_LOADS % LOADS == 0, "a wave's loads are all keys or all values");
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * STAGE];
+
+    // Workgroups start in the order of their numbers, heads fastest: the long walks (late tiles) of all heads first, so that the
+    // short ones fill the end.  A plain list runs from early tiles to late ones and is taken backwards; a list of pairs names a
+    // late tile, an early one, the next later one, the next earlier one, ...: first its late tiles in their order, then its early
+    // ones backwards.
+    const int n_groups = gridDim.y / n_splits, turn = blockIdx.y / n_splits, split = blockIdx.y % n_splits;
+    const int group = !list_order ? n_groups - 1 - turn : turn < n_groups / 2 ? 2 * turn : 2 * (n_groups - 1 - turn) + 1;
+    const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int4 tile = tiles[group];
+    const int row0 = tile.x, n_rows = tile.y, pos0 = tile.z, slot = tile.w;
+    if (n_rows == 0) return;                                  // (a tile that only fills a pair)
+    const int head = blockIdx.x, g = head / (n_heads / n_kv);
+    const int col = lane & 31, hf = lane >> 5;
+    const int* tab = table + (size_t)slot * table_stride;
+
+    const int my_row = wv * 32 + col;
+    const bool row_ok = my_row < n_rows;
+    const int my_pos = row_ok ? pos0 + my_row : -1;
+    const int my_lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
+    const int wave_last = pos0 + min(n_rows, wv * 32 + 32) - 1;
+    const bool wave_ok = wv * 32 < n_rows;
+    const bool wave_full = wv * 32 + 32 <= n_rows;
+    const int wave_first = wave_full ? pos0 + wv * 32 : -1;
+    const int wave_lo_max = window > 0 ? max(0, wave_last - window + 1) : 0;
+    const int wave_lo_min = window > 0 ? max(0, pos0 + wv * 32 - window + 1) : 0;
+    const float scale2 = scale * LOG2E;
+
+    bf16x8 qreg[QSTEPS];
+#pragma unroll
+    for (int s = 0; s < QSTEPS; ++s) {
+        uint4 v = {0, 0, 0, 0};
+        if (row_ok) v = load16(q + ((size_t)(row0 + my_row) * n_heads + head) * HD + 16 * s + 8 * hf);
+        qreg[s] = as_bf16x8(v);
+    }
+    floatx16 o[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i) o[i] = floatx16{};
+    float m = -INFINITY, l = 0.f;
+
+    const int last_pos = pos0 + n_rows - 1;
+    const int first_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+    const int range_first = first_lo & ~(KV_TILE - 1);
+    const int per_split = ((last_pos - range_first) / KV_TILE + n_splits) / n_splits * KV_TILE;
+    const int kv_first = range_first + split * per_split, my_last = min(last_pos, kv_first + per_split - 1);
+    const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+    auto page_index = [&](int kv) { return page_shift >= 0 ? kv >> page_shift : kv / page_size; };
+    auto place_of = [&](int kv) { return page_shift >= 0 ? kv & (page_size - 1) : kv % page_size; };
+    const int held_page = tab[page_index(max(my_last, 0))];   // stands in where a position has no page (beyond the end, before a window): finite, and masked
+    const long v_plane = (long)n_kv * page_size * HD;
+
+    // What this wave loads of every tile: LOADS loads of 1 KB, all of the keys' part or all of the values' part.
+    // Keys: load n covers rows n * 64 / CK ..; lane l brings chunk (l % CK) ^ f(row) of row first + l / CK.
+    // Values: load n covers group n / (HD / 32) of 16 positions and 32 channels; lane l brings chunk (l % 2) ^ ((d / 8) % 2) of channel d = first + l / 2.
+    const bool loads_keys = wv * LOADS < K_LOADS;
+    unsigned lane_off[LOADS];                                 // bytes from the group's place 0 in the page's keys (or values) to what this lane brings
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int n = wv * LOADS + i;                         // number of the load within the tile: keys first
+        if (loads_keys) {
+            const int r = n * (64 / CK) + lane / CK, c = (lane % CK) ^ (r & 15);
+            lane_off[i] = 2u * (unsigned)((g * page_size + (r & 15)) * HD + 8 * c);
+        } else {
+            const int d = ((n - K_LOADS) % (HD / 32)) * 32 + lane / 2, h = (lane & 1) ^ ((d >> 3) & 1);
+            lane_off[i] = 2u * (unsigned)((g * HD + d) * page_size + 8 * h);
+        }
+    }
+    typedef __attribute__((address_space(3))) unsigned char* lds_ptr_t;
+    const unsigned lds_base = (unsigned)(size_t)(lds_ptr_t)lds;      // the tiles' offset in LDS
+    // The pages of a tile's four groups of 16 positions: lanes 0 .. 3 look one up each.
+    auto look_up = [&](int kv0) {
+        const int kv = kv0 + 16 * (lane & 3);
+        return kv <= my_last ? tab[page_index(kv)] : -1;
+    };
+    auto send_for = [&](int kv0, int pages_v, int stage) {    // the loads of the tile at kv0 into `stage`, with what look_up(kv0) gave
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            const int n = wv * LOADS + i;
+            const int grp = loads_keys ? (n * (64 / CK)) >> 4 : (n - K_LOADS) / (HD / 32);      // which 16 positions of the tile (the same for the wave)
+            int pg = __builtin_amdgcn_readlane(pages_v, grp);
+            pg = pg >= 0 ? pg : held_page;
+            const int place = place_of(kv0 + 16 * grp);
+            const bf16_t* base = cache + (long)pg * page_stride + (loads_keys ? (long)place * HD : v_plane + place);
+            const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + stage * STAGE + n * 1024);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off[i]), "s"(base) : "memory", "m0");
+        }
+    };
+    auto landed_barrier = [&]() {                             // this wave's loads have landed; then everybody's, and everybody has read the other stage
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+
+    int pages_v = look_up(kv_first);
+    send_for(kv_first, pages_v, 0);
+    pages_v = look_up(kv_first + KV_TILE);
+    landed_barrier();
+    int stage = 0;
+    for (int kv0 = kv_first; kv0 <= my_last; kv0 += KV_TILE, stage ^= 1) {
+        // The loads of the next tile first (also behind the last one: they bring a held page's keys into the stage nobody reads any
+        // more).  A wave that issues such a load is held while the memory pipeline takes it, some 200 clocks each here; issuing
+        // them behind the matrix instructions of the scores, or half of them there and half behind those of the values, or all
+        // at the end of the step, was 2 to 8 % slower than here, where they have the whole step to land.
+        const bool active = wave_ok && kv0 <= wave_last && kv0 + KV_TILE > wave_lo_min;      // else: no row of this wave sees a key of the tile
+        const unsigned char* Ks = lds + stage * STAGE;
+        const unsigned char* Vs = Ks + K_BYTES;
+        floatx16 s[2] = {floatx16{}, floatx16{}};
+        send_for(kv0 + KV_TILE, pages_v, stage ^ 1);
+        pages_v = look_up(kv0 + 2 * KV_TILE);
+        if (active) {
+            // scores of the tile's two halves of 32 keys: two chains of matrix instructions that do not wait for each other
+            const int pi = (col & 16) | ((col & 4) << 1) | ((col & 8) >> 1) | (col & 3);       // the key this lane's row of the product reads
+#pragma unroll
+            for (int k = 0; k < QSTEPS; ++k) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int r = 32 * h + pi, c = (2 * k + hf) ^ (r & 15);
+                    const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(Ks + r * (HD * 2) + 16 * c));
+                    s[h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[k], s[h], 0, 0, 0);
+                }
+            }
+            // element v of s[h]: key kv0 + 32 h + 16 (v / 8) + 8 hf + v % 8, query row `col`; in units of log2 e after scale2
+            float mx = -INFINITY;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int kv_base = kv0 + 32 * h;
+                const bool inside = kv_base + 31 <= wave_first && kv_base >= wave_lo_max;
+                if (inside) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[h][v]);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int kv = kv_base + 16 * (v / 8) + 8 * hf + (v & 7);
+                        s[h][v] = (kv <= my_pos && kv >= my_lo) ? s[h][v] : -INFINITY;
+                        mx = fmaxf(mx, s[h][v]);
+                    }
+                }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale2;
+            const float m_new = fmaxf(m, mx);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            float sum = 0.f;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    s[h][v] = exp2_fast(fmaf(s[h][v], scale2, -m_use));
+                    sum += s[h][v];
+                }
+            if (__any(m_new != m)) {
+                const float corr = exp2_fast(m - m_use);
+                l *= corr;
+#pragma unroll
+                for (int i = 0; i < DT; ++i)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) o[i][v] *= corr;
+                m = m_new;
+            }
+            l += sum;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {                     // four groups of 16 keys: slot e of this lane is key 16 t + 8 hf + e
+                const floatx16& sh = s[t >> 1];
+                const int e0 = 8 * (t & 1);
+                const uint4 pb = {pack2(sh[e0], sh[e0 + 1]), pack2(sh[e0 + 2], sh[e0 + 3]), pack2(sh[e0 + 4], sh[e0 + 5]), pack2(sh[e0 + 6], sh[e0 + 7])};
+#pragma unroll
+                for (int i = 0; i < DT; ++i) {
+                    const int d = 32 * i + col;
+                    const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(Vs + (t * HD + d) * 32 + 16 * (hf ^ ((d >> 3) & 1))));
+                    o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, as_bf16x8(pb), o[i], 0, 0, 0);
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave's reads of the stage are done before anybody overwrites it
+        landed_barrier();
+    }
+    l += __shfl_xor(l, 32, 64);
+    if (!row_ok) return;
+    if (n_splits > 1) {                                       // part[row of the split tiles][head][split] = {m, l, O[HD]}
+        float* dst = part + (((size_t)(tile_first[group] + my_row) * n_heads + head) * n_splits + split) * (HD + 2);
+        if (hf == 0) {
+            dst[0] = m;
+            dst[1] = l;
+        }
+#pragma unroll
+        for (int i = 0; i < DT; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) dst[2 + 32 * i + 8 * (v / 4) + 4 * hf + (v & 3)] = o[i][v];
+        return;
+    }
+    const float inv = 1.0f / l;
+    bf16_t* orow = out + ((size_t)(row0 + my_row) * n_heads + head) * HD;
+#pragma unroll
+    for (int i = 0; i < DT; ++i)
+#pragma unroll
+        for (int v4 = 0; v4 < 4; ++v4) {                      // element v: channel 32*i + 8*(v/4) + 4*hf + v%4
+            const int d = 32 * i + 8 * v4 + 4 * hf;
+            *reinterpret_cast<uint2*>(orow + d) = uint2{pack2(o[i][4 * v4] * inv, o[i][4 * v4 + 1] * inv),
+                                                        pack2(o[i][4 * v4 + 2] * inv, o[i][4 * v4 + 3] * inv)};
+        }
+}
+
 // =========================================================================================== decode
 // One workgroup per (row, key/value head, query-head group of up to 16, split of the context); its
 // waves cut the split's range further, one piece each.  Keys and values stream from global memory
@@ -678,6 +913,25 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
     GI_REQUIRE(!paired || n_tiles % 2 == 0, "attention_prompt: %d tiles cannot go in pairs", n_tiles);
     // Two tiles share a workgroup of 1024 threads up to head size 64; larger heads need more registers than such a
     // workgroup leaves a thread, and take the same list tile by tile (a filling tile of 0 rows then does nothing).
+    // Head size 128 takes the wide kernel (measured at 8,192 rows: 762 against 1,577 us a layer of 32 heads); head size 64, where the
+    // exponentials bound the kernel and pairs of tiles balance the work, stays with the first one (51 against 70 us at 2,048 rows).
+    if (hd == 128) {
+        GI_REQUIRE((long)n_tiles * n_splits <= 65535, "attention_prompt: %d tiles in %d splits are too many for one launch", n_tiles, n_splits);
+        dim3 wgrid(n_heads, n_tiles * n_splits);
+#define WIDE(HD, NW)                                                                                                                    \
+    attention_prompt_wide_kernel<HD, NW><<<wgrid, 64 * NW, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
+                                                                       table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits, \
+                                                                       tile_first, part, paired ? 1 : 0)
+        if (rows_per_tile == 64) WIDE(128, 2); else WIDE(128, 4);
+#undef WIDE
+        GI_CHECK_LAUNCH("attention_prompt (wide)");
+        if (n_splits > 1) {
+            dim3 cgrid(n_rows, n_heads);
+            attention_decode_combine_kernel<<<cgrid, 64, 0, stream>>>(part, (bf16_t*)out, rows, n_heads, hd, n_splits);
+            GI_CHECK_LAUNCH("attention_prompt (combine)");
+        }
+        return 0;
+    }
     const bool pairs = paired && hd <= 64;
     dim3 grid((pairs ? n_tiles / 2 : n_tiles) * n_splits, n_heads);
 #define GO_(HD, NW, PAIR)                                                                                                               \
@@ -700,6 +954,7 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
     }
     return 0;
 }
+
 
 // Waves a workgroup of the decode kernel may have for this head size.
 GI_API int gi_attention_decode_max_waves(int hd) { return hd <= 128 ? 8 : 4; }

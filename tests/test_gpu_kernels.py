@@ -247,7 +247,7 @@ def plain_attention_rows(q, dense, rows, n_heads, n_kv, hd, window):
 
 ATT_CASES = [  # n_heads, n_kv, hd, page_size, window
     (4, 2, 64, 16, None), (3, 1, 32, 16, None), (8, 8, 128, 32, None), (6, 2, 96, 16, None), (4, 4, 64, 16, 40), (32, 8, 64, 16, None),
-    (5, 5, 48, 16, None), (2, 1, 16, 4, 9), (4, 2, 256, 16, None),
+    (5, 5, 48, 16, None), (2, 1, 16, 4, 9), (4, 2, 256, 16, None), (8, 2, 128, 16, 50), (6, 3, 128, 48, None),
 ]
 
 
@@ -298,7 +298,8 @@ def test_attention_over_pages(n_heads, n_kv, hd, ps, window, dtype, portions, ti
     assert torch.equal(torch.nan_to_num(cache, nan=-1.0), torch.nan_to_num(before, nan=-1.0)), "attention wrote into the cache"
 
 
-@pytest.mark.parametrize("n_heads,n_kv,hd,ps,window", [(4, 2, 64, 16, None), (3, 1, 32, 16, None), (8, 8, 128, 32, None), (6, 2, 96, 16, 700), (4, 4, 64, 16, 450)])
+@pytest.mark.parametrize("n_heads,n_kv,hd,ps,window", [(4, 2, 64, 16, None), (3, 1, 32, 16, None), (8, 8, 128, 32, None), (6, 2, 96, 16, 700), (4, 4, 64, 16, 450),
+                                                       (4, 1, 128, 16, 600)])
 def test_few_prompt_tiles_over_a_long_context_share_their_keys_out(n_heads, n_kv, hd, ps, window):
     """Two portions on top of long cached contexts: few tiles, so each tile's keys go to several workgroups and a combine
     kernel; among the keys one far one is scaled so that a lost share would show."""
