@@ -326,19 +326,18 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
 }
 
 // ------------------------------------------------------------------------------------- prompt, wide
-// The same attention for head size 128 with another division of the work: a wave owns 32 rows and takes whole tiles of
-// 64 keys, a workgroup of NW waves owns one row tile, and a compute unit holds two workgroups that do not wait for each
-// other: where the kernel above ties all waves of a compute unit to one barrier per tile, so that they load together and
-// then multiply together, here a wave multiplies while its neighbour on the SIMD, of the other workgroup, loads or
-// exponentiates.  Nothing is merged at the end, a row's statistics stay in its two lanes.  (At head size 64 the exponentials
-// bound either kernel, and the first one's pairs of tiles balance the work better: measured, and left with the first.)
+// The same attention for head sizes 64 and 128 with another division of the work: a wave owns 32 rows and takes whole
+// tiles of 64 keys, a workgroup of NW waves owns one row tile, and a compute unit holds several workgroups that do not wait
+// for each other (two at head size 128, three at 64): where the kernel above ties all waves of a compute unit to one barrier
+// per tile, so that they load together and then multiply together, here a wave multiplies while its neighbours on the SIMD,
+// of other workgroups, load or exponentiate.  Nothing is merged at the end, a row's statistics stay in its two lanes.
 //
 // Key and value tiles go from the cache straight into LDS (global_load_lds_dwordx4: lane l of a load lands at the load's
 // LDS address + 16 l, whatever it read), two stages: the loads of tile t + 1 are issued at the start of the step that
 // multiplies tile t and waited for at its end, before the barrier.  LDS rows are not padded (a load cannot pad); instead
 // the 16-byte chunk c of a row lies at chunk position c ^ f(row), so that the 16 lanes a clock serves, which read one
-// chunk column of 16 consecutive rows, hit 16 different bank groups: for the keys (rows of 128 channels, 256 bytes)
-// f(r) = r % 16.  The values (transposed in the cache: per channel, a page's positions) lie in LDS as
+// chunk column of 16 consecutive rows, hit 16 different bank groups: for the keys f(r) = r % 16 at 256 bytes a row
+// (128 channels), (r / 2) % 8 at 128 bytes.  The values (transposed in the cache: per channel, a page's positions) lie in LDS as
 // [group of 16 positions][channel][2 chunks of 8 positions], with the two chunks swapped for channels with (d / 8) % 2 = 1.
 // A wave-wide load so covers 4 or 8 key rows or 32 channels of one group of 16 positions, which lie in one page (pages hold
 // multiples of 16): the page's address and the place in it are worked out by the scalar unit, and a lane adds an offset
@@ -348,13 +347,13 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
 // pi(i) = 16 (i / 16) + 8 ((i / 4) % 2) + 4 ((i / 8) % 2) + i % 4 of its 32, so that the 8 scores a lane holds for the
 // next product's k index are 8 consecutive keys, and the value operand is one 16-byte read (8 positions of a channel).
 template <int HD, int NW>
-__global__ __launch_bounds__(64 * NW, 2) void attention_prompt_wide_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
+__global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_wide_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
                                                                        bf16_t* __restrict__ out, const int4* __restrict__ tiles,
                                                                        const int* __restrict__ table, int table_stride, long page_stride,
                                                                        int page_size, int n_heads, int n_kv, int window, float scale,
                                                                        int n_splits, const int* __restrict__ tile_first, float* __restrict__ part,
                                                                        int list_order) {
-    static_assert(HD == 128, "the chunk swizzle is made for key rows of 256 bytes");
+    static_assert(HD == 128 || HD == 64, "the chunk swizzle is made for key rows of 256 or 128 bytes");
     constexpr int QSTEPS = HD / 16, DT = HD / 32;
     constexpr int K_BYTES = KV_TILE * HD * 2, V_BYTES = HD * KV_TILE * 2, STAGE = K_BYTES + V_BYTES;
     constexpr int CK = HD / 8;                               // 16-byte chunks of a key row
@@ -420,7 +419,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attention_prompt_wide_kernel(const
     for (int i = 0; i < LOADS; ++i) {
         const int n = wv * LOADS + i;                         // number of the load within the tile: keys first
         if (loads_keys) {
-            const int r = n * (64 / CK) + lane / CK, c = (lane % CK) ^ (r & 15);
+            const int r = n * (64 / CK) + lane / CK, c = (lane % CK) ^ (HD == 128 ? (r & 15) : ((r >> 1) & 7));
             lane_off[i] = 2u * (unsigned)((g * page_size + (r & 15)) * HD + 8 * c);
         } else {
             const int d = ((n - K_LOADS) % (HD / 32)) * 32 + lane / 2, h = (lane & 1) ^ ((d >> 3) & 1);
@@ -474,7 +473,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attention_prompt_wide_kernel(const
             for (int k = 0; k < QSTEPS; ++k) {
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
-                    const int r = 32 * h + pi, c = (2 * k + hf) ^ (r & 15);
+                    const int r = 32 * h + pi, c = (2 * k + hf) ^ (HD == 128 ? (r & 15) : ((r >> 1) & 7));
                     const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(Ks + r * (HD * 2) + 16 * c));
                     s[h] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[k], s[h], 0, 0, 0);
                 }
@@ -913,16 +912,20 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
     GI_REQUIRE(!paired || n_tiles % 2 == 0, "attention_prompt: %d tiles cannot go in pairs", n_tiles);
     // Two tiles share a workgroup of 1024 threads up to head size 64; larger heads need more registers than such a
     // workgroup leaves a thread, and take the same list tile by tile (a filling tile of 0 rows then does nothing).
-    // Head size 128 takes the wide kernel (measured at 8,192 rows: 762 against 1,577 us a layer of 32 heads); head size 64, where the
-    // exponentials bound the kernel and pairs of tiles balance the work, stays with the first one (51 against 70 us at 2,048 rows).
-    if (hd == 128) {
+    // Head size 128 takes the wide kernel (measured at 8,192 rows: 762 against 1,577 us a layer of 32 heads).  At head size 64 the
+    // first kernel's pairs of tiles are the better balance while they fit the chip in one round (a workgroup of 16 waves a compute
+    // unit: 2,048 rows of 32 heads take 56 against 61 us) and where few tiles share their keys out; beyond one round its time
+    // doubles at once and the wide kernel's many small workgroups win (2,560 rows: 73 against 100 us; 8,192: 423 against 572).
+    const bool one_round = (long)(paired ? n_tiles / 2 : n_tiles) * n_heads <= 256;
+    if (hd == 128 || (hd == 64 && n_splits == 1 && !one_round)) {
         GI_REQUIRE((long)n_tiles * n_splits <= 65535, "attention_prompt: %d tiles in %d splits are too many for one launch", n_tiles, n_splits);
         dim3 wgrid(n_heads, n_tiles * n_splits);
 #define WIDE(HD, NW)                                                                                                                    \
     attention_prompt_wide_kernel<HD, NW><<<wgrid, 64 * NW, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
                                                                        table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits, \
                                                                        tile_first, part, paired ? 1 : 0)
-        if (rows_per_tile == 64) WIDE(128, 2); else WIDE(128, 4);
+        if (hd == 64) { if (rows_per_tile == 64) WIDE(64, 2); else WIDE(64, 4); }
+        else if (rows_per_tile == 64) WIDE(128, 2); else WIDE(128, 4);
 #undef WIDE
         GI_CHECK_LAUNCH("attention_prompt (wide)");
         if (n_splits > 1) {

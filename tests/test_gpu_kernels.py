@@ -326,6 +326,35 @@ def test_few_prompt_tiles_over_a_long_context_share_their_keys_out(n_heads, n_kv
     assert rel(out, want) < 8e-3, rel(out, want)
 
 
+@pytest.mark.parametrize("window", [None, 200])
+def test_many_prompt_tiles_of_many_heads(window):
+    """More workgroups than compute units at head size 64 (5 pairs of tiles x 64 heads): the step takes the kernel with a
+    workgroup per tile, several to a compute unit, which head size 128 always takes.  A whole prompt of 900 rows, a portion of
+    130 rows on 300 cached positions and a single row; with a window the pages behind it are gone."""
+    from geneinfer_amd.parts import StepContext
+    n_heads, n_kv, hd, ps = 64, 16, 64, 16
+    contexts = [900, 430, 50]
+    segs = [(0, 0, 900), (1, 300, 130), (2, 49, 1)]
+    gone = {slot: max(0, pos0 - window + 1) for slot, pos0, _ in segs} if window else None
+    cache, table, dense = build_paged(contexts, n_kv, hd, ps, torch.bfloat16, seed=5, scale_one=(77, 3.0), gone_before=gone)
+    rows, seg_start, seg_len, seg_pos0, seg_slot = [], [], [], [], []
+    for slot, pos0, n in segs:
+        seg_start.append(len(rows)); seg_len.append(n); seg_pos0.append(pos0); seg_slot.append(slot + 1)
+        rows += [(slot, pos0 + i) for i in range(n)]
+    T = len(rows)
+    q = randn(T, n_heads * hd, dtype=torch.bfloat16, seed=3)
+    pos = torch.tensor([p for _, p in rows], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([s_ + 1 for s_, _ in rows], dtype=torch.int32, device=DEV)
+    ctx = StepContext(n_rows=T, dtype=torch.bfloat16, device=torch.device(DEV), tokens=pos, row_pos=pos, row_slot=slots, seg_slot=seg_slot,
+                      seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0)
+    plan = ops().AttentionPlan(seg_start, seg_len, seg_pos0, seg_slot, DEV)
+    assert plan.paired and plan.tile == 128 and plan.n_tiles // 2 * n_heads > 256
+    out = torch.full((T, n_heads * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window)
+    want = plain_attention_rows(q, dense, rows, n_heads, n_kv, hd, window)
+    assert rel(out, want) < 8e-3, rel(out, want)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_attention_finds_one_far_key(dtype):
     """Among 700 keys one is scaled so that its score stands out: the output must be its value."""
