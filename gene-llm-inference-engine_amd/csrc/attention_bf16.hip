@@ -359,6 +359,7 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
     constexpr int CK = HD / 8;                               // 16-byte chunks of a key row
     constexpr int K_LOADS = K_BYTES / 1024, V_LOADS = V_BYTES / 1024, LOADS = (K_LOADS + V_LOADS) / NW;      // wave-wide loads of 1 KB: per tile, per wave
     static_assert((K_LOADS + V_LOADS) % NW == 0 && K_LOADS % LOADS == 0, "a wave's loads are all keys or all values");
+    static_assert(LOADS % (16 / (64 / CK)) == 0, "a wave's loads begin with a group's first rows");
     __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * STAGE];
 
     // Workgroups start in the order of their numbers, heads fastest: the long walks (late tiles) of all heads first, so that the
@@ -414,16 +415,19 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
     // Keys: load n covers rows n * 64 / CK ..; lane l brings chunk (l % CK) ^ f(row) of row first + l / CK.
     // Values: load n covers group n / (HD / 32) of 16 positions and 32 channels; lane l brings chunk (l % 2) ^ ((d / 8) % 2) of channel d = first + l / 2.
     const bool loads_keys = wv * LOADS < K_LOADS;
-    unsigned lane_off[LOADS];                                 // bytes from the group's place 0 in the page's keys (or values) to what this lane brings
+    // Bytes from the group's place 0 in the page's keys (or values) to what this lane brings.  The key loads of a group of 16
+    // positions differ in which of its rows they cover (KP loads a group, and the swizzle goes by the row): one offset each.
+    // The value loads of a group differ in their 32 channels only, which the scalar unit adds to the page's address.
+    constexpr int KP = 16 / (64 / CK);
+    unsigned lane_off[KP];
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-        const int n = wv * LOADS + i;                         // number of the load within the tile: keys first
+    for (int j = 0; j < KP; ++j) {
         if (loads_keys) {
-            const int r = n * (64 / CK) + lane / CK, c = (lane % CK) ^ (HD == 128 ? (r & 15) : ((r >> 1) & 7));
-            lane_off[i] = 2u * (unsigned)((g * page_size + (r & 15)) * HD + 8 * c);
-        } else {
-            const int d = ((n - K_LOADS) % (HD / 32)) * 32 + lane / 2, h = (lane & 1) ^ ((d >> 3) & 1);
-            lane_off[i] = 2u * (unsigned)((g * HD + d) * page_size + 8 * h);
+            const int r = j * (64 / CK) + lane / CK, c = (lane % CK) ^ (HD == 128 ? (r & 15) : ((r >> 1) & 7));      // (row within its group of 16)
+            lane_off[j] = 2u * (unsigned)((g * page_size + r) * HD + 8 * c);
+        } else {                                              // (the same for every j)
+            const int d = lane / 2, h = (lane & 1) ^ ((d >> 3) & 1);
+            lane_off[j] = 2u * (unsigned)((g * HD + d) * page_size + 8 * h);
         }
     }
     typedef __attribute__((address_space(3))) unsigned char* lds_ptr_t;
@@ -441,9 +445,10 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
             int pg = __builtin_amdgcn_readlane(pages_v, grp);
             pg = pg >= 0 ? pg : held_page;
             const int place = place_of(kv0 + 16 * grp);
-            const bf16_t* base = cache + (long)pg * page_stride + (loads_keys ? (long)place * HD : v_plane + place);
+            const bf16_t* base = cache + (long)pg * page_stride +
+                                 (loads_keys ? (long)place * HD : v_plane + place + (long)((n - K_LOADS) % (HD / 32)) * 32 * page_size);
             const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + stage * STAGE + n * 1024);
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off[i]), "s"(base) : "memory", "m0");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(lane_off[i % KP]), "s"(base) : "memory", "m0");
         }
     };
     auto landed_barrier = [&]() {                             // this wave's loads have landed; then everybody's, and everybody has read the other stage
@@ -925,7 +930,7 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
                                                                        table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits, \
                                                                        tile_first, part, paired ? 1 : 0)
         if (hd == 64) { if (rows_per_tile == 64) WIDE(64, 2); else WIDE(64, 4); }
-        else if (rows_per_tile == 64) WIDE(128, 2); else WIDE(128, 4);
+        else WIDE(128, 4);      // (tiles of 64 rows too: two of its waves then only load; a workgroup of two waves would need 16 loads a wave and more registers than two to a SIMD leave)
 #undef WIDE
         GI_CHECK_LAUNCH("attention_prompt (wide)");
         if (n_splits > 1) {
