@@ -432,19 +432,20 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
     }
     typedef __attribute__((address_space(3))) unsigned char* lds_ptr_t;
     const unsigned lds_base = (unsigned)(size_t)(lds_ptr_t)lds;      // the tiles' offset in LDS
-    // The pages of a tile's four groups of 16 positions: lanes 0 .. 3 look one up each.
-    auto look_up = [&](int kv0) {
-        const int kv = kv0 + 16 * (lane & 3);
-        return kv <= my_last ? tab[page_index(kv)] : -1;
+    // A tile's four groups of 16 positions: lanes 0 .. 3 work out one group's page and place in it each (a division, if the page
+    // size is no power of two, and a load: once a tile, by the vector unit), and the loads read them from those lanes.
+    auto look_up = [&](int kv0, int& pages_v, int& places_v) {
+        const int kv = kv0 + 16 * (lane & 3), index = page_index(kv);
+        const int pg = kv <= my_last ? tab[index] : -1;
+        pages_v = pg >= 0 ? pg : held_page;
+        places_v = kv - index * page_size;
     };
-    auto send_for = [&](int kv0, int pages_v, int stage) {    // the loads of the tile at kv0 into `stage`, with what look_up(kv0) gave
+    auto send_for = [&](int pages_v, int places_v, int stage) {      // the loads of a tile into `stage`, with what look_up gave for it
 #pragma unroll
         for (int i = 0; i < LOADS; ++i) {
             const int n = wv * LOADS + i;
             const int grp = loads_keys ? (n * (64 / CK)) >> 4 : (n - K_LOADS) / (HD / 32);      // which 16 positions of the tile (the same for the wave)
-            int pg = __builtin_amdgcn_readlane(pages_v, grp);
-            pg = pg >= 0 ? pg : held_page;
-            const int place = place_of(kv0 + 16 * grp);
+            const int pg = __builtin_amdgcn_readlane(pages_v, grp), place = __builtin_amdgcn_readlane(places_v, grp);
             const bf16_t* base = cache + (long)pg * page_stride +
                                  (loads_keys ? (long)place * HD : v_plane + place + (long)((n - K_LOADS) % (HD / 32)) * 32 * page_size);
             const unsigned dst = __builtin_amdgcn_readfirstlane(lds_base + stage * STAGE + n * 1024);
@@ -455,9 +456,10 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
         asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     };
 
-    int pages_v = look_up(kv_first);
-    send_for(kv_first, pages_v, 0);
-    pages_v = look_up(kv_first + KV_TILE);
+    int pages_v, places_v;
+    look_up(kv_first, pages_v, places_v);
+    send_for(pages_v, places_v, 0);
+    look_up(kv_first + KV_TILE, pages_v, places_v);
     landed_barrier();
     int stage = 0;
     for (int kv0 = kv_first; kv0 <= my_last; kv0 += KV_TILE, stage ^= 1) {
@@ -468,10 +470,10 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
         const bool active = wave_ok && kv0 <= wave_last && kv0 + KV_TILE > wave_lo_min;      // else: no row of this wave sees a key of the tile
         const unsigned char* Ks = lds + stage * STAGE;
         const unsigned char* Vs = Ks + K_BYTES;
-        floatx16 s[2] = {floatx16{}, floatx16{}};
-        send_for(kv0 + KV_TILE, pages_v, stage ^ 1);
-        pages_v = look_up(kv0 + 2 * KV_TILE);
+        send_for(pages_v, places_v, stage ^ 1);
+        look_up(kv0 + 2 * KV_TILE, pages_v, places_v);
         if (active) {
+            floatx16 s[2] = {floatx16{}, floatx16{}};
             // scores of the tile's two halves of 32 keys: two chains of matrix instructions that do not wait for each other
             const int pi = (col & 16) | ((col & 4) << 1) | ((col & 8) >> 1) | (col & 3);       // the key this lane's row of the product reads
 #pragma unroll
@@ -484,23 +486,23 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
                 }
             }
             // element v of s[h]: key kv0 + 32 h + 16 (v / 8) + 8 hf + v % 8, query row `col`; in units of log2 e after scale2
-            float mx = -INFINITY;
+            // (keys some row of the wave does not see are masked where they stand, before the part that every tile walks)
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int kv_base = kv0 + 32 * h;
-                const bool inside = kv_base + 31 <= wave_first && kv_base >= wave_lo_max;
-                if (inside) {
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[h][v]);
-                } else {
+                if (!(kv_base + 31 <= wave_first && kv_base >= wave_lo_max)) {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int kv = kv_base + 16 * (v / 8) + 8 * hf + (v & 7);
                         s[h][v] = (kv <= my_pos && kv >= my_lo) ? s[h][v] : -INFINITY;
-                        mx = fmaxf(mx, s[h][v]);
                     }
                 }
             }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[h][v]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale2;
             const float m_new = fmaxf(m, mx);
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -917,10 +919,10 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
     GI_REQUIRE(!paired || n_tiles % 2 == 0, "attention_prompt: %d tiles cannot go in pairs", n_tiles);
     // Two tiles share a workgroup of 1024 threads up to head size 64; larger heads need more registers than such a
     // workgroup leaves a thread, and take the same list tile by tile (a filling tile of 0 rows then does nothing).
-    // Head size 128 takes the wide kernel (measured at 8,192 rows: 762 against 1,577 us a layer of 32 heads).  At head size 64 the
+    // Head size 128 takes the wide kernel (measured at 8,192 rows: 726 against 1,577 us a layer of 32 heads).  At head size 64 the
     // first kernel's pairs of tiles are the better balance while they fit the chip in one round (a workgroup of 16 waves a compute
     // unit: 2,048 rows of 32 heads take 56 against 61 us) and where few tiles share their keys out; beyond one round its time
-    // doubles at once and the wide kernel's many small workgroups win (2,560 rows: 73 against 100 us; 8,192: 423 against 572).
+    // doubles at once and the wide kernel's many small workgroups win (2,560 rows: 68 against 100 us; 8,192: 360 against 572).
     const bool one_round = (long)(paired ? n_tiles / 2 : n_tiles) * n_heads <= 256;
     if (hd == 128 || (hd == 64 && n_splits == 1 && !one_round)) {
         GI_REQUIRE((long)n_tiles * n_splits <= 65535, "attention_prompt: %d tiles in %d splits are too many for one launch", n_tiles, n_splits);
