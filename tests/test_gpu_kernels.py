@@ -65,7 +65,9 @@ def test_gemm_exact_rows_alone_have_the_same_bits(w_dtype, k):
                                    # the ping-pong kernel (a 256 x 256 tile or more for every compute unit): one block of k, an odd number of them, edges
                                    (4100, 4104, 64), (4096, 4100, 320),
                                    # ... and with k shared out over workgroups because the tiles are few
-                                   (72, 256, 1024), (300, 2048, 2048), (65, 130, 512),
+                                   (200, 256, 1024), (300, 2048, 2048), (129, 130, 512),
+                                   # 65 to 128 rows: the skinny kernel with six or eight tiles of rows, narrow outputs (k shared out) and wide ones
+                                   (72, 256, 1024), (65, 130, 512), (72, 2048, 2048), (96, 3072, 2048), (128, 2048, 8192), (80, 12300, 264), (113, 12288, 520),
                                    # wide outputs finished by the skinny kernel itself, from 12 rows and from 5
                                    (12, 12300, 520), (40, 12300, 264), (5, 65600, 72), (16, 12288, 256),
                                    # 17 to 32 rows, narrow outputs, short k: the slim kernel with two tiles of rows
@@ -83,6 +85,7 @@ def test_gemm_bf16(m, n, k, out_dtype, accumulate):
 
 
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 8), (5, 48, 136), (16, 160, 96), (17, 176, 64), (64, 32, 264), (70, 192, 128), (300, 8192 // 16, 2048 // 8),
+                                       (72, 8192, 2048), (128, 6144, 264), (100, 288, 136),
                                        (40, 6144, 264), (13, 6160, 72), (64, 8192, 512), (2048, 1024, 192), (600, 288, 64), (200, 512, 1024),
                                        (4100, 2064, 128)])
 def test_gemm_bf16_gated(m, inter, k):
