@@ -53,8 +53,7 @@ def generate(runner: Runner, sampler: Sampler, prompt_tokens: Sequence[int], max
             runner.step([StepEntry(request, prompt[pos:pos + n], ())])
             pos += n
         token = prompt[pos] if pos < len(prompt) else None
-        ahead = (sample is None and pos < steps and getattr(runner, "can_step_from_device", False) and sampler.kind in ("greedy", "plain")
-                 and runner.model.device.type == "cuda")
+        ahead = sample is None and pos < steps and getattr(runner, "can_step_from_device", False) and runner.model.device.type == "cuda"
 
         def took(nxt) -> bool:
             """Books for one generated token; False when it ends the request."""

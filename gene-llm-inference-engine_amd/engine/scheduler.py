@@ -244,10 +244,8 @@ class Engine:
 
         if self._landing_strips is not None and len(wanting) == len(taken) == len(self.running) and self.runner.can_step_from_device:
             # every running request decodes: its token may stay on the device for the next step
-            tokens = sample_rows_on_device(logits, [j.sampler for j in wanting])
-            if tokens is not None:
-                self._flight = self._take_off(taken, tokens)
-                return True
+            self._flight = self._take_off(taken, sample_rows_on_device(logits, [j.sampler for j in wanting]))
+            return True
         sampled = self._sample(logits, [j.sampler for j in wanting]) if wanting else []
         next_token = {j.id: t for j, t in zip(wanting, sampled)}
         for job in [job for job, n in taken if self._after_rows(job, n, next_token.get(job.id), self.stats.passes)]:

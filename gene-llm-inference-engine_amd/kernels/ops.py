@@ -44,6 +44,7 @@ _SIGNATURES = {
     "gi_probe_mfma": [c_int, c_void_p, c_int, c_void_p],
     "gi_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
+    "gi_sample_filtered": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
 }
 
 _lib = None
@@ -59,6 +60,8 @@ def lib():
             fn.restype = c_int
         l.gi_argmax_chunks.argtypes = [c_int]
         l.gi_argmax_chunks.restype = c_int
+        l.gi_sample_filtered_histogram_bytes.argtypes = []
+        l.gi_sample_filtered_histogram_bytes.restype = c_int
         l.gi_attention_bf16_supports.argtypes = [c_int, c_int, c_int]
         l.gi_attention_bf16_supports.restype = c_int
         l.gi_gemm_bf16_scratch_floats.argtypes = [c_int, c_int, c_int]
@@ -607,6 +610,28 @@ def sample_temperature(logits, temperature, uniform, out):
     part_s = torch.empty(n * chunks, dtype=torch.float64, device=logits.device)
     _call("gi_sample_temperature", logits.data_ptr(), temperature.data_ptr(), uniform.data_ptr(), out.data_ptr(), part_m.data_ptr(),
           part_s.data_ptr(), n, vocab, logits.stride(0), _stream())
+    return out
+
+
+def sample_filtered(logits, temperature, top_k, top_p, uniform, out):
+    """Top-k, then top-p, then the draw, for rows that each have one of the two filters (top_k in 1..vocab-1, or
+    top_p < 1): a row without a filter is drawn in index order, which `sample_temperature` does."""
+    _dev(logits, temperature, top_k, top_p, uniform, out)
+    n, vocab = logits.shape
+    if not (logits.dtype == torch.float32 and logits.stride(1) == 1):
+        raise KernelError("sample: logits must be float32 with unit inner stride")
+    for t, name in ((temperature, "temperature"), (top_p, "top_p"), (uniform, "uniform")):
+        if not (t.dtype == torch.float32 and t.is_contiguous() and t.numel() >= n):
+            raise KernelError(f"sample: {name} must be float32 [n]")
+    _i32(top_k, "sample: top_k", n)
+    _i32(out, "sample: out", n)
+    chunks = lib().gi_argmax_chunks(vocab)
+    part_m = torch.empty(n * chunks, dtype=torch.float32, device=logits.device)
+    part_s = torch.empty(n * chunks, dtype=torch.float64, device=logits.device)
+    kept = torch.empty(n * vocab, dtype=torch.float32, device=logits.device)
+    tops = torch.empty(n * lib().gi_sample_filtered_histogram_bytes() // 8, dtype=torch.int64, device=logits.device)
+    _call("gi_sample_filtered", logits.data_ptr(), temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), uniform.data_ptr(),
+          out.data_ptr(), part_m.data_ptr(), part_s.data_ptr(), kept.data_ptr(), tops.data_ptr(), n, vocab, logits.stride(0), _stream())
     return out
 
 

@@ -8,9 +8,8 @@ Rules (src/sampler/sampler.h:1-14, src/sampler/sampler.cpp:25-129):
      descending, index ascending) whose mass reaches top_p times the kept mass.
   4. a token is drawn by walking the kept tokens until the cumulative probability exceeds
      u times the kept mass; without filtering the walk is in index order.
-Greedy and plain temperature sampling run on the device on the logits where the step left
-them; a request with top-k or top-p has its row brought to the host and filtered there, as the
-reference samples every row.
+All of it runs on the device, on the logits where the step left them; `filtered_draw` states
+steps 2-4 on the host as the reference has them, for one row.
 """
 from __future__ import annotations
 
@@ -104,7 +103,7 @@ class Sampler:
         config.validate(vocab_size)
         self.config, self.vocab_size = config, vocab_size
         self.stream = UniformStream(config.seed)
-        # where this sampler's rows go in `sample_rows`: arg max, plain temperature (both on the device), filtered (host)
+        # which kernels this sampler's rows go through in `sample_rows`: arg max, plain temperature, top-k / top-p
         self.kind = "greedy" if config.greedy else "filtered" if config.filters(vocab_size) else "plain"
         self.temperature = float(config.temperature)
 
@@ -116,58 +115,56 @@ class Sampler:
         return sample_rows(logits.reshape(1, -1), [self])[0]
 
 
-def sample_rows_on_device(logits: torch.Tensor, samplers: Sequence[Sampler]):
-    """The tokens of `sample_rows`, left on the device (int32 [n]) without waiting for them, when every
-    sampler is greedy or every one samples the plain softmax (each then draws its uniform number now);
-    None, with nothing drawn, when a row needs the host (top-k, top-p) or the kinds are mixed."""
-    n, vocab = logits.shape
-    if n != len(samplers):
-        raise ValueError(f"{n} rows of logits for {len(samplers)} samplers")
-    kinds = {s.kind for s in samplers}
-    out = torch.empty(n, dtype=torch.int32, device=logits.device)
-    if kinds == {"greedy"}:
-        return ops.argmax(logits, out)
-    if kinds == {"plain"}:
-        both = torch.tensor([[s.temperature for s in samplers], [s.stream.next_uniform() for s in samplers]], dtype=torch.float32).to(logits.device)
-        return ops.sample_temperature(logits, both[0], both[1], out)
-    return None
+_KIND_ORDER = {"greedy": 0, "plain": 1, "filtered": 2}
 
 
-def sample_rows(logits: torch.Tensor, samplers: Sequence[Sampler]) -> List[int]:
-    """Row i of `logits` (float32 [n, vocab], on the device) is sampled with samplers[i].
-    A sampler draws one uniform number per call unless it is greedy."""
+def sample_rows_on_device(logits: torch.Tensor, samplers: Sequence[Sampler]) -> torch.Tensor:
+    """Row i of `logits` (float32 [n, vocab], on the device) is sampled with samplers[i]; the tokens stay on the
+    device (int32 [n]) and nothing waits for them.  A sampler draws one uniform number per call unless it is greedy.
+    Rows of one kind (arg max; the plain softmax; top-k or top-p) go through that kind's kernels together; where
+    kinds are mixed, each kind's rows are gathered first."""
     n, vocab = logits.shape
     if n != len(samplers):
         raise ValueError(f"{n} rows of logits for {len(samplers)} samplers")
     dev = logits.device
-    kinds = {s.kind for s in samplers}
-    if kinds == {"greedy"}:                                      # the two common cases without a list per kind
-        return ops.argmax(logits, torch.empty(n, dtype=torch.int32, device=dev)).tolist()
-    if kinds == {"plain"}:
-        both = torch.tensor([[s.temperature for s in samplers], [s.stream.next_uniform() for s in samplers]], dtype=torch.float32).to(dev)
-        return ops.sample_temperature(logits, both[0], both[1], torch.empty(n, dtype=torch.int32, device=dev)).tolist()
-    out: List[int] = [0] * n
-    greedy = [i for i, s in enumerate(samplers) if s.kind == "greedy"]
-    host = [i for i, s in enumerate(samplers) if s.kind == "filtered"]
-    plain = [i for i, s in enumerate(samplers) if s.kind == "plain"]
-    pending = []
-    if greedy:
-        rows = logits if len(greedy) == n else logits[torch.tensor(greedy, device=dev)]
-        res = torch.empty(len(greedy), dtype=torch.int32, device=dev)
-        ops.argmax(rows, res)
-        pending.append((greedy, res))
-    if plain:
-        rows = logits if len(plain) == n else logits[torch.tensor(plain, device=dev)]
-        both = torch.tensor([[samplers[i].temperature for i in plain], [samplers[i].next_uniform() for i in plain]],
-                            dtype=torch.float32).to(dev)                       # one copy for temperatures and uniform numbers
-        res = torch.empty(len(plain), dtype=torch.int32, device=dev)
-        ops.sample_temperature(rows, both[0], both[1], res)
-        pending.append((plain, res))
-    if host:
-        rows = logits[torch.tensor(host, device=dev)].cpu().numpy()
-        for i, row in zip(host, rows):
-            out[i] = filtered_draw(row, samplers[i].config, samplers[i].next_uniform())
-    for idx, res in pending:
-        for i, t in zip(idx, res.tolist()):
-            out[i] = int(t)
+    out = torch.empty(n, dtype=torch.int32, device=dev)
+    kinds = [s.kind for s in samplers]
+    if all(k == "greedy" for k in kinds):
+        return ops.argmax(logits, out)
+    # One copy to the device for everything the rows' kernels need, rows grouped by kind: temperature, uniform number,
+    # top-p, top-k, and the row in `logits`.
+    order = sorted(range(n), key=lambda i: _KIND_ORDER[kinds[i]])
+    host = np.zeros((5, n), dtype=np.float32)
+    ints = host.view(np.int32)
+    for col, i in enumerate(order):
+        s = samplers[i]
+        if s.kind != "greedy":
+            host[0, col], host[1, col], host[2, col] = s.temperature, s.next_uniform(), s.config.top_p
+            ints[3, col] = s.config.top_k if 0 < s.config.top_k < vocab else 0
+        ints[4, col] = i
+    params = torch.from_numpy(host).to(dev)
+    sorted_kinds = [kinds[i] for i in order]
+    start = 0
+    while start < n:
+        kind = sorted_kinds[start]
+        stop = start + sorted_kinds.count(kind)
+        whole = stop - start == n                                 # then the rows are in their own order
+        where = None if whole else params[4, start:stop].view(torch.int32).long()
+        rows = logits if whole else logits.index_select(0, where)
+        res = out if whole else torch.empty(stop - start, dtype=torch.int32, device=dev)
+        if kind == "greedy":
+            ops.argmax(rows, res)
+        elif kind == "plain":
+            ops.sample_temperature(rows, params[0, start:stop], params[1, start:stop], res)
+        else:
+            ops.sample_filtered(rows, params[0, start:stop], params[3, start:stop].view(torch.int32), params[2, start:stop],
+                                params[1, start:stop], res)
+        if not whole:
+            out.index_copy_(0, where, res)
+        start = stop
     return out
+
+
+def sample_rows(logits: torch.Tensor, samplers: Sequence[Sampler]) -> List[int]:
+    """`sample_rows_on_device`, with the tokens brought to the host."""
+    return sample_rows_on_device(logits, samplers).tolist()

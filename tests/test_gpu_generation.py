@@ -97,8 +97,20 @@ def test_temperature_sampling_follows_the_seeded_stream(folders):
                 cum = torch.cumsum(p, 0)
                 assert abs(tok - want) == 1 and float((cum - float(us[step])).abs().min()) < 1e-5
             toks.append(tok)
-    top = llm.generate(prompts_for("B", [9])[0], steps=20, temperature=0.8, top_k=5, top_p=0.9, seed=3).generated_tokens
-    assert len(top) == 12 and all(0 <= t < CONFIGS["B"]["vocab_size"] for t in top)
+    for k, p, seed in ((5, 0.9, 3), (0, 0.7, 4), (3, 1.0, 5)):        # with filters: the same, the order of nearly equal tokens aside
+        prompt = prompts_for("B", [9])[0]
+        top = llm.generate(prompt, steps=20, temperature=0.8, top_k=k, top_p=p, seed=seed).generated_tokens
+        assert len(top) == 12
+        us = plain_sampler.uniforms(seed, 12)
+        toks = list(prompt)
+        for step, tok in enumerate(top):
+            row = plain.logits(toks)[-1].float().numpy()
+            want = plain_sampler.sample(row, 0.8, k, p, us[step])
+            if tok != want:
+                near = {plain_sampler.sample(row, 0.8, k, min(max(p + dp, 1e-6), 1.0 - 1e-7) if p < 1.0 else p, min(max(float(us[step]) + du, 0.0), 1.0 - 2.0 ** -24))
+                        for dp in (-1e-5, 0.0, 1e-5) for du in (-1e-5, 0.0, 1e-5)}
+                assert tok in near, (k, p, step, tok, want)
+            toks.append(tok)
 
 
 @pytest.mark.parametrize("name,temperature", [("A", 0.0), ("B", 0.8)])

@@ -2,6 +2,7 @@
 the engine's test models: primes, sizes that are no multiple of a tile, single rows."""
 import math
 
+import numpy as np
 import pytest
 import torch
 
@@ -200,6 +201,98 @@ def test_sample_temperature_matches_the_inverse_distribution():
                 p = torch.softmax(logits[i].double() / float(temps[i]), 0)
                 cum = torch.cumsum(p, 0)
                 assert abs(got - want) == 1 and float((cum - float(us[i])).abs().min()) < 1e-6, (vocab, i, got, want)
+
+
+def on_an_edge(logits, temperature, top_k, top_p, u, got, want):
+    """Whether the plain sampler could give `got` for `want` by rounding alone: two tokens whose probabilities differ in the
+    last bits change places in the order, or u, or top_p times the kept mass, falls within 2e-6 of a boundary."""
+    from plain_sampler import sample
+    p = torch.softmax(torch.from_numpy(logits).double() / temperature, 0)
+    if abs(float(p[got]) - float(p[want])) <= 1e-6 * float(p[want]):
+        return True
+    near = set()
+    for dp in (-2e-6, 0.0, 2e-6):
+        for du in (-2e-6, 0.0, 2e-6):
+            near.add(sample(logits, temperature, top_k, top_p if top_p >= 1.0 else min(max(top_p + dp, 1e-6), 1.0 - 1e-7),
+                            min(max(u + du, 0.0), 1.0 - 2.0 ** -24)))
+    return got in near
+
+
+def filtered_on_device(logits, temps, ks, ps, us):
+    n = logits.shape[0]
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    ops().sample_filtered(logits.to(DEV), torch.tensor(temps, dtype=torch.float32, device=DEV), torch.tensor(ks, dtype=torch.int32, device=DEV),
+                          torch.tensor(ps, dtype=torch.float32, device=DEV), torch.tensor(us, dtype=torch.float32, device=DEV), out)
+    return out.tolist()
+
+
+def test_filters_on_the_device_keep_what_they_should():
+    """The sets that the filters leave, as the reference's test states them (tests/verify_sampler.py:161-166): among equal
+    probabilities the lowest indices stay."""
+    g = torch.Generator().manual_seed(3)
+    us = torch.rand(300, generator=g).tolist()
+    flat = torch.zeros(300, 10)
+    assert set(filtered_on_device(flat, [1.0] * 300, [3] * 300, [1.0] * 300, us)) == {0, 1, 2}
+    assert set(filtered_on_device(flat, [1.0] * 300, [0] * 300, [0.35] * 300, us)) == {0, 1, 2, 3}
+    assert set(filtered_on_device(flat, [1.0] * 300, [7] * 300, [0.35] * 300, us)) == {0, 1, 2}          # 0.35 of the mass of seven
+    peaked = torch.zeros(300, 20)
+    peaked[:, 13] = 30.0
+    assert set(filtered_on_device(peaked, [1.0] * 300, [0] * 300, [0.9] * 300, us)) == {13}
+    assert set(filtered_on_device(peaked, [1.0] * 300, [1] * 300, [1.0] * 300, us)) == {13}
+    wide = torch.zeros(300, 5000)                                   # equal probabilities far beyond one wave's reach
+    wide[:, 4000:] = 1.0
+    got = filtered_on_device(wide, [1.0] * 300, [600] * 300, [1.0] * 300, us)
+    assert min(got) >= 4000 and max(got) < 4600 and len(set(got)) > 150
+    got = filtered_on_device(wide, [1.0] * 300, [1300] * 300, [1.0] * 300, us)                            # all of the likely ones and 300 of the rest
+    assert set(t for t in got if t < 4000) <= set(range(300)) and any(t < 4000 for t in got) and max(got) < 5000
+
+
+def test_sample_filtered_matches_the_plain_sampler():
+    """Top-k and top-p on the device against the plain sampler, row by row: random logits, logits on a coarse grid (many
+    tokens of exactly equal probability, so that the filters cut through groups of equals), and the real vocabulary."""
+    from plain_sampler import sample
+    g = torch.Generator().manual_seed(1)
+    settings = [(1.0, 0, 0.9), (0.8, 0, 0.5), (1.0, 0, 0.05), (1.0, 3, 1.0), (1.5, 50, 1.0), (1.0, 5, 0.9), (0.7, 1, 1.0), (1.0, 4, 0.3),
+                (0.3, 0, 0.999), (2.0, 40, 0.95), (1.0, 10 ** 6, 0.7), (1.0, 0, 2.0 ** -20)]
+    exact = total = 0
+    for vocab, coarse in ((2, False), (5, False), (100, False), (100, True), (3001, False), (3001, True), (128256, False), (128256, True)):
+        rows = []
+        for t, k, p in settings:
+            if not (0 < k < vocab or p < 1.0):
+                continue
+            for u in torch.rand(2 if vocab > 100000 else 6, generator=g).tolist() + [0.0, 1.0 - 2.0 ** -24]:
+                rows.append((t, k, p, u))
+        logits = 2 * torch.randn(len(rows), vocab, generator=g)
+        if coarse:
+            logits = torch.round(logits * 2) / 2
+        got = filtered_on_device(logits, *zip(*rows))
+        for i, (t, k, p, u) in enumerate(rows):
+            row = logits[i].numpy()
+            want = sample(row, t, k, p, np.float32(u))
+            total += 1
+            exact += got[i] == want
+            assert got[i] == want or on_an_edge(row, t, k, p, u, got[i], want), (vocab, coarse, i, (t, k, p, u), got[i], want)
+    assert exact >= 0.98 * total, (exact, total)
+
+
+def test_rows_of_every_kind_of_sampler_in_one_call():
+    """Greedy, plain and filtered samplers side by side get what each gets alone, and every one draws from its own stream."""
+    from geneinfer_amd.sampling import Sampler, SamplerConfig, sample_rows
+    g = torch.Generator().manual_seed(5)
+    vocab = 777
+    configs = [SamplerConfig(0.0), SamplerConfig(0.9, seed=4), SamplerConfig(1.0, top_k=7, seed=5), SamplerConfig(0.0), SamplerConfig(0.7, top_p=0.8, seed=6),
+               SamplerConfig(1.2, seed=7), SamplerConfig(1.0, top_k=20, top_p=0.5, seed=8)]
+    together = [Sampler(c, vocab) for c in configs]
+    alone = [Sampler(c, vocab) for c in configs]
+    for step in range(5):
+        logits = (2 * torch.randn(len(configs), vocab, generator=g)).to(DEV)
+        got = sample_rows(logits, together)
+        want = [sample_rows(logits[i:i + 1], [alone[i]])[0] for i in range(len(configs))]
+        assert got == want, (step, got, want)
+        assert [s.stream.state for s in together] == [s.stream.state for s in alone]
+    some = [together[i] for i in (2, 4, 6)]                           # only filtered ones: no gathering
+    logits = (2 * torch.randn(3, vocab, generator=g)).to(DEV)
+    assert sample_rows(logits, some) == [sample_rows(logits[i:i + 1], [alone[j]])[0] for i, j in enumerate((2, 4, 6))]
 
 
 # ------------------------------------------------------------------------------------- attention
