@@ -189,6 +189,39 @@ def test_decoding_ahead_changes_no_token(folders, temperature):
     assert 0 <= outcomes[(True, 1024, 6)].rows - outcomes[(False, 1024, 6)].rows <= sum(a.stopped_by_end_token for a in alone)
 
 
+def test_samplers_of_every_kind_side_by_side(folders):
+    """Greedy, plain and filtering (top-k, top-p, both) requests in one engine, their decode steps queued ahead: each ends
+    with the tokens it gets alone, and a filtering request alone decodes ahead as well."""
+    import geneinfer_amd as gi
+    from geneinfer_amd.engine import EngineConfig, EngineRequest
+    from geneinfer_amd.sampling import SamplerConfig
+    name, new, ps = "B", 24, PAGE_SIZE["B"]
+    prompts = prompts_for(name, [7, 19, 3, 30, 12, 5], seed=78)
+    samplers = [SamplerConfig(0.0), SamplerConfig(0.8, seed=11), SamplerConfig(0.9, top_k=6, seed=12), SamplerConfig(1.1, top_p=0.6, seed=13),
+                SamplerConfig(0.7, top_k=12, top_p=0.8, seed=14), SamplerConfig(0.0)]
+    roomy = gi.LLM(folders[name], dtype="float32", page_size=ps, max_tokens=512, max_running=1)
+    alone = [roomy.generate(p, steps=len(p) + new - 1, temperature=c.temperature, top_k=c.top_k, top_p=c.top_p, seed=c.seed).generated_tokens
+             for p, c in zip(prompts, samplers)]
+    assert all(len(a) == new for a in alone) and len({tuple(a) for a in alone}) == len(alone)
+    for max_running in (6, 3):
+        llm = gi.LLM(folders[name], dtype="float32", page_size=ps, max_tokens=1024, max_running=max_running, max_rows=64)
+        eng = llm.engine(EngineConfig(max_running=max_running))
+        ids = [eng.submit(EngineRequest(p, len(p) + new - 1, c)) for p, c in zip(prompts, samplers)]
+        flights = 0
+        while eng.step():
+            flights += eng._flight is not None
+        assert flights > 10
+        for j, want in zip(ids, alone):
+            assert eng.result(j).generated_tokens == want, (max_running, j)
+    llm = gi.LLM(folders[name], dtype="float32", page_size=ps, max_tokens=512, max_running=2, max_rows=64)
+    eng = llm.engine(EngineConfig(max_running=2))
+    ids = [eng.submit(EngineRequest(prompts[i], len(prompts[i]) + new - 1, samplers[i])) for i in (2, 4)]
+    flights = 0
+    while eng.step():
+        flights += eng._flight is not None
+    assert flights > 10 and [eng.result(j).generated_tokens for j in ids] == [alone[2], alone[4]]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_requests_with_an_equal_beginning_share_its_pages(folders, dtype):
     """Requests that begin alike take the pages an earlier one computed: fewer rows are fed, and every request still
