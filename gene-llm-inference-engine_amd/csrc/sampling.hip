@@ -243,17 +243,39 @@ __device__ __forceinline__ void add_tokens(Histogram& h, bool take, unsigned dig
 }
 
 // Every thread of the workgroup calls `f(i, pattern of p_i, i < vocab)` for its share of a row's tokens (and for a few places
-// beyond the row's end, so that whole waves call it), eight loads in flight at a time: a pass over a row is a chain of loads
-// from the second-level cache, and one load per turn would wait out each one's latency.
+// beyond the row's end, so that whole waves call it; there the pattern is that of a negative number, which no probability
+// has), in no particular order.  A pass over a row is a chain of loads from the second-level cache, each waited for: a thread
+// has eight loads in flight at a time, of four tokens each where the row allows.
 template <typename F>
 __device__ __forceinline__ void for_each_token(const float* __restrict__ e, float inv, int vocab, F f) {
     constexpr int AT_ONCE = 8;
+    if ((vocab & 3) == 0 && ((size_t)e & 15) == 0) {
+        const int fours = vocab >> 2;
+        for (int first = 0; first < fours; first += FT * AT_ONCE) {
+            float4 v[AT_ONCE];
+#pragma unroll
+            for (int u = 0; u < AT_ONCE; ++u) {
+                const int at = first + u * FT + (int)threadIdx.x;
+                v[u] = at < fours ? reinterpret_cast<const float4*>(e)[at] : float4{-1.0f, -1.0f, -1.0f, -1.0f};
+            }
+#pragma unroll
+            for (int u = 0; u < AT_ONCE; ++u) {
+                const int at = first + u * FT + (int)threadIdx.x;
+                if (first + u * FT >= fours) break;
+                f(4 * at, __float_as_uint(v[u].x * inv), at < fours);
+                f(4 * at + 1, __float_as_uint(v[u].y * inv), at < fours);
+                f(4 * at + 2, __float_as_uint(v[u].z * inv), at < fours);
+                f(4 * at + 3, __float_as_uint(v[u].w * inv), at < fours);
+            }
+        }
+        return;
+    }
     for (int first = 0; first < vocab; first += FT * AT_ONCE) {
         float v[AT_ONCE];
 #pragma unroll
         for (int u = 0; u < AT_ONCE; ++u) {
             const int i = first + u * FT + (int)threadIdx.x;
-            v[u] = i < vocab ? e[i] : -1.0f;                  // no probability is negative
+            v[u] = i < vocab ? e[i] : -1.0f;
         }
 #pragma unroll
         for (int u = 0; u < AT_ONCE; ++u) {

@@ -118,6 +118,45 @@ class Sampler:
 _KIND_ORDER = {"greedy": 0, "plain": 1, "filtered": 2}
 
 
+class _Staging:
+    """The rows' parameters go to the device through pinned memory with a copy that does not wait.  (A copy from ordinary
+    memory makes the host wait until the device has reached it, that is until the step before it has run: the host could then
+    queue nothing ahead.)  A ring of buffers; one is taken again only after its last copy has finished."""
+    DEPTH, FLOATS = 8, 5 * 1024
+
+    def __init__(self, device):
+        self.device = device
+        self.host = [torch.empty(self.FLOATS, dtype=torch.float32, pin_memory=True) for _ in range(self.DEPTH)]
+        self.done = [None] * self.DEPTH
+        self.turn = 0
+
+    def upload(self, values: np.ndarray) -> torch.Tensor:
+        if values.size > self.FLOATS:
+            return torch.from_numpy(values).to(self.device)
+        self.turn = (self.turn + 1) % self.DEPTH
+        if self.done[self.turn] is None:
+            self.done[self.turn] = torch.cuda.Event()
+        else:
+            self.done[self.turn].synchronize()
+        staged = self.host[self.turn][:values.size].view(values.shape)
+        staged.copy_(torch.from_numpy(values))
+        out = torch.empty(values.shape, dtype=torch.float32, device=self.device)
+        out.copy_(staged, non_blocking=True)
+        self.done[self.turn].record()
+        return out
+
+
+_staging = {}
+
+
+def _to_device(values: np.ndarray, device) -> torch.Tensor:
+    if device.type != "cuda":
+        return torch.from_numpy(values).to(device)
+    if device not in _staging:
+        _staging[device] = _Staging(device)
+    return _staging[device].upload(values)
+
+
 def sample_rows_on_device(logits: torch.Tensor, samplers: Sequence[Sampler]) -> torch.Tensor:
     """Row i of `logits` (float32 [n, vocab], on the device) is sampled with samplers[i]; the tokens stay on the
     device (int32 [n]) and nothing waits for them.  A sampler draws one uniform number per call unless it is greedy.
@@ -142,7 +181,7 @@ def sample_rows_on_device(logits: torch.Tensor, samplers: Sequence[Sampler]) -> 
             host[0, col], host[1, col], host[2, col] = s.temperature, s.next_uniform(), s.config.top_p
             ints[3, col] = s.config.top_k if 0 < s.config.top_k < vocab else 0
         ints[4, col] = i
-    params = torch.from_numpy(host).to(dev)
+    params = _to_device(host, dev)
     sorted_kinds = [kinds[i] for i in order]
     start = 0
     while start < n:

@@ -113,6 +113,9 @@ def test_benches_take_a_configuration_alone_and_requests_of_their_own_lengths(tm
     quick = subprocess.run([str(ROOT / "bin" / "gi_serve_bench"), "--config", str(cfg), "--concurrency", "3", "--runs", "1", "--no-compare"],
                            capture_output=True, text=True, timeout=170)
     assert quick.returncode == 0 and "not compared" in quick.stdout, quick.stdout + quick.stderr
+    drawn = subprocess.run([str(ROOT / "bin" / "gi_serve_bench"), "--config", str(cfg), "--concurrency", "3", "--runs", "1", "--weights", "f32",
+                            "--temperature", "0.8", "--top-k", "5", "--top-p", "0.9", "--seed", "4"], capture_output=True, text=True, timeout=170)
+    assert drawn.returncode == 0 and "temperature 0.8, top-k 5, top-p 0.9" in drawn.stdout and "identical to running alone" in drawn.stdout, drawn.stdout + drawn.stderr
     one = subprocess.run([str(ROOT / "bin" / "gi_bench"), "--config", str(cfg), "--prompt-tokens", "20", "--decode-tokens", "5", "--runs", "1"],
                          capture_output=True, text=True, timeout=170)
     assert one.returncode == 0 and "workload: 20 prompt + 5 decode positions" in one.stdout and "random weights (seed 0)" in one.stdout, one.stdout + one.stderr
@@ -122,7 +125,8 @@ def test_gi_serve_bench_usage_errors():
     exe = str(ROOT / "bin" / "gi_serve_bench")
     for args, msg in (([], "give --model DIR, or --config FILE"), (["--model", "x", "--prompt-tokens", "9:3"], "LO not above HI"),
                       (["--model", "x", "--config", "y"], "give --model DIR, or --config FILE"), (["--model", "x", "--concurrency", "0"], "--concurrency needs positive integers"),
-                      (["--model", "x", "--weights", "int8"], "--weights must be native or f32"), (["--model", "x", "--runs"], "missing value for --runs"),
+                      (["--model", "x", "--weights", "int8"], "--weights must be native or f32"), (["--model", "x", "--runs"], "missing value for --runs"), (["--model", "x", "--top-p", "2"], "--top-p must be in (0, 1]"),
+                      (["--model", "x", "--temperature", "hot"], "invalid number for --temperature"),
                       (["--model", "x", "--max-seq-len", "8"], "--max-seq-len is shorter"), (["--model", "x", "--what"], "unknown option --what")):
         r = subprocess.run([exe, *args], capture_output=True, text=True, timeout=60)
         assert r.returncode == 2 and msg in r.stderr and "usage: gi_serve_bench" in r.stderr
