@@ -672,11 +672,34 @@ __global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* 
 // and of activation row r, so the four lanes of a row read 64 contiguous bytes per load.  Loads run
 // two blocks ahead of the products.  The slices' sums meet in LDS and are added in slice order.
 // ROWS = 8 leaves half of each product idle and doubles the number of workgroups for narrow outputs.
-template <int STRIPS, int ROWS, int EPI>
+//
+// HAND: an RMS norm between two such products without a kernel of its own.  The norm of a row x is g * x * r with
+// r = rsqrt(mean(x^2) + eps), and r, one number a row, commutes with the product that reads the normed row.  A product that adds
+// onto the rows x (EPI_ADD_F32) also writes g * x of the sums it has just made, in bfloat16, and what its columns give to the
+// sum of squares of every row, one number per row and workgroup (`norm_out`); the product that reads those rows multiplies its
+// results by r, which it gets from those numbers, added in a fixed order (`norm_in`).
+struct NormOut {                 // for a product that adds onto x: all null if it does not hand the norm on
+    const float* g;              // the norm's weights [N]
+    bf16_t* scaled;              // out: g * x, [M, ld]
+    long ld;
+    float* squares;              // out: [M, parts], parts = the number of workgroups (times STRIPS)
+};
+struct NormIn {                  // for a product whose rows A are g * x without r: squares null if they are ready-made rows
+    const float* squares;        // [M, parts]
+    int parts;                   // at most slim_max_parts(M)
+    float eps;                   // r = rsqrt(sum / K + eps)
+};
+// A thread keeps 8 pieces while the products run (more would cost the kernel its second workgroup per compute unit); 64 threads
+// share a row where there are at most 8 rows, 32 otherwise.
+constexpr int SLIM_PIECES = 8;
+__host__ __device__ constexpr int slim_max_parts(int M) { return SLIM_PIECES * (M <= 8 ? 64 : 32); }
+
+template <int STRIPS, int ROWS, int EPI, bool HAND>
 __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
-                                                            int M, int N, int K, long lda, long ldw, long ldc) {
+                                                            int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in, NormOut norm_out) {
     constexpr int SLICES = 8 / STRIPS, STEP = SLICES * SK, DEPTH = 3;
     __shared__ float red[8][64][4];
+    __shared__ float row_scale[16];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int strip = wave % STRIPS, slice = wave / STRIPS;
     const int r = lane & 15, q = lane >> 4;
@@ -698,6 +721,19 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
     const int k_first = slice * SK;
 #pragma unroll
     for (int d = 0; d < DEPTH - 1; ++d) fetch(k_first + d * STEP, w_buf[d], x_buf[d]);      // beyond K: zeros, no loads
+    // The pieces of the rows' sums of squares, 32 or 64 threads a row: asked for behind the first weights, they have come when
+    // the products are done.
+    float piece[HAND ? SLIM_PIECES : 1];
+    const int sharing = M <= 8 ? 64 : 32, piece_row = M <= 8 ? tid >> 6 : tid >> 5;
+    if constexpr (HAND) {
+        if (norm_in.squares != nullptr) {
+#pragma unroll
+            for (int i = 0; i < SLIM_PIECES; ++i) {
+                const int p = (tid & (sharing - 1)) + sharing * i;
+                piece[i] = (piece_row < M && p < norm_in.parts) ? norm_in.squares[(size_t)piece_row * norm_in.parts + p] : 0.f;
+            }
+        }
+    }
     for (int k0 = k_first; k0 < K; k0 += DEPTH * STEP) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {                     // buffer d holds block k0 + d*STEP
@@ -709,11 +745,25 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
     }
 #pragma unroll
     for (int v = 0; v < 4; ++v) red[wave][lane][v] = acc[v];
+    if constexpr (HAND) {
+        if (norm_in.squares != nullptr) {
+            float sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < SLIM_PIECES; ++i) sum += piece[i];
+            if (sharing == 64) sum += __shfl_xor(sum, 32, 64);
+#pragma unroll
+            for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+            if ((tid & (sharing - 1)) == 0 && piece_row < 16) row_scale[piece_row] = 1.0f / sqrtf(sum / (float)K + norm_in.eps);
+        }
+    }
     __syncthreads();
     // Element v of a lane's result: activation row 4*q + v, weight row r of the strip.
     if (tid < 256 * (EPI == EPI_GATED_BF16 ? 1 : STRIPS)) {
         const int st = tid >> 8, e = tid & 255, m = e >> 4, c = e & 15;
         const int src_lane = c + 16 * (m >> 2), v = m & 3;
+        float r = 1.0f;
+        if constexpr (HAND) r = norm_in.squares != nullptr ? row_scale[m] : 1.0f;
+        float square = 0.f;
         if (m < M && c < ROWS) {
             if constexpr (EPI == EPI_GATED_BF16) {
                 float gate = 0.f, up = 0.f;
@@ -722,13 +772,36 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
                     gate += red[s * STRIPS + 0][src_lane][v];
                     up += red[s * STRIPS + 1][src_lane][v];
                 }
+                if constexpr (HAND) { gate *= r; up *= r; }
                 ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 16 + c] = f32_to_bf16(silu_gate(gate, up));
             } else {
                 float sum = 0.f;
 #pragma unroll
                 for (int s = 0; s < SLICES; ++s) sum += red[s * STRIPS + st][src_lane][v];
+                if constexpr (HAND) sum *= r;
                 const int col = (blockIdx.x * STRIPS + st) * ROWS + c;
-                if (col < N) write_out<EPI>(C, (size_t)m * ldc + col, sum);
+                if (col < N) {
+                    if constexpr (HAND && EPI == EPI_ADD_F32) {
+                        if (norm_out.scaled != nullptr) {
+                            float* at = (float*)C + (size_t)m * ldc + col;
+                            const float x = *at + sum;
+                            *at = x;
+                            norm_out.scaled[(size_t)m * norm_out.ld + col] = f32_to_bf16(norm_out.g[col] * x);
+                            square = x * x;
+                        } else {
+                            write_out<EPI>(C, (size_t)m * ldc + col, sum);
+                        }
+                    } else {
+                        write_out<EPI>(C, (size_t)m * ldc + col, sum);
+                    }
+                }
+            }
+        }
+        if constexpr (HAND && EPI == EPI_ADD_F32) {
+            if (norm_out.scaled != nullptr) {                   // the 16 threads of a row: its columns of this workgroup
+#pragma unroll
+                for (int off = 8; off > 0; off >>= 1) square += __shfl_xor(square, off, 64);
+                if (c == 0 && m < M) norm_out.squares[(size_t)m * (gridDim.x * STRIPS) + blockIdx.x * STRIPS + st] = square;
             }
         }
     }
@@ -855,6 +928,77 @@ static int reduce_partials(const float* scratch, void* C, int epi, int M, int N,
     return 0;
 }
 
+// Up to 16 rows the slim kernel (no LDS staging, one launch) is the faster one, except for wide outputs with more
+// than a few rows, where its per-workgroup reading of the activations costs more than the skinny kernel's staging
+// (measured crossovers at K = 2048: 12 rows for 256 strips of 64 columns, 5 rows for 2004 strips).
+static bool takes_slim(int M, int N, int K) {
+    const int strips64 = (N + 63) / 64;
+    const bool wide_skinny = gi_gemm_bf16_skinny_splits(N, K) == 0 && (M >= 12 || (M >= 5 && strips64 >= 1024));
+    return M <= 16 && !wide_skinny;
+}
+
+// Workgroups of the slim kernel for an output of N columns that is not gated: the pieces a row's sum of squares comes in.
+static int slim_parts(int N) { return (N + 15) / 16 >= 256 ? (N + 15) / 16 : (N + 7) / 8; }
+
+static int launch_slim(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in,
+                       NormOut norm_out, hipStream_t stream) {
+    const bool hand = norm_in.squares != nullptr || norm_out.scaled != nullptr;
+#define SLIM(STRIPS_, ROWS_, EPI_)                                                                                                                     \
+    do {                                                                                                                                               \
+        if (hand) gemm_bf16_slim_kernel<STRIPS_, ROWS_, EPI_, true><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out); \
+        else gemm_bf16_slim_kernel<STRIPS_, ROWS_, EPI_, false><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out);     \
+    } while (0)
+    if (epi == EPI_GATED_BF16) {
+        dim3 grid(N / 32);
+        SLIM(2, 16, EPI_GATED_BF16);
+    } else if ((N + 15) / 16 >= 256) {
+        dim3 grid((N + 15) / 16);
+        if (epi == EPI_STORE_F32) SLIM(1, 16, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 16, EPI_ADD_F32); else SLIM(1, 16, EPI_STORE_BF16);
+    } else {                                   // a narrow output: strips of 8 rows, twice the workgroups
+        dim3 grid((N + 7) / 8);
+        if (epi == EPI_STORE_F32) SLIM(1, 8, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 8, EPI_ADD_F32); else SLIM(1, 8, EPI_STORE_BF16);
+    }
+#undef SLIM
+    GI_CHECK_LAUNCH("gemm_bf16 (slim)");
+    return 0;
+}
+
+// The pieces per row that a product of these sizes writes when it hands a norm on (gi_gemm_bf16_handing with `scaled_out`);
+// 0 if it cannot: more than 16 rows, or a shape that the slim kernel does not take.
+GI_API int gi_gemm_bf16_norm_parts(int M, int N, int K) {
+    if (!takes_slim(M, N, K)) return 0;
+    const int parts = slim_parts(N);
+    return parts <= slim_max_parts(M) ? parts : 0;
+}
+
+// Whether a product of these sizes can read rows whose norm was handed on (gi_gemm_bf16_handing with `squares_in`).
+GI_API int gi_gemm_bf16_takes_norm(int M, int N, int K) { return takes_slim(M, N, K) ? 1 : 0; }
+
+// gi_gemm_bf16 for at most 16 rows, with an RMS norm handed from one product to the next instead of a kernel of its own.
+// squares_in != null: the rows A are g * x of some rows x, in bfloat16, and squares_in [M, parts_in] holds the pieces of every
+// row's sum of x^2; the results are multiplied by rsqrt(sum / K + eps).  scaled_out != null (needs accumulate onto 32-bit C):
+// beside C += A W^T, scaled_out [M, ld_scaled] = bfloat16(g * C) and squares_out [M, gi_gemm_bf16_norm_parts(M, N, K)] = the
+// pieces of the rows' sums of C^2, for the next product.
+GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dtype, int accumulate, int gated, int M, int N, int K, long lda,
+                                long ldw, long ldc, const float* squares_in, int parts_in, float eps, const float* g, void* scaled_out,
+                                long ld_scaled, float* squares_out, hipStream_t stream) {
+    GI_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: M %d, N %d, K %d must be positive", M, N, K);
+    GI_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_bf16: K %d and the row strides (%ld, %ld) must be multiples of 8", K, lda, ldw);
+    GI_REQUIRE(((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_bf16: operands must be 16-byte aligned");
+    GI_REQUIRE(lda >= K && ldw >= K && ldc >= (gated ? N / 2 : N), "gemm_bf16: leading dimensions too small");
+    int epi = epilogue_of(c_dtype, accumulate);
+    if (gated) {
+        GI_REQUIRE(N % 32 == 0 && c_dtype == GI_BF16 && !accumulate, "gemm_bf16: the gated product needs N %% 32 == 0 and a bfloat16 output");
+        epi = EPI_GATED_BF16;
+    }
+    GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
+    GI_REQUIRE(takes_slim(M, N, K), "gemm_bf16: a norm is handed on between products of at most 16 rows (M %d, N %d, K %d)", M, N, K);
+    GI_REQUIRE(squares_in == nullptr || (parts_in > 0 && parts_in <= slim_max_parts(M)), "gemm_bf16: %d pieces of a sum of squares, at most %d", parts_in, slim_max_parts(M));
+    GI_REQUIRE(scaled_out == nullptr || (epi == EPI_ADD_F32 && g != nullptr && squares_out != nullptr && ld_scaled >= N && slim_parts(N) <= slim_max_parts(M)),
+               "gemm_bf16: handing a norm on needs a product that adds onto 32-bit rows, the norm's weights and room for the sums of squares");
+    return launch_slim(A, W, C, epi, M, N, K, lda, ldw, ldc, NormIn{squares_in, parts_in, eps}, NormOut{g, (bf16_t*)scaled_out, ld_scaled, squares_out}, stream);
+}
+
 // `gated` != 0: W is [gate; up] interleaved in groups of 16 rows (N rows in all, a multiple of 32)
 // and C is bfloat16 [M, N/2] = silu(gate) * up.
 GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int accumulate, int gated, int M, int N, int K, long lda,
@@ -870,28 +1014,7 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     }
     GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
 
-    // Up to 16 rows the slim kernel (no LDS staging, one launch) is the faster one, except for wide outputs with more
-    // than a few rows, where its per-workgroup reading of the activations costs more than the skinny kernel's staging
-    // (measured crossovers at K = 2048: 12 rows for 256 strips of 64 columns, 5 rows for 2004 strips).
-    const int strips64 = (N + 63) / 64;
-    const bool wide_skinny = gi_gemm_bf16_skinny_splits(N, K) == 0 && (M >= 12 || (M >= 5 && strips64 >= 1024));
-    if (M <= 16 && !wide_skinny) {
-#define SLIM(STRIPS_, ROWS_, EPI_) \
-    gemm_bf16_slim_kernel<STRIPS_, ROWS_, EPI_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
-        if (epi == EPI_GATED_BF16) {
-            dim3 grid(N / 32);
-            SLIM(2, 16, EPI_GATED_BF16);
-        } else if ((N + 15) / 16 >= 256) {
-            dim3 grid((N + 15) / 16);
-            if (epi == EPI_STORE_F32) SLIM(1, 16, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 16, EPI_ADD_F32); else SLIM(1, 16, EPI_STORE_BF16);
-        } else {                                   // a narrow output: strips of 8 rows, twice the workgroups
-            dim3 grid((N + 7) / 8);
-            if (epi == EPI_STORE_F32) SLIM(1, 8, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 8, EPI_ADD_F32); else SLIM(1, 8, EPI_STORE_BF16);
-        }
-#undef SLIM
-        GI_CHECK_LAUNCH("gemm_bf16 (slim)");
-        return 0;
-    }
+    if (takes_slim(M, N, K)) return launch_slim(A, W, C, epi, M, N, K, lda, ldw, ldc, NormIn{nullptr, 0, 0.f}, NormOut{nullptr, nullptr, 0, nullptr}, stream);
 
     // 17 to 32 rows, a narrow output and a short k: one launch of the slim kernel with two tiles of activation rows.  Measured at
     // N = 3072 and 2048, K = 2048 against the skinny kernel's partial sums and their second kernel: 9 against 13 us at 17 and 32 rows,

@@ -61,9 +61,17 @@ class DecoderModel:
         trace = self.trace
         if trace is not None:
             trace("embedding", -1, x)
+        handed = None                     # the next block's first norm, where the block before could leave it half applied
         for i, entry in enumerate(self.run_order):
             ctx.trace = None if trace is None else (lambda tag, rows, i=i: trace(tag, i, rows))
-            self.layers[entry.layer].forward(x, ctx, cache.layer_cache(i))
+            layer = self.layers[entry.layer]
+            if getattr(layer, "hands_norm_on", False):
+                after = self.layers[self.run_order[i + 1].layer] if i + 1 < len(self.run_order) else None
+                handed = layer.forward(x, ctx, cache.layer_cache(i), handed=handed,
+                                       next_reader=after.first_reader() if getattr(after, "hands_norm_on", False) else None)
+            else:
+                layer.forward(x, ctx, cache.layer_cache(i))
+                handed = None
         ctx.trace = None
         if n_logit_rows == 0:
             return None

@@ -42,6 +42,8 @@ _SIGNATURES = {
                                  c_float, c_int, c_int, c_void_p],
     "gi_probe_stream": [c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p],
     "gi_probe_mfma": [c_int, c_void_p, c_int, c_void_p],
+    "gi_gemm_bf16_handing": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_int, c_float,
+                             c_void_p, c_void_p, c_long, c_void_p, c_void_p],
     "gi_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_filtered": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
@@ -66,6 +68,9 @@ def lib():
         l.gi_attention_bf16_supports.restype = c_int
         l.gi_gemm_bf16_scratch_floats.argtypes = [c_int, c_int, c_int]
         l.gi_gemm_bf16_scratch_floats.restype = c_long
+        for fn in (l.gi_gemm_bf16_norm_parts, l.gi_gemm_bf16_takes_norm):
+            fn.argtypes = [c_int, c_int, c_int]
+            fn.restype = c_int
         l.gi_probe_mfma_flops.argtypes = [c_int, c_int]
         l.gi_probe_mfma_flops.restype = c_long
         _lib = l
@@ -85,6 +90,9 @@ def _call(name, *args):
         raise KernelError(lib().gi_last_error().decode())
 
 
+_PROFILE_LABEL = {"gi_gemm_bf16_handing": "gemm_bf16"}        # the same products, with a norm's share on top
+
+
 class KernelProfile:
     """Time per kernel entry point, with the device waited for before and after every call (so the times add up, and
     a step takes longer than it does unobserved).  What the reference's device model reports with --profile
@@ -98,7 +106,7 @@ class KernelProfile:
 
     def timed(self, name, fn, args):
         import time
-        label, nbytes = name[3:], 0
+        label, nbytes = _PROFILE_LABEL.get(name, name[3:]), 0
         if self.note is not None:
             label, nbytes = f"{label} {self.note[0]}", self.note[1]
             self.note = None
@@ -554,9 +562,25 @@ def gemm_bf16_supports(a, w, out) -> bool:
             and (out.dtype == torch.float32 or out.dtype == torch.bfloat16) and out.stride(1) == 1)
 
 
-def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False):
+def gemm_bf16_norm_parts(m, n, k) -> int:
+    """The pieces per row in which a product [m, k] x [n, k] that adds onto rows writes their sums of squares when it hands
+    the next norm on (`gemm_bf16(..., norm_out=...)`); 0 if a product of these sizes cannot."""
+    return lib().gi_gemm_bf16_norm_parts(m, n, k)
+
+
+def gemm_bf16_takes_norm(m, n, k) -> bool:
+    """Whether a product of these sizes can read rows whose norm was handed on (`gemm_bf16(..., norm_in=...)`)."""
+    return bool(lib().gi_gemm_bf16_takes_norm(m, n, k))
+
+
+def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=None, norm_out=None):
     """out (=|+=) a @ w.T with bfloat16 operands on the matrix cores, float32 sums.
-    gated: w is [gate; up] interleaved in groups of 16 rows and out = silu(a @ gate.T) * (a @ up.T), bfloat16 [m, n/2]."""
+    gated: w is [gate; up] interleaved in groups of 16 rows and out = silu(a @ gate.T) * (a @ up.T), bfloat16 [m, n/2].
+
+    An RMS norm between two products of a few rows, without a kernel of its own:
+    norm_out = (g, scaled, squares), with accumulate: beside out += a @ w.T, scaled = bfloat16(g * out) and squares
+    [m, gemm_bf16_norm_parts(m, n, k)] = the pieces of the rows' sums of out^2;
+    norm_in = (squares, eps): a is such a `scaled`, and the results are multiplied by rsqrt(sum of the row's pieces / k + eps)."""
     _dev(a, w, out)
     m, k = a.shape
     n = w.shape[0]
@@ -570,6 +594,23 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False):
     scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device) if n_scratch else None
     if _profile is not None:
         _profile.note = (f"{n}x{k}{' gated' if gated else ''}", n * k * w.element_size())
+    if norm_in is not None or norm_out is not None:
+        squares_in, eps = norm_in if norm_in is not None else (None, 0.0)
+        g, scaled, squares_out = norm_out if norm_out is not None else (None, None, None)
+        if squares_in is not None and not (squares_in.dtype == torch.float32 and squares_in.is_contiguous() and squares_in.dim() == 2 and squares_in.shape[0] == m):
+            raise KernelError("gemm: the pieces of the sums of squares must be float32 [m, pieces]")
+        if norm_out is not None:
+            parts = gemm_bf16_norm_parts(m, n, k)
+            if not (parts and accumulate and out.dtype == torch.float32 and g.dtype == torch.float32 and g.is_contiguous() and g.numel() == n
+                    and scaled.dtype == torch.bfloat16 and scaled.shape == (m, n) and scaled.stride(1) == 1
+                    and squares_out.dtype == torch.float32 and squares_out.is_contiguous() and squares_out.shape == (m, parts)):
+                raise KernelError("gemm: handing a norm on needs a product of a few rows that adds onto float32 rows, float32 weights of the norm, "
+                                  "bfloat16 [m, n] for the scaled rows and float32 [m, gemm_bf16_norm_parts] for the sums of squares")
+            _dev(g, scaled, squares_out)
+        _call("gi_gemm_bf16_handing", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,
+              m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(squares_in), squares_in.shape[1] if squares_in is not None else 0, float(eps),
+              _ptr(g), _ptr(scaled), scaled.stride(0) if scaled is not None else 0, _ptr(squares_out), _stream())
+        return out
     _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,
           m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _stream())
     return out

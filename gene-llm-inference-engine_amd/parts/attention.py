@@ -17,11 +17,12 @@ from ..cache.needs import PagedKvNeed
 from ..kernels import ops
 from ..weights.loader import TensorNeed
 from .base import Mixer, position_class, register_mixer
-from .linear import activation_dtype_for, linear
+from .linear import activation_dtype_for, linear, linear_onto
 
 
 class Attention(Mixer):
     accepts_deferred_norm = True      # its input goes into `linear` only
+    hands_norm_on = True              # `forward` takes `then`, the norm that reads the residual next
 
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
@@ -46,7 +47,10 @@ class Attention(Mixer):
     def cache_need(cls, spec):
         return PagedKvNeed(spec.n_kv_heads, spec.head_dim, spec.window)
 
-    def forward(self, h, residual, ctx, cache):
+    def takes_handed_norm(self, n_rows: int) -> bool:
+        return self.in_dtype == torch.bfloat16 and ops.gemm_bf16_takes_norm(n_rows, self.w_qkv.shape[0], self.w_qkv.shape[1])
+
+    def forward(self, h, residual, ctx, cache, then=None):
         s, T = self.spec, ctx.n_rows
         tables = self.position.half_split_tables(ctx) if self.position is not None else None
         cos, sin = tables if tables is not None else (None, None)
@@ -67,7 +71,7 @@ class Attention(Mixer):
             ops.attention(q_rot, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, s.window)
         if att.dtype != self.att_dtype:
             att = att.to(self.att_dtype)
-        linear(att, self.w_o, residual, accumulate=True)
+        return linear_onto(att, self.w_o, residual, then)
 
 
 register_mixer("attention", Attention)

@@ -112,6 +112,14 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+# Optional, for a mixer or feed-forward (none of it is needed; a part without it is served the ordinary way):
+#   accepts_deferred_norm = True   `h` may be a norm not yet applied (parts/norm.py: `NormedRows`), which the part passes to `linear`
+#                                  unchanged; it may then also be a norm half applied by whoever wrote the rows (`HandedRows`), if
+#   takes_handed_norm(n_rows)      says that the part's first product can finish such a norm at this number of rows.
+#   hands_norm_on = True           `forward` takes a keyword `then`, the norm that will read `residual` next, adds onto the residual with
+#                                  `linear_onto(..., then)` and returns what that returns (the `HandedRows`, or None).
+
+
 class Norm(Part):
     def __call__(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
         raise NotImplementedError

@@ -38,13 +38,40 @@ class PreNormBlock:
             return norm.deferred(x, dtype)
         return norm(x, dtype)
 
-    def forward(self, x, ctx, cache):
-        self.mixer.forward(self._normed(self.mixer_norm, self.mixer, x, ctx), x, ctx, cache)
+    # A part that adds onto the residual may do the next norm's share on the way (`HandedRows` in parts/norm.py), if that
+    # norm can be applied so (`handed_weight`), its reader takes rows so normed (`takes_handed_norm`) and the part knows how
+    # (`hands_norm_on`: its `forward` takes `then` and returns the handed rows, or None where its product could not).
+    hands_norm_on = True
+
+    def first_reader(self):
+        """The norm that reads the residual first in this block, and the part that reads the normed rows."""
+        return self.mixer_norm, self.mixer
+
+    @staticmethod
+    def _then(part, reader, n_rows):
+        norm, consumer = reader if reader is not None else (None, None)
+        if (norm is None or not getattr(part, "hands_norm_on", False) or not hasattr(norm, "handed_weight")
+                or not getattr(consumer, "accepts_deferred_norm", False) or not hasattr(consumer, "takes_handed_norm")
+                or not consumer.takes_handed_norm(n_rows)):
+            return None
+        return norm
+
+    def forward(self, x, ctx, cache, handed=None, next_reader=None):
+        """handed: this block's first norm as whoever wrote x last left it, or None.  next_reader: `first_reader()` of whatever
+        reads x after this block, or None.  Returns that reader's norm handed on, or None."""
+        if handed is None or handed.norm is not self.mixer_norm:
+            handed = self._normed(self.mixer_norm, self.mixer, x, ctx)
+        then = self._then(self.mixer, (self.feed_forward_norm, self.feed_forward), ctx.n_rows)
+        handed = self.mixer.forward(handed, x, ctx, cache) if then is None else self.mixer.forward(handed, x, ctx, cache, then=then)
         if ctx.trace is not None:
             ctx.trace("attn_out", x)
-        self.feed_forward.forward(self._normed(self.feed_forward_norm, self.feed_forward, x, ctx), x, ctx)
+        if handed is None or then is None:
+            handed = self._normed(self.feed_forward_norm, self.feed_forward, x, ctx)
+        then = self._then(self.feed_forward, next_reader, ctx.n_rows)
+        handed = self.feed_forward.forward(handed, x, ctx) if then is None else self.feed_forward.forward(handed, x, ctx, then=then)
         if ctx.trace is not None:
             ctx.trace("ffn_out", x)
+        return handed if then is not None else None
 
 
 register_block("prenorm", PreNormBlock)

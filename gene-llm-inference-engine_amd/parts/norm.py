@@ -3,7 +3,14 @@
 
 A norm may be handed on *unapplied* (`deferred`): `NormedRows` names the rows (optionally a
 selection of them), the weight and eps; whoever consumes it asks for the rows (`materialize`), and
-the norm's kernel gathers the selection itself."""
+the norm's kernel gathers the selection itself.
+
+A norm may also be *half applied* by the product that wrote the rows last (`HandedRows`): that
+product, when it adds onto the rows x, also writes w * x in bfloat16 and the pieces of every row's
+sum of squares, and the product that reads the normed rows multiplies its results by
+rsqrt(mean(x^2) + eps), which is one number a row and commutes with it.  For a few rows (decoding)
+this saves the norm's kernel; `linear` decides where it applies, and `materialize` still gives the
+rows the ordinary way."""
 from __future__ import annotations
 
 import torch
@@ -27,6 +34,14 @@ class NormedRows:
         return self._value
 
 
+class HandedRows(NormedRows):
+    """norm(x) as bfloat16, half applied: `scaled` = w * x, `squares` [rows, pieces] = the pieces of the rows' sums of x^2."""
+
+    def __init__(self, norm: "RmsNorm", x: torch.Tensor, scaled: torch.Tensor, squares: torch.Tensor):
+        super().__init__(norm, x, torch.bfloat16)
+        self.scaled, self.squares, self.eps = scaled, squares, norm.eps
+
+
 class RmsNorm(Norm):
     graph_safe = True
 
@@ -34,6 +49,7 @@ class RmsNorm(Norm):
         super().__init__(spec, tensors, dtype, device)
         self.weight = tensors[spec.weight]
         self.eps = float(spec.eps)
+        self._weight_f32 = None
 
     @classmethod
     def tensor_needs(cls, spec):
@@ -49,6 +65,12 @@ class RmsNorm(Norm):
 
     def deferred(self, x, out_dtype, rows=None) -> NormedRows:
         return NormedRows(self, x, out_dtype, rows)
+
+    def handed_weight(self) -> torch.Tensor:
+        """The weights in 32-bit, for a product that applies them to the rows it has just written."""
+        if self._weight_f32 is None:
+            self._weight_f32 = self.weight.float().contiguous()
+        return self._weight_f32
 
 
 register_norm("rmsnorm", RmsNorm)

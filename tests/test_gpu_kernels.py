@@ -171,6 +171,45 @@ def test_rope_cos_sin_uses_64_bit_angles():
     assert (cos.double() - torch.cos(ang)).abs().max() < 1e-7 and (sin.double() - torch.sin(ang)).abs().max() < 1e-7
 
 
+@pytest.mark.parametrize("m,d,k1,n2,gated", [(1, 2048, 2048, 3072, False), (8, 2048, 8192, 16384, True), (8, 2048, 2048, 16384, True), (9, 2048, 2048, 3072, False),
+                                            (16, 136, 264, 96, False), (5, 3072, 3072, 5120, False), (3, 4096, 4096, 6144, False), (7, 264, 136, 64, True)])
+def test_norm_handed_from_one_product_to_the_next(m, d, k1, n2, gated):
+    """A product that adds onto rows x also writes g * x and the pieces of the rows' sums of squares; the next product reads
+    g * x and multiplies its results by rsqrt(mean(x^2) + eps).  The rows x are what the plain product leaves, bit for bit; the
+    second product's results are as near the 64-bit norm and product as those of the norm's own kernel followed by the product."""
+    o = ops()
+    eps = 1e-5
+    a = randn(m, k1, dtype=torch.bfloat16, seed=1)
+    w1 = randn(d, k1, dtype=torch.bfloat16, seed=2, scale=0.05)
+    w2 = randn(n2, d, dtype=torch.bfloat16, seed=3, scale=0.05)
+    g = (1 + 0.1 * randn(d, seed=4)).float()
+    x0 = randn(m, d, seed=5)
+    parts = o.gemm_bf16_norm_parts(m, d, k1)
+    assert parts and o.gemm_bf16_takes_norm(m, n2, d), "every case here is one the kernels take"
+    plain_x = x0.clone()
+    o.gemm_bf16(a, w1, plain_x, accumulate=True)
+    x, scaled, squares = x0.clone(), torch.full((m, d), float("nan"), dtype=torch.bfloat16, device=DEV), torch.full((m, parts), float("nan"), device=DEV)
+    o.gemm_bf16(a, w1, x, accumulate=True, norm_out=(g, scaled, squares))
+    assert torch.equal(x, plain_x)
+    assert torch.equal(scaled, (g * x).to(torch.bfloat16))
+    assert rel(squares.double().sum(1), (x.double() ** 2).sum(1)) < 1e-6
+    out_shape = (m, n2 // 2) if gated else (m, n2)
+    out_dtype = torch.bfloat16 if gated else torch.float32
+    w2k = o.interleave_gate_up(w2[:n2 // 2], w2[n2 // 2:]) if gated else w2
+    handed = torch.empty(out_shape, dtype=out_dtype, device=DEV)
+    o.gemm_bf16(scaled, w2k, handed, gated=gated, norm_in=(squares, eps))
+    normed = torch.empty((m, d), dtype=torch.bfloat16, device=DEV)
+    o.rmsnorm(x, g, eps, normed)
+    usual = torch.empty(out_shape, dtype=out_dtype, device=DEV)
+    o.gemm_bf16(normed, w2k, usual, gated=gated)
+    xd = x.double()
+    exact = (g.double() * xd * torch.rsqrt((xd ** 2).mean(1, keepdim=True) + eps)) @ w2.double().T
+    if gated:
+        exact = torch.nn.functional.silu(exact[:, :n2 // 2]) * exact[:, n2 // 2:]
+    err_handed, err_usual = rel(handed, exact), rel(usual, exact)
+    assert err_handed < 1.5 * err_usual + 1e-6, (err_handed, err_usual)
+
+
 # -------------------------------------------------------------------------------------- sampling
 def test_argmax_lowest_index_on_ties():
     rows = [[1, 5, 5, 2], [3, 3, 3, 3], [-7, -8, -9, -10], [0, -1, 9, 9]]          # tests/verify_sampler.py:173-178
