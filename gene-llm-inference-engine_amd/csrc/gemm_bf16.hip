@@ -497,12 +497,45 @@ constexpr int SK = 128;                               // k per product group of 
 constexpr int SKINNY_MAX_ROWS = 128;                  // rows of A the skinny kernel takes (8 tiles of 16)
 constexpr int KB = 2 * SK, X_STRIDE = KB + 8;         // k per block of the workgroup; +8 bf16 of padding
 
+// ----------------------------------------------------------------- an RMS norm between two products of a few rows
+// The norm of a row x is g * x * r with r = rsqrt(mean(x^2) + eps), and r, one number a row, commutes with the product that reads
+// the normed row.  A product that adds onto the rows x also writes g * x of the sums it has just made, in bfloat16, and what its
+// columns give to the sum of squares of every row, one number per row and piece of the row (`NormOut`); the product that reads
+// those rows multiplies its results by r, which it gets from those numbers, added in a fixed order (`NormIn`).  No kernel for
+// the norm, no second pass over the rows.
+struct NormOut {                 // for a product that adds onto x: all null if it does not hand the norm on
+    const float* g;              // the norm's weights [N]
+    bf16_t* scaled;              // out: g * x, [M, ld]
+    long ld;
+    float* squares;              // out: [M, parts]
+};
+struct NormIn {                  // for a product whose rows A are g * x without r: squares null if they are ready-made rows
+    const float* squares;        // [M, parts]
+    int parts;
+    float eps;
+    int dim;                     // r = rsqrt(sum / dim + eps)
+};
+// The kernel for at most 16 rows: a thread keeps 8 pieces while the products run (more would cost the kernel its second
+// workgroup per compute unit); 64 threads share a row where there are at most 8 rows, 32 otherwise.
+constexpr int SLIM_PIECES = 8;
+__host__ __device__ constexpr int slim_max_parts(int M) { return SLIM_PIECES * (M <= 8 ? 64 : 32); }
+// The kernels for 17 to 128 rows: the kernel that adds the partial sums onto x writes one piece per 1024 columns.
+constexpr int REDUCE_COLUMNS = 1024, REDUCE_MAX_PARTS = 8;
+
+__device__ __forceinline__ float row_scale_of(const NormIn& n, int row) {      // a few pieces: read and added one by one
+    float sum = 0.f;
+    for (int p = 0; p < n.parts; ++p) sum += n.squares[(size_t)row * n.parts + p];
+    return 1.0f / sqrtf(sum / (float)n.dim + n.eps);
+}
+
 template <int MT, int EPI, bool PARTIAL>
 __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
                                                               float* __restrict__ P, int M, int N, int K, long lda, long ldw, long ldc,
-                                                              int k_per_split) {
+                                                              int k_per_split, NormIn norm_in) {
     __shared__ __attribute__((aligned(16))) bf16_t Xs[MT * 16 * X_STRIDE];
     __shared__ float other[4][MT][64][4];
+    __shared__ float row_scale[MT * 16];
+    const bool scaled_rows = !PARTIAL && norm_in.squares != nullptr;       // the rows of A lack their norm's rsqrt(mean square + eps)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int strip = wave & 3, half = wave >> 2;
     const int r = lane & 15, q = lane >> 4;
@@ -529,6 +562,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __r
     fetch_x(k_begin);
     fetch_w(k_begin, w_buf[0]);
     fetch_w(k_begin + KB, w_buf[1]);
+    if (scaled_rows && tid < MT * 16) row_scale[tid] = tid < M ? row_scale_of(norm_in, tid) : 0.f;     // (the loop's barriers lie before its use)
     for (int k0 = k_begin; k0 < k_end; k0 += 3 * KB) {
 #pragma unroll
         for (int d = 0; d < 3; ++d) {                 // buffer d holds the weights of block k0 + d*KB
@@ -586,7 +620,8 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __r
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const int m = t * 16 + 4 * q + v;
-                    if (m < M) ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 32 + (strip >> 1) * 16 + r] = f32_to_bf16(silu_gate(acc[t][v], other[strip + 1][t][lane][v]));
+                    const float rs = scaled_rows ? row_scale[m] : 1.0f;
+                    if (m < M) ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 32 + (strip >> 1) * 16 + r] = f32_to_bf16(silu_gate(acc[t][v] * rs, other[strip + 1][t][lane][v] * rs));
                 }
         }
     } else if (half == 0 && n < N) {
@@ -597,15 +632,19 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __r
                 const int m = t * 16 + 4 * q + v;
                 if (m >= M) continue;
                 if constexpr (PARTIAL) P[((size_t)blockIdx.y * M + m) * N + n] = acc[t][v];
-                else write_out<EPI>(C, (size_t)m * ldc + n, acc[t][v]);
+                else write_out<EPI>(C, (size_t)m * ldc + n, scaled_rows ? acc[t][v] * row_scale[m] : acc[t][v]);
             }
     }
 }
 
 // Adds the k-split partial sums [splits][M][N] in ascending split order and writes the result.  A thread takes VEC neighbouring
 // columns and asks for its values of up to eight splits at once: the kernel is one round trip to memory, not one per split.
+// With `norm_in` the sums are multiplied by their row's rsqrt(mean square + eps).  With `norm_out` (adding onto 32-bit rows, four
+// columns a thread, rows of a multiple of 1024 columns: a workgroup then lies in one row, and no workgroup is cut short) the rows'
+// new values times g go out in bfloat16 beside them, and the workgroup's share of the row's sum of squares.
 template <int EPI, int VEC>
-__global__ void skinny_reduce_kernel(const float* __restrict__ P, void* __restrict__ C, int M, int N, int splits, long ldc) {
+__global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restrict__ P, void* __restrict__ C, int M, int N, int splits, long ldc,
+                                                            NormIn norm_in, NormOut norm_out) {
     const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC, slab = (size_t)M * N;
     if (i >= slab) return;
     float s[VEC];
@@ -631,6 +670,11 @@ __global__ void skinny_reduce_kernel(const float* __restrict__ P, void* __restri
             }
     }
     const size_t row = i / N, col = i % N, o = row * ldc + col;      // (VEC divides N: the VEC columns lie in one row)
+    if (norm_in.squares != nullptr) {
+        const float rs = row_scale_of(norm_in, (int)row);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) s[v] *= rs;
+    }
     if constexpr (VEC == 4) {                                        // (the host has checked that rows of C start at multiples of 16 bytes)
         if constexpr (EPI == EPI_STORE_BF16) {
             uint2 packed;
@@ -642,6 +686,25 @@ __global__ void skinny_reduce_kernel(const float* __restrict__ P, void* __restri
             float4 x = EPI == EPI_ADD_F32 ? *dst : float4{0.f, 0.f, 0.f, 0.f};
             x.x += s[0]; x.y += s[1]; x.z += s[2]; x.w += s[3];
             *dst = x;
+            if constexpr (EPI == EPI_ADD_F32) {
+                if (norm_out.scaled != nullptr) {                    // (the same for every thread of the kernel)
+                    __shared__ float wave_squares[4];
+                    const float4 g = *reinterpret_cast<const float4*>(norm_out.g + col);
+                    uint2 packed;
+                    packed.x = (unsigned)f32_to_bf16(g.x * x.x) | ((unsigned)f32_to_bf16(g.y * x.y) << 16);
+                    packed.y = (unsigned)f32_to_bf16(g.z * x.z) | ((unsigned)f32_to_bf16(g.w * x.w) << 16);
+                    *reinterpret_cast<uint2*>(norm_out.scaled + row * norm_out.ld + col) = packed;
+                    float square = (x.x * x.x + x.y * x.y) + (x.z * x.z + x.w * x.w);
+#pragma unroll
+                    for (int off = 32; off > 0; off >>= 1) square += __shfl_xor(square, off, 64);
+                    if ((threadIdx.x & 63) == 0) wave_squares[threadIdx.x >> 6] = square;
+                    __syncthreads();
+                    if (threadIdx.x == 0) {
+                        const int per_row = N / REDUCE_COLUMNS;
+                        norm_out.squares[row * per_row + blockIdx.x % per_row] = (wave_squares[0] + wave_squares[1]) + (wave_squares[2] + wave_squares[3]);
+                    }
+                }
+            }
         }
     } else {
         write_out<EPI>(C, o, s[0]);
@@ -672,28 +735,7 @@ __global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* 
 // and of activation row r, so the four lanes of a row read 64 contiguous bytes per load.  Loads run
 // two blocks ahead of the products.  The slices' sums meet in LDS and are added in slice order.
 // ROWS = 8 leaves half of each product idle and doubles the number of workgroups for narrow outputs.
-//
-// HAND: an RMS norm between two such products without a kernel of its own.  The norm of a row x is g * x * r with
-// r = rsqrt(mean(x^2) + eps), and r, one number a row, commutes with the product that reads the normed row.  A product that adds
-// onto the rows x (EPI_ADD_F32) also writes g * x of the sums it has just made, in bfloat16, and what its columns give to the
-// sum of squares of every row, one number per row and workgroup (`norm_out`); the product that reads those rows multiplies its
-// results by r, which it gets from those numbers, added in a fixed order (`norm_in`).
-struct NormOut {                 // for a product that adds onto x: all null if it does not hand the norm on
-    const float* g;              // the norm's weights [N]
-    bf16_t* scaled;              // out: g * x, [M, ld]
-    long ld;
-    float* squares;              // out: [M, parts], parts = the number of workgroups (times STRIPS)
-};
-struct NormIn {                  // for a product whose rows A are g * x without r: squares null if they are ready-made rows
-    const float* squares;        // [M, parts]
-    int parts;                   // at most slim_max_parts(M)
-    float eps;                   // r = rsqrt(sum / K + eps)
-};
-// A thread keeps 8 pieces while the products run (more would cost the kernel its second workgroup per compute unit); 64 threads
-// share a row where there are at most 8 rows, 32 otherwise.
-constexpr int SLIM_PIECES = 8;
-__host__ __device__ constexpr int slim_max_parts(int M) { return SLIM_PIECES * (M <= 8 ? 64 : 32); }
-
+// HAND: with the two halves of a norm handed from product to product (`NormIn`, `NormOut` above).
 template <int STRIPS, int ROWS, int EPI, bool HAND>
 __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
                                                             int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in, NormOut norm_out) {
@@ -753,7 +795,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
             if (sharing == 64) sum += __shfl_xor(sum, 32, 64);
 #pragma unroll
             for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
-            if ((tid & (sharing - 1)) == 0 && piece_row < 16) row_scale[piece_row] = 1.0f / sqrtf(sum / (float)K + norm_in.eps);
+            if ((tid & (sharing - 1)) == 0 && piece_row < 16) row_scale[piece_row] = 1.0f / sqrtf(sum / (float)norm_in.dim + norm_in.eps);
         }
     }
     __syncthreads();
@@ -910,18 +952,28 @@ GI_API long gi_gemm_bf16_scratch_floats(int M, int N, int K) {
     return splits > 1 ? (long)splits * M * N : 0;
 }
 
-static int reduce_partials(const float* scratch, void* C, int epi, int M, int N, int splits, long ldc, hipStream_t stream) {
+static const NormIn NO_NORM_IN = {nullptr, 0, 0.f, 1};
+static const NormOut NO_NORM_OUT = {nullptr, nullptr, 0, nullptr};
+
+static int reduce_partials(const float* scratch, void* C, int epi, int M, int N, int splits, long ldc, hipStream_t stream, NormIn norm_in = NO_NORM_IN,
+                           NormOut norm_out = NO_NORM_OUT) {
     if (epi == EPI_GATED_BF16) {
+        GI_REQUIRE(norm_in.squares == nullptr, "gemm_bf16: a gated product whose k is shared out cannot finish a norm handed on");
         skinny_reduce_gated_kernel<<<(unsigned)(((size_t)M * (N / 2) + 255) / 256), 256, 0, stream>>>(scratch, (bf16_t*)C, M, N, splits, ldc);
     } else {
 #define REDUCE(VEC_)                                                                                                                    \
     do {                                                                                                                                \
         const unsigned blocks = (unsigned)(((size_t)M * N / VEC_ + 255) / 256);                                                         \
-        if (epi == EPI_STORE_F32) skinny_reduce_kernel<EPI_STORE_F32, VEC_><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);  \
-        else if (epi == EPI_ADD_F32) skinny_reduce_kernel<EPI_ADD_F32, VEC_><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc); \
-        else skinny_reduce_kernel<EPI_STORE_BF16, VEC_><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc);                      \
+        if (epi == EPI_STORE_F32) skinny_reduce_kernel<EPI_STORE_F32, VEC_><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc, norm_in, norm_out);  \
+        else if (epi == EPI_ADD_F32) skinny_reduce_kernel<EPI_ADD_F32, VEC_><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc, norm_in, norm_out); \
+        else skinny_reduce_kernel<EPI_STORE_BF16, VEC_><<<blocks, 256, 0, stream>>>(scratch, C, M, N, splits, ldc, norm_in, norm_out);                      \
     } while (0)
-        if (N % 4 == 0 && ldc % 4 == 0 && ((uintptr_t)scratch & 15) == 0 && ((uintptr_t)C & 15) == 0) REDUCE(4); else REDUCE(1);
+        const bool four = N % 4 == 0 && ldc % 4 == 0 && ((uintptr_t)scratch & 15) == 0 && ((uintptr_t)C & 15) == 0;
+        GI_REQUIRE(norm_out.scaled == nullptr || (four && epi == EPI_ADD_F32 && N % REDUCE_COLUMNS == 0 && N / REDUCE_COLUMNS <= REDUCE_MAX_PARTS && norm_out.ld % 4 == 0 &&
+                                                  ((uintptr_t)norm_out.scaled & 7) == 0 && ((uintptr_t)norm_out.g & 15) == 0),
+                   "gemm_bf16: handing a norm on from %d rows needs rows of a multiple of %d columns, at most %d, and aligned operands", M, REDUCE_COLUMNS,
+                   REDUCE_COLUMNS * REDUCE_MAX_PARTS);
+        if (four) REDUCE(4); else REDUCE(1);
 #undef REDUCE
     }
     GI_CHECK_LAUNCH("gemm_bf16 (reduce)");
@@ -963,25 +1015,92 @@ static int launch_slim(const void* A, const void* W, void* C, int epi, int M, in
     return 0;
 }
 
-// The pieces per row that a product of these sizes writes when it hands a norm on (gi_gemm_bf16_handing with `scaled_out`);
-// 0 if it cannot: more than 16 rows, or a shape that the slim kernel does not take.
-GI_API int gi_gemm_bf16_norm_parts(int M, int N, int K) {
-    if (!takes_slim(M, N, K)) return 0;
-    const int parts = slim_parts(N);
-    return parts <= slim_max_parts(M) ? parts : 0;
+// 17 to 32 rows, a narrow output and a short k: one launch of the slim kernel with two tiles of activation rows.  Measured at
+// N = 3072 and 2048, K = 2048 against the skinny kernel's partial sums and their second kernel: 9 against 13 us at 17 and 32 rows,
+// 11 against 13 at 48, 13 against 13 at 64; at K = 8192 (every workgroup reads all the activations: 1 MB at 64 rows) 21 to 43 us
+// against 16 to 19, so longer k and more rows stay with the skinny kernel.
+static bool takes_slim_tiles(int M, int N, int K, int epi) {
+    return !takes_slim(M, N, K) && M <= 32 && K <= 2048 && epi != EPI_GATED_BF16 && gi_gemm_bf16_skinny_splits(N, K) > 0;
 }
 
-// Whether a product of these sizes can read rows whose norm was handed on (gi_gemm_bf16_handing with `squares_in`).
-GI_API int gi_gemm_bf16_takes_norm(int M, int N, int K) { return takes_slim(M, N, K) ? 1 : 0; }
+static int launch_slim_tiles(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, hipStream_t stream) {
+    dim3 grid((N + 15) / 16);
+#define SLIM_TILES(MT_)                                                                                                                             \
+    do {                                                                                                                                            \
+        if (epi == EPI_STORE_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+        else if (epi == EPI_ADD_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_ADD_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+        else gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_BF16><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+    } while (0)
+    SLIM_TILES(2);
+#undef SLIM_TILES
+    GI_CHECK_LAUNCH("gemm_bf16 (slim, tiles)");
+    return 0;
+}
 
-// gi_gemm_bf16 for at most 16 rows, with an RMS norm handed from one product to the next instead of a kernel of its own.
+// Up to 128 rows the weights are the traffic and every workgroup streams its share of them once (measured on the decode step of
+// the Llama-3.2-1B shape: 72 rows took 2.69 ms through the tiles of 128 rows of the kernels for more rows, against 2.11 ms at 64 rows).
+static int launch_skinny(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, float* scratch,
+                         long scratch_floats, NormIn norm_in, NormOut norm_out, hipStream_t stream) {
+    const int splits = gi_gemm_bf16_skinny_splits(N, K), mt = (M + 15) / 16;
+#define SKINNY_MT(EPI_, PARTIAL_)                                                                                                   \
+    do {                                                                                                                            \
+        if (mt == 1) gemm_bf16_skinny_kernel<1, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
+        else if (mt == 2) gemm_bf16_skinny_kernel<2, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
+        else if (mt == 3) gemm_bf16_skinny_kernel<3, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
+        else if (mt == 4) gemm_bf16_skinny_kernel<4, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
+        else if (mt <= 6) gemm_bf16_skinny_kernel<6, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
+        else gemm_bf16_skinny_kernel<8, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
+    } while (0)
+    GI_REQUIRE(norm_in.squares == nullptr || norm_in.parts <= REDUCE_MAX_PARTS, "gemm_bf16: %d pieces of a sum of squares, at most %d for more than 16 rows",
+               norm_in.parts, REDUCE_MAX_PARTS);
+    if (splits == 0) {                             // a wide output: every workgroup sees all of k and finishes its columns
+        GI_REQUIRE(norm_out.scaled == nullptr, "gemm_bf16: a product this wide does not hand a norm on");
+        const int k_per_split = K;
+        dim3 grid((N + 63) / 64, 1);
+        if (epi == EPI_GATED_BF16) SKINNY_MT(EPI_GATED_BF16, false); else if (epi == EPI_STORE_F32) SKINNY_MT(EPI_STORE_F32, false);
+        else if (epi == EPI_ADD_F32) SKINNY_MT(EPI_ADD_F32, false); else SKINNY_MT(EPI_STORE_BF16, false);
+        GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
+        return 0;
+    }
+    GI_REQUIRE(scratch != nullptr && scratch_floats >= (long)splits * M * N, "gemm_bf16: scratch of %ld floats needed, %ld given",
+               (long)splits * M * N, scratch_floats);
+    int k_per_split = (K + splits - 1) / splits;
+    k_per_split = (k_per_split + KB - 1) / KB * KB;
+    dim3 grid((N + 63) / 64, splits);
+    SKINNY_MT(EPI_STORE_F32, true);
+#undef SKINNY_MT
+    GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
+    return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream, norm_in, norm_out);
+}
+
+// The pieces per row that a product of these sizes writes when it hands a norm on (gi_gemm_bf16_handing with `scaled_out`);
+// 0 if it cannot: a shape whose kernel does not do it.  Up to 16 rows one piece per workgroup of the slim kernel; up to 128 rows
+// one per 1024 columns, from the kernel that adds the partial sums of the shares of k onto the rows.
+GI_API int gi_gemm_bf16_norm_parts(int M, int N, int K) {
+    if (takes_slim(M, N, K)) {
+        const int parts = slim_parts(N);
+        return parts <= slim_max_parts(M) ? parts : 0;
+    }
+    if (M <= 16 || M > SKINNY_MAX_ROWS || takes_slim_tiles(M, N, K, EPI_ADD_F32) || gi_gemm_bf16_skinny_splits(N, K) == 0) return 0;
+    return N % REDUCE_COLUMNS == 0 && N / REDUCE_COLUMNS <= REDUCE_MAX_PARTS ? N / REDUCE_COLUMNS : 0;
+}
+
+// Whether a product of these sizes can read rows whose norm was handed on (gi_gemm_bf16_handing with `squares_in`) by a product
+// of as many rows.
+GI_API int gi_gemm_bf16_takes_norm(int M, int N, int K, int gated) {
+    if (takes_slim(M, N, K)) return 1;
+    if (M <= 16 || M > SKINNY_MAX_ROWS || takes_slim_tiles(M, N, K, gated ? EPI_GATED_BF16 : EPI_STORE_F32)) return 0;
+    return gi_gemm_bf16_skinny_splits(N, K) == 0 || !gated ? 1 : 0;
+}
+
+// gi_gemm_bf16 for at most 128 rows, with an RMS norm handed from one product to the next instead of a kernel of its own.
 // squares_in != null: the rows A are g * x of some rows x, in bfloat16, and squares_in [M, parts_in] holds the pieces of every
 // row's sum of x^2; the results are multiplied by rsqrt(sum / K + eps).  scaled_out != null (needs accumulate onto 32-bit C):
 // beside C += A W^T, scaled_out [M, ld_scaled] = bfloat16(g * C) and squares_out [M, gi_gemm_bf16_norm_parts(M, N, K)] = the
-// pieces of the rows' sums of C^2, for the next product.
+// pieces of the rows' sums of C^2, for the next product.  Where the two queries above say no, it fails.
 GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dtype, int accumulate, int gated, int M, int N, int K, long lda,
-                                long ldw, long ldc, const float* squares_in, int parts_in, float eps, const float* g, void* scaled_out,
-                                long ld_scaled, float* squares_out, hipStream_t stream) {
+                                long ldw, long ldc, float* scratch, long scratch_floats, const float* squares_in, int parts_in, float eps,
+                                const float* g, void* scaled_out, long ld_scaled, float* squares_out, hipStream_t stream) {
     GI_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: M %d, N %d, K %d must be positive", M, N, K);
     GI_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_bf16: K %d and the row strides (%ld, %ld) must be multiples of 8", K, lda, ldw);
     GI_REQUIRE(((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_bf16: operands must be 16-byte aligned");
@@ -992,11 +1111,19 @@ GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dty
         epi = EPI_GATED_BF16;
     }
     GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
-    GI_REQUIRE(takes_slim(M, N, K), "gemm_bf16: a norm is handed on between products of at most 16 rows (M %d, N %d, K %d)", M, N, K);
-    GI_REQUIRE(squares_in == nullptr || (parts_in > 0 && parts_in <= slim_max_parts(M)), "gemm_bf16: %d pieces of a sum of squares, at most %d", parts_in, slim_max_parts(M));
-    GI_REQUIRE(scaled_out == nullptr || (epi == EPI_ADD_F32 && g != nullptr && squares_out != nullptr && ld_scaled >= N && slim_parts(N) <= slim_max_parts(M)),
-               "gemm_bf16: handing a norm on needs a product that adds onto 32-bit rows, the norm's weights and room for the sums of squares");
-    return launch_slim(A, W, C, epi, M, N, K, lda, ldw, ldc, NormIn{squares_in, parts_in, eps}, NormOut{g, (bf16_t*)scaled_out, ld_scaled, squares_out}, stream);
+    GI_REQUIRE(squares_in == nullptr || (parts_in > 0 && gi_gemm_bf16_takes_norm(M, N, K, gated)),
+               "gemm_bf16: a product of these sizes (M %d, N %d, K %d%s) cannot finish a norm handed on", M, N, K, gated ? ", gated" : "");
+    GI_REQUIRE(scaled_out == nullptr || (epi == EPI_ADD_F32 && g != nullptr && squares_out != nullptr && ld_scaled >= N && gi_gemm_bf16_norm_parts(M, N, K) > 0),
+               "gemm_bf16: handing a norm on needs a product that adds onto 32-bit rows, of sizes that allow it (M %d, N %d, K %d), the norm's weights and "
+               "room for the sums of squares", M, N, K);
+    const NormIn norm_in = {squares_in, parts_in, eps, K};
+    const NormOut norm_out = {g, (bf16_t*)scaled_out, ld_scaled, squares_out};
+    if (takes_slim(M, N, K)) {
+        GI_REQUIRE(squares_in == nullptr || parts_in <= slim_max_parts(M), "gemm_bf16: %d pieces of a sum of squares, at most %d", parts_in, slim_max_parts(M));
+        return launch_slim(A, W, C, epi, M, N, K, lda, ldw, ldc, norm_in, norm_out, stream);
+    }
+    GI_REQUIRE(!takes_slim_tiles(M, N, K, epi) && M <= SKINNY_MAX_ROWS, "gemm_bf16: no norm is handed on by or to a product of these sizes (M %d, N %d, K %d)", M, N, K);
+    return launch_skinny(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, norm_in, norm_out, stream);
 }
 
 // `gated` != 0: W is [gate; up] interleaved in groups of 16 rows (N rows in all, a multiple of 32)
@@ -1014,56 +1141,10 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     }
     GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
 
-    if (takes_slim(M, N, K)) return launch_slim(A, W, C, epi, M, N, K, lda, ldw, ldc, NormIn{nullptr, 0, 0.f}, NormOut{nullptr, nullptr, 0, nullptr}, stream);
+    if (takes_slim(M, N, K)) return launch_slim(A, W, C, epi, M, N, K, lda, ldw, ldc, NO_NORM_IN, NO_NORM_OUT, stream);
 
-    // 17 to 32 rows, a narrow output and a short k: one launch of the slim kernel with two tiles of activation rows.  Measured at
-    // N = 3072 and 2048, K = 2048 against the skinny kernel's partial sums and their second kernel: 9 against 13 us at 17 and 32 rows,
-    // 11 against 13 at 48, 13 against 13 at 64; at K = 8192 (every workgroup reads all the activations: 1 MB at 64 rows) 21 to 43 us
-    // against 16 to 19, so longer k and more rows stay with the skinny kernel.
-    if (M <= 32 && K <= 2048 && epi != EPI_GATED_BF16 && gi_gemm_bf16_skinny_splits(N, K) > 0) {
-        dim3 grid((N + 15) / 16);
-#define SLIM_TILES(MT_)                                                                                                                             \
-    do {                                                                                                                                            \
-        if (epi == EPI_STORE_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
-        else if (epi == EPI_ADD_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_ADD_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
-        else gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_BF16><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
-    } while (0)
-        SLIM_TILES(2);
-#undef SLIM_TILES
-        GI_CHECK_LAUNCH("gemm_bf16 (slim, tiles)");
-        return 0;
-    }
-    // Up to 128 rows the weights are the traffic and every workgroup streams its share of them once (measured on the decode step of
-    // the Llama-3.2-1B shape: 72 rows took 2.69 ms through the tiles of 128 rows of the kernels below, against 2.11 ms at 64 rows).
-    if (M <= SKINNY_MAX_ROWS) {
-        const int splits = gi_gemm_bf16_skinny_splits(N, K), mt = (M + 15) / 16;
-#define SKINNY_MT(EPI_, PARTIAL_)                                                                                                   \
-    do {                                                                                                                            \
-        if (mt == 1) gemm_bf16_skinny_kernel<1, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split); \
-        else if (mt == 2) gemm_bf16_skinny_kernel<2, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split); \
-        else if (mt == 3) gemm_bf16_skinny_kernel<3, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split); \
-        else if (mt == 4) gemm_bf16_skinny_kernel<4, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split); \
-        else if (mt <= 6) gemm_bf16_skinny_kernel<6, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split); \
-        else gemm_bf16_skinny_kernel<8, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split); \
-    } while (0)
-        if (splits == 0) {                             // a wide output: every workgroup sees all of k and finishes its columns
-            const int k_per_split = K;
-            dim3 grid((N + 63) / 64, 1);
-            if (epi == EPI_GATED_BF16) SKINNY_MT(EPI_GATED_BF16, false); else if (epi == EPI_STORE_F32) SKINNY_MT(EPI_STORE_F32, false);
-            else if (epi == EPI_ADD_F32) SKINNY_MT(EPI_ADD_F32, false); else SKINNY_MT(EPI_STORE_BF16, false);
-            GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
-            return 0;
-        }
-        GI_REQUIRE(scratch != nullptr && scratch_floats >= (long)splits * M * N, "gemm_bf16: scratch of %ld floats needed, %ld given",
-                   (long)splits * M * N, scratch_floats);
-        int k_per_split = (K + splits - 1) / splits;
-        k_per_split = (k_per_split + KB - 1) / KB * KB;
-        dim3 grid((N + 63) / 64, splits);
-        SKINNY_MT(EPI_STORE_F32, true);
-#undef SKINNY_MT
-        GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
-        return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream);
-    }
+    if (takes_slim_tiles(M, N, K, epi)) return launch_slim_tiles(A, W, C, epi, M, N, K, lda, ldw, ldc, stream);
+    if (M <= SKINNY_MAX_ROWS) return launch_skinny(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, NO_NORM_IN, NO_NORM_OUT, stream);
 
     GI_REQUIRE((M + 63) / 64 <= 65535, "gemm_bf16: M %d is too large", M);
     if (K % PK == 0 && N >= 128) {

@@ -42,8 +42,8 @@ _SIGNATURES = {
                                  c_float, c_int, c_int, c_void_p],
     "gi_probe_stream": [c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p],
     "gi_probe_mfma": [c_int, c_void_p, c_int, c_void_p],
-    "gi_gemm_bf16_handing": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_int, c_float,
-                             c_void_p, c_void_p, c_long, c_void_p, c_void_p],
+    "gi_gemm_bf16_handing": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long,
+                             c_void_p, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p, c_void_p],
     "gi_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_filtered": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
@@ -68,9 +68,10 @@ def lib():
         l.gi_attention_bf16_supports.restype = c_int
         l.gi_gemm_bf16_scratch_floats.argtypes = [c_int, c_int, c_int]
         l.gi_gemm_bf16_scratch_floats.restype = c_long
-        for fn in (l.gi_gemm_bf16_norm_parts, l.gi_gemm_bf16_takes_norm):
-            fn.argtypes = [c_int, c_int, c_int]
-            fn.restype = c_int
+        l.gi_gemm_bf16_norm_parts.argtypes = [c_int, c_int, c_int]
+        l.gi_gemm_bf16_norm_parts.restype = c_int
+        l.gi_gemm_bf16_takes_norm.argtypes = [c_int, c_int, c_int, c_int]
+        l.gi_gemm_bf16_takes_norm.restype = c_int
         l.gi_probe_mfma_flops.argtypes = [c_int, c_int]
         l.gi_probe_mfma_flops.restype = c_long
         _lib = l
@@ -568,9 +569,10 @@ def gemm_bf16_norm_parts(m, n, k) -> int:
     return lib().gi_gemm_bf16_norm_parts(m, n, k)
 
 
-def gemm_bf16_takes_norm(m, n, k) -> bool:
-    """Whether a product of these sizes can read rows whose norm was handed on (`gemm_bf16(..., norm_in=...)`)."""
-    return bool(lib().gi_gemm_bf16_takes_norm(m, n, k))
+def gemm_bf16_takes_norm(m, n, k, gated=False) -> bool:
+    """Whether a product of these sizes can read rows whose norm was handed on (`gemm_bf16(..., norm_in=...)`) by a product
+    of as many rows."""
+    return bool(lib().gi_gemm_bf16_takes_norm(m, n, k, 1 if gated else 0))
 
 
 def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=None, norm_out=None):
@@ -608,7 +610,7 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=N
                                   "bfloat16 [m, n] for the scaled rows and float32 [m, gemm_bf16_norm_parts] for the sums of squares")
             _dev(g, scaled, squares_out)
         _call("gi_gemm_bf16_handing", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,
-              m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(squares_in), squares_in.shape[1] if squares_in is not None else 0, float(eps),
+              m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _ptr(squares_in), squares_in.shape[1] if squares_in is not None else 0, float(eps),
               _ptr(g), _ptr(scaled), scaled.stride(0) if scaled is not None else 0, _ptr(squares_out), _stream())
         return out
     _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,

@@ -21,7 +21,7 @@ def linear(a, weight: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
     """gated: weight is [gate; up] interleaved by `ops.interleave_gate_up` and out = silu(gate) * up (bfloat16 only)."""
     if isinstance(a, HandedRows):
         if (weight.dtype == torch.bfloat16 and ops.gemm_bf16_supports(a.scaled, weight, out)
-                and ops.gemm_bf16_takes_norm(a.scaled.shape[0], weight.shape[0], weight.shape[1])):
+                and ops.gemm_bf16_takes_norm(a.scaled.shape[0], weight.shape[0], weight.shape[1], gated)):
             return ops.gemm_bf16(a.scaled, weight, out, accumulate, gated, checked=True, norm_in=(a.squares, a.eps))
     if isinstance(a, NormedRows):
         a = a.materialize()

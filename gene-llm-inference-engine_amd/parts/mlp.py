@@ -33,7 +33,7 @@ class SwiGlu(FeedForward):
         return [TensorNeed(spec.gate_proj, (i, d)), TensorNeed(spec.up_proj, (i, d)), TensorNeed(spec.down_proj, (d, i))]
 
     def takes_handed_norm(self, n_rows: int) -> bool:
-        return self.in_dtype == torch.bfloat16 and ops.gemm_bf16_takes_norm(n_rows, self.w_gate_up.shape[0], self.w_gate_up.shape[1])
+        return self.in_dtype == torch.bfloat16 and ops.gemm_bf16_takes_norm(n_rows, self.w_gate_up.shape[0], self.w_gate_up.shape[1], self.fused)
 
     def forward(self, h, residual, ctx, then=None):
         T, inter = ctx.n_rows, self.spec.intermediate_size
