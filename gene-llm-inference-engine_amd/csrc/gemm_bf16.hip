@@ -528,13 +528,39 @@ __device__ __forceinline__ float row_scale_of(const NormIn& n, int row) {      /
     return 1.0f / sqrtf(sum / (float)n.dim + n.eps);
 }
 
+// The same for all M rows into `scales` (LDS, at least 32 floats or M), by a workgroup of 512 threads; the caller puts a barrier
+// before the use.  With many pieces (the writer was a kernel for at most 32 rows with a piece per workgroup: at most
+// TILES_MAX_PARTS for 17 to 32 rows, slim_max_parts for fewer) 16 or 32 threads share a row and ask for 16 pieces each at once.
+constexpr int TILES_MAX_PARTS = 256;
+__device__ __forceinline__ void row_scales_into(float* scales, const NormIn& n, int M) {
+    const int tid = threadIdx.x;
+    if (n.parts <= REDUCE_MAX_PARTS) {
+        if (tid < M) scales[tid] = row_scale_of(n, tid);
+        return;
+    }
+    const int sharing = M <= 16 ? 32 : 16, row = tid / sharing, at = tid % sharing;        // M <= 32 here
+    float piece[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int p = at + sharing * i;
+        piece[i] = (row < M && p < n.parts) ? n.squares[(size_t)row * n.parts + p] : 0.f;
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sum += piece[i];
+    if (sharing == 32) sum += __shfl_xor(sum, 16, 64);
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    if (at == 0 && row < M) scales[row] = 1.0f / sqrtf(sum / (float)n.dim + n.eps);
+}
+
 template <int MT, int EPI, bool PARTIAL>
 __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
                                                               float* __restrict__ P, int M, int N, int K, long lda, long ldw, long ldc,
                                                               int k_per_split, NormIn norm_in) {
     __shared__ __attribute__((aligned(16))) bf16_t Xs[MT * 16 * X_STRIDE];
     __shared__ float other[4][MT][64][4];
-    __shared__ float row_scale[MT * 16];
+    __shared__ float row_scale[MT * 16 < 32 ? 32 : MT * 16];
     const bool scaled_rows = !PARTIAL && norm_in.squares != nullptr;       // the rows of A lack their norm's rsqrt(mean square + eps)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int strip = wave & 3, half = wave >> 2;
@@ -562,7 +588,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __r
     fetch_x(k_begin);
     fetch_w(k_begin, w_buf[0]);
     fetch_w(k_begin + KB, w_buf[1]);
-    if (scaled_rows && tid < MT * 16) row_scale[tid] = tid < M ? row_scale_of(norm_in, tid) : 0.f;     // (the loop's barriers lie before its use)
+    if (scaled_rows) row_scales_into(row_scale, norm_in, M);                   // (the loop's barriers lie before its use)
     for (int k0 = k_begin; k0 < k_end; k0 += 3 * KB) {
 #pragma unroll
         for (int d = 0; d < 3; ++d) {                 // buffer d holds the weights of block k0 + d*KB
@@ -857,9 +883,11 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
 // second kernel to add them, costs that kernel's launch and as many bytes of partial sums as the output projection has weights.
 template <int MT, int EPI>
 __global__ __launch_bounds__(512) void gemm_bf16_slim_tiles_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
-                                                                  int M, int N, int K, long lda, long ldw, long ldc) {
+                                                                  int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in, NormOut norm_out) {
     constexpr int SLICES = 8, STEP = SLICES * SK, DEPTH = 2;
     __shared__ float red[SLICES][MT][64][4];
+    __shared__ float row_scale[MT * 16 < 32 ? 32 : MT * 16];
+    static_assert(MT == 2, "the epilogue's sums of squares take every thread's one result to lie in one row of 16 threads");
     const int tid = threadIdx.x, lane = tid & 63, slice = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
     const int n = blockIdx.x * 16 + r;
@@ -887,6 +915,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_tiles_kernel(const bf16_t*
     };
     const int k_first = slice * SK;
     fetch(k_first, w_buf[0], x_buf[0]);
+    if (norm_in.squares != nullptr) row_scales_into(row_scale, norm_in, M);      // (the barrier behind the products lies before its use)
     for (int k0 = k_first; k0 < K; k0 += DEPTH * STEP) {
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d) {                     // buffer d holds block k0 + d*STEP
@@ -910,6 +939,23 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_tiles_kernel(const bf16_t*
         float sum = 0.f;
 #pragma unroll
         for (int s = 0; s < SLICES; ++s) sum += red[s][t][src_lane][v];
+        if (norm_in.squares != nullptr && row < M) sum *= row_scale[row];
+        if constexpr (EPI == EPI_ADD_F32) {
+            if (norm_out.scaled != nullptr) {                   // (every thread comes here once: MT * 256 results, 512 threads)
+                float square = 0.f;
+                if (row < M && col < N) {
+                    float* at = (float*)C + (size_t)row * ldc + col;
+                    const float x = *at + sum;
+                    *at = x;
+                    norm_out.scaled[(size_t)row * norm_out.ld + col] = f32_to_bf16(norm_out.g[col] * x);
+                    square = x * x;
+                }
+#pragma unroll
+                for (int off = 8; off > 0; off >>= 1) square += __shfl_xor(square, off, 64);
+                if (c == 0 && row < M) norm_out.squares[(size_t)row * gridDim.x + blockIdx.x] = square;
+                continue;
+            }
+        }
         if (row < M && col < N) write_out<EPI>(C, (size_t)row * ldc + col, sum);
     }
 }
@@ -951,6 +997,9 @@ GI_API long gi_gemm_bf16_scratch_floats(int M, int N, int K) {
     const int splits = gi_gemm_bf16_piped_splits(M, N, K);
     return splits > 1 ? (long)splits * M * N : 0;
 }
+
+// The most pieces a reader of M rows takes: what a writer of as many rows makes.
+static int consumer_max_parts(int M) { return M <= 16 ? slim_max_parts(M) : M <= 32 ? TILES_MAX_PARTS : REDUCE_MAX_PARTS; }
 
 static const NormIn NO_NORM_IN = {nullptr, 0, 0.f, 1};
 static const NormOut NO_NORM_OUT = {nullptr, nullptr, 0, nullptr};
@@ -1023,13 +1072,14 @@ static bool takes_slim_tiles(int M, int N, int K, int epi) {
     return !takes_slim(M, N, K) && M <= 32 && K <= 2048 && epi != EPI_GATED_BF16 && gi_gemm_bf16_skinny_splits(N, K) > 0;
 }
 
-static int launch_slim_tiles(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, hipStream_t stream) {
+static int launch_slim_tiles(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in,
+                             NormOut norm_out, hipStream_t stream) {
     dim3 grid((N + 15) / 16);
 #define SLIM_TILES(MT_)                                                                                                                             \
     do {                                                                                                                                            \
-        if (epi == EPI_STORE_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
-        else if (epi == EPI_ADD_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_ADD_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
-        else gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_BF16><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+        if (epi == EPI_STORE_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out); \
+        else if (epi == EPI_ADD_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_ADD_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out); \
+        else gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_BF16><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out); \
     } while (0)
     SLIM_TILES(2);
 #undef SLIM_TILES
@@ -1051,8 +1101,8 @@ static int launch_skinny(const void* A, const void* W, void* C, int epi, int M, 
         else if (mt <= 6) gemm_bf16_skinny_kernel<6, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
         else gemm_bf16_skinny_kernel<8, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
     } while (0)
-    GI_REQUIRE(norm_in.squares == nullptr || norm_in.parts <= REDUCE_MAX_PARTS, "gemm_bf16: %d pieces of a sum of squares, at most %d for more than 16 rows",
-               norm_in.parts, REDUCE_MAX_PARTS);
+    GI_REQUIRE(norm_in.squares == nullptr || norm_in.parts <= consumer_max_parts(M), "gemm_bf16: %d pieces of a sum of squares, at most %d for %d rows",
+               norm_in.parts, consumer_max_parts(M), M);
     if (splits == 0) {                             // a wide output: every workgroup sees all of k and finishes its columns
         GI_REQUIRE(norm_out.scaled == nullptr, "gemm_bf16: a product this wide does not hand a norm on");
         const int k_per_split = K;
@@ -1074,23 +1124,26 @@ static int launch_skinny(const void* A, const void* W, void* C, int epi, int M, 
 }
 
 // The pieces per row that a product of these sizes writes when it hands a norm on (gi_gemm_bf16_handing with `scaled_out`);
-// 0 if it cannot: a shape whose kernel does not do it.  Up to 16 rows one piece per workgroup of the slim kernel; up to 128 rows
-// one per 1024 columns, from the kernel that adds the partial sums of the shares of k onto the rows.
+// 0 if it cannot: a shape whose kernel does not do it.  One piece per workgroup from the kernels that finish a product of up to
+// 16 or 32 rows in one launch; up to 128 rows one per 1024 columns, from the kernel that adds the partial sums of the shares of k
+// onto the rows.
 GI_API int gi_gemm_bf16_norm_parts(int M, int N, int K) {
     if (takes_slim(M, N, K)) {
         const int parts = slim_parts(N);
         return parts <= slim_max_parts(M) ? parts : 0;
     }
-    if (M <= 16 || M > SKINNY_MAX_ROWS || takes_slim_tiles(M, N, K, EPI_ADD_F32) || gi_gemm_bf16_skinny_splits(N, K) == 0) return 0;
+    if (takes_slim_tiles(M, N, K, EPI_ADD_F32)) return (N + 15) / 16 <= TILES_MAX_PARTS ? (N + 15) / 16 : 0;
+    if (M <= 16 || M > SKINNY_MAX_ROWS || gi_gemm_bf16_skinny_splits(N, K) == 0) return 0;
     return N % REDUCE_COLUMNS == 0 && N / REDUCE_COLUMNS <= REDUCE_MAX_PARTS ? N / REDUCE_COLUMNS : 0;
 }
 
 // Whether a product of these sizes can read rows whose norm was handed on (gi_gemm_bf16_handing with `squares_in`) by a product
 // of as many rows.
 GI_API int gi_gemm_bf16_takes_norm(int M, int N, int K, int gated) {
-    if (takes_slim(M, N, K)) return 1;
-    if (M <= 16 || M > SKINNY_MAX_ROWS || takes_slim_tiles(M, N, K, gated ? EPI_GATED_BF16 : EPI_STORE_F32)) return 0;
-    return gi_gemm_bf16_skinny_splits(N, K) == 0 || !gated ? 1 : 0;
+    if (takes_slim(M, N, K) || takes_slim_tiles(M, N, K, gated ? EPI_GATED_BF16 : EPI_STORE_F32)) return 1;
+    if (M > SKINNY_MAX_ROWS) return 0;
+    if (gi_gemm_bf16_skinny_splits(N, K) == 0) return 1;      // the weight-streaming kernel finishes its columns and scales them
+    return M > 32 && !gated ? 1 : 0;                          // the kernel that adds the shares of k scales: with a few pieces only
 }
 
 // gi_gemm_bf16 for at most 128 rows, with an RMS norm handed from one product to the next instead of a kernel of its own.
@@ -1122,7 +1175,11 @@ GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dty
         GI_REQUIRE(squares_in == nullptr || parts_in <= slim_max_parts(M), "gemm_bf16: %d pieces of a sum of squares, at most %d", parts_in, slim_max_parts(M));
         return launch_slim(A, W, C, epi, M, N, K, lda, ldw, ldc, norm_in, norm_out, stream);
     }
-    GI_REQUIRE(!takes_slim_tiles(M, N, K, epi) && M <= SKINNY_MAX_ROWS, "gemm_bf16: no norm is handed on by or to a product of these sizes (M %d, N %d, K %d)", M, N, K);
+    if (takes_slim_tiles(M, N, K, epi)) {
+        GI_REQUIRE(squares_in == nullptr || parts_in <= consumer_max_parts(M), "gemm_bf16: %d pieces of a sum of squares, at most %d", parts_in, consumer_max_parts(M));
+        return launch_slim_tiles(A, W, C, epi, M, N, K, lda, ldw, ldc, norm_in, norm_out, stream);
+    }
+    GI_REQUIRE(M <= SKINNY_MAX_ROWS, "gemm_bf16: no norm is handed on by or to a product of %d rows", M);
     return launch_skinny(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, norm_in, norm_out, stream);
 }
 
@@ -1143,7 +1200,7 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
 
     if (takes_slim(M, N, K)) return launch_slim(A, W, C, epi, M, N, K, lda, ldw, ldc, NO_NORM_IN, NO_NORM_OUT, stream);
 
-    if (takes_slim_tiles(M, N, K, epi)) return launch_slim_tiles(A, W, C, epi, M, N, K, lda, ldw, ldc, stream);
+    if (takes_slim_tiles(M, N, K, epi)) return launch_slim_tiles(A, W, C, epi, M, N, K, lda, ldw, ldc, NO_NORM_IN, NO_NORM_OUT, stream);
     if (M <= SKINNY_MAX_ROWS) return launch_skinny(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, NO_NORM_IN, NO_NORM_OUT, stream);
 
     GI_REQUIRE((M + 63) / 64 <= 65535, "gemm_bf16: M %d is too large", M);

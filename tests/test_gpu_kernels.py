@@ -174,7 +174,9 @@ def test_rope_cos_sin_uses_64_bit_angles():
 @pytest.mark.parametrize("m,d,k1,n2,gated", [(1, 2048, 2048, 3072, False), (8, 2048, 8192, 16384, True), (8, 2048, 2048, 16384, True), (9, 2048, 2048, 3072, False),
                                             (16, 136, 264, 96, False), (5, 3072, 3072, 5120, False), (3, 4096, 4096, 6144, False), (7, 264, 136, 64, True),
                                             (64, 2048, 8192, 16384, True), (64, 2048, 2048, 3072, False), (40, 2048, 8192, 3072, False), (17, 2048, 8192, 16384, True),
-                                            (100, 4096, 14336, 6144, False), (128, 3072, 8192, 16384, True), (33, 1024, 512, 12288, False)])
+                                            (100, 4096, 14336, 6144, False), (128, 3072, 8192, 16384, True), (33, 1024, 512, 12288, False),
+                                            (24, 2048, 2048, 16384, True), (24, 2048, 8192, 3072, False), (14, 2048, 2048, 16384, True), (32, 2048, 2048, 2048, False),
+                                            (17, 264, 136, 12288, False), (13, 4096, 4096, 28672, True)])
 def test_norm_handed_from_one_product_to_the_next(m, d, k1, n2, gated):
     """A product that adds onto rows x also writes g * x and the pieces of the rows' sums of squares; the next product reads
     g * x and multiplies its results by rsqrt(mean(x^2) + eps).  The rows x are what the plain product leaves, bit for bit; the
