@@ -24,6 +24,17 @@ def compute_dtype(name) -> torch.dtype:
         raise ValueError(f"unknown dtype {name!r}: bfloat16 or float32") from None
 
 
+class _Head:
+    """The output head as the reader of the final norm: asked, like a part, whether it takes that norm half applied."""
+    accepts_deferred_norm = True
+
+    def __init__(self, weight: torch.Tensor, in_dtype: torch.dtype):
+        self.weight, self.in_dtype = weight, in_dtype
+
+    def takes_handed_norm(self, n_rows: int) -> bool:
+        return self.in_dtype == torch.bfloat16 and ops.gemm_bf16_takes_norm(n_rows, self.weight.shape[0], self.weight.shape[1])
+
+
 class DecoderModel:
     def __init__(self, spec: ModelSpec, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device):
         self.spec, self.dtype, self.device = spec, dtype, torch.device(device)
@@ -32,6 +43,7 @@ class DecoderModel:
         self.layers = [block_class(l.block)(l, tensors, dtype, device) for l in spec.layers]
         self.final_norm = norm_class(spec.final_norm)(spec.final_norm, tensors, dtype, device)
         self.head_in_dtype = activation_dtype_for(self.lm_head, dtype)
+        self.head = _Head(self.lm_head, self.head_in_dtype)
         self.after_embedding = [row_transform_class(t)(t, tensors, dtype, device) for t in spec.after_embedding]
         self.after_head = [row_transform_class(t)(t, tensors, dtype, device) for t in spec.after_head]
         self.run_order = spec.run_order
@@ -66,9 +78,12 @@ class DecoderModel:
             ctx.trace = None if trace is None else (lambda tag, rows, i=i: trace(tag, i, rows))
             layer = self.layers[entry.layer]
             if getattr(layer, "hands_norm_on", False):
-                after = self.layers[self.run_order[i + 1].layer] if i + 1 < len(self.run_order) else None
-                handed = layer.forward(x, ctx, cache.layer_cache(i), handed=handed,
-                                       next_reader=after.first_reader() if getattr(after, "hands_norm_on", False) else None)
+                if i + 1 < len(self.run_order):
+                    after = self.layers[self.run_order[i + 1].layer]
+                    reader = after.first_reader() if getattr(after, "hands_norm_on", False) else None
+                else:                     # the head reads every row of the final norm, or a selection, which is not handed on
+                    reader = (self.final_norm, self.head) if ctx.every_row_wanted and trace is None else None
+                handed = layer.forward(x, ctx, cache.layer_cache(i), handed=handed, next_reader=reader)
             else:
                 layer.forward(x, ctx, cache.layer_cache(i))
                 handed = None
@@ -76,7 +91,9 @@ class DecoderModel:
         if n_logit_rows == 0:
             return None
         logits = torch.empty((n_logit_rows, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-        if hasattr(self.final_norm, "deferred"):
+        if handed is not None and handed.norm is self.final_norm and ctx.every_row_wanted:
+            normed = handed
+        elif hasattr(self.final_norm, "deferred"):
             normed = self.final_norm.deferred(x, self.head_in_dtype, rows=logit_rows)
         else:
             picked = torch.empty((n_logit_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device)

@@ -170,7 +170,7 @@ class Runner:
         meta_dev = meta_dev.view(3, n_rows)
         ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
                           row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0,
-                          upload=self._uploads.put)
+                          upload=self._uploads.put, every_row_wanted=logit_rows == list(range(n_rows)))
         logits = self._forward(ctx, rows_dev, len(logit_rows))
         self._uploads.end_step()
         for e in entries:
@@ -362,7 +362,7 @@ class _DecodeGraph:
     def _context(self, seg_slot, seg_pos0) -> StepContext:
         m, b = self.model, self.batch
         ctx = StepContext(n_rows=b, dtype=m.dtype, device=m.device, tokens=self.meta[0], row_pos=self.meta[1], row_slot=self.meta[2],
-                          seg_slot=list(seg_slot), seg_start=list(range(b)), seg_len=[1] * b, seg_pos0=list(seg_pos0))
+                          seg_slot=list(seg_slot), seg_start=list(range(b)), seg_len=[1] * b, seg_pos0=list(seg_pos0), every_row_wanted=True)
         ctx.memo["attention_plan"] = self.plan
         return ctx
 

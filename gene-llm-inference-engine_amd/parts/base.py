@@ -48,6 +48,7 @@ class StepContext:
     memo: Dict[Any, Any] = field(default_factory=dict)     # per-step tables shared by layers (rotary cos/sin)
     upload: Optional[Callable[..., Any]] = None    # the runner's way of bringing int32 step data to the device: upload(a) -> tensor, upload(a, b) -> (tensor, tensor) in one copy
     trace: Optional[Callable[[str, torch.Tensor], None]] = None        # debugging: a block reports (tag, residual stream [T, hidden]) after each of its two halves
+    every_row_wanted: bool = False           # the step's logits are asked for at every row, in the rows' order
 
     def to_device(self, *values):
         """int32 data made on the host for this step (row lists, tile lists) as device tensors, valid during the step:
