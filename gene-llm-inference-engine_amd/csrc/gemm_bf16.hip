@@ -753,6 +753,89 @@ __global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* 
     C[m * ldc + c] = f32_to_bf16(silu_gate(gate, up));
 }
 
+// The same for the q/k/v product of an attention layer, N = (n_heads + 2 n_kv) * hd columns: the sums of a row are its queries,
+// keys and values, and instead of writing them out for a kernel that rotates them and puts them into the cache, this one does
+// that itself: queries rotated into q_out, keys rotated and values as they are into the page table[slot][pos / page_size] at
+// place pos % page_size (pairs (i, i + hd/2): a' = a cos - b sin, b' = a sin + b cos; the page's layout as the attention
+// kernels read it: keys [kv_head][place][hd], then values [kv_head][hd][place]).  A thread has four neighbouring columns; the
+// other half of its pairs is with the thread hd/8 lanes away, in the same wave (hd a power of two from 8 to 256, and rows of a
+// multiple of 256 columns, so that a wave lies in one row and holds whole heads).
+struct RopeStore {
+    const float* cos_t;          // [M, hd/2], or null with sin_t: no rotation
+    const float* sin_t;
+    const int* pos;              // [M]
+    const int* slot;             // [M]
+    const int* table;
+    int table_stride;
+    bf16_t* q_out;               // [M, n_heads * hd]
+    bf16_t* cache;
+    long page_stride;
+    int page_size, n_heads, n_kv, hd;
+};
+
+__global__ __launch_bounds__(256) void skinny_reduce_rope_store_kernel(const float* __restrict__ P, int M, int N, int splits, NormIn norm_in, RopeStore rs) {
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4, slab = (size_t)M * N;
+    const bool live = i < slab;                              // (whole waves are live or not: 256 divides N)
+    const size_t row = live ? i / N : 0;
+    const int col = live ? (int)(i % N) : 0;
+    int p = 0, slot = 0;
+    if (live) {
+        p = rs.pos[row];
+        slot = rs.slot[row];
+    }
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int sp0 = 0; live && sp0 < splits; sp0 += 8) {
+        float4 part[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) part[u] = *reinterpret_cast<const float4*>(P + (size_t)min(sp0 + u, splits - 1) * slab + i);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (sp0 + u < splits) {
+                s[0] += part[u].x; s[1] += part[u].y; s[2] += part[u].z; s[3] += part[u].w;
+            }
+    }
+    if (live && norm_in.squares != nullptr) {
+        const float scale = row_scale_of(norm_in, (int)row);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) s[v] *= scale;
+    }
+    const int a_dim = rs.n_heads * rs.hd, kv_dim = rs.n_kv * rs.hd, half = rs.hd / 2;
+    const int which = col < a_dim ? 0 : col < a_dim + kv_dim ? 1 : 2;                        // queries, keys, values
+    const int c = which == 0 ? col : which == 1 ? col - a_dim : col - a_dim - kv_dim;        // the column among them
+    const int h = c / rs.hd, kk = c % rs.hd;
+    float out[4] = {s[0], s[1], s[2], s[3]};
+    if (rs.cos_t != nullptr) {                               // (every lane takes part in the exchange, whatever it holds)
+        float other[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) other[v] = __shfl_xor(s[v], half / 4, 64);
+        if (live && which != 2) {
+            const float4 cc = *reinterpret_cast<const float4*>(rs.cos_t + row * half + kk % half);
+            const float4 ss = *reinterpret_cast<const float4*>(rs.sin_t + row * half + kk % half);
+            const float cs[4] = {cc.x, cc.y, cc.z, cc.w}, sn[4] = {ss.x, ss.y, ss.z, ss.w};
+#pragma unroll
+            for (int v = 0; v < 4; ++v) out[v] = kk < half ? s[v] * cs[v] - other[v] * sn[v] : other[v] * sn[v] + s[v] * cs[v];
+        }
+    }
+    if (!live) return;
+    uint2 packed;
+    packed.x = (unsigned)f32_to_bf16(out[0]) | ((unsigned)f32_to_bf16(out[1]) << 16);
+    packed.y = (unsigned)f32_to_bf16(out[2]) | ((unsigned)f32_to_bf16(out[3]) << 16);
+    if (which == 0) {
+        *reinterpret_cast<uint2*>(rs.q_out + row * a_dim + c) = packed;
+        return;
+    }
+    const long page = rs.table[(size_t)slot * rs.table_stride + p / rs.page_size];
+    const int place = p % rs.page_size;
+    bf16_t* keys = rs.cache + page * rs.page_stride;
+    bf16_t* values = keys + (size_t)rs.n_kv * rs.page_size * rs.hd;
+    if (which == 1) {
+        *reinterpret_cast<uint2*>(keys + ((size_t)h * rs.page_size + place) * rs.hd + kk) = packed;
+    } else {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) values[((size_t)h * rs.hd + kk + v) * rs.page_size + place] = f32_to_bf16(out[v]);
+    }
+}
+
 // ------------------------------------------------------------------------------------------- slim
 // At most 16 rows of A.  Workgroup: 8 waves = STRIPS strips of ROWS weight rows x (8 / STRIPS)
 // slices of k; slice s takes the 128-wide blocks of k numbered s, s + slices, ...  Both operands go
@@ -1090,7 +1173,7 @@ static int launch_slim_tiles(const void* A, const void* W, void* C, int epi, int
 // Up to 128 rows the weights are the traffic and every workgroup streams its share of them once (measured on the decode step of
 // the Llama-3.2-1B shape: 72 rows took 2.69 ms through the tiles of 128 rows of the kernels for more rows, against 2.11 ms at 64 rows).
 static int launch_skinny(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, float* scratch,
-                         long scratch_floats, NormIn norm_in, NormOut norm_out, hipStream_t stream) {
+                         long scratch_floats, NormIn norm_in, NormOut norm_out, hipStream_t stream, const RopeStore* rope = nullptr) {
     const int splits = gi_gemm_bf16_skinny_splits(N, K), mt = (M + 15) / 16;
 #define SKINNY_MT(EPI_, PARTIAL_)                                                                                                   \
     do {                                                                                                                            \
@@ -1104,7 +1187,7 @@ static int launch_skinny(const void* A, const void* W, void* C, int epi, int M, 
     GI_REQUIRE(norm_in.squares == nullptr || norm_in.parts <= consumer_max_parts(M), "gemm_bf16: %d pieces of a sum of squares, at most %d for %d rows",
                norm_in.parts, consumer_max_parts(M), M);
     if (splits == 0) {                             // a wide output: every workgroup sees all of k and finishes its columns
-        GI_REQUIRE(norm_out.scaled == nullptr, "gemm_bf16: a product this wide does not hand a norm on");
+        GI_REQUIRE(norm_out.scaled == nullptr && rope == nullptr, "gemm_bf16: a product this wide does not hand a norm on, or its rows to the cache");
         const int k_per_split = K;
         dim3 grid((N + 63) / 64, 1);
         if (epi == EPI_GATED_BF16) SKINNY_MT(EPI_GATED_BF16, false); else if (epi == EPI_STORE_F32) SKINNY_MT(EPI_STORE_F32, false);
@@ -1120,6 +1203,11 @@ static int launch_skinny(const void* A, const void* W, void* C, int epi, int M, 
     SKINNY_MT(EPI_STORE_F32, true);
 #undef SKINNY_MT
     GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
+    if (rope != nullptr) {                         // the sums go where an attention layer wants its queries, keys and values
+        skinny_reduce_rope_store_kernel<<<(unsigned)(((size_t)M * N / 4 + 255) / 256), 256, 0, stream>>>(scratch, M, N, splits, norm_in, *rope);
+        GI_CHECK_LAUNCH("gemm_bf16 (reduce, rotate, store)");
+        return 0;
+    }
     return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream, norm_in, norm_out);
 }
 
@@ -1181,6 +1269,38 @@ GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dty
     }
     GI_REQUIRE(M <= SKINNY_MAX_ROWS, "gemm_bf16: no norm is handed on by or to a product of %d rows", M);
     return launch_skinny(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, norm_in, norm_out, stream);
+}
+
+// Whether gi_gemm_bf16_qkv_rope_store takes a q/k/v product of these sizes with heads of hd channels: the shapes whose k is shared out
+// over workgroups (17 or 33 to 128 rows), whose sums a second kernel adds up anyway.
+GI_API int gi_gemm_bf16_qkv_rope_store_takes(int M, int N, int K, int hd) {
+    return !takes_slim(M, N, K) && !takes_slim_tiles(M, N, K, EPI_STORE_F32) && M <= SKINNY_MAX_ROWS && gi_gemm_bf16_skinny_splits(N, K) > 0 &&
+           N % 256 == 0 && hd >= 8 && hd <= 256 && (hd & (hd - 1)) == 0 ? 1 : 0;
+}
+
+// The q/k/v product of an attention layer, A [M, K] x W [N, K]^T with N = (n_heads + 2 n_kv) * hd, whose results do not come back:
+// the queries go, rotated, to q_out [M, n_heads * hd] in bfloat16, the keys (rotated) and values into the pages of a bfloat16
+// cache, as gi_rope_store would put them (cos_t, sin_t [M, hd/2] or both null; pos, slot [M]; table, cache, page_stride, page_size
+// as there).  squares_in, parts_in, eps: a norm handed on, as for gi_gemm_bf16_handing (null: none).
+GI_API int gi_gemm_bf16_qkv_rope_store(const void* A, const void* W, int M, int N, int K, long lda, long ldw, float* scratch, long scratch_floats,
+                                       const float* squares_in, int parts_in, float eps, const float* cos_t, const float* sin_t, const int* pos,
+                                       const int* slot, const int* table, int table_stride, void* q_out, void* cache, long page_stride, int page_size,
+                                       int n_heads, int n_kv, int hd, hipStream_t stream) {
+    GI_REQUIRE(M > 0 && N > 0 && K > 0 && n_heads > 0 && n_kv > 0 && hd > 0 && N == (n_heads + 2 * n_kv) * hd,
+               "gemm_bf16 (q/k/v): M %d, N %d, K %d, %d heads, %d key/value heads of %d do not fit together", M, N, K, n_heads, n_kv, hd);
+    GI_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K, "gemm_bf16: K %d and the row strides (%ld, %ld) must be multiples of 8", K, lda, ldw);
+    GI_REQUIRE(((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0 && ((uintptr_t)scratch & 15) == 0, "gemm_bf16: operands must be 16-byte aligned");
+    GI_REQUIRE(gi_gemm_bf16_qkv_rope_store_takes(M, N, K, hd), "gemm_bf16 (q/k/v): sizes M %d, N %d, K %d, heads of %d are not taken", M, N, K, hd);
+    GI_REQUIRE((cos_t == nullptr) == (sin_t == nullptr) && ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0,
+               "gemm_bf16 (q/k/v): cos and sin must both be given or both be absent, 16-byte aligned");
+    GI_REQUIRE(pos != nullptr && slot != nullptr && table != nullptr && q_out != nullptr && cache != nullptr && page_size > 0 &&
+               page_stride >= 2L * n_kv * page_size * hd && ((uintptr_t)q_out & 7) == 0 && ((uintptr_t)cache & 7) == 0 && page_stride % 4 == 0,
+               "gemm_bf16 (q/k/v): positions, slots, a table, q_out and a cache with a page stride of at least 2*n_kv*page_size*hd are needed");
+    GI_REQUIRE(squares_in == nullptr || (parts_in > 0 && parts_in <= REDUCE_MAX_PARTS), "gemm_bf16 (q/k/v): %d pieces of a sum of squares, at most %d", parts_in,
+               REDUCE_MAX_PARTS);
+    const RopeStore rope = {cos_t, sin_t, pos, slot, table, table_stride, (bf16_t*)q_out, (bf16_t*)cache, page_stride, page_size, n_heads, n_kv, hd};
+    return launch_skinny(A, W, nullptr, EPI_STORE_F32, M, N, K, lda, ldw, (long)N, scratch, scratch_floats, NormIn{squares_in, parts_in, eps, K}, NO_NORM_OUT,
+                         stream, &rope);
 }
 
 // `gated` != 0: W is [gate; up] interleaved in groups of 16 rows (N rows in all, a multiple of 32)

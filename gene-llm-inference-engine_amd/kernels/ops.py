@@ -44,6 +44,8 @@ _SIGNATURES = {
     "gi_probe_mfma": [c_int, c_void_p, c_int, c_void_p],
     "gi_gemm_bf16_handing": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long,
                              c_void_p, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p, c_void_p],
+    "gi_gemm_bf16_qkv_rope_store": [c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p,
+                                    c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p],
     "gi_argmax": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_temperature": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gi_sample_filtered": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
@@ -72,6 +74,8 @@ def lib():
         l.gi_gemm_bf16_norm_parts.restype = c_int
         l.gi_gemm_bf16_takes_norm.argtypes = [c_int, c_int, c_int, c_int]
         l.gi_gemm_bf16_takes_norm.restype = c_int
+        l.gi_gemm_bf16_qkv_rope_store_takes.argtypes = [c_int, c_int, c_int, c_int]
+        l.gi_gemm_bf16_qkv_rope_store_takes.restype = c_int
         l.gi_probe_mfma_flops.argtypes = [c_int, c_int]
         l.gi_probe_mfma_flops.restype = c_long
         _lib = l
@@ -91,7 +95,7 @@ def _call(name, *args):
         raise KernelError(lib().gi_last_error().decode())
 
 
-_PROFILE_LABEL = {"gi_gemm_bf16_handing": "gemm_bf16"}        # the same products, with a norm's share on top
+_PROFILE_LABEL = {"gi_gemm_bf16_handing": "gemm_bf16", "gi_gemm_bf16_qkv_rope_store": "gemm_bf16"}        # the same products, with a norm's share on top
 
 
 class KernelProfile:
@@ -616,6 +620,43 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=N
     _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, 1 if gated else 0,
           m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _stream())
     return out
+
+
+def gemm_bf16_qkv_rope_store_takes(m, n, k, hd) -> bool:
+    """Whether `gemm_bf16_qkv_rope_store` takes a q/k/v product of m rows, n = (heads + 2 kv heads) * hd columns and k."""
+    return bool(lib().gi_gemm_bf16_qkv_rope_store_takes(m, n, k, hd))
+
+
+def gemm_bf16_qkv_rope_store(a, w, cos, sin, positions, slots, table, q_out, cache, n_heads, n_kv, hd, norm_in=None):
+    """The q/k/v product a @ w.T of an attention layer whose results do not come back: the queries go, rotated, into q_out
+    (bfloat16 [m, heads*hd]), the keys (rotated) and the values into the cache's pages, as `rope_store` puts them.
+    cos, sin: float32 [m, hd/2] or None; norm_in as for `gemm_bf16`."""
+    _dev(a, w, cos, sin, positions, slots, table, q_out, cache)
+    m, k = a.shape
+    n = w.shape[0]
+    if not (gemm_bf16_supports(a, w, q_out) and w.shape == (n, k) and n == (n_heads + 2 * n_kv) * hd and gemm_bf16_qkv_rope_store_takes(m, n, k, hd)):
+        raise KernelError(f"gemm (q/k/v): a product of {m} x {n} x {k} with heads of {hd} is not taken")
+    if not (q_out.dtype == torch.bfloat16 and q_out.shape == (m, n_heads * hd) and q_out.is_contiguous() and cache.dtype == torch.bfloat16):
+        raise KernelError("gemm (q/k/v): q_out must be bfloat16 [m, heads*hd], contiguous, and the cache bfloat16")
+    if cos is not None:
+        for t in (cos, sin):
+            if not (t.dtype == torch.float32 and t.shape == (m, hd // 2) and t.is_contiguous()):
+                raise KernelError("gemm (q/k/v): cos/sin must be float32 [m, hd/2]")
+    page_size = cache.shape[3]
+    _check_cache(cache, table, page_size, n_kv, hd, "gemm (q/k/v)")
+    _i32(positions, "gemm (q/k/v): positions", m)
+    _i32(slots, "gemm (q/k/v): slots", m)
+    squares_in, eps = norm_in if norm_in is not None else (None, 0.0)
+    if squares_in is not None and not (squares_in.dtype == torch.float32 and squares_in.is_contiguous() and squares_in.dim() == 2 and squares_in.shape[0] == m):
+        raise KernelError("gemm: the pieces of the sums of squares must be float32 [m, pieces]")
+    n_scratch = lib().gi_gemm_bf16_scratch_floats(m, n, k)
+    scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device)
+    if _profile is not None:
+        _profile.note = (f"{n}x{k}", n * k * w.element_size())
+    _call("gi_gemm_bf16_qkv_rope_store", a.data_ptr(), w.data_ptr(), m, n, k, a.stride(0), w.stride(0), scratch.data_ptr(), n_scratch,
+          _ptr(squares_in), squares_in.shape[1] if squares_in is not None else 0, float(eps), _ptr(cos), _ptr(sin), positions.data_ptr(),
+          slots.data_ptr(), table.data_ptr(), table.stride(0), q_out.data_ptr(), cache.data_ptr(), cache.stride(0), page_size, n_heads, n_kv, hd, _stream())
+    return q_out
 
 
 def interleave_gate_up(gate, up):

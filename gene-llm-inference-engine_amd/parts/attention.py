@@ -17,7 +17,7 @@ from ..cache.needs import PagedKvNeed
 from ..kernels import ops
 from ..weights.loader import TensorNeed
 from .base import Mixer, position_class, register_mixer
-from .linear import activation_dtype_for, linear, linear_onto
+from .linear import activation_dtype_for, linear, linear_onto, rows_for_product
 
 
 class Attention(Mixer):
@@ -55,6 +55,22 @@ class Attention(Mixer):
         tables = self.position.half_split_tables(ctx) if self.position is not None else None
         cos, sin = tables if tables is not None else (None, None)
         att = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
+        if (cache.writes and (tables is not None or self.position is None) and self.w_qkv.dtype == torch.bfloat16 and cache.kv.dtype == torch.bfloat16
+                and self.in_dtype == torch.bfloat16 and ops.gemm_bf16_qkv_rope_store_takes(T, self.w_qkv.shape[0], self.w_qkv.shape[1], s.head_dim)):
+            # some tens of rows: the product's second kernel, which adds up the shares of k, rotates and writes the pages itself
+            rows, norm_in = rows_for_product(h, self.w_qkv)
+            if norm_in is not None and norm_in[0].shape[1] > 8:          # (that kernel reads a norm's pieces one by one)
+                rows, norm_in = h.materialize(), None
+            if ops.gemm_bf16_supports(rows, self.w_qkv, att):
+                q_rot = torch.empty((T, self.a_dim), dtype=torch.bfloat16, device=ctx.device)
+                ops.gemm_bf16_qkv_rope_store(rows, self.w_qkv, cos, sin, ctx.row_pos, ctx.row_slot, cache.table, q_rot, cache.kv, s.n_heads, s.n_kv_heads,
+                                             s.head_dim, norm_in)
+                ops.attention(q_rot, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, s.window)
+                if att.dtype != self.att_dtype:
+                    att = att.to(self.att_dtype)
+                return linear_onto(att, self.w_o, residual, then)
+            if norm_in is None:
+                h = rows                  # (whole rows: what `linear` below would make of h)
         if cache.writes:
             qkv = torch.empty((T, self.a_dim + 2 * self.kv_dim), dtype=torch.float32, device=ctx.device)
             linear(h, self.w_qkv, qkv)

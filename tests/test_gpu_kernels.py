@@ -214,6 +214,53 @@ def test_norm_handed_from_one_product_to_the_next(m, d, k1, n2, gated):
     assert err_handed < 1.5 * err_usual + 1e-6, (err_handed, err_usual)
 
 
+@pytest.mark.parametrize("m,hidden,n_heads,n_kv,hd,page_size,rotate,handed", [(64, 2048, 32, 8, 64, 16, True, True), (40, 2048, 32, 8, 64, 16, True, False),
+                                                                              (128, 3072, 24, 8, 128, 16, True, True), (33, 512, 6, 1, 32, 8, False, False),
+                                                                              (17, 4096, 32, 8, 128, 32, True, False), (100, 1024, 2, 1, 256, 16, True, True)])
+def test_qkv_product_that_rotates_and_fills_the_pages(m, hidden, n_heads, n_kv, hd, page_size, rotate, handed):
+    """The q/k/v product whose second kernel rotates and writes the pages itself against the product followed by the kernel
+    that does that: the same queries and the same pages (the sums are added in the same order), also with a norm handed on."""
+    o = ops()
+    n = (n_heads + 2 * n_kv) * hd
+    assert o.gemm_bf16_qkv_rope_store_takes(m, n, hidden, hd)
+    a = randn(m, hidden, dtype=torch.bfloat16, seed=1)
+    w = randn(n, hidden, dtype=torch.bfloat16, seed=2, scale=0.05)
+    g = torch.Generator().manual_seed(9)
+    ang = torch.rand(m, hd // 2, generator=g) * 6.28
+    cos, sin = (torch.cos(ang).to(DEV), torch.sin(ang).to(DEV)) if rotate else (None, None)
+    n_slots, pages_per = 5, 4
+    n_pages = n_slots * pages_per + 2
+    table = torch.randperm(n_pages, generator=g)[:n_slots * pages_per].view(n_slots, pages_per).to(torch.int32).to(DEV)
+    slots = torch.randint(0, n_slots, (m,), generator=g).to(torch.int32)
+    positions = torch.empty(m, dtype=torch.int32)
+    seen = {}
+    for i in range(m):                                                # distinct (slot, position) per row
+        while True:
+            p = int(torch.randint(0, pages_per * page_size, (1,), generator=g))
+            if (int(slots[i]), p) not in seen:
+                seen[(int(slots[i]), p)] = True
+                positions[i] = p
+                break
+    slots, positions = slots.to(DEV), positions.to(DEV)
+    norm_in = None
+    if handed:
+        squares = (torch.rand(m, 2, generator=g) * hidden).to(DEV)
+        norm_in = (squares, 1e-5)
+    fill = lambda: torch.full((n_pages, 2, n_kv, page_size, hd), 7.0, dtype=torch.bfloat16, device=DEV)
+    want_cache, got_cache = fill(), fill()
+    qkv = torch.empty(m, n, device=DEV)
+    o.gemm_bf16(a, w, qkv, norm_in=norm_in)
+    a_dim, kv_dim = n_heads * hd, n_kv * hd
+    want_q = torch.empty(m, a_dim, dtype=torch.bfloat16, device=DEV)
+    o.rope_store(qkv[:, :a_dim], qkv[:, a_dim:a_dim + kv_dim], qkv[:, a_dim + kv_dim:], cos, sin, positions, slots, table, want_q, want_cache, n_heads, n_kv, hd)
+    got_q = torch.full((m, a_dim), float("nan"), dtype=torch.bfloat16, device=DEV)
+    o.gemm_bf16_qkv_rope_store(a, w, cos, sin, positions, slots, table, got_q, got_cache, n_heads, n_kv, hd, norm_in)
+    step = lambda t: t.float().abs().clamp_min(1e-3) * 2.0 ** -7          # a rounding step of bfloat16 at most: the two kernels may fuse a * cos - b * sin differently
+    assert ((got_q.float() - want_q.float()).abs() <= step(want_q)).all()
+    assert ((got_cache.float() - want_cache.float()).abs() <= step(want_cache)).all()
+    assert float((got_q.float() != want_q.float()).float().mean()) < 0.01 and float((got_cache.float() != want_cache.float()).float().mean()) < 0.01
+
+
 # -------------------------------------------------------------------------------------- sampling
 def test_argmax_lowest_index_on_ties():
     rows = [[1, 5, 5, 2], [3, 3, 3, 3], [-7, -8, -9, -10], [0, -1, 9, 9]]          # tests/verify_sampler.py:173-178
