@@ -295,6 +295,14 @@ class CacheManager:
     def open_requests(self):
         return list(self._slot)
 
+    def slots_and_lengths(self, requests: Sequence[Hashable]) -> Tuple[List[int], List[int]]:
+        """The slots and the lengths of the named requests, in their order (what a decode step asks of every request
+        of its batch, in one call); `CacheError` names the first request that is not open."""
+        try:
+            return [self._slot[r] for r in requests], [self._length[r] for r in requests]
+        except KeyError as err:
+            raise CacheError(f"request {err.args[0]!r} is not open") from None
+
     @property
     def free_slots(self) -> int:
         return len(self._free_slots)

@@ -9,13 +9,13 @@ tie_word_embeddings (false).
 from __future__ import annotations
 
 import json
+import math
 from dataclasses import dataclass, asdict
 from typing import Optional
 
 from .errors import ConfigError
 from .registry import register_architecture
-from .spec import (AttentionSpec, LayerSpec, Llama3Scaling, ModelSpec, RmsNormSpec, RotarySpec,
-                   RunEntry, SwiGluSpec)
+from .spec import AttentionSpec, LayerSpec, ModelSpec, RmsNormSpec, RotarySpec, RunEntry, SwiGluSpec
 
 
 _MAX_INT = 100_000_000   # src/loader/hf_checkpoint.cpp:31
@@ -49,6 +49,34 @@ def _optional_number(cfg, key, fallback):
     if isinstance(v, bool) or not isinstance(v, (int, float)):
         raise ConfigError(f"config.json: '{key}' is not a number")
     return float(v)
+
+
+@dataclass(frozen=True)
+class Llama3Scaling:
+    """Per-frequency stretch of rotary frequencies (reference: src/common/rope_style.h:13-19)."""
+    factor: float
+    low_freq_factor: float
+    high_freq_factor: float
+    original_max_position_embeddings: int
+
+
+def rotary_frequencies(head_dim: int, theta: float, scaling: Optional[Llama3Scaling] = None):
+    """f_k = theta^(-2k/head_dim) in 64-bit, and with scaling the reference's rule per frequency
+    (src/kernels/kernels.cpp:142-158): a wavelength 2*pi/f above original/low_freq_factor divides f by `factor`, one
+    below original/high_freq_factor leaves it, and between the two f is blended."""
+    out = []
+    for k in range(head_dim // 2):
+        f = 1.0 / math.pow(float(theta), 2.0 * k / head_dim)
+        if scaling is not None:
+            wavelength = 6.283185307179586476925 / f
+            original = float(scaling.original_max_position_embeddings)
+            if wavelength > original / scaling.low_freq_factor:
+                f /= scaling.factor
+            elif not wavelength < original / scaling.high_freq_factor:
+                smooth = (original / wavelength - scaling.low_freq_factor) / (scaling.high_freq_factor - scaling.low_freq_factor)
+                f = (1.0 - smooth) * f / scaling.factor + smooth * f
+        out.append(f)
+    return tuple(out)
 
 
 def _parse_rope_scaling(s) -> Optional[Llama3Scaling]:
@@ -169,7 +197,8 @@ class LlamaConfig:
         """The decoder as parts: per layer pre-norm attention with rotary positions and a SwiGLU
         feed-forward, tensor names as a Hugging Face Llama folder stores them
         (src/loader/hf_checkpoint.cpp:214-235)."""
-        rotary = RotarySpec(self.head_dim, self.rope_theta, self.rope_scaling)
+        rotary = RotarySpec(self.head_dim, self.rope_theta,
+                            None if self.rope_scaling is None else rotary_frequencies(self.head_dim, self.rope_theta, self.rope_scaling))
         layers = []
         for l in range(self.num_hidden_layers):
             p = f"model.layers.{l}."

@@ -16,21 +16,18 @@ from typing import Any, ClassVar, Optional, Tuple
 
 
 @dataclass(frozen=True)
-class Llama3Scaling:
-    """Per-frequency stretch of rotary frequencies (reference: src/common/rope_style.h:13-19)."""
-    factor: float
-    low_freq_factor: float
-    high_freq_factor: float
-    original_max_position_embeddings: int
-
-
-@dataclass(frozen=True)
 class RotarySpec:
-    """Rotation of the pairs (k, k + head_dim/2) of every head by pos * theta^(-2k/head_dim)."""
+    """Rotation of the pairs (k, k + head_dim/2) of every head by pos * f_k, with f_k = theta^(-2k/head_dim) unless the
+    architecture gives its own `frequencies` (head_dim/2 numbers: whatever rule stretches or blends them is the
+    architecture's, applied where it builds this spec)."""
     kind: ClassVar[str] = "rotary_half_split"
     head_dim: int
     theta: float
-    scaling: Optional[Llama3Scaling] = None
+    frequencies: Optional[Tuple[float, ...]] = None
+
+    def __post_init__(self):
+        if self.frequencies is not None and len(self.frequencies) != self.head_dim // 2:
+            raise ValueError(f"a rotation of heads of {self.head_dim} channels needs {self.head_dim // 2} frequencies, not {len(self.frequencies)}")
 
 
 @dataclass(frozen=True)

@@ -923,7 +923,7 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
     // first kernel's pairs of tiles are the better balance while they fit the chip in one round (a workgroup of 16 waves a compute
     // unit: 2,048 rows of 32 heads take 56 against 61 us) and where few tiles share their keys out; beyond one round its time
     // doubles at once and the wide kernel's many small workgroups win (2,560 rows: 68 against 100 us; 8,192: 360 against 572).
-    const bool one_round = (long)(paired ? n_tiles / 2 : n_tiles) * n_heads <= 256;
+    const bool one_round = (long)(paired ? n_tiles / 2 : n_tiles) * n_heads <= gi_compute_units();
     if (hd == 128 || (hd == 64 && n_splits == 1 && !one_round)) {
         GI_REQUIRE((long)n_tiles * n_splits <= 65535, "attention_prompt: %d tiles in %d splits are too many for one launch", n_tiles, n_splits);
         dim3 wgrid(n_heads, n_tiles * n_splits);

@@ -81,6 +81,8 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
 
 }  // namespace
 
+GI_API int gi_attention_exact_max_head_size() { return MAX_HD; }
+
 GI_API int gi_attention_exact(const void* q, int q_dtype, const void* cache, int cache_dtype, void* out, int out_dtype, const int* pos,
                               const int* slot, const int* table, int table_stride, long page_stride, int page_size, int n_rows,
                               int n_heads, int n_kv, int hd, int window, float scale, hipStream_t stream) {

@@ -17,6 +17,9 @@ typedef uint16_t bf16_t;   // storage of a bfloat16: the high half of a float
 // Records the message and returns -1 (defined in elementwise.hip).
 int gi_fail(const char* fmt, ...);
 
+// Compute units of the current device (defined in elementwise.hip).
+GI_API int gi_compute_units();
+
 #define GI_REQUIRE(cond, ...)                  \
     do {                                       \
         if (!(cond)) return gi_fail(__VA_ARGS__); \

@@ -18,6 +18,25 @@ int gi_fail(const char* fmt, ...) {
 
 GI_API const char* gi_last_error() { return g_error; }
 
+// Compute units of the current device, asked for once per device; where no device answers, those of an MI355X.  Dispatch
+// rules that speak of "one round of workgroups" or "three quarters of the chip" are stated in terms of this number.
+GI_API int gi_compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        (void)hipGetLastError();
+        return 256;
+    }
+    int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if (n > 0) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        n = 256;
+    }
+    __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+    return n;
+}
+
 GI_API int gi_device_arch(char* out, int cap) {
     hipDeviceProp_t p;
     int dev = 0;

@@ -1054,23 +1054,24 @@ int epilogue_of(int c_dtype, int accumulate) {
 // Number of k-splits of the skinny kernel for a product with 17..64 rows, so that the caller can size
 // the scratch (splits * M * N floats); 0: the output is wide enough to fill the chip without a split,
 // no scratch is needed.  Workgroups for three quarters of the chip or more, each with at least one block of k (measured at 33 to
-// 64 rows, product and reduce kernel together: 192 to 384 workgroups with two blocks of k each take 11 us for N = 3072, K = 2048 and
+// 64 rows, product and reduce kernel together: 192 to 384 workgroups on 256 compute units, with two blocks of k each, take 11 us for N = 3072, K = 2048 and
 // 16 us for N = 2048, K = 8192; twice the workgroups with one block each 12.5 and 17.5 us, half of them 13 and 22 us).
 GI_API int gi_gemm_bf16_skinny_splits(int N, int K) {
-    const int strips = (N + 63) / 64;
-    if (strips >= 192) return 0;
+    const int strips = (N + 63) / 64, most_of_the_chip = gi_compute_units() * 3 / 4;
+    if (strips >= most_of_the_chip) return 0;
     int splits = 1;
-    while (strips * splits < 192 && K / (splits * 2) >= KB) splits *= 2;
+    while (strips * splits < most_of_the_chip && K / (splits * 2) >= KB) splits *= 2;
     return splits;
 }
 
-// Splits of k for the LDS-ring kernel (more than 64 rows): with fewer than 192 tiles of 128 x 128 the tiles alone
+// Splits of k for the LDS-ring kernel (more than 64 rows): with fewer tiles of 128 x 128 than three quarters of the compute units the tiles alone
 // leave compute units idle and the weights stream too slowly; every share keeps at least 256 of k.
 GI_API int gi_gemm_bf16_piped_splits(int M, int N, int K) {
     if (M <= SKINNY_MAX_ROWS || K % PK != 0 || N < 128) return 1;
     const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+    const int most_of_the_chip = gi_compute_units() * 3 / 4;
     int splits = 1;
-    while (tiles * splits < 192 && K % (splits * 2 * PK) == 0 && K / (splits * 2) >= 256) splits *= 2;
+    while (tiles * splits < most_of_the_chip && K % (splits * 2 * PK) == 0 && K / (splits * 2) >= 256) splits *= 2;
     return splits;
 }
 

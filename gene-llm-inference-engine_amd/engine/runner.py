@@ -17,7 +17,7 @@ from typing import Hashable, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..cache import CacheManager
+from ..cache import CacheError, CacheManager
 from ..kernels import ops
 from ..parts import LayerCache, StepContext
 from .model import DecoderModel
@@ -62,9 +62,12 @@ class Runner:
     max_positions longest request; defaults to the model's limit
     use_graphs   replay decode steps (one token per request, all logits wanted) from captured HIP graphs,
                  if every part of the model allows it (`graph_safe`)
-    max_graphs   most captured graphs kept (one per batch size and bracket of the longest context); the one used
-                 longest ago goes when another is needed.  All graphs take their memory from one pool, so what they
-                 hold is what the largest of them needs (a pass's activations and its logits), not the sum.
+    max_graphs   most captured graphs kept (one per batch size and bracket of the longest context, at least two); the
+                 one used longest ago goes when another is needed.  All graphs take their memory from one pool, so what
+                 they hold is what the largest of them needs (a pass's activations and its logits), not the sum.
+
+    The logits a step returns are the caller's until the next step of this runner, of whatever batch size: captured
+    steps write theirs into the graphs' common pool, where the next step's activations may lie.
     """
 
     def __init__(self, model: DecoderModel, *, page_size: int = 16, max_tokens: int = 4096, max_requests: int = 8,
@@ -82,7 +85,7 @@ class Runner:
         self.rows_run = 0
         self.use_graphs = bool(use_graphs) and model.graph_safe
         self._graphs = {}
-        self.max_graphs = max(1, int(max_graphs))
+        self.max_graphs = max(2, int(max_graphs))       # (two at least: the graph that goes is then never the one replayed last, whose logits a step queued ahead may still be read from)
         self._graph_pool = None
         self._uploads = _StepUploads(model.device, min(8 * self.max_rows + 1024, 1 << 18))       # at most 1 MiB a buffer; what is larger is copied the ordinary way
 
@@ -222,10 +225,9 @@ class Runner:
         if len(set(requests)) != n:
             raise StepError("a request appears twice in one step")
         try:
-            slots = [cache._slot[r] for r in requests]
-        except KeyError as err:
-            raise StepError(f"request {err.args[0]!r} is not open") from None
-        lengths = [cache._length[r] for r in requests]
+            slots, lengths = cache.slots_and_lengths(requests)
+        except CacheError as err:
+            raise StepError(str(err)) from None
         tokens = [int(e.tokens[0]) for e in entries]
         vocab = self.model.spec.vocab_size
         if min(tokens) < 0 or max(tokens) >= vocab:

@@ -66,6 +66,8 @@ def lib():
         l.gi_argmax_chunks.restype = c_int
         l.gi_sample_filtered_histogram_bytes.argtypes = []
         l.gi_sample_filtered_histogram_bytes.restype = c_int
+        l.gi_attention_exact_max_head_size.argtypes = []
+        l.gi_attention_exact_max_head_size.restype = c_int
         l.gi_attention_bf16_supports.argtypes = [c_int, c_int, c_int]
         l.gi_attention_bf16_supports.restype = c_int
         l.gi_gemm_bf16_scratch_floats.argtypes = [c_int, c_int, c_int]
@@ -353,6 +355,12 @@ def gemm_exact(a, w, out, accumulate=False):
     _call("gi_gemm_exact", a.data_ptr(), _code(a, "gemm: a"), w.data_ptr(), _code(w, "gemm: w"), out.data_ptr(), _code(out, "gemm: out"),
           1 if accumulate else 0, m, n, k, a.stride(0), w.stride(0), out.stride(0), _stream())
     return out
+
+
+def attention_max_head_size() -> int:
+    """The largest head the attention kernels take (the exact kernel's limit; the matrix-core kernels take fewer sizes and
+    leave the others to it)."""
+    return lib().gi_attention_exact_max_head_size()
 
 
 def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None):

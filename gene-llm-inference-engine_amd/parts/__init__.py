@@ -4,7 +4,8 @@ from .base import (FeedForward, LayerCache, Mixer, Norm, Part, PositionEncoding,
                    register_mixer, register_norm, register_position_encoding, register_row_transform, row_transform_class,
                    weight_bytes, weight_tensors)
 from . import norm, rope, attention, mlp, block, transform          # registers the built-in kinds
-from .linear import linear
+from .linear import linear, linear_onto
+from .attention import qkv_rotate_store_attend
 from ..weights.loader import TensorNeed
 
 

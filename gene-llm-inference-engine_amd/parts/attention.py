@@ -20,6 +20,58 @@ from .base import Mixer, position_class, register_mixer
 from .linear import activation_dtype_for, linear, linear_onto, rows_for_product
 
 
+def qkv_rotate_store_attend(h, w_qkv, ctx, cache, *, n_heads, n_kv_heads, head_dim, position=None, window=None, in_dtype=None,
+                            before_rotation=None):
+    """The front half of an attention-like mixer, for any mixer to call: the product with the stacked matrix [q; k; v], the
+    position encoding on queries and keys, the new keys and values into the entry's pages, and every row's attention over its
+    request's pages up to its own position.  Returns the heads' outputs [rows, n_heads*head_dim] in the cache's dtype.
+
+    h                the mixer's input: rows, or a norm not yet (or half) applied, as `linear` takes it
+    position         a `PositionEncoding` or None; one with `half_split_tables` is applied by the kernels that store and attend
+    before_rotation  `f(q, k)`: changes the 32-bit products in place before the rotation (a norm or a scale per head; k is None
+                     where the pages are another entry's).  With it the products are always written out in 32-bit; the kernels
+                     that rotate, store and attend from them still serve.
+    Which kernels serve is decided here by storage and shape alone: for some tens of rows the product's second kernel rotates
+    and fills the pages itself; for a few decoded rows one kernel rotates, stores and attends; otherwise product, rotation +
+    store and attention are three launches."""
+    T, a_dim, kv_dim = ctx.n_rows, n_heads * head_dim, n_kv_heads * head_dim
+    in_dtype = in_dtype if in_dtype is not None else activation_dtype_for(w_qkv, ctx.dtype)
+    tables = position.half_split_tables(ctx) if position is not None else None
+    cos, sin = tables if tables is not None else (None, None)
+    att = torch.empty((T, a_dim), dtype=cache.kv.dtype, device=ctx.device)
+    if (before_rotation is None and cache.writes and (tables is not None or position is None) and w_qkv.dtype == torch.bfloat16
+            and cache.kv.dtype == torch.bfloat16 and in_dtype == torch.bfloat16
+            and ops.gemm_bf16_qkv_rope_store_takes(T, w_qkv.shape[0], w_qkv.shape[1], head_dim)):
+        # some tens of rows: the product's second kernel, which adds up the shares of k, rotates and writes the pages itself
+        rows, norm_in = rows_for_product(h, w_qkv)
+        if norm_in is not None and norm_in[0].shape[1] > 8:          # (that kernel reads a norm's pieces one by one)
+            rows, norm_in = h.materialize(), None
+        if ops.gemm_bf16_supports(rows, w_qkv, att):
+            q_rot = torch.empty((T, a_dim), dtype=torch.bfloat16, device=ctx.device)
+            ops.gemm_bf16_qkv_rope_store(rows, w_qkv, cos, sin, ctx.row_pos, ctx.row_slot, cache.table, q_rot, cache.kv, n_heads, n_kv_heads,
+                                         head_dim, norm_in)
+            return ops.attention(q_rot, cache.kv, att, ctx, cache.table, n_heads, n_kv_heads, head_dim, window)
+        if norm_in is None:
+            h = rows                  # (whole rows: what `linear` below would make of h)
+    if cache.writes:
+        qkv = torch.empty((T, a_dim + 2 * kv_dim), dtype=torch.float32, device=ctx.device)
+        linear(h, w_qkv, qkv)
+        q, k, v = qkv[:, :a_dim], qkv[:, a_dim:a_dim + kv_dim], qkv[:, a_dim + kv_dim:]
+    else:                       # the pages are another layer's: only the queries are made
+        q, k, v = torch.empty((T, a_dim), dtype=torch.float32, device=ctx.device), None, None
+        linear(h, w_qkv[:a_dim], q)
+    if before_rotation is not None:
+        before_rotation(q, k)
+    if position is not None and tables is None:          # an encoding with kernels of its own: q and k are turned in place
+        position.apply(q, k, ctx, n_heads, n_kv_heads, head_dim)
+    # a step of single decoded rows: one kernel rotates, writes the pages and attends
+    if not ops.attention_from_products(q, k, v, cos, sin, cache.kv, att, ctx, cache.table, n_heads, n_kv_heads, head_dim, window):
+        q_rot = torch.empty((T, a_dim), dtype=cache.kv.dtype, device=ctx.device)
+        ops.rope_store(q, k, v, cos, sin, ctx.row_pos, ctx.row_slot, cache.table, q_rot, cache.kv, n_heads, n_kv_heads, head_dim)
+        ops.attention(q_rot, cache.kv, att, ctx, cache.table, n_heads, n_kv_heads, head_dim, window)
+    return att
+
+
 class Attention(Mixer):
     accepts_deferred_norm = True      # its input goes into `linear` only
     hands_norm_on = True              # `forward` takes `then`, the norm that reads the residual next
@@ -29,6 +81,8 @@ class Attention(Mixer):
         s = spec
         if s.n_heads % s.n_kv_heads:
             raise ValueError("the number of heads must be a multiple of the number of key/value heads")
+        if not 0 < s.head_dim <= ops.attention_max_head_size():
+            raise ValueError(f"attention: head_dim = {s.head_dim} is outside what the attention kernels take (1 to {ops.attention_max_head_size()} channels a head)")
         self.a_dim, self.kv_dim = s.n_heads * s.head_dim, s.n_kv_heads * s.head_dim
         self.w_qkv = torch.cat([tensors[s.q_proj], tensors[s.k_proj], tensors[s.v_proj]], dim=0).contiguous()
         self.w_o = tensors[s.o_proj]
@@ -51,40 +105,9 @@ class Attention(Mixer):
         return self.in_dtype == torch.bfloat16 and ops.gemm_bf16_takes_norm(n_rows, self.w_qkv.shape[0], self.w_qkv.shape[1])
 
     def forward(self, h, residual, ctx, cache, then=None):
-        s, T = self.spec, ctx.n_rows
-        tables = self.position.half_split_tables(ctx) if self.position is not None else None
-        cos, sin = tables if tables is not None else (None, None)
-        att = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
-        if (cache.writes and (tables is not None or self.position is None) and self.w_qkv.dtype == torch.bfloat16 and cache.kv.dtype == torch.bfloat16
-                and self.in_dtype == torch.bfloat16 and ops.gemm_bf16_qkv_rope_store_takes(T, self.w_qkv.shape[0], self.w_qkv.shape[1], s.head_dim)):
-            # some tens of rows: the product's second kernel, which adds up the shares of k, rotates and writes the pages itself
-            rows, norm_in = rows_for_product(h, self.w_qkv)
-            if norm_in is not None and norm_in[0].shape[1] > 8:          # (that kernel reads a norm's pieces one by one)
-                rows, norm_in = h.materialize(), None
-            if ops.gemm_bf16_supports(rows, self.w_qkv, att):
-                q_rot = torch.empty((T, self.a_dim), dtype=torch.bfloat16, device=ctx.device)
-                ops.gemm_bf16_qkv_rope_store(rows, self.w_qkv, cos, sin, ctx.row_pos, ctx.row_slot, cache.table, q_rot, cache.kv, s.n_heads, s.n_kv_heads,
-                                             s.head_dim, norm_in)
-                ops.attention(q_rot, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, s.window)
-                if att.dtype != self.att_dtype:
-                    att = att.to(self.att_dtype)
-                return linear_onto(att, self.w_o, residual, then)
-            if norm_in is None:
-                h = rows                  # (whole rows: what `linear` below would make of h)
-        if cache.writes:
-            qkv = torch.empty((T, self.a_dim + 2 * self.kv_dim), dtype=torch.float32, device=ctx.device)
-            linear(h, self.w_qkv, qkv)
-            q, k, v = qkv[:, :self.a_dim], qkv[:, self.a_dim:self.a_dim + self.kv_dim], qkv[:, self.a_dim + self.kv_dim:]
-        else:                       # the pages are another layer's: only the queries are made
-            q, k, v = torch.empty((T, self.a_dim), dtype=torch.float32, device=ctx.device), None, None
-            linear(h, self.w_qkv[:self.a_dim], q)
-        if self.position is not None and tables is None:          # an encoding with kernels of its own: q and k are turned in place
-            self.position.apply(q, k, ctx, s.n_heads, s.n_kv_heads, s.head_dim)
-        # a step of single decoded rows: one kernel rotates, writes the pages and attends
-        if not ops.attention_from_products(q, k, v, cos, sin, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, s.window):
-            q_rot = torch.empty((T, self.a_dim), dtype=cache.kv.dtype, device=ctx.device)
-            ops.rope_store(q, k, v, cos, sin, ctx.row_pos, ctx.row_slot, cache.table, q_rot, cache.kv, s.n_heads, s.n_kv_heads, s.head_dim)
-            ops.attention(q_rot, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, s.window)
+        s = self.spec
+        att = qkv_rotate_store_attend(h, self.w_qkv, ctx, cache, n_heads=s.n_heads, n_kv_heads=s.n_kv_heads, head_dim=s.head_dim,
+                                      position=self.position, window=s.window, in_dtype=self.in_dtype)
         if att.dtype != self.att_dtype:
             att = att.to(self.att_dtype)
         return linear_onto(att, self.w_o, residual, then)

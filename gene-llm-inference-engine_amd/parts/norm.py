@@ -49,7 +49,9 @@ class RmsNorm(Norm):
         super().__init__(spec, tensors, dtype, device)
         self.weight = tensors[spec.weight]
         self.eps = float(spec.eps)
-        self._weight_f32 = None
+        # the weights once more in 32-bit, for a product that applies them to rows it has just written (`handed_weight`); made
+        # here, not at first use, which might fall into the capture of a graph
+        self._handed_weight = self.weight if self.weight.dtype == torch.float32 else self.weight.float().contiguous()
 
     @classmethod
     def tensor_needs(cls, spec):
@@ -68,9 +70,12 @@ class RmsNorm(Norm):
 
     def handed_weight(self) -> torch.Tensor:
         """The weights in 32-bit, for a product that applies them to the rows it has just written."""
-        if self._weight_f32 is None:
-            self._weight_f32 = self.weight.float().contiguous()
-        return self._weight_f32
+        return self._handed_weight
+
+    def weights_read_per_step(self):
+        """One copy of the weights: a step reads them as stored (the norm's kernel) or in 32-bit (a product that does the
+        norm's share), never both."""
+        return [self.weight]
 
 
 register_norm("rmsnorm", RmsNorm)

@@ -1,11 +1,10 @@
-"""Rotary position encoding with half-split pairs and the optional llama3 change of frequencies.
+"""Rotary position encoding with half-split pairs.
 
-Frequencies are computed once, in 64-bit on the host, as the reference computes them per
-frequency (src/kernels/kernels.cpp:142-158): f_k = theta^(-2k/head_dim); with scaling, a
-wavelength 2*pi/f above original/low_freq_factor divides f by `factor`, one below
-original/high_freq_factor leaves it, and between the two f is blended.  Per step, cos and sin
-of pos*f_k are made on the device from 64-bit angles for the step's rows and shared by every
-layer with the same spec."""
+Frequencies are computed once, in 64-bit on the host, as the reference computes them
+(src/kernels/kernels.cpp:142-147): f_k = theta^(-2k/head_dim), unless the spec brings the
+frequencies an architecture's own rule has made of them.  Per step, cos and sin of pos*f_k are
+made on the device from 64-bit angles for the step's rows and shared by every layer with the
+same spec."""
 from __future__ import annotations
 
 import math
@@ -15,23 +14,8 @@ import torch
 from ..kernels import ops
 from .base import PositionEncoding, register_position_encoding
 
-_TWO_PI = 6.283185307179586476925
-
-
-def inverse_frequencies(head_dim: int, theta: float, scaling=None):
-    out = []
-    for k in range(head_dim // 2):
-        f = 1.0 / math.pow(float(theta), 2.0 * k / head_dim)
-        if scaling is not None:
-            wavelength = _TWO_PI / f
-            original = float(scaling.original_max_position_embeddings)
-            if wavelength > original / scaling.low_freq_factor:
-                f /= scaling.factor
-            elif not wavelength < original / scaling.high_freq_factor:
-                smooth = (original / wavelength - scaling.low_freq_factor) / (scaling.high_freq_factor - scaling.low_freq_factor)
-                f = (1.0 - smooth) * f / scaling.factor + smooth * f
-        out.append(f)
-    return out
+def inverse_frequencies(head_dim: int, theta: float):
+    return [1.0 / math.pow(float(theta), 2.0 * k / head_dim) for k in range(head_dim // 2)]
 
 
 class RotaryHalfSplit(PositionEncoding):
@@ -42,7 +26,8 @@ class RotaryHalfSplit(PositionEncoding):
         if spec.head_dim % 2:
             raise ValueError("rotary encoding needs an even head size")
         self.half = spec.head_dim // 2
-        self.inv_freq = torch.tensor(inverse_frequencies(spec.head_dim, spec.theta, spec.scaling), dtype=torch.float64, device=device)
+        frequencies = spec.frequencies if spec.frequencies is not None else inverse_frequencies(spec.head_dim, spec.theta)
+        self.inv_freq = torch.tensor(list(frequencies), dtype=torch.float64, device=device)
 
     def half_split_tables(self, ctx):
         """(cos, sin), float32 [T, head_dim/2], for the rows of this step."""

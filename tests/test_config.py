@@ -105,7 +105,11 @@ def test_model_spec_names_and_shapes():
     assert isinstance(spec, ModelSpec) and len(spec.layers) == 3 and spec.run_order == tuple(RunEntry(i) for i in range(3))
     m = spec.layers[1].mixer
     assert isinstance(m, AttentionSpec) and (m.n_heads, m.n_kv_heads, m.head_dim, m.window) == (3, 1, 32, None)
-    assert m.q_proj == "model.layers.1.self_attn.q_proj.weight" and m.position.scaling.factor == 4.0
+    assert m.q_proj == "model.layers.1.self_attn.q_proj.weight" and c.rope_scaling.factor == 4.0
+    # the neutral spec carries the frequencies the architecture's rule has made: the first as theta gives it, the last a quarter of it
+    f = m.position.frequencies
+    assert len(f) == 16 and f[0] == 1.0 and abs(f[-1] * 4.0 * 500000.0 ** (30 / 32) - 1.0) < 1e-12
+    assert parse_config(full_config(CONFIGS["A"])).model_spec().layers[0].mixer.position.frequencies is None
     assert spec.lm_head == "lm_head.weight" and spec.embedding == "model.embed_tokens.weight"
     tied = parse_config(full_config(CONFIGS["A"])).model_spec()
     assert tied.lm_head == tied.embedding and any("lm_head" in p for p in tied.ignorable_tensors)

@@ -236,19 +236,38 @@ def test_requests_with_an_equal_beginning_share_its_pages(folders, dtype):
     system = prompts_for(name, [70], seed=31)[0]
     tails = prompts_for(name, [5, 1, 12, 30], seed=32)
     prompts = [system + t for t in tails] + [system[:40], tails[3] + system]
-    def run(prefix_cache, max_tokens):
+    def run(prefix_cache, max_tokens, watch=False):
+        from geneinfer_amd.engine import Engine
+        from geneinfer_amd.sampling import sample_rows
         llm = gi.LLM(folders[name], dtype=dtype, page_size=16, max_tokens=max_tokens, max_running=3, max_rows=64)
-        eng = llm.engine(EngineConfig(max_running=3, step_rows=48, prefix_cache=prefix_cache))
+        seen = []                                                    # (sampler, logits row) of every draw, when watched (no step is then queued ahead)
+        def watching(logits, samplers):
+            seen.extend(zip(samplers, logits.cpu()))
+            return sample_rows(logits, samplers)
+        cfg = EngineConfig(max_running=3, step_rows=48, prefix_cache=prefix_cache)
+        eng = Engine(llm.runner, cfg, llm.end_tokens, sample=watching) if watch else llm.engine(cfg)
         ids = [eng.submit(EngineRequest(prompts[0], len(prompts[0]) + new - 1, SamplerConfig(0.0)))]
         eng.run_until_idle()                                         # the first one has finished when the others arrive
         ids += [eng.submit(EngineRequest(p, len(p) + new - 1, SamplerConfig(0.0))) for p in prompts[1:]]
         eng.run_until_idle()
         llm.runner.cache.check_consistency()
-        return llm, eng, [eng.result(j) for j in ids]
-    _, plain_eng, plain = run(False, 1024)
+        by_sampler = {}
+        for sampler, row in seen:
+            by_sampler.setdefault(id(sampler), []).append(row)
+        return llm, eng, [eng.result(j) for j in ids], [by_sampler.get(id(eng.jobs[j].sampler), []) for j in ids]
+    _, plain_eng, plain, _ = run(False, 1024)
     exact, rounded = PlainLlama(folders[name]), PlainLlama(folders[name], storage=torch.bfloat16)
-    for max_tokens in (1024, 192):                                   # roomy; and so tight that named pages must be given back
-        llm, eng, shared = run(True, max_tokens)
+
+    def compare(got, want, near, what):
+        if dtype == "float32":
+            worst = max(relative_error(row, want[key]) for key, row in got.items())
+            assert worst < 2e-5, (what, worst)
+        else:
+            assert_within_bfloat16_noise(got, want.__getitem__, near.__getitem__, what)
+
+    # roomy; so tight that named pages must be given back; and tight again with the logits of every draw watched
+    for max_tokens, watch in ((1024, False), (192, False), (192, True)):
+        llm, eng, shared, drawn_from = run(True, max_tokens, watch)
         assert eng.prefix is not None and eng.stats.prefix_hits >= 4 and eng.stats.prefix_tokens >= 3 * 64 + 32
         assert eng.stats.rows <= plain_eng.stats.rows - (3 * 64 + 32) + 64 * eng.stats.preemptions
         for a, b in zip(shared, plain):
@@ -258,13 +277,26 @@ def test_requests_with_an_equal_beginning_share_its_pages(folders, dtype):
         assert sum(r.cached_tokens for r in shared) == eng.stats.prefix_tokens
         if max_tokens == 192:
             assert eng.stats.evicted_pages > 0 or eng.stats.preemptions > 0
-            continue
+        if watch:
+            # Every token was drawn from the plain model's logits for the request's tokens so far, whichever pages were shared,
+            # given back and computed again on the way (a request fed again after a preemption draws its next new token only).
+            got, want, near = {}, {}, {}
+            for i, (r, rows) in enumerate(zip(shared, drawn_from)):
+                tokens = prompts[i] + r.generated_tokens
+                assert len(rows) == len(r.generated_tokens) == new
+                e, nr = exact.logits(tokens[:-1]), rounded.logits(tokens[:-1])
+                for k, row in enumerate(rows):
+                    at = len(prompts[i]) - 1 + k
+                    got[(i, k)], want[(i, k)], near[(i, k)] = row, e[at], nr[at]
+                    assert int(torch.argmax(row)) == r.generated_tokens[k]
+            compare(got, want, near, f"draws behind shared pages, pool of {max_tokens}")
         # What the shared pages hold, in either precision: every prompt again, opened on the pages the index still names for
         # it, the rest fed in one step; the logits behind the shared pages are the plain model's for the whole prompt.
-        runner, index, got, want, near = llm.runner, llm.runner.cache.prefix, {}, {}, {}
+        runner, index, got, want, near, found = llm.runner, llm.runner.cache.prefix, {}, {}, {}, 0
         for i, prompt in enumerate(prompts):
             pages = index.match(prompt, len(prompt) - 1)
-            if i != 5:
+            found += len(pages)
+            if i != 5 and max_tokens == 1024:
                 assert len(pages) >= (2 if i == 4 else 4)            # 70 equal tokens are four full pages of 16, 40 are two
             runner.open(("again", i), pages)
             held = runner.length(("again", i))
@@ -273,11 +305,9 @@ def test_requests_with_an_equal_beginning_share_its_pages(folders, dtype):
             e, r = exact.logits(prompt), rounded.logits(prompt)
             for k, row in enumerate(rows):
                 got[(i, held + k)], want[(i, held + k)], near[(i, held + k)] = row, e[held + k], r[held + k]
-        if dtype == "float32":
-            worst = max(relative_error(row, want[key]) for key, row in got.items())
-            assert worst < 2e-5, worst
-        else:
-            assert_within_bfloat16_noise(got, want.__getitem__, near.__getitem__, "rows behind shared pages")
+        assert found >= 4, "the index names no page of the prompts it has just served"
+        compare(got, want, near, f"rows behind shared pages, pool of {max_tokens}")
+        runner.cache.check_consistency()
 
 
 def test_scheduler_in_bfloat16_runs_mixed_batches(folders):

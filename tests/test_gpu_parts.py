@@ -47,8 +47,9 @@ def test_norm_part(dtype):
 
 def test_rotary_part_tables_are_shared_within_a_step():
     from geneinfer_amd.config import Llama3Scaling, RotarySpec
+    from geneinfer_amd.config.llama import rotary_frequencies
     from geneinfer_amd.parts import position_class
-    spec = RotarySpec(32, 500000.0, Llama3Scaling(4.0, 1.0, 4.0, 32))
+    spec = RotarySpec(32, 500000.0, rotary_frequencies(32, 500000.0, Llama3Scaling(4.0, 1.0, 4.0, 32)))
     part = position_class(spec)(spec, {}, torch.float32, DEV)
     ctx = step_context([(0, 35, 4), (1, 0, 1)], torch.float32)
     cos, sin = part.half_split_tables(ctx)
@@ -103,6 +104,66 @@ def test_attention_part_over_two_steps(dtype, window):
         v = store((hx @ wd["v"].T).reshape(T, KV, hd))
         want = store(causal_attention(q, k, v, window)).reshape(T, H * hd) @ wd["o"].T
         assert relative_error(torch.cat(got[r]), want) < (3e-6 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_mixer_of_ones_own_uses_the_attention_front_half_with_a_hook(dtype):
+    """An attention-like mixer defined here (it scales every query head and every key head by a number of its own before
+    the rotation, as a per-head norm would) calls `qkv_rotate_store_attend` with that hook and gets the framework's kernels
+    for product, rotation, page write and attention: a portion of 40 rows (tiles), then single rows (the kernel that
+    rotates, stores and attends from the 32-bit products), against the plain functions."""
+    from geneinfer_amd.cache import CacheManager, PagedKvNeed
+    from geneinfer_amd.config import RotarySpec
+    from geneinfer_amd.kernels import ops
+    from geneinfer_amd.parts import LayerCache, position_class, qkv_rotate_store_attend
+    D, H, KV, hd = 128, 4, 2, 64
+    q_scale, k_scale = [0.5, 1.5, -1.0, 2.0], [1.25, 0.75]
+    rot = RotarySpec(hd, 10000.0)
+    position = position_class(rot)(rot, {}, dtype, DEV)
+    w = {"q": randn(H * hd, D, seed=1, scale=0.2), "k": randn(KV * hd, D, seed=2, scale=0.2), "v": randn(KV * hd, D, seed=3, scale=0.2)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    w_qkv = torch.cat([w["q"], w["k"], w["v"]]).to(DEV).contiguous()
+    calls = []
+
+    def per_head(q, k):
+        calls.append((tuple(q.shape), None if k is None else tuple(k.shape)))
+        for h, c in enumerate(q_scale):
+            ops.scale_rows(q[:, h * hd:(h + 1) * hd], c)
+        for g, c in enumerate(k_scale):
+            ops.scale_rows(k[:, g * hd:(g + 1) * hd], c)
+
+    cache = CacheManager([PagedKvNeed(KV, hd, None)], [None], page_size=16, n_pages=4, max_requests=1, max_positions=64, dtype=dtype, device=DEV)
+    kv, table, _ = cache.kv(0)
+    T = 44
+    hs = randn(T, D, seed=5).to(dtype)
+    cache.open("a")
+    got, fed = [], 0
+    for n in (40, 1, 1, 2):
+        cache.reserve([("a", n)]); cache.sync()
+        ctx = step_context([(cache.slot("a"), fed, n)], dtype)
+        att = qkv_rotate_store_attend(hs[fed:fed + n].to(DEV), w_qkv, ctx, LayerCache(kv=kv, table=table, writes=True), n_heads=H, n_kv_heads=KV,
+                                      head_dim=hd, position=position, before_rotation=per_head)
+        got.append(att.float().cpu())
+        cache.advance("a", n)
+        fed += n
+    assert calls == [((n, H * hd), (n, KV * hd)) for n in (40, 1, 1, 2)]
+    inv = rope_inverse_frequencies(hd, 10000.0)
+    store = (lambda t: t.to(torch.bfloat16).double()) if dtype == torch.bfloat16 else (lambda t: t)
+    hx, wd = hs.double(), {k: v.double() for k, v in w.items()}
+    q = (hx @ wd["q"].T).reshape(T, H, hd) * torch.tensor(q_scale, dtype=torch.float64)[None, :, None]
+    k = (hx @ wd["k"].T).reshape(T, KV, hd) * torch.tensor(k_scale, dtype=torch.float64)[None, :, None]
+    q, k = store(rope_rotate(q, torch.arange(T), inv)), store(rope_rotate(k, torch.arange(T), inv))
+    want = causal_attention(q, k, store((hx @ wd["v"].T).reshape(T, KV, hd))).reshape(T, H * hd)
+    assert relative_error(torch.cat(got), want) < (3e-6 if dtype == torch.float32 else 1e-2)
+
+
+def test_attention_refuses_a_head_size_its_kernels_do_not_take():
+    from geneinfer_amd.config import AttentionSpec
+    from geneinfer_amd.parts import mixer_class
+    spec = AttentionSpec(64, 1, 1, 272, "q", "k", "v", "o")
+    w = {"q": torch.zeros(272, 64, device=DEV), "k": torch.zeros(272, 64, device=DEV), "v": torch.zeros(272, 64, device=DEV), "o": torch.zeros(64, 272, device=DEV)}
+    with pytest.raises(ValueError, match="head_dim = 272"):
+        mixer_class(spec)(spec, w, torch.float32, DEV)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

@@ -6,7 +6,13 @@ with split contexts) meet the plain model under every way of cutting the work, i
 compared at every 16th position and at the last of each request.  What tests/verify_forward.py:72-117 does for the
 reference at its sizes.  The layer shape of Llama 3.2 3B (hidden 3072, 24 query heads over 8 key/value heads of 128
 channels, one layer, a cut vocabulary) follows in bfloat16 under the cuts that differ most: whole prompts, and long
-portions beside single tokens with pages used again."""
+portions beside single tokens with pages used again.
+
+Then the steps that serve many requests at once: 72 requests decode together, one token each, and close in groups, so that
+steps of 72, 65, 64, 40, 24 and 17 rows run, each size three times (as it comes, captured, replayed), through the runner's
+captured graphs with their fill rows, against the plain model row by row; and the same prompts through the scheduler with 64
+running requests and steps queued ahead, against the single-request loop.  What tools/engine_check_main.cpp:179-211 does
+for the reference: every request through the engine gets what it gets alone."""
 import random
 
 import pytest
@@ -22,6 +28,9 @@ EVERY = 16
 PAGE = 16
 
 
+_PLAIN = {}                       # folder -> its plain model, kept for the tests that ask it about other requests
+
+
 def make_case(folder, sizes, seed):
     write_model(folder, sizes, seed=seed, dtype=torch.bfloat16, std=0.02)
     rng = random.Random(9)
@@ -34,6 +43,7 @@ def make_case(folder, sizes, seed):
         for dtype, model in (("float32", plain), ("bfloat16", rounded)):
             for p, row in zip(places, model.logits_at(toks, places)):
                 want[dtype][(rid, p)] = row
+    _PLAIN[str(folder)] = plain
     return folder, requests, want, {}
 
 
@@ -116,3 +126,143 @@ def test_llama_3b_layer_shape_in_bfloat16(case_3b, mode):
     assert set(got) == set(want["bfloat16"])
     mean_e, mean_n = assert_within_bfloat16_noise(got, want["float32"].__getitem__, want["bfloat16"].__getitem__, f"3B shape, {mode}")
     print(f"3B shape bfloat16 {mode}: mean error {mean_e:.2e} (rounding noise {mean_n:.2e}), {len(steps)} steps")
+
+
+# ------------------------------------------------------------------------------------------------ many requests decoding at once
+WIDE_SIZES = [72, 65, 64, 40, 24, 17]          # rows of the all-decode steps, in this order
+WIDE_STEPS_EACH = 3                            # a size runs as it comes, is captured at its second step, and replayed at its third
+
+
+def wide_requests(vocab, seed=12):
+    """72 requests: request i has a prompt of 20 to 60 tokens and then one given token for every step it lives through
+    (it closes when the step size falls to i or below)."""
+    rng = random.Random(seed)
+    requests, alive = {}, {}
+    for i in range(max(WIDE_SIZES)):
+        alive[f"w{i}"] = WIDE_STEPS_EACH * sum(1 for n in WIDE_SIZES if n > i)
+        requests[f"w{i}"] = [rng.randrange(vocab) for _ in range(rng.randint(20, 60) + alive[f"w{i}"])]
+    return requests, alive
+
+
+def wide_decode(model, requests, alive, use_graphs):
+    """Prompts in steps of eight requests (nothing wanted), then the all-decode steps.  Returns {(request, position): logits row},
+    and the runner."""
+    from geneinfer_amd.engine import Runner, StepEntry
+    ids = list(requests)
+    pool = sum(-(-len(requests[r]) // PAGE) * PAGE for r in ids)                      # every request's final length, in whole pages: nothing to spare
+    runner = Runner(model, page_size=PAGE, max_tokens=pool, max_requests=len(ids), max_rows=1024, use_graphs=use_graphs)
+    fed = {}
+    for first in range(0, len(ids), 8):
+        group = ids[first:first + 8]
+        for r in group:
+            runner.open(r)
+            fed[r] = len(requests[r]) - alive[r]
+        runner.step([StepEntry(r, requests[r][:fed[r]], ()) for r in group])
+    got = {}
+    for size in WIDE_SIZES:
+        for r in ids[size:]:
+            if runner.is_open(r):
+                assert fed[r] == len(requests[r])
+                runner.close(r)
+        live = ids[:size]
+        for _ in range(WIDE_STEPS_EACH):
+            logits = runner.step([StepEntry(r, [requests[r][fed[r]]], (0,)) for r in live]).cpu()
+            for r, row in zip(live, logits):
+                got[(r, fed[r])] = row
+                fed[r] += 1
+    for r in ids[:WIDE_SIZES[-1]]:
+        runner.close(r)
+    runner.cache.check_consistency()
+    assert runner.cache.free_pages() == [g.pool.n_pages for g in runner.cache.groups], "pages were not all given back"
+    return got, runner
+
+
+_WIDE_WANT = {}
+
+
+def wide_want(plain, requests, alive, storage=None):
+    key = (id(plain), storage)
+    if key not in _WIDE_WANT:
+        _WIDE_WANT[key] = _wide_want(plain, requests, alive, storage)
+    return _WIDE_WANT[key]
+
+
+def _wide_want(plain, requests, alive, storage):
+    model = plain if storage is None else plain.with_storage(storage)
+    want = {}
+    for r, toks in requests.items():
+        places = list(range(len(toks) - alive[r], len(toks)))
+        for p, row in zip(places, model.logits_at(toks, places)):
+            want[(r, p)] = row.float()
+    return want
+
+
+def assert_wide_graphs(runner):
+    """Which captured steps served the run: 72 rows (also for 65 requests, filled up), 64, 40, 24 and 20 (for 17)."""
+    sizes = sorted(batch for batch, _ in runner._graphs)
+    assert sizes == [20, 24, 40, 64, 72], f"captured batch sizes {sizes}"
+    for (batch, bracket), g in runner._graphs.items():
+        assert g.graph is not None and g.calls == WIDE_STEPS_EACH * (2 if batch == 72 else 1), f"the graph of {batch} rows was not captured and replayed"
+    return sizes
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_llama_1b_layer_shape_many_requests_decode_at_once(case, dtype):
+    folder, _, _, _ = case
+    requests, alive = wide_requests(LLAMA_1B_SHAPE["vocab_size"])
+    model = model_of(case, dtype)
+    got, runner = wide_decode(model, requests, alive, use_graphs=True)
+    sizes = assert_wide_graphs(runner)
+    exact = wide_want(_PLAIN[str(folder)], requests, alive)
+    assert set(got) == set(exact) and len(got) == WIDE_STEPS_EACH * sum(WIDE_SIZES)
+    if dtype == "float32":
+        worst = max(relative_error(row, exact[key]) for key, row in got.items())
+        assert worst < 2e-5, f"worst relative error {worst:.3e}"
+        plain_steps, other = wide_decode(model, requests, alive, use_graphs=False)
+        assert not other._graphs
+        for key, row in got.items():
+            assert torch.equal(row, plain_steps[key]), f"logits of {key} differ in bits between the captured steps and steps run as they are"
+        print(f"1B shape float32, steps of {WIDE_SIZES} rows through graphs of {sizes}: worst relative error {worst:.2e}")
+    else:
+        rounded = wide_want(_PLAIN[str(folder)], requests, alive, torch.bfloat16)
+        mean_e, mean_n = assert_within_bfloat16_noise(got, exact.__getitem__, rounded.__getitem__, "1B shape, many requests decoding")
+        print(f"1B shape bfloat16, steps of {WIDE_SIZES} rows through graphs of {sizes}: mean error {mean_e:.2e} (rounding noise {mean_n:.2e})")
+
+
+def test_llama_3b_layer_shape_many_requests_decode_at_once(case_3b):
+    folder, _, _, _ = case_3b
+    requests, alive = wide_requests(LLAMA_3B_SHAPE["vocab_size"])
+    got, runner = wide_decode(model_of(case_3b, "bfloat16"), requests, alive, use_graphs=True)
+    sizes = assert_wide_graphs(runner)
+    exact = wide_want(_PLAIN[str(folder)], requests, alive)
+    rounded = wide_want(_PLAIN[str(folder)], requests, alive, torch.bfloat16)
+    assert set(got) == set(exact)
+    mean_e, mean_n = assert_within_bfloat16_noise(got, exact.__getitem__, rounded.__getitem__, "3B shape, many requests decoding")
+    print(f"3B shape bfloat16, steps of {WIDE_SIZES} rows through graphs of {sizes}: mean error {mean_e:.2e} (rounding noise {mean_n:.2e})")
+
+
+def test_llama_1b_layer_shape_scheduler_with_64_running_requests(case):
+    """The 72 prompts through the scheduler, 64 running at a time, decode steps queued ahead of the host, graphs on: every
+    request ends with the tokens the single-request loop gives it, bit for bit in 32-bit.  Requests generate 6 to 24 tokens,
+    so the batch drains and the last eight are admitted as others finish."""
+    import geneinfer_amd as gi
+    from geneinfer_amd.engine import EngineConfig, EngineRequest
+    from geneinfer_amd.sampling import SamplerConfig
+    requests, alive = wide_requests(LLAMA_1B_SHAPE["vocab_size"])
+    rng = random.Random(3)
+    prompts = [toks[:len(toks) - alive[r]] for r, toks in requests.items()]
+    new = [rng.randint(6, 24) for _ in prompts]
+    llm = gi.LLM(model_of(case, "float32"), page_size=PAGE, max_tokens=64 * 96, max_running=64, max_rows=1024)
+    alone = [llm.generate(p, steps=len(p) + n - 1, temperature=0.0).generated_tokens for p, n in zip(prompts, new)]
+    assert [len(a) for a in alone] == new
+    eng = llm.engine(EngineConfig(max_running=64, step_rows=512))
+    ids = [eng.submit(EngineRequest(p, len(p) + n - 1, SamplerConfig(0.0))) for p, n in zip(prompts, new)]
+    flights = 0
+    while eng.step():
+        flights += eng._flight is not None
+    out = [eng.result(j) for j in ids]
+    assert all(r.finished and r.error == "" for r in out)
+    assert eng.stats.max_running_seen == 64 and flights > 10, "the scheduler did not run 64 requests with steps queued ahead"
+    assert any(batch >= 40 for batch, _ in llm.runner._graphs), f"captured batch sizes {sorted(llm.runner._graphs)}"
+    assert [r.generated_tokens for r in out] == alone
+    llm.runner.cache.check_consistency()

@@ -77,9 +77,10 @@ def test_llama3_frequencies_in_another_formulation(theta, factor, low, high, ori
 
 def test_the_engine_computes_the_same_frequencies():
     from geneinfer_amd.config import Llama3Scaling
+    from geneinfer_amd.config.llama import rotary_frequencies
     from geneinfer_amd.parts.rope import inverse_frequencies
     for theta, factor, low, high, original, hd in LLAMA3_CASES:
-        got = inverse_frequencies(hd, theta, Llama3Scaling(factor, low, high, original))
+        got = rotary_frequencies(hd, theta, Llama3Scaling(factor, low, high, original))
         want = rope_inverse_frequencies(hd, theta, dict(factor=factor, low_freq_factor=low, high_freq_factor=high,
                                                         original_max_position_embeddings=original))
         assert np.allclose(got, want.numpy(), rtol=1e-15)
