@@ -5,7 +5,9 @@
 // and 0 without; query head h uses key/value head h / (n_heads / n_kv).  Scores are scaled by
 // 1/sqrt(hd) after the dot product, softmax is taken with a running maximum over tiles of 64
 // keys, and the weighted sum of the values follows in position order
-// (src/model/transformer.cpp:228-255, src/gpu/device_kernels.inc:377-449).
+// (src/model/transformer.cpp:228-255, src/gpu/device_kernels.inc:377-449).  The softmax's
+// denominator is a 64-bit sum, as the reference's (src/kernels/kernels.cpp:95-100): a 32-bit
+// running sum over tens of thousands of keys loses digits that every output of the head then lacks.
 // The order of every sum depends on (pos, window, hd) only, so a row's result has the same bits
 // whatever else is in the batch and whichever pages hold its request.
 //
@@ -34,7 +36,8 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
     __syncthreads();
 
     const long v_plane = (long)n_kv * page_size * hd;   // from a page's keys to its values
-    float m = -INFINITY, l = 0.f;
+    float m = -INFINITY;
+    double l = 0.0;
     float acc[MAX_HD / 64] = {};
     for (int j0 = lo; j0 <= p_row; j0 += 64) {
         const int j = j0 + lane;
@@ -52,7 +55,7 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
         const float m_new = fmaxf(m, wave_max(s));
         const float p = valid ? expf(s - m_new) : 0.f;
         const float corr = expf(m - m_new);      // 0 at the first tile (m = -inf)
-        l = l * corr + wave_sum(p);
+        l = l * (double)corr + (double)wave_sum(p);
         m = m_new;
         __syncthreads();                         // the previous tile's p_s and v_off have been read
         p_s[lane] = p;
@@ -71,7 +74,7 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
             }
         }
     }
-    const float inv = 1.0f / l;
+    const float inv = 1.0f / (float)l;
 #pragma unroll
     for (int i = 0; i < MAX_HD / 64; ++i) {
         const int d = lane + 64 * i;

@@ -295,3 +295,35 @@ GI_API int gi_softcap_rows(float* x, int n_rows, int dim, long stride, float cap
     GI_CHECK_LAUNCH("softcap_rows");
     return 0;
 }
+
+// ------------------------------------------------------------------------------- random weights
+// out[i] = offset + scale * z_i with z_i a standard normal number that is a function of (key, i) alone, so that a model's random
+// weights can be re-made anywhere from the seed and the tensors' names (the key is made of both on the host):
+//   r  = mix(key + (i + 1) * 0x9E3779B97F4A7C15)      mix: the splitmix64 finaliser
+//   u1 = ((r >> 40) + 1) / 2^24  in (0, 1],  u2 = ((r >> 8) & 0xFFFFFF) / 2^24  in [0, 1)
+//   z  = sqrt(-2 ln u1) * cos(2 pi u2)                 in 64-bit; offset + scale * z is rounded to 32-bit, then to the storage type
+__device__ __forceinline__ uint64_t splitmix_finish(uint64_t z) {
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void random_normal_kernel(T* __restrict__ out, size_t n, uint64_t key, double offset, double scale) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const uint64_t r = splitmix_finish(key + (uint64_t)(i + 1) * 0x9E3779B97F4A7C15ull);
+        const double u1 = (double)((r >> 40) + 1) * (1.0 / 16777216.0), u2 = (double)((r >> 8) & 0xFFFFFFull) * (1.0 / 16777216.0);
+        const double z = sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925 * u2);
+        store_f32(out, i, (float)(offset + scale * z));
+    }
+}
+
+GI_API int gi_random_normal(void* out, int dtype, long n, unsigned long long key, double offset, double scale, hipStream_t stream) {
+    GI_REQUIRE(out != nullptr && n > 0, "random_normal: bad arguments (n %ld)", n);
+    const unsigned grid = (unsigned)min((n + 255) / 256, (long)gi_compute_units() * 16);
+    if (dtype == GI_F32) random_normal_kernel<float><<<grid, 256, 0, stream>>>((float*)out, (size_t)n, key, offset, scale);
+    else if (dtype == GI_BF16) random_normal_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, (size_t)n, key, offset, scale);
+    else return gi_fail("random_normal: unknown dtype %d", dtype);
+    GI_CHECK_LAUNCH("random_normal");
+    return 0;
+}

@@ -9,18 +9,21 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-// Every thread walks the buffer in strides of the grid, four 16-byte loads in flight; with `dst` it stores what it
-// read, without it folds it into one word per thread (so that the loads cannot be dropped).
+// Every thread walks the buffer in strides of the grid, U 16-byte loads in flight; with `dst` it stores what it read, without it
+// folds it into one word per thread (so that the loads cannot be dropped).
+template <int U>
 __global__ __launch_bounds__(256) void stream_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16, uint32_t* __restrict__ sink) {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     uint32_t fold = 0;
-    for (; i + 3 * stride < n16; i += 4 * stride) {
-        const uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
-        if (dst) {
-            dst[i] = a; dst[i + stride] = b; dst[i + 2 * stride] = c; dst[i + 3 * stride] = d;
-        } else {
-            fold ^= a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w ^ c.x ^ c.y ^ c.z ^ c.w ^ d.x ^ d.y ^ d.z ^ d.w;
+    for (; i + (U - 1) * stride < n16; i += U * stride) {
+        uint4 v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = src[i + u * stride];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (dst) dst[i + u * stride] = v[u];
+            else fold ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
         }
     }
     for (; i < n16; i += stride) {
@@ -57,12 +60,16 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, float* __rest
 }  // namespace
 
 // Streams `bytes` (a multiple of 16) from `src`, into `dst` if that is given (a copy: `bytes` read and as many written)
-// or nowhere (a read).  `sink` takes one word per thread of a read: n_blocks * 256 words.
-GI_API int gi_probe_stream(const void* src, void* dst, long bytes, void* sink, int n_blocks, hipStream_t stream) {
+// or nowhere (a read), with `in_flight` (4, 8 or 16) loads of 16 bytes a thread.  `sink` takes one word per thread of a read:
+// n_blocks * 256 words.
+GI_API int gi_probe_stream(const void* src, void* dst, long bytes, void* sink, int n_blocks, int in_flight, hipStream_t stream) {
     GI_REQUIRE(src != nullptr && bytes > 0 && bytes % 16 == 0 && n_blocks > 0, "probe_stream: bad arguments (bytes %ld, blocks %d)", bytes, n_blocks);
+    GI_REQUIRE(in_flight == 4 || in_flight == 8 || in_flight == 16, "probe_stream: %d loads in flight (4, 8 or 16)", in_flight);
     GI_REQUIRE(((uintptr_t)src & 15) == 0 && ((uintptr_t)dst & 15) == 0, "probe_stream: buffers must be 16-byte aligned");
     GI_REQUIRE(dst != nullptr || sink != nullptr, "probe_stream: a read needs a sink of n_blocks * 256 words");
-    stream_kernel<<<n_blocks, 256, 0, stream>>>((const uint4*)src, (uint4*)dst, (size_t)bytes / 16, (uint32_t*)sink);
+    if (in_flight == 4) stream_kernel<4><<<n_blocks, 256, 0, stream>>>((const uint4*)src, (uint4*)dst, (size_t)bytes / 16, (uint32_t*)sink);
+    else if (in_flight == 8) stream_kernel<8><<<n_blocks, 256, 0, stream>>>((const uint4*)src, (uint4*)dst, (size_t)bytes / 16, (uint32_t*)sink);
+    else stream_kernel<16><<<n_blocks, 256, 0, stream>>>((const uint4*)src, (uint4*)dst, (size_t)bytes / 16, (uint32_t*)sink);
     GI_CHECK_LAUNCH("probe_stream");
     return 0;
 }

@@ -128,18 +128,14 @@ def load_model(folder, dtype="bfloat16", device="cuda:0") -> DecoderModel:
 
 def random_model(config, seed: int, dtype="bfloat16", device="cuda:0", std: float = 0.02, draw_on_device: bool = False) -> DecoderModel:
     """A model of `config` with seeded random weights, without a folder in between.  With
-    `draw_on_device` the numbers come from the device's generator (fast for large models; other
-    numbers than the host generator gives for the same seed)."""
+    `draw_on_device` the numbers are made on the device by a formula of (seed, tensor name, element index)
+    (`weights.random_init`: fast for large models, and anybody can re-make them; other numbers than the
+    host generator gives for the same seed)."""
     dtype = compute_dtype(dtype)
     spec = config.model_spec()
     if draw_on_device:
-        from ..weights import merge_needs
-        gen = torch.Generator(device=device)
-        gen.manual_seed(int(seed))
-        tensors = {}
-        for name, need in merge_needs(model_tensor_needs(spec)).items():
-            t = torch.randn(need.shape, generator=gen, dtype=torch.float32, device=device)
-            tensors[name] = (1.0 + 0.1 * t if need.role == "norm" else std * t).to(dtype)
+        from ..weights import formula_tensors
+        tensors = formula_tensors(model_tensor_needs(spec), seed, dtype, std, device)
     else:
         host = random_tensors(model_tensor_needs(spec), seed, dtype, std)
         tensors = {k: v.to(device) for k, v in host.items()}

@@ -7,6 +7,7 @@ from __future__ import annotations
 import ctypes
 from ctypes import c_float, c_int, c_long, c_void_p
 
+from functools import lru_cache
 from typing import Optional
 
 import torch
@@ -40,7 +41,8 @@ _SIGNATURES = {
     "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
                                  c_float, c_int, c_int, c_void_p],
-    "gi_probe_stream": [c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p],
+    "gi_random_normal": [c_void_p, c_int, c_long, ctypes.c_ulonglong, ctypes.c_double, ctypes.c_double, c_void_p],
+    "gi_probe_stream": [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p],
     "gi_probe_mfma": [c_int, c_void_p, c_int, c_void_p],
     "gi_gemm_bf16_handing": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long,
                              c_void_p, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p, c_void_p],
@@ -78,6 +80,8 @@ def lib():
         l.gi_gemm_bf16_takes_norm.restype = c_int
         l.gi_gemm_bf16_qkv_rope_store_takes.argtypes = [c_int, c_int, c_int, c_int]
         l.gi_gemm_bf16_qkv_rope_store_takes.restype = c_int
+        l.gi_compute_units.argtypes = []
+        l.gi_compute_units.restype = c_int
         l.gi_probe_mfma_flops.argtypes = [c_int, c_int]
         l.gi_probe_mfma_flops.restype = c_long
         _lib = l
@@ -339,6 +343,16 @@ def softcap_rows(x, cap):
     return _rows_in_place("softcap_rows", x, cap)
 
 
+def random_normal(out, key: int, offset: float, scale: float):
+    """out[i] = offset + scale * z_i, z_i the standard normal number that (key, i) give (`weights.random_init` states the formula);
+    out is a contiguous float32 or bfloat16 tensor of any shape, filled in the order of its memory."""
+    _dev(out)
+    if not out.is_contiguous():
+        raise KernelError("random_normal: out must be contiguous")
+    _call("gi_random_normal", out.data_ptr(), _code(out, "random_normal: out"), out.numel(), int(key) & 0xFFFFFFFFFFFFFFFF, float(offset), float(scale), _stream())
+    return out
+
+
 def gemm_exact(a, w, out, accumulate=False):
     """out (=|+=) a @ w.T in 32-bit arithmetic with one summation order for every batch size."""
     _dev(a, w, out)
@@ -443,6 +457,7 @@ class AttentionPlan:
             self.decode_rows = rest[0] if rest else None
 
 
+@lru_cache(maxsize=None)
 def attention_bf16_supports(hd, page_size, prompt: bool) -> bool:
     return bool(lib().gi_attention_bf16_supports(hd, page_size, 1 if prompt else 0))
 
@@ -575,12 +590,21 @@ def gemm_bf16_supports(a, w, out) -> bool:
             and (out.dtype == torch.float32 or out.dtype == torch.bfloat16) and out.stride(1) == 1)
 
 
+# What the library says about a shape does not change while the process lives, and a step asks it some hundred times: the answers
+# are kept (a question costs a call through ctypes, about a microsecond of the host's time each).
+@lru_cache(maxsize=None)
+def _scratch_floats(m, n, k) -> int:
+    return lib().gi_gemm_bf16_scratch_floats(m, n, k)
+
+
+@lru_cache(maxsize=None)
 def gemm_bf16_norm_parts(m, n, k) -> int:
     """The pieces per row in which a product [m, k] x [n, k] that adds onto rows writes their sums of squares when it hands
     the next norm on (`gemm_bf16(..., norm_out=...)`); 0 if a product of these sizes cannot."""
     return lib().gi_gemm_bf16_norm_parts(m, n, k)
 
 
+@lru_cache(maxsize=None)
 def gemm_bf16_takes_norm(m, n, k, gated=False) -> bool:
     """Whether a product of these sizes can read rows whose norm was handed on (`gemm_bf16(..., norm_in=...)`) by a product
     of as many rows."""
@@ -604,7 +628,7 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=N
         raise KernelError(f"gemm: out is {tuple(out.shape)}, ({m}, {n // 2 if gated else n}) is needed")
     if not (checked or gemm_bf16_supports(a, w, out)):
         raise KernelError("gemm_bf16: operands must be bfloat16 with K and row strides multiples of 8, 16-byte aligned")
-    n_scratch = lib().gi_gemm_bf16_scratch_floats(m, n, k)           # partial sums where k is split over workgroups
+    n_scratch = _scratch_floats(m, n, k)                             # partial sums where k is split over workgroups
     scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device) if n_scratch else None
     if _profile is not None:
         _profile.note = (f"{n}x{k}{' gated' if gated else ''}", n * k * w.element_size())
@@ -630,6 +654,7 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=N
     return out
 
 
+@lru_cache(maxsize=None)
 def gemm_bf16_qkv_rope_store_takes(m, n, k, hd) -> bool:
     """Whether `gemm_bf16_qkv_rope_store` takes a q/k/v product of m rows, n = (heads + 2 kv heads) * hd columns and k."""
     return bool(lib().gi_gemm_bf16_qkv_rope_store_takes(m, n, k, hd))
@@ -657,7 +682,7 @@ def gemm_bf16_qkv_rope_store(a, w, cos, sin, positions, slots, table, q_out, cac
     squares_in, eps = norm_in if norm_in is not None else (None, 0.0)
     if squares_in is not None and not (squares_in.dtype == torch.float32 and squares_in.is_contiguous() and squares_in.dim() == 2 and squares_in.shape[0] == m):
         raise KernelError("gemm: the pieces of the sums of squares must be float32 [m, pieces]")
-    n_scratch = lib().gi_gemm_bf16_scratch_floats(m, n, k)
+    n_scratch = _scratch_floats(m, n, k)
     scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device)
     if _profile is not None:
         _profile.note = (f"{n}x{k}", n * k * w.element_size())
@@ -742,15 +767,24 @@ def _timed_ms(launch, repeats):
     return sorted(times)[len(times) // 2]
 
 
-def measured_read_bandwidth(device="cuda:0", n_bytes: int = 2 << 30, repeats: int = 5, copy: bool = False) -> float:
+# (workgroups of 256 threads per compute unit, loads of 16 bytes in flight per thread) of the plain read.  On an MI355X few
+# waves with many loads each read fastest (measured over 1 to 64 workgroups a unit and 4, 8, 16 loads: 6.3 TB/s with one
+# workgroup and 8 loads, 6.2 with two and 4; 5.3 to 5.8 with 4 to 16 workgroups; 6.0 with 32 and 64); a copy reaches 5.1 to 5.3.
+STREAM_SHAPES = ((1, 8), (2, 4), (1, 16), (64, 4))
+
+
+def measured_read_bandwidth(device="cuda:0", n_bytes: int = 2 << 30, repeats: int = 5, copy: bool = False, shapes=STREAM_SHAPES) -> float:
     """GB/s at which a plain kernel of this library reads `n_bytes` of device memory (much more than the caches hold);
-    with `copy`, reads and writes them (bytes moved = 2 * n_bytes)."""
+    with `copy`, reads and writes them (bytes moved = 2 * n_bytes): the best of a few shapes of the kernel (`STREAM_SHAPES`)."""
     src = torch.empty(n_bytes // 4, dtype=torch.int32, device=device).fill_(1)
     dst = torch.empty_like(src) if copy else None
-    n_blocks = 256 * 16
-    sink = torch.empty(n_blocks * 256, dtype=torch.int32, device=device)
-    ms = _timed_ms(lambda: _call("gi_probe_stream", src.data_ptr(), _ptr(dst), n_bytes, sink.data_ptr(), n_blocks, _stream()), repeats)
-    return (2 if copy else 1) * n_bytes / (ms * 1e-3) / 1e9
+    best = 0.0
+    for blocks_per_unit, in_flight in shapes:
+        n_blocks = lib().gi_compute_units() * blocks_per_unit
+        sink = torch.empty(n_blocks * 256, dtype=torch.int32, device=device)
+        ms = _timed_ms(lambda: _call("gi_probe_stream", src.data_ptr(), _ptr(dst), n_bytes, sink.data_ptr(), n_blocks, in_flight, _stream()), repeats)
+        best = max(best, (2 if copy else 1) * n_bytes / (ms * 1e-3) / 1e9)
+    return best
 
 
 def measured_mfma_rate(device="cuda:0", iters: int = 20000, repeats: int = 5) -> float:

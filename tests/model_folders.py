@@ -83,6 +83,35 @@ def random_weights(cfg: dict, seed: int, std: float = 0.2):
     return w
 
 
+def formula_weights(cfg: dict, seed: int, std: float = 0.02):
+    """The weights that the engine draws on the device for `seed` (`random_model(..., draw_on_device=True)`), re-made here from the
+    formula its documentation states, in this file's own words: key = fnv1a64(name) + (seed + 1) * golden; element i (row-major)
+    takes r = splitmix64's finaliser of key + (i + 1) * golden, u1 = ((r >> 40) + 1) / 2^24, u2 = ((r >> 8) & 0xFFFFFF) / 2^24,
+    z = sqrt(-2 ln u1) cos(2 pi u2) in 64-bit; matrices std * z, norm weights 1 + 0.1 z, rounded to 32-bit."""
+    golden, mask = 0x9E3779B97F4A7C15, (1 << 64) - 1
+    out = {}
+    for name, shape in tensor_layout(cfg):
+        key = 0xCBF29CE484222325
+        for byte in name.encode():
+            key = ((key ^ byte) * 0x100000001B3) & mask
+        key = (key + (seed + 1) * golden) & mask
+        n = int(np.prod(shape))
+        values = np.empty(n, dtype=np.float32)
+        offset, scale = (1.0, 0.1) if name.endswith("norm.weight") else (0.0, std)
+        with np.errstate(over="ignore"):
+            for start in range(0, n, 1 << 24):
+                i = np.arange(start + 1, min(n, start + (1 << 24)) + 1, dtype=np.uint64)
+                z = np.uint64(key) + i * np.uint64(golden)
+                z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+                z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+                z = z ^ (z >> np.uint64(31))
+                u1 = ((z >> np.uint64(40)).astype(np.float64) + 1.0) / 2.0 ** 24
+                u2 = ((z >> np.uint64(8)) & np.uint64(0xFFFFFF)).astype(np.float64) / 2.0 ** 24
+                values[start:start + len(i)] = (offset + scale * (np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * np.pi * u2))).astype(np.float32)
+        out[name] = torch.from_numpy(values).reshape(shape)
+    return out
+
+
 _NAMES = {torch.float32: "F32", torch.bfloat16: "BF16", torch.float16: "F16", torch.int32: "I32", torch.int64: "I64", torch.float64: "F64"}
 
 

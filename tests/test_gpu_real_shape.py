@@ -19,7 +19,8 @@ import pytest
 import torch
 
 import traces
-from model_folders import LLAMA_1B_SHAPE, LLAMA_3B_SHAPE, assert_within_bfloat16_noise, relative_error, write_model
+from model_folders import (LLAMA_1B_SHAPE, LLAMA_3B_SHAPE, assert_within_bfloat16_noise, formula_weights, full_config, relative_error,
+                           write_model)
 from plain_llama import PlainLlama
 
 pytestmark = pytest.mark.gpu
@@ -266,3 +267,33 @@ def test_llama_1b_layer_shape_scheduler_with_64_running_requests(case):
     assert any(batch >= 40 for batch, _ in llm.runner._graphs), f"captured batch sizes {sorted(llm.runner._graphs)}"
     assert [r.generated_tokens for r in out] == alone
     llm.runner.cache.check_consistency()
+
+
+def test_the_weights_the_benchmark_draws_can_be_remade_and_give_the_plain_logits(tmp_path):
+    """`random_model(..., draw_on_device=True)`, what bench.py runs, at the 1B layer shape: the tensors on the device are, bit for
+    bit, the ones this suite re-makes from the stated formula, and the model's bfloat16 logits for a prompt and decoded tokens
+    are the plain model's on the re-made weights."""
+    from geneinfer_amd.config import LlamaConfig
+    from geneinfer_amd.engine import Runner, StepEntry, random_model
+    sizes = dict(LLAMA_1B_SHAPE, num_hidden_layers=1)
+    model = random_model(LlamaConfig.from_dict(sizes), seed=5, dtype="bfloat16", device="cuda:0", draw_on_device=True)
+    remade = formula_weights(full_config(sizes), seed=5, std=0.02)
+    assert torch.equal(model.embedding.cpu(), remade["model.embed_tokens.weight"].to(torch.bfloat16))
+    layer = model.layers[0]
+    assert torch.equal(layer.mixer.w_o.cpu(), remade["model.layers.0.self_attn.o_proj.weight"].to(torch.bfloat16))
+    assert torch.equal(layer.mixer_norm.weight.cpu(), remade["model.layers.0.input_layernorm.weight"].to(torch.bfloat16))
+    assert torch.equal(layer.feed_forward.w_down.cpu(), remade["model.layers.0.mlp.down_proj.weight"].to(torch.bfloat16))
+    write_model(tmp_path, sizes, dtype=torch.bfloat16, weights=remade)
+    plain = PlainLlama(tmp_path)
+    rng = random.Random(2)
+    toks = [rng.randrange(sizes["vocab_size"]) for _ in range(150)]
+    places = list(range(0, 140, 20)) + list(range(140, 150))
+    exact, rounded = plain.logits_at(toks, places), plain.with_storage(torch.bfloat16).logits_at(toks, places)
+    runner = Runner(model, page_size=PAGE, max_tokens=160, max_requests=1, max_rows=256)
+    runner.open("r")
+    got = dict(zip(range(0, 140, 20), runner.step([StepEntry("r", toks[:140], tuple(range(0, 140, 20)))]).cpu()))
+    for p in range(140, 150):
+        got[p] = runner.step([StepEntry("r", [toks[p]], (0,))])[0].cpu()
+    runner.close("r")
+    at = {p: i for i, p in enumerate(places)}
+    assert_within_bfloat16_noise(got, lambda p: exact[at[p]], lambda p: rounded[at[p]], "the benchmark's random model")

@@ -157,3 +157,33 @@ def test_random_model_folder_is_seeded_and_complete(tmp_path, dtype):
 def test_random_tensors_refuse_integer_tables():
     with pytest.raises(ValueError, match="integer tables"):
         random_tensors([TensorNeed("t", (2,), "table")], 0)
+
+
+def test_the_formula_of_the_weights_drawn_on_the_device_is_the_stated_one():
+    """`formula_values` (the product's statement of what the device kernel draws) against this suite's own restatement
+    (`model_folders.formula_weights`) and, for three elements, against the formula worked with Python's integers and math."""
+    import math
+    from geneinfer_amd.weights import formula_values, tensor_key
+    from model_folders import TINY_C, formula_weights, full_config, tensor_layout
+    cfg = full_config(TINY_C)
+    ours = formula_weights(cfg, seed=11, std=0.03)
+    for name, shape in tensor_layout(cfg):
+        offset, scale = (1.0, 0.1) if name.endswith("norm.weight") else (0.0, 0.03)
+        assert torch.equal(formula_values(name, shape, 11, offset, scale), ours[name]), name
+    name, golden, mask = "model.layers.0.mlp.up_proj.weight", 0x9E3779B97F4A7C15, (1 << 64) - 1
+    key = 0xCBF29CE484222325
+    for byte in name.encode():
+        key = ((key ^ byte) * 0x100000001B3) & mask
+    key = (key + 12 * golden) & mask
+    assert key == tensor_key(name, 11)
+    flat = ours[name].reshape(-1)
+    for i in (0, 1, 4000):
+        z = (key + (i + 1) * golden) & mask
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & mask
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & mask
+        z ^= z >> 31
+        u1, u2 = ((z >> 40) + 1) / 2 ** 24, ((z >> 8) & 0xFFFFFF) / 2 ** 24
+        want = 0.03 * math.sqrt(-2.0 * math.log(u1)) * math.cos(2.0 * math.pi * u2)
+        assert abs(float(flat[i]) - want) <= 1e-9 + 1e-7 * abs(want)
+    every = torch.cat([t.reshape(-1) for n, t in ours.items() if not n.endswith("norm.weight")])
+    assert abs(float(every.mean())) < 3e-4 and abs(float(every.std()) - 0.03) < 3e-4               # N(0, std)
