@@ -34,7 +34,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-enum Epilogue : int { EPI_STORE_F32 = 0, EPI_ADD_F32 = 1, EPI_STORE_BF16 = 2, EPI_GATED_BF16 = 3 };
+enum Epilogue : int { EPI_STORE_F32 = 0, EPI_ADD_F32 = 1, EPI_STORE_BF16 = 2, EPI_GATED_BF16 = 3, EPI_QKV_ROPE = 4 };
 
 __device__ __forceinline__ float silu_gate(float g, float u) { return (g * (1.0f / (1.0f + expf(-g)))) * u; }
 // The same with the hardware's exp2 and reciprocal (each within a unit or two in the last place of 32 bits): for results
@@ -52,6 +52,154 @@ __device__ __forceinline__ void write_out(void* C, size_t o, float v) {
     if constexpr (EPI == EPI_STORE_F32) ((float*)C)[o] = v;
     else if constexpr (EPI == EPI_ADD_F32) ((float*)C)[o] += v;
     else ((bf16_t*)C)[o] = f32_to_bf16(v);
+}
+
+// ----------------------------------------------------------------- an RMS norm between two products of a few rows
+// The norm of a row x is g * x * r with r = rsqrt(mean(x^2) + eps), and r, one number a row, commutes with the product that reads
+// the normed row.  A product that adds onto the rows x also writes g * x of the sums it has just made, in bfloat16, and what its
+// columns give to the sum of squares of every row, one number per row and piece of the row (`NormOut`); the product that reads
+// those rows multiplies its results by r, which it gets from those numbers, added in a fixed order (`NormIn`).  No kernel for
+// the norm, no second pass over the rows.
+struct NormOut {                 // for a product that adds onto x: all null if it does not hand the norm on
+    const float* g;              // the norm's weights [N]
+    bf16_t* scaled;              // out: g * x, [M, ld]
+    long ld;
+    float* squares;              // out: [M, parts]
+};
+struct NormIn {                  // for a product whose rows A are g * x without r: squares null if they are ready-made rows
+    const float* squares;        // [M, parts]
+    int parts;
+    float eps;
+    int dim;                     // r = rsqrt(sum / dim + eps)
+};
+
+// Where an attention layer wants the sums of its q/k/v product (columns: n_heads * hd queries, n_kv * hd keys, n_kv * hd values):
+// queries rotated into q_out, keys rotated and values as they are into the page table[slot][pos / page_size] at place
+// pos % page_size (pairs (i, i + hd/2): a' = a cos - b sin, b' = a sin + b cos; the page's layout as the attention kernels read
+// it: keys [kv_head][place][hd], then values [kv_head][hd][place]).
+struct RopeStore {
+    const float* cos_t;          // [M, hd/2], or null with sin_t: no rotation
+    const float* sin_t;
+    const int* pos;              // [M]
+    const int* slot;             // [M]
+    const int* table;
+    int table_stride;
+    bf16_t* q_out;               // [M, n_heads * hd]
+    bf16_t* cache;
+    long page_stride;
+    int page_size, n_heads, n_kv, hd;
+};
+
+
+constexpr int PIPED_MAX_PARTS = 64;            // pieces of a row's sum of squares that a kernel for more than 128 rows reads
+
+// r = rsqrt(mean square + eps) of the `rows` rows from `first` on into `scales` (LDS), by a workgroup of NT threads; rows
+// beyond M get 1.  The caller puts a barrier before the use.
+template <int NT>
+__device__ __forceinline__ void tile_row_scales(float* scales, const NormIn& n, int first, int rows, int M) {
+    for (int row = threadIdx.x; row < rows; row += NT) {
+        float sum = 0.f;
+        if (first + row < M)
+            for (int p = 0; p < n.parts; ++p) sum += n.squares[(size_t)(first + row) * n.parts + p];
+        scales[row] = first + row < M ? 1.0f / sqrtf(sum / (float)n.dim + n.eps) : 1.0f;
+    }
+}
+
+// Where the rows of a tile of 128 go in the cache: per row the page's offset and the place in the page, and per group of
+// eight rows whether they are eight consecutive positions of one request that begin at a multiple of eight (rows of a prompt).
+struct TilePlaces {
+    long page[128];              // page * page_stride
+    int place[128];
+    int run[16];
+};
+
+// Filled by the workgroup's first 128 threads (each row's page is two loads that depend on each other: done once per row here,
+// not once per piece of a row); the caller puts a barrier before the use.
+__device__ __forceinline__ void tile_places(TilePlaces& t, int m0, int M, const RopeStore& rs) {
+    const int row = threadIdx.x;
+    if (row >= 128) return;
+    const int m = min(m0 + row, M - 1), p = rs.pos[m], slot = rs.slot[m];
+    t.page[row] = (long)rs.table[(size_t)slot * rs.table_stride + p / rs.page_size] * rs.page_stride;
+    t.place[row] = p % rs.page_size;
+    // the eight lanes of a group agree on the first row's slot and position
+    const int first = row & ~7, p0 = __shfl(p, first & 63, 64), slot0 = __shfl(slot, first & 63, 64);
+    const bool fits = m0 + row < M && slot == slot0 && p == p0 + (row & 7);
+    const unsigned long long all = __ballot(fits);
+    if ((row & 7) == 0) t.run[row >> 3] = ((all >> (row & 63)) & 0xffull) == 0xffull && p % 8 == 0 && rs.page_size % 8 == 0;
+}
+
+// A tile of 128 x 128 sums of a q/k/v product, row-major in LDS, goes where `RopeStore` says.  Whole heads lie inside the
+// tile (hd divides 128, the tile starts at a multiple of 128 columns), so the other half of every pair is in LDS too.  Queries
+// and keys: a thread takes four pairs of a row at a time, whose two halves leave as 8-byte pieces of contiguous rows; the
+// cosines and sines of four such items are asked for at once.  Values are stored transposed in their pages ([hd][place]),
+// so they are taken column by column, eight rows at a time: where those are a run of eight positions (`TilePlaces`), they
+// leave as one 16-byte piece, otherwise one by one.
+template <int NT>
+__device__ __forceinline__ void qkv_tile_rope_store(const float* tile, const TilePlaces& at, int m0, int n0, int M, int N, const RopeStore& rs) {
+    const int a_dim = rs.n_heads * rs.hd, kv_dim = rs.n_kv * rs.hd, half = rs.hd / 2;
+    if (n0 < a_dim + kv_dim && rs.cos_t != nullptr) {
+        // An item is four pairs (i, i + hd/2) of a row: two pieces of four columns, hd/2 apart, that share their cosines and sines.
+        constexpr int BATCH = 4;
+        const int per_head = rs.hd / 8;                                          // items of a head; 16 items a row of the tile
+        for (int e0 = threadIdx.x; e0 < 128 * 16; e0 += NT * BATCH) {
+            float4 cc[BATCH], ss[BATCH];
+#pragma unroll
+            for (int b = 0; b < BATCH; ++b) {
+                const int e = min(e0 + b * NT, 128 * 16 - 1), m = min(m0 + (e >> 4), M - 1), kq = (e & 15) % per_head;
+                cc[b] = *reinterpret_cast<const float4*>(rs.cos_t + (size_t)m * half + kq * 4);
+                ss[b] = *reinterpret_cast<const float4*>(rs.sin_t + (size_t)m * half + kq * 4);
+            }
+#pragma unroll
+            for (int b = 0; b < BATCH; ++b) {
+                const int e = e0 + b * NT, row = e >> 4, item = e & 15, m = m0 + row;
+                const int c_lo = (item / per_head) * rs.hd + (item % per_head) * 4, col = n0 + c_lo;      // in the tile; in the product
+                if (e >= 128 * 16 || m >= M || col >= a_dim + kv_dim) continue;
+                const float4 a = *reinterpret_cast<const float4*>(tile + row * 128 + c_lo);
+                const float4 o = *reinterpret_cast<const float4*>(tile + row * 128 + c_lo + half);
+                const uint2 lo = {f32x2_to_bf16x2(a.x * cc[b].x - o.x * ss[b].x, a.y * cc[b].y - o.y * ss[b].y),
+                                  f32x2_to_bf16x2(a.z * cc[b].z - o.z * ss[b].z, a.w * cc[b].w - o.w * ss[b].w)};
+                const uint2 hi = {f32x2_to_bf16x2(a.x * ss[b].x + o.x * cc[b].x, a.y * ss[b].y + o.y * cc[b].y),
+                                  f32x2_to_bf16x2(a.z * ss[b].z + o.z * cc[b].z, a.w * ss[b].w + o.w * cc[b].w)};
+                const bool key = col >= a_dim;
+                const int c = key ? col - a_dim : col;                           // the column among the queries, or the keys
+                bf16_t* dst = key ? rs.cache + at.page[row] + ((size_t)(c / rs.hd) * rs.page_size + at.place[row]) * rs.hd + c % rs.hd
+                                  : rs.q_out + (size_t)m * a_dim + c;
+                *reinterpret_cast<uint2*>(dst) = lo;
+                *reinterpret_cast<uint2*>(dst + half) = hi;
+            }
+        }
+    } else if (n0 < a_dim + kv_dim) {                                            // no rotation: the sums as they are
+        for (int e = threadIdx.x; e < 128 * 32; e += NT) {
+            const int row = e >> 5, c4 = (e & 31) * 4, m = m0 + row, col = n0 + c4;
+            if (m >= M || col >= a_dim + kv_dim) continue;
+            const float4 v = *reinterpret_cast<const float4*>(tile + row * 128 + c4);
+            const uint2 packed = {f32x2_to_bf16x2(v.x, v.y), f32x2_to_bf16x2(v.z, v.w)};
+            const bool key = col >= a_dim;
+            const int c = key ? col - a_dim : col;
+            bf16_t* dst = key ? rs.cache + at.page[row] + ((size_t)(c / rs.hd) * rs.page_size + at.place[row]) * rs.hd + c % rs.hd
+                              : rs.q_out + (size_t)m * a_dim + c;
+            *reinterpret_cast<uint2*>(dst) = packed;
+        }
+    }
+    if (n0 + 128 > a_dim + kv_dim) {
+        const size_t v_plane = (size_t)rs.n_kv * rs.page_size * rs.hd;           // from a page's keys to its values
+        const bool aligned = ((uintptr_t)rs.cache & 15) == 0 && rs.page_stride % 8 == 0;
+        for (int e = threadIdx.x; e < 16 * 128; e += NT) {
+            const int rows = (e >> 7) * 8, c1 = e & 127, m = m0 + rows, col = n0 + c1;
+            if (m >= M || col >= N || col < a_dim + kv_dim) continue;
+            const size_t c = (size_t)(col - a_dim - kv_dim) * rs.page_size;     // (h * hd + kk) * page_size
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = tile[(rows + i) * 128 + c1];
+            if (aligned && at.run[e >> 7]) {
+                const uint4 packed = {f32x2_to_bf16x2(v[0], v[1]), f32x2_to_bf16x2(v[2], v[3]), f32x2_to_bf16x2(v[4], v[5]), f32x2_to_bf16x2(v[6], v[7])};
+                *reinterpret_cast<uint4*>(rs.cache + at.page[rows] + v_plane + c + at.place[rows]) = packed;
+            } else {
+                const int last = min(7, M - 1 - m);
+                for (int i = 0; i <= last; ++i) rs.cache[at.page[rows + i] + v_plane + c + at.place[rows + i]] = f32_to_bf16(v[i]);
+            }
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------ tiled
@@ -162,7 +310,7 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int EPI>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
                                                              int M, int N, int K, long lda, long ldw, long ldc, int k_per_split,
-                                                             long split_stride) {
+                                                             long split_stride, NormIn norm_in, RopeStore rope) {
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int ROWS = BM + BN, STAGE_BYTES = ROWS * 128, LOADS = ROWS / 8 / (WAVES_M * WAVES_N);      // loads per wave and stage
     static_assert(ROWS % (8 * WAVES_M * WAVES_N) == 0, "the rows of a stage must divide among the waves' loads");
@@ -235,6 +383,31 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
         }
     }
     // Element v of a lane's 32x32 result: row 8*(v/4) + 4*(lane/32) + v%4, column lane%32.
+    if constexpr (EPI == EPI_QKV_ROPE) {
+        // The sums of a q/k/v product do not go out as they are: the tile is laid into LDS (the ring is free once everyone has
+        // read the last block), scaled by a norm handed on if there is one, and leaves rotated, queries to their rows, keys and
+        // values to their pages.
+        static_assert(BM == 128 && BN == 128 && STAGES * STAGE_BYTES >= 128 * 128 * 4, "the tile in LDS is 128 x 128 floats");
+        __shared__ float row_scale[128];
+        __shared__ TilePlaces places;
+        const bool scaled_rows = norm_in.squares != nullptr;
+        if (scaled_rows) tile_row_scales<64 * WAVES_M * WAVES_N>(row_scale, norm_in, m0, 128, M);
+        if (n0 + 128 > rope.n_heads * rope.hd) tile_places(places, m0, M, rope);       // (a tile of queries alone needs no pages)
+        __syncthreads();
+        float* tile = reinterpret_cast<float*>(ring);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = wm + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3);
+                    tile[row * 128 + wn + j * 32 + (lane & 31)] = scaled_rows ? acc[i][j][v] * row_scale[row] : acc[i][j][v];
+                }
+        __syncthreads();
+        qkv_tile_rope_store<64 * WAVES_M * WAVES_N>(tile, places, m0, n0, M, N, rope);
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -247,7 +420,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
                     const float up = __shfl_xor(acc[i][j][v], 16, 64);
                     if ((lane & 16) == 0 && m < M && n < N)
                         ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(silu_gate(acc[i][j][v], up));
-                } else {
+                } else if constexpr (EPI != EPI_QKV_ROPE) {
                     if (m < M && n < N) write_out<EPI>(C, (size_t)m * ldc + n, acc[i][j][v]);
                 }
             }
@@ -497,24 +670,6 @@ constexpr int SK = 128;                               // k per product group of 
 constexpr int SKINNY_MAX_ROWS = 128;                  // rows of A the skinny kernel takes (8 tiles of 16)
 constexpr int KB = 2 * SK, X_STRIDE = KB + 8;         // k per block of the workgroup; +8 bf16 of padding
 
-// ----------------------------------------------------------------- an RMS norm between two products of a few rows
-// The norm of a row x is g * x * r with r = rsqrt(mean(x^2) + eps), and r, one number a row, commutes with the product that reads
-// the normed row.  A product that adds onto the rows x also writes g * x of the sums it has just made, in bfloat16, and what its
-// columns give to the sum of squares of every row, one number per row and piece of the row (`NormOut`); the product that reads
-// those rows multiplies its results by r, which it gets from those numbers, added in a fixed order (`NormIn`).  No kernel for
-// the norm, no second pass over the rows.
-struct NormOut {                 // for a product that adds onto x: all null if it does not hand the norm on
-    const float* g;              // the norm's weights [N]
-    bf16_t* scaled;              // out: g * x, [M, ld]
-    long ld;
-    float* squares;              // out: [M, parts]
-};
-struct NormIn {                  // for a product whose rows A are g * x without r: squares null if they are ready-made rows
-    const float* squares;        // [M, parts]
-    int parts;
-    float eps;
-    int dim;                     // r = rsqrt(sum / dim + eps)
-};
 // The kernel for at most 16 rows: a thread keeps 8 pieces while the products run (more would cost the kernel its second
 // workgroup per compute unit); 64 threads share a row where there are at most 8 rows, 32 otherwise.
 constexpr int SLIM_PIECES = 8;
@@ -760,19 +915,6 @@ __global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* 
 // kernels read it: keys [kv_head][place][hd], then values [kv_head][hd][place]).  A thread has four neighbouring columns; the
 // other half of its pairs is with the thread hd/8 lanes away, in the same wave (hd a power of two from 8 to 256, and rows of a
 // multiple of 256 columns, so that a wave lies in one row and holds whole heads).
-struct RopeStore {
-    const float* cos_t;          // [M, hd/2], or null with sin_t: no rotation
-    const float* sin_t;
-    const int* pos;              // [M]
-    const int* slot;             // [M]
-    const int* table;
-    int table_stride;
-    bf16_t* q_out;               // [M, n_heads * hd]
-    bf16_t* cache;
-    long page_stride;
-    int page_size, n_heads, n_kv, hd;
-};
-
 __global__ __launch_bounds__(256) void skinny_reduce_rope_store_kernel(const float* __restrict__ P, int M, int N, int splits, NormIn norm_in, RopeStore rs) {
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4, slab = (size_t)M * N;
     const bool live = i < slab;                              // (whole waves are live or not: 256 divides N)
@@ -1085,6 +1227,9 @@ GI_API long gi_gemm_bf16_scratch_floats(int M, int N, int K) {
 // The most pieces a reader of M rows takes: what a writer of as many rows makes.
 static int consumer_max_parts(int M) { return M <= 16 ? slim_max_parts(M) : M <= 32 ? TILES_MAX_PARTS : REDUCE_MAX_PARTS; }
 
+// Whether a product of more than 128 rows takes the ping-pong kernel: a 256 x 256 tile or more for every compute unit.
+static bool takes_pingpong(int M, int N) { return (long)((M + 255) / 256) * ((N + 255) / 256) >= gi_compute_units(); }
+
 static const NormIn NO_NORM_IN = {nullptr, 0, 0.f, 1};
 static const NormOut NO_NORM_OUT = {nullptr, nullptr, 0, nullptr};
 
@@ -1212,6 +1357,79 @@ static int launch_skinny(const void* A, const void* W, void* C, int epi, int M, 
     return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream, norm_in, norm_out);
 }
 
+static const RopeStore NO_ROPE = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, nullptr, nullptr, 0, 0, 0, 0, 0};
+
+// More than 128 rows, K a multiple of 64, 128 columns or more: the kernels that load their operands straight into LDS.
+// `rope` != null: the sums are those of an attention layer's q/k/v product and go where it says (`epi` is then not looked at).
+static int launch_large(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, float* scratch,
+                        long scratch_floats, NormIn norm_in, const RopeStore* rope, hipStream_t stream) {
+#define PIPED(BM_, BN_, WM_, WN_, ST_, EPI_, OUT_, LDC_, SPLITS_, KPS_, SLAB_, NORM_, ROPE_)                                            \
+    do {                                                                                                                                \
+        constexpr int bytes = ST_ * (BM_ + BN_) * 128;                                                                                  \
+        static bool raised = false;                                                                                                     \
+        if (!raised) {                                                                                                                  \
+            if (hipFuncSetAttribute((const void*)gemm_bf16_piped_kernel<BM_, BN_, WM_, WN_, ST_, EPI_>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) \
+                return gi_fail("gemm_bf16: cannot reserve %d bytes of LDS", bytes);                                                     \
+            raised = true;                                                                                                              \
+        }                                                                                                                               \
+        dim3 grid((N + BN_ - 1) / BN_, (M + BM_ - 1) / BM_, SPLITS_);                                                                   \
+        gemm_bf16_piped_kernel<BM_, BN_, WM_, WN_, ST_, EPI_><<<grid, 64 * WM_ * WN_, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, OUT_, M, N, K, lda, \
+                                                                                                        ldw, LDC_, KPS_, SLAB_, NORM_, ROPE_); \
+    } while (0)
+#define PIPED_EPI(BM_, BN_, WM_, WN_, ST_)                                                                                              \
+    do {                                                                                                                                \
+        if (rope != nullptr) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_QKV_ROPE, nullptr, 0L, 1, K, 0L, norm_in, *rope);                       \
+        else if (epi == EPI_STORE_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_F32, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);            \
+        else if (epi == EPI_ADD_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_ADD_F32, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);                \
+        else if (epi == EPI_STORE_BF16) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_BF16, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);          \
+        else PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_BF16, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);                                     \
+    } while (0)
+    const int splits = gi_gemm_bf16_piped_splits(M, N, K);
+    if (splits > 1) {                              // few tiles: k is shared out, the sums are finished by the reduce kernel
+        GI_REQUIRE(scratch != nullptr && scratch_floats >= (long)splits * M * N, "gemm_bf16: scratch of %ld floats needed, %ld given",
+                   (long)splits * M * N, scratch_floats);
+        const int k_per_split = K / splits;
+        PIPED(128, 128, 2, 2, 2, EPI_STORE_F32, scratch, (long)N, splits, k_per_split, (long)M * N, NO_NORM_IN, NO_ROPE);
+        GI_CHECK_LAUNCH("gemm_bf16 (piped, split)");
+        if (rope != nullptr) {
+            skinny_reduce_rope_store_kernel<<<(unsigned)(((size_t)M * N / 4 + 255) / 256), 256, 0, stream>>>(scratch, M, N, splits, norm_in, *rope);
+            GI_CHECK_LAUNCH("gemm_bf16 (reduce, rotate, store)");
+            return 0;
+        }
+        return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream, norm_in);
+    }
+    // Measured at 2,048 rows (K = 2048 and 8192): where 256 x 256 tiles give every compute unit one or more, they halve
+    // the traffic into LDS and run the two groups of waves out of step (the ping-pong kernel); otherwise 128 x 128, two
+    // workgroups per unit with two stages each when there are enough tiles, else one workgroup of eight waves with four stages.
+    const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    if (takes_pingpong(M, N) && rope == nullptr) {     // a 256 x 256 tile or more for every compute unit: the ping-pong kernel
+#define PINGPONG(EPI_)                                                                                                                  \
+    do {                                                                                                                                \
+        constexpr int bytes = 2 * 512 * 128;                                                                                            \
+        static bool raised = false;                                                                                                     \
+        if (!raised) {                                                                                                                  \
+            if (hipFuncSetAttribute((const void*)gemm_bf16_pingpong_kernel<256, EPI_>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) \
+                return gi_fail("gemm_bf16: cannot reserve %d bytes of LDS", bytes);                                                     \
+            raised = true;                                                                                                              \
+        }                                                                                                                               \
+        dim3 grid((N + 255) / 256, (M + 255) / 256);                                                                                    \
+        gemm_bf16_pingpong_kernel<256, EPI_><<<grid, 512, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+    } while (0)
+        GI_REQUIRE(lda < (1L << 22) && ldw < (1L << 22), "gemm_bf16: row strides %ld, %ld are too large for the tile-relative addressing", lda, ldw);
+        if (epi == EPI_STORE_F32) PINGPONG(EPI_STORE_F32); else if (epi == EPI_ADD_F32) PINGPONG(EPI_ADD_F32);
+        else if (epi == EPI_STORE_BF16) PINGPONG(EPI_STORE_BF16); else PINGPONG(EPI_GATED_BF16);
+#undef PINGPONG
+        GI_CHECK_LAUNCH("gemm_bf16 (pingpong)");
+        return 0;
+    }
+    if (tiles128 > gi_compute_units()) PIPED_EPI(128, 128, 2, 2, 2);
+    else PIPED_EPI(128, 128, 2, 4, 4);
+#undef PIPED_EPI
+#undef PIPED
+    GI_CHECK_LAUNCH("gemm_bf16 (piped)");
+    return 0;
+}
+
 // The pieces per row that a product of these sizes writes when it hands a norm on (gi_gemm_bf16_handing with `scaled_out`);
 // 0 if it cannot: a shape whose kernel does not do it.  One piece per workgroup from the kernels that finish a product of up to
 // 16 or 32 rows in one launch; up to 128 rows one per 1024 columns, from the kernel that adds the partial sums of the shares of k
@@ -1272,11 +1490,21 @@ GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dty
     return launch_skinny(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, norm_in, norm_out, stream);
 }
 
-// Whether gi_gemm_bf16_qkv_rope_store takes a q/k/v product of these sizes with heads of hd channels: the shapes whose k is shared out
-// over workgroups (17 or 33 to 128 rows), whose sums a second kernel adds up anyway.
+// Whether gi_gemm_bf16_qkv_rope_store takes a q/k/v product of these sizes with heads of hd channels.  17 or 33 to 128 rows: the
+// shapes whose k is shared out over workgroups, whose sums a second kernel adds up anyway.  More rows: the kernels with tiles of
+// 128 x 128, whose epilogue lays the tile into LDS and sends it off rotated (whole heads must lie inside a tile), or, where they
+// share k out, that second kernel again; not where the ping-pong kernel with its larger tiles is the faster product.
 GI_API int gi_gemm_bf16_qkv_rope_store_takes(int M, int N, int K, int hd) {
-    return !takes_slim(M, N, K) && !takes_slim_tiles(M, N, K, EPI_STORE_F32) && M <= SKINNY_MAX_ROWS && gi_gemm_bf16_skinny_splits(N, K) > 0 &&
-           N % 256 == 0 && hd >= 8 && hd <= 256 && (hd & (hd - 1)) == 0 ? 1 : 0;
+    if (hd < 8 || hd > 256 || (hd & (hd - 1)) != 0) return 0;
+    if (M <= SKINNY_MAX_ROWS)
+        return !takes_slim(M, N, K) && !takes_slim_tiles(M, N, K, EPI_STORE_F32) && gi_gemm_bf16_skinny_splits(N, K) > 0 && N % 256 == 0 ? 1 : 0;
+    if (K % PK != 0 || N < 128 || takes_pingpong(M, N)) return 0;
+    return gi_gemm_bf16_piped_splits(M, N, K) > 1 ? N % 256 == 0 : hd <= 128;
+}
+
+// The most pieces of a row's sum of squares that gi_gemm_bf16_qkv_rope_store reads for a product of M rows.
+GI_API int gi_gemm_bf16_qkv_rope_store_max_parts(int M, int N, int K) {
+    return M <= SKINNY_MAX_ROWS || gi_gemm_bf16_piped_splits(M, N, K) > 1 ? REDUCE_MAX_PARTS : PIPED_MAX_PARTS;
 }
 
 // The q/k/v product of an attention layer, A [M, K] x W [N, K]^T with N = (n_heads + 2 n_kv) * hd, whose results do not come back:
@@ -1297,9 +1525,11 @@ GI_API int gi_gemm_bf16_qkv_rope_store(const void* A, const void* W, int M, int 
     GI_REQUIRE(pos != nullptr && slot != nullptr && table != nullptr && q_out != nullptr && cache != nullptr && page_size > 0 &&
                page_stride >= 2L * n_kv * page_size * hd && ((uintptr_t)q_out & 7) == 0 && ((uintptr_t)cache & 7) == 0 && page_stride % 4 == 0,
                "gemm_bf16 (q/k/v): positions, slots, a table, q_out and a cache with a page stride of at least 2*n_kv*page_size*hd are needed");
-    GI_REQUIRE(squares_in == nullptr || (parts_in > 0 && parts_in <= REDUCE_MAX_PARTS), "gemm_bf16 (q/k/v): %d pieces of a sum of squares, at most %d", parts_in,
-               REDUCE_MAX_PARTS);
+    GI_REQUIRE(squares_in == nullptr || (parts_in > 0 && parts_in <= gi_gemm_bf16_qkv_rope_store_max_parts(M, N, K)),
+               "gemm_bf16 (q/k/v): %d pieces of a sum of squares, at most %d", parts_in, gi_gemm_bf16_qkv_rope_store_max_parts(M, N, K));
     const RopeStore rope = {cos_t, sin_t, pos, slot, table, table_stride, (bf16_t*)q_out, (bf16_t*)cache, page_stride, page_size, n_heads, n_kv, hd};
+    if (M > SKINNY_MAX_ROWS)
+        return launch_large(A, W, nullptr, EPI_STORE_F32, M, N, K, lda, ldw, (long)N, scratch, scratch_floats, NormIn{squares_in, parts_in, eps, K}, &rope, stream);
     return launch_skinny(A, W, nullptr, EPI_STORE_F32, M, N, K, lda, ldw, (long)N, scratch, scratch_floats, NormIn{squares_in, parts_in, eps, K}, NO_NORM_OUT,
                          stream, &rope);
 }
@@ -1325,67 +1555,7 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     if (M <= SKINNY_MAX_ROWS) return launch_skinny(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, NO_NORM_IN, NO_NORM_OUT, stream);
 
     GI_REQUIRE((M + 63) / 64 <= 65535, "gemm_bf16: M %d is too large", M);
-    if (K % PK == 0 && N >= 128) {
-#define PIPED(BM_, BN_, WM_, WN_, ST_, EPI_, OUT_, LDC_, SPLITS_, KPS_, SLAB_)                                                          \
-    do {                                                                                                                                \
-        constexpr int bytes = ST_ * (BM_ + BN_) * 128;                                                                                  \
-        static bool raised = false;                                                                                                     \
-        if (!raised) {                                                                                                                  \
-            if (hipFuncSetAttribute((const void*)gemm_bf16_piped_kernel<BM_, BN_, WM_, WN_, ST_, EPI_>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) \
-                return gi_fail("gemm_bf16: cannot reserve %d bytes of LDS", bytes);                                                     \
-            raised = true;                                                                                                              \
-        }                                                                                                                               \
-        dim3 grid((N + BN_ - 1) / BN_, (M + BM_ - 1) / BM_, SPLITS_);                                                                   \
-        gemm_bf16_piped_kernel<BM_, BN_, WM_, WN_, ST_, EPI_><<<grid, 64 * WM_ * WN_, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, OUT_, M, N, K, lda, \
-                                                                                                        ldw, LDC_, KPS_, SLAB_);        \
-    } while (0)
-#define PIPED_EPI(BM_, BN_, WM_, WN_, ST_)                                                                                              \
-    do {                                                                                                                                \
-        if (epi == EPI_STORE_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_F32, C, ldc, 1, K, 0L);                                      \
-        else if (epi == EPI_ADD_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_ADD_F32, C, ldc, 1, K, 0L);                                     \
-        else if (epi == EPI_STORE_BF16) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_BF16, C, ldc, 1, K, 0L);                               \
-        else PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_BF16, C, ldc, 1, K, 0L);                                                          \
-    } while (0)
-        const int splits = gi_gemm_bf16_piped_splits(M, N, K);
-        if (splits > 1) {                              // few tiles: k is shared out, the sums are finished by the reduce kernel
-            GI_REQUIRE(scratch != nullptr && scratch_floats >= (long)splits * M * N, "gemm_bf16: scratch of %ld floats needed, %ld given",
-                       (long)splits * M * N, scratch_floats);
-            const int k_per_split = K / splits;
-            PIPED(128, 128, 2, 2, 2, EPI_STORE_F32, scratch, (long)N, splits, k_per_split, (long)M * N);
-            GI_CHECK_LAUNCH("gemm_bf16 (piped, split)");
-            return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream);
-        }
-        // Measured at 2,048 rows (K = 2048 and 8192): where 256 x 256 tiles give every compute unit one or more, they halve
-        // the traffic into LDS and run the two groups of waves out of step (the ping-pong kernel); otherwise 128 x 128, two
-        // workgroups per unit with two stages each when there are enough tiles, else one workgroup of eight waves with four stages.
-        const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128), tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-        if (tiles256 >= 256) {                         // a 256 x 256 tile or more for every compute unit: the ping-pong kernel
-#define PINGPONG(EPI_)                                                                                                                  \
-    do {                                                                                                                                \
-        constexpr int bytes = 2 * 512 * 128;                                                                                            \
-        static bool raised = false;                                                                                                     \
-        if (!raised) {                                                                                                                  \
-            if (hipFuncSetAttribute((const void*)gemm_bf16_pingpong_kernel<256, EPI_>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) \
-                return gi_fail("gemm_bf16: cannot reserve %d bytes of LDS", bytes);                                                     \
-            raised = true;                                                                                                              \
-        }                                                                                                                               \
-        dim3 grid((N + 255) / 256, (M + 255) / 256);                                                                                    \
-        gemm_bf16_pingpong_kernel<256, EPI_><<<grid, 512, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
-    } while (0)
-            GI_REQUIRE(lda < (1L << 22) && ldw < (1L << 22), "gemm_bf16: row strides %ld, %ld are too large for the tile-relative addressing", lda, ldw);
-            if (epi == EPI_STORE_F32) PINGPONG(EPI_STORE_F32); else if (epi == EPI_ADD_F32) PINGPONG(EPI_ADD_F32);
-            else if (epi == EPI_STORE_BF16) PINGPONG(EPI_STORE_BF16); else PINGPONG(EPI_GATED_BF16);
-#undef PINGPONG
-            GI_CHECK_LAUNCH("gemm_bf16 (pingpong)");
-            return 0;
-        }
-        if (tiles128 > 256) PIPED_EPI(128, 128, 2, 2, 2);
-        else PIPED_EPI(128, 128, 2, 4, 4);
-#undef PIPED_EPI
-#undef PIPED
-        GI_CHECK_LAUNCH("gemm_bf16 (piped)");
-        return 0;
-    }
+    if (K % PK == 0 && N >= 128) return launch_large(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, NO_NORM_IN, nullptr, stream);
 #define TILED(BM_, EPI_) gemm_bf16_tiled_kernel<BM_, EPI_><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
     if ((long)((M + 127) / 128) * ((N + BN - 1) / BN) < 512) {   // few tiles: smaller ones fill more of the chip
         dim3 grid((N + BN - 1) / BN, (M + 63) / 64);

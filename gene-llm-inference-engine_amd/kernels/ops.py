@@ -82,6 +82,8 @@ def lib():
         l.gi_gemm_bf16_qkv_rope_store_takes.restype = c_int
         l.gi_compute_units.argtypes = []
         l.gi_compute_units.restype = c_int
+        l.gi_gemm_bf16_qkv_rope_store_max_parts.argtypes = [c_int, c_int, c_int]
+        l.gi_gemm_bf16_qkv_rope_store_max_parts.restype = c_int
         l.gi_probe_mfma_flops.argtypes = [c_int, c_int]
         l.gi_probe_mfma_flops.restype = c_long
         _lib = l
@@ -660,6 +662,12 @@ def gemm_bf16_qkv_rope_store_takes(m, n, k, hd) -> bool:
     return bool(lib().gi_gemm_bf16_qkv_rope_store_takes(m, n, k, hd))
 
 
+@lru_cache(maxsize=None)
+def gemm_bf16_qkv_rope_store_max_parts(m, n, k) -> int:
+    """The most pieces of a row's sum of squares (`norm_in`) that `gemm_bf16_qkv_rope_store` reads for these sizes."""
+    return lib().gi_gemm_bf16_qkv_rope_store_max_parts(m, n, k)
+
+
 def gemm_bf16_qkv_rope_store(a, w, cos, sin, positions, slots, table, q_out, cache, n_heads, n_kv, hd, norm_in=None):
     """The q/k/v product a @ w.T of an attention layer whose results do not come back: the queries go, rotated, into q_out
     (bfloat16 [m, heads*hd]), the keys (rotated) and the values into the cache's pages, as `rope_store` puts them.
@@ -683,10 +691,10 @@ def gemm_bf16_qkv_rope_store(a, w, cos, sin, positions, slots, table, q_out, cac
     if squares_in is not None and not (squares_in.dtype == torch.float32 and squares_in.is_contiguous() and squares_in.dim() == 2 and squares_in.shape[0] == m):
         raise KernelError("gemm: the pieces of the sums of squares must be float32 [m, pieces]")
     n_scratch = _scratch_floats(m, n, k)
-    scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device)
+    scratch = torch.empty(n_scratch, dtype=torch.float32, device=a.device) if n_scratch else None
     if _profile is not None:
         _profile.note = (f"{n}x{k}", n * k * w.element_size())
-    _call("gi_gemm_bf16_qkv_rope_store", a.data_ptr(), w.data_ptr(), m, n, k, a.stride(0), w.stride(0), scratch.data_ptr(), n_scratch,
+    _call("gi_gemm_bf16_qkv_rope_store", a.data_ptr(), w.data_ptr(), m, n, k, a.stride(0), w.stride(0), _ptr(scratch), n_scratch,
           _ptr(squares_in), squares_in.shape[1] if squares_in is not None else 0, float(eps), _ptr(cos), _ptr(sin), positions.data_ptr(),
           slots.data_ptr(), table.data_ptr(), table.stride(0), q_out.data_ptr(), cache.data_ptr(), cache.stride(0), page_size, n_heads, n_kv, hd, _stream())
     return q_out

@@ -31,9 +31,9 @@ def qkv_rotate_store_attend(h, w_qkv, ctx, cache, *, n_heads, n_kv_heads, head_d
     before_rotation  `f(q, k)`: changes the 32-bit products in place before the rotation (a norm or a scale per head; k is None
                      where the pages are another entry's).  With it the products are always written out in 32-bit; the kernels
                      that rotate, store and attend from them still serve.
-    Which kernels serve is decided here by storage and shape alone: for some tens of rows the product's second kernel rotates
-    and fills the pages itself; for a few decoded rows one kernel rotates, stores and attends; otherwise product, rotation +
-    store and attention are three launches."""
+    Which kernels serve is decided here by storage and shape alone: for some tens of rows and for the rows of prompts the
+    product's own last step rotates and fills the pages; for a few decoded rows one kernel rotates, stores and attends;
+    otherwise product, rotation + store and attention are three launches."""
     T, a_dim, kv_dim = ctx.n_rows, n_heads * head_dim, n_kv_heads * head_dim
     in_dtype = in_dtype if in_dtype is not None else activation_dtype_for(w_qkv, ctx.dtype)
     tables = position.half_split_tables(ctx) if position is not None else None
@@ -42,9 +42,9 @@ def qkv_rotate_store_attend(h, w_qkv, ctx, cache, *, n_heads, n_kv_heads, head_d
     if (before_rotation is None and cache.writes and (tables is not None or position is None) and w_qkv.dtype == torch.bfloat16
             and cache.kv.dtype == torch.bfloat16 and in_dtype == torch.bfloat16
             and ops.gemm_bf16_qkv_rope_store_takes(T, w_qkv.shape[0], w_qkv.shape[1], head_dim)):
-        # some tens of rows: the product's second kernel, which adds up the shares of k, rotates and writes the pages itself
+        # the product's own last step (the kernel that adds up the shares of k, or the epilogue over a tile) rotates and writes the pages
         rows, norm_in = rows_for_product(h, w_qkv)
-        if norm_in is not None and norm_in[0].shape[1] > 8:          # (that kernel reads a norm's pieces one by one)
+        if norm_in is not None and norm_in[0].shape[1] > ops.gemm_bf16_qkv_rope_store_max_parts(T, w_qkv.shape[0], w_qkv.shape[1]):
             rows, norm_in = h.materialize(), None
         if ops.gemm_bf16_supports(rows, w_qkv, att):
             q_rot = torch.empty((T, a_dim), dtype=torch.bfloat16, device=ctx.device)

@@ -216,10 +216,17 @@ def test_norm_handed_from_one_product_to_the_next(m, d, k1, n2, gated):
 
 @pytest.mark.parametrize("m,hidden,n_heads,n_kv,hd,page_size,rotate,handed", [(64, 2048, 32, 8, 64, 16, True, True), (40, 2048, 32, 8, 64, 16, True, False),
                                                                               (128, 3072, 24, 8, 128, 16, True, True), (33, 512, 6, 1, 32, 8, False, False),
-                                                                              (17, 4096, 32, 8, 128, 32, True, False), (100, 1024, 2, 1, 256, 16, True, True)])
+                                                                              (17, 4096, 32, 8, 128, 32, True, False), (100, 1024, 2, 1, 256, 16, True, True),
+                                                                              # rows of prompts: tiles of 128 x 128 whose epilogue rotates and stores (two workgroups
+                                                                              # of four waves a unit; one of eight), and shapes whose k is shared out over workgroups
+                                                                              (2048, 2048, 32, 8, 64, 16, True, False), (1100, 256, 20, 2, 128, 16, True, True),
+                                                                              (1100, 256, 80, 8, 32, 8, False, True), (300, 3072, 24, 8, 128, 16, True, True),
+                                                                              (520, 512, 28, 2, 64, 16, True, False), (129, 2048, 32, 8, 64, 16, True, True)])
 def test_qkv_product_that_rotates_and_fills_the_pages(m, hidden, n_heads, n_kv, hd, page_size, rotate, handed):
-    """The q/k/v product whose second kernel rotates and writes the pages itself against the product followed by the kernel
-    that does that: the same queries and the same pages (the sums are added in the same order), also with a norm handed on."""
+    """The q/k/v product whose last step rotates and writes the pages itself (the kernel that adds up the shares of k, or the
+    epilogue over a tile of a prompt's rows) against the product followed by the kernel that does that, which
+    `test_rope_store_writes_the_right_places` holds against the plain statement: the same queries and the same pages, also with
+    a norm handed on."""
     o = ops()
     n = (n_heads + 2 * n_kv) * hd
     assert o.gemm_bf16_qkv_rope_store_takes(m, n, hidden, hd)
@@ -228,7 +235,8 @@ def test_qkv_product_that_rotates_and_fills_the_pages(m, hidden, n_heads, n_kv, 
     g = torch.Generator().manual_seed(9)
     ang = torch.rand(m, hd // 2, generator=g) * 6.28
     cos, sin = (torch.cos(ang).to(DEV), torch.sin(ang).to(DEV)) if rotate else (None, None)
-    n_slots, pages_per = 5, 4
+    n_slots = 5
+    pages_per = max(4, -(-2 * m // (n_slots * page_size)))
     n_pages = n_slots * pages_per + 2
     table = torch.randperm(n_pages, generator=g)[:n_slots * pages_per].view(n_slots, pages_per).to(torch.int32).to(DEV)
     slots = torch.randint(0, n_slots, (m,), generator=g).to(torch.int32)
@@ -243,13 +251,15 @@ def test_qkv_product_that_rotates_and_fills_the_pages(m, hidden, n_heads, n_kv, 
                 break
     slots, positions = slots.to(DEV), positions.to(DEV)
     norm_in = None
-    if handed:
-        squares = (torch.rand(m, 2, generator=g) * hidden).to(DEV)
-        norm_in = (squares, 1e-5)
     fill = lambda: torch.full((n_pages, 2, n_kv, page_size, hd), 7.0, dtype=torch.bfloat16, device=DEV)
     want_cache, got_cache = fill(), fill()
     qkv = torch.empty(m, n, device=DEV)
-    o.gemm_bf16(a, w, qkv, norm_in=norm_in)
+    o.gemm_bf16(a, w, qkv)
+    if handed:
+        parts = min(16, o.gemm_bf16_qkv_rope_store_max_parts(m, n, hidden))
+        squares = (torch.rand(m, parts, generator=g) * hidden / parts).to(DEV)
+        norm_in = (squares, 1e-5)
+        qkv *= torch.rsqrt(squares.sum(1, keepdim=True) / hidden + 1e-5)
     a_dim, kv_dim = n_heads * hd, n_kv * hd
     want_q = torch.empty(m, a_dim, dtype=torch.bfloat16, device=DEV)
     o.rope_store(qkv[:, :a_dim], qkv[:, a_dim:a_dim + kv_dim], qkv[:, a_dim + kv_dim:], cos, sin, positions, slots, table, want_q, want_cache, n_heads, n_kv, hd)
