@@ -66,6 +66,38 @@ GI_API int gi_embed(const void* table, int table_dtype, const int* tokens, float
     return 0;
 }
 
+// The same for a step of a few rows whose first norm the product behind it finishes (see the products' `NormIn`): beside x the
+// row goes out times the norm's weights in bfloat16, and its sum of squares as one number.
+template <typename TT>
+__global__ __launch_bounds__(256) void embed_handing_kernel(const TT* __restrict__ table, const int* __restrict__ tokens, float* __restrict__ x, int dim,
+                                                            const float* __restrict__ g, bf16_t* __restrict__ scaled, float* __restrict__ squares) {
+    __shared__ float red[4];
+    const int t = blockIdx.x;
+    const TT* row = table + (size_t)tokens[t] * dim;
+    float sum = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 256) {
+        const float v = load_f32(row, d);
+        x[(size_t)t * dim + d] = v;
+        scaled[(size_t)t * dim + d] = f32_to_bf16(g[d] * v);
+        sum = fmaf(v, v, sum);
+    }
+    sum = block_sum<256>(sum, red);
+    if (threadIdx.x == 0) squares[t] = sum;
+}
+
+GI_API int gi_embed_handing(const void* table, int table_dtype, const int* tokens, float* x, int n_rows, int dim, const float* g, void* scaled,
+                            float* squares, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && dim > 0 && g != nullptr && scaled != nullptr && squares != nullptr, "embed: n_rows %d and dim %d must be positive, and the norm's operands given", n_rows, dim);
+    if (table_dtype == GI_F32)
+        embed_handing_kernel<float><<<n_rows, 256, 0, stream>>>((const float*)table, tokens, x, dim, g, (bf16_t*)scaled, squares);
+    else if (table_dtype == GI_BF16)
+        embed_handing_kernel<bf16_t><<<n_rows, 256, 0, stream>>>((const bf16_t*)table, tokens, x, dim, g, (bf16_t*)scaled, squares);
+    else
+        return gi_fail("embed: unknown table dtype %d", table_dtype);
+    GI_CHECK_LAUNCH("embed");
+    return 0;
+}
+
 // -------------------------------------------------------------------------------------- RMS norm
 // out = w * (x * rsqrt(mean(x^2) + eps)), one workgroup per row; the sum of squares is taken in
 // 32-bit in an order that depends on the row's length only.  Reference: src/kernels/kernels.cpp:72-83.

@@ -11,6 +11,7 @@ from ..config import ModelSpec, read_config
 from ..kernels import ops
 from ..parts import LayerCache, StepContext, block_class, linear, model_tensor_needs, norm_class, row_transform_class, weight_bytes
 from ..parts.linear import activation_dtype_for
+from ..parts.norm import HandedRows
 from ..weights import load_tensors, random_tensors
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
@@ -67,13 +68,10 @@ class DecoderModel:
         """Runs the step's rows through every layer of the run order; returns float32 logits
         [n_logit_rows, vocab] of the rows listed in `logit_rows`, or None if there are none."""
         x = torch.empty((ctx.n_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device)
-        ops.embed(self.embedding, ctx.tokens, x)
-        for transform in self.after_embedding:
-            transform(x)
         trace = self.trace
+        handed = self._embed(ctx, x)      # the next block's first norm, where whoever wrote x could leave it half applied
         if trace is not None:
             trace("embedding", -1, x)
-        handed = None                     # the next block's first norm, where the block before could leave it half applied
         for i, entry in enumerate(self.run_order):
             ctx.trace = None if trace is None else (lambda tag, rows, i=i: trace(tag, i, rows))
             layer = self.layers[entry.layer]
@@ -105,6 +103,25 @@ class DecoderModel:
         for transform in self.after_head:
             transform(logits)
         return logits
+
+    def _embed(self, ctx: StepContext, x: torch.Tensor):
+        """The rows of the token table into x.  Where the first block's first norm can be taken half applied (`HandedRows`: a few
+        single rows of decoding requests in bfloat16, a norm of the form g * x * rsqrt(mean square + eps), a reader whose product
+        finishes it), the kernel that fetches the rows does the norm's first half too and the `HandedRows` are returned; None otherwise."""
+        first = self.layers[self.run_order[0].layer] if self.run_order else None
+        if (first is not None and not self.after_embedding and self.trace is None and self.dtype == torch.bfloat16
+                and getattr(first, "hands_norm_on", False) and ctx.max_seg_len == 1):         # (decode steps: the one norm kernel of a step that is all launches)
+            norm, reader = first.first_reader()
+            if (hasattr(norm, "handed_weight") and getattr(reader, "accepts_deferred_norm", False) and hasattr(reader, "takes_handed_norm")
+                    and reader.takes_handed_norm(ctx.n_rows)):
+                scaled = torch.empty((ctx.n_rows, self.spec.hidden_size), dtype=torch.bfloat16, device=self.device)
+                squares = torch.empty((ctx.n_rows, 1), dtype=torch.float32, device=self.device)
+                ops.embed_handing(self.embedding, ctx.tokens, x, norm.handed_weight(), scaled, squares)
+                return HandedRows(norm, x, scaled, squares)
+        ops.embed(self.embedding, ctx.tokens, x)
+        for transform in self.after_embedding:
+            transform(x)
+        return None
 
     def set_trace(self, trace) -> None:
         """Debugging, as the reference's Model::set_trace (src/model/model.h): `trace(tag, run-order entry or -1, rows)` is

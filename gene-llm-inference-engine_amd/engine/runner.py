@@ -111,7 +111,7 @@ class Runner:
     def _validate(self, entries: Sequence[StepEntry]):
         if not entries:
             raise StepError("a step needs at least one entry")
-        seen, n_rows, vocab = set(), 0, self.model.spec.vocab_size
+        seen, n_rows, vocab, token_arrays = set(), 0, self.model.spec.vocab_size, []
         for e in entries:
             if e.request in seen:
                 raise StepError(f"request {e.request!r} appears twice in one step")
@@ -120,9 +120,14 @@ class Runner:
                 raise StepError(f"request {e.request!r} is not open")
             if len(e.tokens) == 0:
                 raise StepError(f"request {e.request!r} brings no tokens")
-            for t in e.tokens:
-                if not 0 <= int(t) < vocab:
-                    raise StepError(f"token {t} of request {e.request!r} is outside the vocabulary [0, {vocab})")
+            try:
+                tokens = np.asarray(e.tokens, dtype=np.int64)              # (checked as a whole: a prompt portion has thousands)
+            except (TypeError, ValueError, OverflowError):
+                raise StepError(f"the tokens of request {e.request!r} are not integers") from None
+            if tokens.ndim != 1 or int(tokens.min()) < 0 or int(tokens.max()) >= vocab:
+                bad = next((t for t in e.tokens if not 0 <= int(t) < vocab), None) if tokens.ndim == 1 else None
+                raise StepError(f"token {bad} of request {e.request!r} is outside the vocabulary [0, {vocab})")
+            token_arrays.append(tokens)
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise StepError(f"request {e.request!r} wants logits at place {w} of {len(e.tokens)} tokens")
@@ -140,7 +145,7 @@ class Runner:
             n_rows += len(e.tokens)
         if n_rows > self.max_rows:
             raise StepError(f"the step holds {n_rows} rows, more than max_rows = {self.max_rows}")
-        return n_rows
+        return n_rows, token_arrays
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Runs the batch; returns float32 logits [wanted, vocab] on the device in the order of the
@@ -148,7 +153,7 @@ class Runner:
         until the next step."""
         if self.can_step_from_device and all(len(e.tokens) == 1 and tuple(e.want) == (0,) and e.at is None for e in entries) and entries:
             return self._step_of_single_tokens(entries)
-        n_rows = self._validate(entries)
+        n_rows, token_arrays = self._validate(entries)
         self.cache.reserve([(e.request, len(e.tokens)) for e in entries])       # OutOfPages: nothing changed
         self._uploads.begin_step()
         self.cache.sync(self._uploads.put)
@@ -156,9 +161,9 @@ class Runner:
         meta = np.empty((3, n_rows), dtype=np.int32)                            # tokens, positions, slots
         seg_slot, seg_start, seg_len, seg_pos0, logit_rows = [], [], [], [], []
         row = 0
-        for e in entries:
+        for e, tokens in zip(entries, token_arrays):
             n, slot, pos0 = len(e.tokens), self.cache.slot(e.request), self.cache.length(e.request)
-            meta[0, row:row + n] = np.asarray(e.tokens, dtype=np.int32)
+            meta[0, row:row + n] = tokens
             meta[1, row:row + n] = np.arange(pos0, pos0 + n, dtype=np.int32)
             meta[2, row:row + n] = slot
             seg_slot.append(slot); seg_start.append(row); seg_len.append(n); seg_pos0.append(pos0)

@@ -24,6 +24,7 @@ class KernelError(RuntimeError):
 
 _SIGNATURES = {
     "gi_embed": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "gi_embed_handing": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p],
     "gi_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_long, c_long, c_void_p],
     "gi_rope_cos_sin": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "gi_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -221,6 +222,22 @@ def embed(table, tokens, out):
         raise KernelError("embed: out must be contiguous float32")
     _i32(tokens, "embed: tokens", n)
     _call("gi_embed", table.data_ptr(), _code(table, "embed: table"), tokens.data_ptr(), out.data_ptr(), n, dim, _stream())
+    return out
+
+
+def embed_handing(table, tokens, out, g, scaled, squares):
+    """`embed`, and on the way the first half of an RMS norm of the rows for a product that finishes it (`gemm_bf16(..., norm_in=...)`):
+    scaled = bfloat16(g * out) and squares [n, 1] = the rows' sums of out^2."""
+    _dev(table, tokens, out, g, scaled, squares)
+    n, dim = out.shape
+    if not (table.dim() == 2 and table.shape[1] == dim and table.is_contiguous() and out.dtype == torch.float32 and out.is_contiguous()):
+        raise KernelError("embed: table must be [vocab, dim], contiguous, and out contiguous float32")
+    if not (g.dtype == torch.float32 and g.is_contiguous() and g.numel() == dim and scaled.dtype == torch.bfloat16 and scaled.shape == (n, dim)
+            and scaled.is_contiguous() and squares.dtype == torch.float32 and squares.is_contiguous() and squares.shape == (n, 1)):
+        raise KernelError("embed: handing a norm on needs float32 weights [dim], bfloat16 [n, dim] for the scaled rows and float32 [n, 1] for the sums of squares")
+    _i32(tokens, "embed: tokens", n)
+    _call("gi_embed_handing", table.data_ptr(), _code(table, "embed: table"), tokens.data_ptr(), out.data_ptr(), n, dim, g.data_ptr(), scaled.data_ptr(),
+          squares.data_ptr(), _stream())
     return out
 
 
