@@ -116,13 +116,14 @@ def main() -> int:
 
     # ---- prefill of one 2,048-token prompt (median of 5 after PREFILL_WARMUP untimed ones: the first few run some percent slower)
     runner = make_runner(1, T + 64)
+    greedy = Sampler(SamplerConfig(temperature=0.0), vocab)
     times = []
     for i in range(PREFILL_WARMUP + 5):
         toks = torch.randint(0, vocab, (T,), generator=gen).tolist()            # the prompt is there before the clock starts
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         logits = prefill(runner, i, toks)
-        int(torch.argmax(logits[0]))           # the first token reaches the host
+        sample_rows(logits, [greedy])          # the first token reaches the host, drawn as generation draws it
         times.append(time.perf_counter() - t0)
         runner.close(i)
     prefill_s = sorted(times[PREFILL_WARMUP:])[2]
@@ -160,7 +161,7 @@ def main() -> int:
         "value": round(args.batch * args.steps / dt, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(dt / args.steps * 1e3, 4), "ms_per_step_min": round(windows[0][0] / args.steps * 1e3, 4), "windows": WINDOWS,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02) by a stated formula of seed, tensor name and index, uniform random token ids",
         "config": {"model": f"{name} shape", "layers": L, "layers_of_config": layers_full, "hidden": D, "heads": H,
                    "kv_heads": config.num_key_value_heads, "head_dim": hd, "intermediate": I, "vocab": V, "global_batch": args.batch,
                    "seq_len": context_len, "prompt_len": PROMPT, "decode_context": context, "page_size": PAGE, "tied_embeddings": bool(sizes.get("tie_word_embeddings", False)),

@@ -161,8 +161,9 @@ class PageGroup:
             return
         block = self.table_host[rows, lo:hi]
         if upload is not None:                 # int32 array -> device tensor without waiting for the device
-            idx, data = upload(np.asarray(rows, dtype=np.int32), block)      # (both in one copy)
-            self.table_dev[:, lo:hi].index_copy_(0, idx.long(), data.view(len(rows), hi - lo))
+            # (both in one copy; the rows go as 64-bit numbers, which is what the copy by index wants: no kernel to widen them)
+            idx, data = upload(np.asarray(rows, dtype=np.int64).view(np.int32), block)
+            self.table_dev[:, lo:hi].index_copy_(0, idx.view(torch.int64), data.view(len(rows), hi - lo))
             return
         idx = torch.tensor(rows, dtype=torch.int64)
         self.table_dev[:, lo:hi].index_copy_(0, idx.to(self.table_dev.device), torch.from_numpy(np.ascontiguousarray(block)).to(self.table_dev.device))

@@ -75,11 +75,29 @@ __global__ __launch_bounds__(256) void embed_handing_kernel(const TT* __restrict
     const int t = blockIdx.x;
     const TT* row = table + (size_t)tokens[t] * dim;
     float sum = 0.f;
-    for (int d = threadIdx.x; d < dim; d += 256) {
-        const float v = load_f32(row, d);
-        x[(size_t)t * dim + d] = v;
-        scaled[(size_t)t * dim + d] = f32_to_bf16(g[d] * v);
-        sum = fmaf(v, v, sum);
+    if (dim % 4 == 0 && (((uintptr_t)table | (uintptr_t)x | (uintptr_t)g | (uintptr_t)scaled) & 15) == 0) {      // four neighbouring channels a thread
+        for (int d = threadIdx.x * 4; d < dim; d += 1024) {
+            float v[4];
+            if constexpr (sizeof(TT) == 2) {
+                const uint2 raw = *reinterpret_cast<const uint2*>(row + d);
+                v[0] = __uint_as_float(raw.x << 16); v[1] = __uint_as_float(raw.x & 0xffff0000u);
+                v[2] = __uint_as_float(raw.y << 16); v[3] = __uint_as_float(raw.y & 0xffff0000u);
+            } else {
+                const float4 raw = *reinterpret_cast<const float4*>(row + d);
+                v[0] = raw.x; v[1] = raw.y; v[2] = raw.z; v[3] = raw.w;
+            }
+            const float4 gd = *reinterpret_cast<const float4*>(g + d);
+            *reinterpret_cast<float4*>(x + (size_t)t * dim + d) = float4{v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<uint2*>(scaled + (size_t)t * dim + d) = uint2{f32x2_to_bf16x2(gd.x * v[0], gd.y * v[1]), f32x2_to_bf16x2(gd.z * v[2], gd.w * v[3])};
+            sum += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+        }
+    } else {
+        for (int d = threadIdx.x; d < dim; d += 256) {
+            const float v = load_f32(row, d);
+            x[(size_t)t * dim + d] = v;
+            scaled[(size_t)t * dim + d] = f32_to_bf16(g[d] * v);
+            sum = fmaf(v, v, sum);
+        }
     }
     sum = block_sum<256>(sum, red);
     if (threadIdx.x == 0) squares[t] = sum;
