@@ -1327,7 +1327,9 @@ static int launch_skinny(const void* A, const void* W, void* C, int epi, int M, 
         else if (mt == 2) gemm_bf16_skinny_kernel<2, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
         else if (mt == 3) gemm_bf16_skinny_kernel<3, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
         else if (mt == 4) gemm_bf16_skinny_kernel<4, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
-        else if (mt <= 6) gemm_bf16_skinny_kernel<6, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
+        else if (mt == 5) gemm_bf16_skinny_kernel<5, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
+        else if (mt == 6) gemm_bf16_skinny_kernel<6, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
+        else if (mt == 7) gemm_bf16_skinny_kernel<7, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
         else gemm_bf16_skinny_kernel<8, EPI_, PARTIAL_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, scratch, M, N, K, lda, ldw, ldc, k_per_split, norm_in); \
     } while (0)
     GI_REQUIRE(norm_in.squares == nullptr || norm_in.parts <= consumer_max_parts(M), "gemm_bf16: %d pieces of a sum of squares, at most %d for %d rows",

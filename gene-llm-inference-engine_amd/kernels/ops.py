@@ -493,16 +493,52 @@ def prompt_attention_splits(n_groups, n_heads, span, target_groups=512):
     return max(1, min(-(-target_groups // groups), span // 256, 64))
 
 
+def _decode_piece(span, n_pieces):
+    """Positions a wave of the decode kernel takes when a context of `span` is cut into `n_pieces` (multiples of 32, as the kernel cuts)."""
+    return (-(-span // n_pieces) + 31) & ~31
+
+
+def _decode_shape_time(groups, splits, n_waves, span, hd, units, waves_per_unit):
+    """Microseconds the decode attention takes by a model fitted to measurements at the Llama-3.2-1B shape (1 to 128 rows,
+    contexts of 500 to 30,000): a wave costs 8 us and 0.1 us per position of 64 channels; the workgroups run in as many rounds as
+    a compute unit's wave slots make necessary; more than one split costs the kernel that merges them."""
+    slots = units * (waves_per_unit // n_waves)
+    rounds = -(-groups * splits // slots)
+    wave = 8.0 + 0.1 * (hd / 64.0) * _decode_piece(span, splits * n_waves)
+    return rounds * wave + (4.0 + 0.12 * splits if splits > 1 else 0.0), rounds
+
+
+@lru_cache(maxsize=None)
 def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096):
     """(splits, waves per workgroup) of the decode kernel: about `target_waves` waves in all and pieces of
-    at least 64 positions; a single split (no combine kernel) when a workgroup's waves cover them."""
+    at least 64 positions; a single split (no combine kernel) when a workgroup's waves cover them.  Where that shape
+    needs more workgroups than the chip holds at once (a second round of workgroups, which costs as much as the first,
+    however few it holds), the shape that a fitted model of the kernel's time likes best among those of one round is taken
+    instead (65 to 127 rows at 8 key/value heads: 73 -> 57 us a layer at 65 rows, 90 -> 74 at 96)."""
     groups = n_decode * n_kv * ((n_heads // n_kv + 15) // 16)
     pieces = max(1, min(-(-target_waves // groups), -(-span // 64)))
     max_waves = min(8, lib().gi_attention_decode_max_waves(hd))
     if pieces <= max_waves:
-        return 1, pieces
-    n_waves = min(4, max_waves)
-    return min(-(-pieces // n_waves), 256), n_waves
+        base = (1, pieces)
+    else:
+        n_waves = min(4, max_waves)
+        base = (min(-(-pieces // n_waves), 256), n_waves)
+    units, waves_per_unit = lib().gi_compute_units(), 16 if max_waves == 8 else 8
+    base_time, base_rounds = _decode_shape_time(groups, base[0], base[1], span, hd, units, waves_per_unit)
+    if base_rounds == 1 or target_waves != 4096:
+        return base
+    best, best_time = base, base_time
+    for n_waves in (8, 4, 3, 2):                       # (5 to 7 waves a workgroup measured slower than either neighbour)
+        if n_waves > max_waves:
+            continue
+        most = units * (waves_per_unit // n_waves) // groups           # splits that still fit in one round
+        for splits in range(1, min(most, 256) + 1):
+            if splits > 1 and _decode_piece(span, splits * n_waves) < 64:
+                break
+            t, _ = _decode_shape_time(groups, splits, n_waves, span, hd, units, waves_per_unit)
+            if t < best_time * (0.95 if splits > 1 and best[0] == 1 and best is not base else 1.0):
+                best, best_time = (splits, n_waves), t
+    return best
 
 
 def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None,
