@@ -62,6 +62,11 @@ class Runner:
     max_positions longest request; defaults to the model's limit
     use_graphs   replay decode steps (one token per request, all logits wanted) from captured HIP graphs,
                  if every part of the model allows it (`graph_safe`)
+    graph_rows   steps of other shapes (portions of prompts, alone or beside decoded tokens) of up to this many rows are
+                 captured too when their shape comes again: the same numbers of rows per request in the same order, as many
+                 logits wanted, the same power-of-two bracket of the longest context (at most `max_step_graphs` are kept).
+                 Such a step costs the host one copy and one launch instead of some hundred launches; longer steps keep
+                 the device busy for longer than the host needs to launch them.  0: none.
     max_graphs   most captured graphs kept (one per batch size and bracket of the longest context, at least two); the
                  one used longest ago goes when another is needed.  All graphs take their memory from one pool, so what
                  they hold is what the largest of them needs (a pass's activations and its logits), not the sum.
@@ -71,7 +76,8 @@ class Runner:
     """
 
     def __init__(self, model: DecoderModel, *, page_size: int = 16, max_tokens: int = 4096, max_requests: int = 8,
-                 max_rows: int = 4096, max_positions: Optional[int] = None, use_graphs: bool = True, max_graphs: int = 48):
+                 max_rows: int = 4096, max_positions: Optional[int] = None, use_graphs: bool = True, max_graphs: int = 48,
+                 graph_rows: int = 1024, max_step_graphs: int = 32):
         self.model = model
         self.page_size = int(page_size)
         self.max_rows = int(max_rows)
@@ -83,10 +89,14 @@ class Runner:
         self._view = _CacheView(self.cache, needs, reads_from)
         self.steps_run = 0
         self.rows_run = 0
+        self.steps_replayed = 0                   # of them, served by the replay of a captured pass
         self.use_graphs = bool(use_graphs) and model.graph_safe
         self._graphs = {}
         self.max_graphs = max(2, int(max_graphs))       # (two at least: the graph that goes is then never the one replayed last, whose logits a step queued ahead may still be read from)
         self._graph_pool = None
+        self.graph_rows = int(graph_rows)
+        self.max_step_graphs = max(2, int(max_step_graphs))
+        self._step_graphs = {}
         self._uploads = _StepUploads(model.device, min(8 * self.max_rows + 1024, 1 << 18))       # at most 1 MiB a buffer; what is larger is copied the ordinary way
 
     # -------------------------------------------------------------------------------- requests
@@ -171,15 +181,23 @@ class Runner:
             row += n
 
         dev = self.model.device
-        if logit_rows:
-            meta_dev, rows_dev = self._uploads.put(meta, np.asarray(logit_rows, dtype=np.int32))
+        every_row_wanted = logit_rows == list(range(n_rows))
+        graph = self._step_graph_for(seg_len, seg_pos0, len(logit_rows), every_row_wanted)
+        if graph is not None and graph.calls >= 1:           # a shape that has come before: captured now, replayed from then on
+            logits = graph.run(self._uploads, meta, logit_rows, seg_start, seg_len, seg_pos0, seg_slot)
+            self.steps_replayed += 1
         else:
-            meta_dev, rows_dev = self._uploads.put(meta), None
-        meta_dev = meta_dev.view(3, n_rows)
-        ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
-                          row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0,
-                          upload=self._uploads.put, every_row_wanted=logit_rows == list(range(n_rows)))
-        logits = self._forward(ctx, rows_dev, len(logit_rows))
+            if graph is not None:
+                graph.calls += 1
+            if logit_rows:
+                meta_dev, rows_dev = self._uploads.put(meta, np.asarray(logit_rows, dtype=np.int32))
+            else:
+                meta_dev, rows_dev = self._uploads.put(meta), None
+            meta_dev = meta_dev.view(3, n_rows)
+            ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
+                              row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0,
+                              upload=self._uploads.put, every_row_wanted=every_row_wanted)
+            logits = self._forward(ctx, rows_dev, len(logit_rows))
         self._uploads.end_step()
         for e in entries:
             self.cache.advance(e.request, len(e.tokens))
@@ -202,6 +220,25 @@ class Runner:
             for entry, state in states.items():
                 state.index_copy_(0, slots, kept[entry])
             raise
+
+    # ------------------------------------------------------------------ captured steps of other shapes
+    def _step_graph_for(self, seg_len, seg_pos0, n_logit_rows: int, every_row_wanted: bool):
+        """The captured pass that serves a step of this shape (made at the shape's first coming, captured at its second), or
+        None where such steps are not captured."""
+        n_rows = sum(seg_len)
+        if not (self.can_step_from_device and 0 < n_rows <= self.graph_rows):
+            return None
+        bracket = _context_bracket(max(p + n for p, n in zip(seg_pos0, seg_len)), self.max_positions)
+        key = (tuple(seg_len), n_logit_rows, every_row_wanted, bracket)
+        g = self._step_graphs.get(key)
+        if g is None:
+            if len(self._step_graphs) >= self.max_step_graphs:       # (never during a capture: a graph may not be freed inside one)
+                del self._step_graphs[min(self._step_graphs, key=lambda k: self._step_graphs[k].last_used)]
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            g = self._step_graphs[key] = _StepGraph(self.model, self._view, n_rows, n_logit_rows, every_row_wanted, bracket, self._graph_pool)
+        g.last_used = self.steps_run
+        return g
 
     # --------------------------------------------------------------------------- captured decode
     @property
@@ -266,10 +303,7 @@ class Runner:
         batch = meta.shape[1]
         # The attention kernel's cut of the context into pieces is fixed at capture, for the longest context the graph
         # is to serve well: one graph per batch size and power-of-two bracket of the step's longest context.
-        longest, bracket = max(seg_pos0) + 1, 1024
-        while bracket < longest:
-            bracket *= 2
-        bracket = min(bracket, self.max_positions)
+        bracket = _context_bracket(max(seg_pos0) + 1, self.max_positions)
         g = self._graphs.get((batch, bracket))
         if g is None:
             if len(self._graphs) >= self.max_graphs:         # (never during a capture: a graph may not be freed inside one)
@@ -278,7 +312,16 @@ class Runner:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             g = self._graphs[(batch, bracket)] = _DecodeGraph(self.model, self._view, bracket, batch, self._graph_pool)
         g.last_used = self.steps_run
+        self.steps_replayed += 1 if g.calls >= 1 else 0
         return g.run(meta, seg_slot, seg_pos0, tokens_on_device)
+
+
+def _context_bracket(longest: int, most: int) -> int:
+    """The power of two from 1,024 on that holds `longest` positions (at most `most`): what a captured pass is made for."""
+    bracket = 1024
+    while bracket < longest:
+        bracket *= 2
+    return min(bracket, most)
 
 
 def captured_batch_size(n: int, most: int) -> int:
@@ -342,6 +385,15 @@ class _StepUploads:
         self.host[self.turn][a:b] = torch.from_numpy(flat)
         return self.host[self.turn][a:b]
 
+    def region(self, n: int) -> torch.Tensor:
+        """n ints of this step's pinned buffer in one piece, for a caller that lays several arrays out itself and copies them
+        over at once."""
+        if self.used + n > self.capacity:
+            return torch.empty(n, dtype=torch.int32, pin_memory=torch.device(self.device).type == "cuda")
+        a = self.used
+        self.used = (a + n + 3) & ~3
+        return self.host[self.turn][a:a + n]
+
     def end_step(self) -> None:
         if torch.device(self.device).type == "cuda":
             ev = self.done[self.turn] or torch.cuda.Event()
@@ -392,6 +444,90 @@ class _DecodeGraph:
             try:
                 with torch.cuda.graph(graph, pool=self.pool):
                     self.logits = self.model.forward(self._context(seg_slot, seg_pos0), self.view, self.logit_rows, self.batch)
+            finally:
+                if collecting:
+                    gc.enable()
+            self.graph = graph
+        self.graph.replay()
+        return self.logits
+
+
+class _StepGraph:
+    """The captured pass of one step shape other than the all-decode one: the same numbers of rows per request in the same order
+    (portions of prompts, alone or beside decoded tokens), as many logits wanted, one bracket of the longest context.  Everything
+    the pass reads of the step (tokens, positions, slots, the rows whose logits are wanted, the attention's lists of tiles and
+    rows) lies in one block of device memory at places the shape fixes; a step lays its numbers out in pinned memory, sends them
+    over in one copy and replays.  The attention cuts contexts for the bracket's longest (`AttentionPlan` with its two context
+    lengths set to the bracket), as the captured decode step does."""
+
+    def __init__(self, model: DecoderModel, view, n_rows: int, n_logit_rows: int, every_row_wanted: bool, bracket: int, pool):
+        self.model, self.view, self.n_rows, self.n_logit_rows, self.every_row_wanted = model, view, n_rows, n_logit_rows, every_row_wanted
+        self.bracket, self.pool = bracket, pool
+        self.block, self.places = None, None                 # the device block, and where each array lies in it: [(offset, size)]
+        self.graph, self.logits, self.calls, self.last_used = None, None, 0, 0
+
+    def _lay_out(self, uploads, meta, logit_rows, seg_start, seg_len, seg_pos0, seg_slot) -> StepContext:
+        """The step's numbers into the block (one copy, nobody waits), and the pass's context over the block's views."""
+        from ..kernels.ops import AttentionPlan
+        arrays = [np.ascontiguousarray(meta, dtype=np.int32).reshape(-1)]
+        if self.n_logit_rows:
+            arrays.append(np.asarray(logit_rows, dtype=np.int32))
+        first_of_plan = len(arrays)
+        views = []
+
+        def collect(*lists):                                 # the attention plan's lists: kept for the copy below, views handed back
+            for values in lists:
+                arrays.append(np.asarray(values, dtype=np.int32).reshape(-1))
+            if self.places is None:
+                return tuple(None for _ in lists)            # (the first time round the block does not exist yet: see below)
+            return tuple(self._view(first_of_plan + i) for i in range(len(lists)))
+
+        plan = AttentionPlan(seg_start, seg_len, seg_pos0, seg_slot, self.model.device, to_device=collect)
+        if self.places is None:                              # the shape's layout, fixed from now on: every array at a multiple of 16 bytes
+            offset, places = 0, []
+            for a in arrays:
+                places.append((offset, a.size))
+                offset = (offset + a.size + 3) & ~3
+            self.places, self.block = places, torch.zeros(max(offset, 4), dtype=torch.int32, device=self.model.device)
+            if plan.n_tiles:
+                plan.tiles, plan.tile_first, plan.tile_rows = self._view(first_of_plan), self._view(first_of_plan + 1), self._view(first_of_plan + 2)
+                plan.decode_rows = self._view(first_of_plan + 3) if len(arrays) > first_of_plan + 3 else None
+        if [a.size for a in arrays] != [size for _, size in self.places]:
+            raise StepError("a captured step met a step of another shape")          # (the shape's key should have told them apart)
+        total = self.places[-1][0] + self.places[-1][1]
+        staged = uploads.region(total)
+        flat = staged.numpy()
+        for a, (offset, size) in zip(arrays, self.places):
+            flat[offset:offset + size] = a
+        self.block[:total].copy_(staged, non_blocking=True)
+        if plan.n_tiles:
+            plan.max_tile_context = self.bracket
+        if plan.n_decode:
+            plan.max_decode_context = self.bracket
+        m = self.model
+        meta_dev = self._view(0).view(3, self.n_rows)
+        ctx = StepContext(n_rows=self.n_rows, dtype=m.dtype, device=m.device, tokens=meta_dev[0], row_pos=meta_dev[1], row_slot=meta_dev[2],
+                          seg_slot=list(seg_slot), seg_start=list(seg_start), seg_len=list(seg_len), seg_pos0=list(seg_pos0),
+                          every_row_wanted=self.every_row_wanted)
+        ctx.memo["attention_plan"] = plan
+        return ctx
+
+    def _view(self, i: int) -> torch.Tensor:
+        offset, size = self.places[i]
+        return self.block[offset:offset + size]
+
+    def run(self, uploads, meta, logit_rows, seg_start, seg_len, seg_pos0, seg_slot):
+        ctx = self._lay_out(uploads, meta, logit_rows, seg_start, seg_len, seg_pos0, seg_slot)
+        self.calls += 1
+        if self.graph is None:
+            rows_dev = self._view(1) if self.n_logit_rows else None
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            collecting = gc.isenabled()
+            gc.disable()                                     # (freeing device memory or another graph inside a capture aborts)
+            try:
+                with torch.cuda.graph(graph, pool=self.pool):
+                    self.logits = self.model.forward(ctx, self.view, rows_dev, self.n_logit_rows)
             finally:
                 if collecting:
                     gc.enable()

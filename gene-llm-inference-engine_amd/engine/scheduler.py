@@ -19,6 +19,8 @@ Policy, as the reference's engine (src/runtime/engine.cpp:64-205):
     and any reservation that needs them takes them back (this scheduler's, another one's on the same runner, a lone
     `generate`).  A preempted request is closed like any other, so what it had computed usually serves it again
     when it returns.
+  * with `portion_quantum` > 0 a portion that the budget (not the prompt's end) cuts short is cut at a multiple of that many rows
+    (ours, not the reference's: steps of one shape can be replayed from a captured pass, see `Runner`).
   * only the row of a request's last known token returns logits; the request's own sampler draws
     the next token from them.  A sampled end token finishes the request (it stays the last
     generated token); so does reaching `max_positions` (prompt plus generated tokens).
@@ -50,6 +52,9 @@ class EngineConfig:
     prefill_chunk: int = 0      # most prompt tokens one request adds to a step; 0 = no limit besides step_rows
     prefix_cache: bool = True   # requests with equal first tokens share the pages of that prefix
     decode_ahead: bool = True   # queue the next decode step before the host has read the last one's tokens
+    portion_quantum: int = 0    # > 0: a prompt portion that the budget cuts short is cut at a multiple of this many rows, so that the
+                                # steps of a long prompt beside a steady batch have one shape, which the runner captures and replays
+                                # (off by default: with the device as the bound it costs a few rows of every step and brings nothing)
 
 
 @dataclass
@@ -118,7 +123,7 @@ class Engine:
             raise ValueError("Engine: step_rows and prefill_chunk must be >= 0")
         step_rows = cfg.step_rows if 0 < cfg.step_rows <= runner.max_rows else runner.max_rows
         self.cfg = EngineConfig(min(cfg.max_running, runner.cache.max_requests), step_rows, cfg.prefill_chunk or step_rows, cfg.prefix_cache,
-                                cfg.decode_ahead)
+                                cfg.decode_ahead, max(0, cfg.portion_quantum))
         self.runner = runner
         self.prefix = runner.cache.prefix if cfg.prefix_cache and runner.cache.enable_prefix_sharing() else None
         self.end_tokens = set(int(t) for t in end_tokens)
@@ -208,6 +213,8 @@ class Engine:
                 if (phase == 0) != (pending == 1):
                     continue
                 take = min(pending, job.steps - job.fed, budget, 1 if phase == 0 else self.cfg.prefill_chunk)
+                if phase == 1 and self.cfg.portion_quantum and self.cfg.portion_quantum < take < pending:
+                    take -= take % self.cfg.portion_quantum        # (cut by the budget, not by the prompt's end: cut at a round number)
                 while take > 0 and any(n > f for n, f in zip(cache.pages_needed(job.key, take), free)):
                     take -= 1
                 if take <= 0:

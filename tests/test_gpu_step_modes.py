@@ -164,6 +164,61 @@ def test_rewind_and_go_another_way(case, dtype):
     assert runner.cache.free_pages() == [g.pool.n_pages for g in runner.cache.groups]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_whose_shape_comes_again_are_replayed_from_a_captured_pass(tmp_path, dtype):
+    """Tiny D: three requests decode while a fourth's prompt goes in as portions of 96 rows, the same shape step after step
+    (captured at its second coming, replayed from then on), then alone in portions of 130 rows; every decoded row's logits and
+    each portion's last are the plain model's, and in 32-bit equal in bits to those of a runner that captures no such step."""
+    from geneinfer_amd.engine import Runner, StepEntry, load_model
+    write_model(tmp_path, CONFIGS["D"], seed=3)
+    rng = random.Random(8)
+    vocab = CONFIGS["D"]["vocab_size"]
+    short = {f"s{i}": [rng.randrange(vocab) for _ in range(30 + 7 * i + 8)] for i in range(3)}      # prompts of 30, 37, 44, then 8 single tokens
+    long = {"p": [rng.randrange(vocab) for _ in range(8 * 96)], "q": [rng.randrange(vocab) for _ in range(5 * 130)]}
+    plain = PlainLlama(tmp_path)
+    exact = {r: plain.logits(t) for r, t in {**short, **long}.items()}
+    near = {r: plain.with_storage(torch.bfloat16).logits(t) for r, t in {**short, **long}.items()}
+    model = load_model(tmp_path, dtype, "cuda:0")
+
+    def run(graph_rows):
+        runner = Runner(model, page_size=16, max_tokens=2048, max_requests=4, max_rows=1024, graph_rows=graph_rows)
+        got, fed = {}, {}
+        for r, toks in short.items():
+            runner.open(r)
+            runner.step([StepEntry(r, toks[:len(toks) - 8], ())])
+            fed[r] = len(toks) - 8
+        runner.open("p")
+        for k in range(8):                                            # (1, 1, 1, 96) eight times
+            entries = [StepEntry(r, [short[r][fed[r]]], (0,)) for r in short] + [StepEntry("p", long["p"][96 * k:96 * k + 96], (95,))]
+            rows = runner.step(entries).cpu()
+            for i, r in enumerate(short):
+                got[(r, fed[r])] = rows[i]
+                fed[r] += 1
+            got[("p", 96 * k + 95)] = rows[3]
+        for r in list(short) + ["p"]:
+            runner.close(r)
+        runner.open("q")
+        for k in range(5):                                            # (130,) five times: tiles of 64 rows, in pairs
+            got[("q", 130 * k + 129)] = runner.step([StepEntry("q", long["q"][130 * k:130 * k + 130], (129,))])[0].cpu()
+        runner.close("q")
+        runner.cache.check_consistency()
+        return got, runner
+
+    got, runner = run(1024)
+    shapes = {key[0]: g for key, g in runner._step_graphs.items()}
+    assert shapes[(1, 1, 1, 96)].graph is not None and shapes[(1, 1, 1, 96)].calls == 8, "the mixed step's shape was not captured and replayed"
+    assert shapes[(130,)].graph is not None and shapes[(130,)].calls == 5
+    if dtype == "float32":
+        worst = max(relative_error(row, exact[r][p]) for (r, p), row in got.items())
+        assert worst < TOLERANCE["float32"], f"worst relative error {worst:.3e}"
+        plainly, other = run(0)
+        assert not other._step_graphs
+        for key, row in got.items():
+            assert torch.equal(row, plainly[key]), f"logits of {key} differ in bits between the captured step and the step run as it is"
+    else:
+        assert_within_bfloat16_noise(got, lambda k: exact[k[0]][k[1]], lambda k: near[k[0]][k[1]], "tiny D, captured steps")
+
+
 def test_a_runner_with_captured_steps_is_freed_without_the_cycle_collector(case):
     """A runner and its captured graphs form no reference cycle: dropping the runner frees them at once, not at a
     moment of the cycle collector's choosing (which may fall inside another capture, where freeing aborts)."""

@@ -177,6 +177,22 @@ def test_the_budget_shortens_the_last_portion():
     assert [n for _, n, _ in runner.log[0]] == [7, 3]
 
 
+def test_a_portion_cut_by_the_budget_is_cut_at_a_round_number_when_asked():
+    """With a quantum a portion that the budget cuts short ends at a multiple of it (the steps of a long prompt then have one
+    shape); the prompt's own end is never rounded, and without a quantum the budget is used to the last row."""
+    for quantum, want in ((0, [1, 29, 29, 29, 15]), (8, [1, 24, 24, 24, 24, 6])):
+        runner = FakeRunner(page_size=4, n_pages=64, max_rows=64, max_positions=200)
+        eng = Engine(runner, EngineConfig(max_running=2, step_rows=30, portion_quantum=quantum), sample=host_sample)
+        eng.submit(EngineRequest([1], 200, SamplerConfig(0.0)))                    # decodes beside the prompt below
+        eng.step()
+        eng.submit(EngineRequest([2] * 102, 200, SamplerConfig(0.0)))
+        taken = [1]
+        while eng.jobs[1].fed < 101:
+            eng.step()
+            taken.append(runner.log[-1][1][1])
+        assert taken == want, (quantum, taken)
+
+
 def test_portions_shrink_to_the_free_pages_and_the_youngest_is_preempted():
     runner = FakeRunner(page_size=4, n_pages=6, max_rows=64)                       # 24 positions in all
     eng = Engine(runner, EngineConfig(max_running=3), sample=host_sample)
