@@ -153,6 +153,24 @@ def test_embed_and_gather():
     assert torch.equal(picked, out[[2, 1]])
 
 
+@pytest.mark.parametrize("dim,dtype", [(2048, torch.bfloat16), (24, torch.bfloat16), (37, torch.bfloat16), (100, torch.float32)])
+def test_embed_with_the_first_half_of_a_norm(dim, dtype):
+    """The fetch of token rows that also writes them times a norm's weights in bfloat16 and their sums of squares (widths with and
+    without the four-channel path), against the plain statement; with the product's share (times rsqrt(mean square + eps)) the
+    rows are the norm's."""
+    table = randn(50, dim, dtype=dtype, seed=10)
+    toks = torch.tensor([3, 49, 0, 3, 17], dtype=torch.int32, device=DEV)
+    g = (1 + 0.1 * randn(dim, seed=12)).contiguous()
+    out, scaled, squares = torch.empty(5, dim, device=DEV), torch.empty(5, dim, dtype=torch.bfloat16, device=DEV), torch.empty(5, 1, device=DEV)
+    ops().embed_handing(table, toks, out, g, scaled, squares)
+    rows = table[toks.long()].double()
+    assert torch.equal(out, rows.float())
+    assert torch.equal(scaled, (g * out).to(torch.bfloat16))
+    assert rel(squares[:, 0], (rows ** 2).sum(1)) < 1e-6
+    normed = scaled.double() * torch.rsqrt(squares.double() / dim + 1e-5)
+    assert rel(normed, g.double() * rows * torch.rsqrt((rows ** 2).mean(1, keepdim=True) + 1e-5)) < 5e-3
+
+
 def test_silu_mul():
     gu = randn(5, 2 * 37, seed=11, scale=4.0)
     gu[0, 0], gu[0, 1] = 100.0, -100.0                               # extremes stay finite
