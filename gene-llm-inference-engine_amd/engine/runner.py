@@ -473,7 +473,6 @@ class _StepGraph:
         if self.n_logit_rows:
             arrays.append(np.asarray(logit_rows, dtype=np.int32))
         first_of_plan = len(arrays)
-        views = []
 
         def collect(*lists):                                 # the attention plan's lists: kept for the copy below, views handed back
             for values in lists:
