@@ -969,6 +969,26 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
 // Waves a workgroup of the decode kernel may have for this head size.
 GI_API int gi_attention_decode_max_waves(int hd) { return hd <= 128 ? 8 : 4; }
 
+// Workgroups of `n_waves` waves of the decode kernel that a compute unit holds at once (by the kernel's registers and its LDS for
+// `gh` query heads per key/value head, at most 16), as the runtime works it out; 0 if it cannot say.  The cut of the context
+// over workgroups is chosen by it: workgroups beyond what the chip holds run as a second round.
+GI_API int gi_attention_decode_workgroups_per_unit(int hd, int fused, int n_waves, int gh) {
+    if (n_waves < 1 || n_waves > gi_attention_decode_max_waves(hd) || gh < 1 || gh > 16) return 0;
+    const size_t lds = (size_t)n_waves * gh * (hd + 2) * sizeof(float);
+    int n = 0;
+    hipError_t e = hipErrorInvalidValue;
+#define ASK2(HD, FUSED_) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)attention_decode_kernel<HD, FUSED_>, 64 * n_waves, lds)
+#define ASK(HD) do { if (fused) ASK2(HD, true); else ASK2(HD, false); } while (0)
+    if (hd == 32) ASK(32); else if (hd == 64) ASK(64); else if (hd == 96) ASK(96); else if (hd == 128) ASK(128); else if (hd == 256) ASK(256);
+#undef ASK
+#undef ASK2
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return n;
+}
+
 // Rows `rows[0 .. n_rows)` of the step (`rows` null: rows 0 .. n_rows-1), one new position each.  Either `q` holds their rotated
 // queries in bfloat16 and the cache already holds their keys and values, or (`qf` given) `qf`,
 // `kf`, `vf` hold the unrotated 32-bit products, `cos_t`/`sin_t` the rotation (or null for none),

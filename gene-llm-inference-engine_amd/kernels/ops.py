@@ -71,6 +71,8 @@ def lib():
         l.gi_sample_filtered_histogram_bytes.restype = c_int
         l.gi_attention_exact_max_head_size.argtypes = []
         l.gi_attention_exact_max_head_size.restype = c_int
+        l.gi_attention_decode_workgroups_per_unit.argtypes = [c_int, c_int, c_int, c_int]
+        l.gi_attention_decode_workgroups_per_unit.restype = c_int
         l.gi_attention_bf16_supports.argtypes = [c_int, c_int, c_int]
         l.gi_attention_bf16_supports.restype = c_int
         l.gi_gemm_bf16_scratch_floats.argtypes = [c_int, c_int, c_int]
@@ -498,47 +500,58 @@ def _decode_piece(span, n_pieces):
     return (-(-span // n_pieces) + 31) & ~31
 
 
-def _decode_shape_time(groups, splits, n_waves, span, hd, units, waves_per_unit):
-    """Microseconds the decode attention takes by a model fitted to measurements at the Llama-3.2-1B shape (1 to 128 rows,
-    contexts of 500 to 30,000): a wave costs 8 us and 0.1 us per position of 64 channels; the workgroups run in as many rounds as
-    a compute unit's wave slots make necessary; more than one split costs the kernel that merges them."""
-    slots = units * (waves_per_unit // n_waves)
-    rounds = -(-groups * splits // slots)
-    wave = 8.0 + 0.1 * (hd / 64.0) * _decode_piece(span, splits * n_waves)
-    return rounds * wave + (4.0 + 0.12 * splits if splits > 1 else 0.0), rounds
+@lru_cache(maxsize=None)
+def _decode_places(hd, fused, n_waves, gh):
+    """Workgroups of `n_waves` waves of the decode kernel that the chip holds at once."""
+    per_unit = lib().gi_attention_decode_workgroups_per_unit(hd, 1 if fused else 0, n_waves, gh)
+    return lib().gi_compute_units() * (per_unit if per_unit > 0 else max(1, 16 // n_waves))
+
+
+def _decode_plain_shape(groups, span, max_waves, target_waves=4096):
+    """About `target_waves` waves in all, pieces of at least 64 positions; one split when a workgroup's waves cover them."""
+    pieces = max(1, min(-(-target_waves // groups), -(-span // 64)))
+    if pieces <= max_waves:
+        return (1, pieces)
+    n_waves = min(4, max_waves)
+    return (min(-(-pieces // n_waves), 256), n_waves)
 
 
 @lru_cache(maxsize=None)
-def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096):
+def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096, fused=False):
     """(splits, waves per workgroup) of the decode kernel: about `target_waves` waves in all and pieces of
-    at least 64 positions; a single split (no combine kernel) when a workgroup's waves cover them.  Where that shape
-    needs more workgroups than the chip holds at once (a second round of workgroups, which costs as much as the first,
-    however few it holds), the shape that a fitted model of the kernel's time likes best among those of one round is taken
-    instead (65 to 127 rows at 8 key/value heads: 73 -> 57 us a layer at 65 rows, 90 -> 74 at 96)."""
-    groups = n_decode * n_kv * ((n_heads // n_kv + 15) // 16)
-    pieces = max(1, min(-(-target_waves // groups), -(-span // 64)))
+    at least 64 positions; a single split (no combine kernel) when a workgroup's waves cover them.
+
+    The chip holds so many workgroups of the kernel at once (the runtime's answer for this head size: 16 waves a compute
+    unit at 64 channels, 12 at 128); workgroups beyond that run as a further round, and a round with a few workgroups in it
+    costs as much as a full one (65 requests of 8 key/value heads: 520 workgroups of 8 waves on 512 places took 73 us a layer
+    against 50 at 64).  So where the plain rule leaves a last round less than half full (less than a third where it has one
+    split: there is no combine kernel to save then, and fewer pieces mean longer waves), or workgroups of 5 to 7 waves (which
+    measured slower than either neighbour), the context is cut into as many pieces as fit in one round instead, in workgroups
+    of 8, 4, 3 or 2 waves, with as few splits as that allows: 65 rows 73 -> 57 us a layer, 96 rows 90 -> 74, 40 rows 46 -> 38,
+    56 rows 2.10 -> 1.92 ms a step (heads of 64 channels); 65 rows 127 -> 111 us (heads of 128).  The small batches whose kernel
+    also rotates and stores the new key keep the plain rule: their workgroups are short, and 8 and 16 rows measured 5 and 3 %
+    slower with one round."""
+    group = n_heads // n_kv
+    groups = n_decode * n_kv * ((group + 15) // 16)
     max_waves = min(8, lib().gi_attention_decode_max_waves(hd))
-    if pieces <= max_waves:
-        base = (1, pieces)
-    else:
-        n_waves = min(4, max_waves)
-        base = (min(-(-pieces // n_waves), 256), n_waves)
-    units, waves_per_unit = lib().gi_compute_units(), 16 if max_waves == 8 else 8
-    base_time, base_rounds = _decode_shape_time(groups, base[0], base[1], span, hd, units, waves_per_unit)
-    if base_rounds == 1 or target_waves != 4096:
+    base = _decode_plain_shape(groups, span, max_waves, target_waves)
+    if target_waves != 4096 or fused:
         return base
-    best, best_time = base, base_time
-    for n_waves in (8, 4, 3, 2):                       # (5 to 7 waves a workgroup measured slower than either neighbour)
+    gh = min(group, 16)
+    rounds = groups * base[0] / _decode_places(hd, fused, base[1], gh)
+    short_last_round = rounds > 1 and 0 < rounds - int(rounds) < (0.5 if base[0] > 1 else 0.3)
+    if not (short_last_round or 5 <= base[1] <= 7):
+        return base
+    best = None
+    for n_waves in (8, 4, 3, 2):
         if n_waves > max_waves:
             continue
-        most = units * (waves_per_unit // n_waves) // groups           # splits that still fit in one round
-        for splits in range(1, min(most, 256) + 1):
-            if splits > 1 and _decode_piece(span, splits * n_waves) < 64:
-                break
-            t, _ = _decode_shape_time(groups, splits, n_waves, span, hd, units, waves_per_unit)
-            if t < best_time * (0.95 if splits > 1 and best[0] == 1 and best is not base else 1.0):
-                best, best_time = (splits, n_waves), t
-    return best
+        splits = min(_decode_places(hd, fused, n_waves, gh) // groups, 256)         # as many as still fit in one round
+        while splits > 1 and _decode_piece(span, splits * n_waves) < 64:
+            splits -= 1
+        if splits >= 1 and (best is None or splits * n_waves > best[0] * best[1] or (splits * n_waves == best[0] * best[1] and splits < best[0])):
+            best = (splits, n_waves)
+    return best or base
 
 
 def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None,
@@ -589,7 +602,7 @@ def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, 
               _ptr(plan.tile_first), _ptr(plan.tile_rows), plan.n_tile_rows, _ptr(part), n_part, _stream())
     if plan.n_decode:
         span = plan.max_decode_context if not window else min(plan.max_decode_context, window + 31)
-        n_splits, n_waves = decode_attention_shape(plan.n_decode, n_heads, n_kv, hd, span, target_waves)
+        n_splits, n_waves = decode_attention_shape(plan.n_decode, n_heads, n_kv, hd, span, target_waves, products is not None)
         n_part = plan.n_decode * n_heads * n_splits * (hd + 2) if n_splits > 1 else 0
         part = torch.empty(n_part, dtype=torch.float32, device=out.device) if n_part else None
         _call("gi_attention_decode_bf16", _ptr(q), _ptr(qf), _ptr(kf), _ptr(vf), qf.stride(0) if qf is not None else 0,

@@ -645,6 +645,26 @@ def test_decode_attention_from_unrotated_products(n_heads, n_kv, hd, ps, window,
     assert torch.equal(torch.nan_to_num(cache, nan=-1.0), torch.nan_to_num(before, nan=-1.0))
 
 
+@pytest.mark.parametrize("hd", [64, 128])
+def test_decode_attention_shape_leaves_no_nearly_empty_round(hd):
+    """The cut of the context over workgroups: whatever the number of rows, the workgroups either fit the chip at once, or their
+    last round is not a small remainder; pieces never fall under 64 positions and the waves cover the span."""
+    o = ops()
+    n_heads, n_kv, span = 32, 8, 4096
+    for rows in list(range(17, 130)) + [192, 256, 500]:
+        splits, n_waves = o.decode_attention_shape(rows, n_heads, n_kv, hd, span)
+        assert 1 <= n_waves <= 8 and splits >= 1 and not 5 <= n_waves <= 7
+        assert splits * n_waves == 1 or o._decode_piece(span, splits * n_waves) >= 64
+        rounds = rows * n_kv * splits / o._decode_places(hd, False, n_waves, 4)
+        plain = o._decode_plain_shape(rows * n_kv, span, 8)
+        if (splits, n_waves) != plain:
+            assert rounds <= 1, (rows, splits, n_waves, rounds)
+        else:
+            assert rounds <= 1 or rounds - int(rounds) == 0 or rounds - int(rounds) >= 0.3, (rows, splits, n_waves, rounds)
+    for rows in range(1, 17):                              # the kernel that also rotates and stores keeps the plain rule
+        assert o.decode_attention_shape(rows, n_heads, n_kv, hd, span, fused=True) == o._decode_plain_shape(rows * n_kv, span, 8)
+
+
 def test_rope_store_writes_the_right_places():
     n_heads, n_kv, hd, ps = 4, 2, 32, 16
     n_pages = 5
