@@ -206,20 +206,7 @@ class Runner:
         return logits
 
     def _forward(self, ctx: StepContext, rows_dev, n_logit_rows: int):
-        """The pass.  Fixed-size state is committed only by a pass that succeeds: parts write their state slots as they
-        go, so the slots of the step's requests are kept aside first and put back if the pass raises (the requests'
-        lengths have not moved yet, and pages reserved for the step stay with their requests for the next try)."""
-        states = self.cache.states
-        if not states:
-            return self.model.forward(ctx, self._view, rows_dev, n_logit_rows)
-        slots = torch.tensor(sorted(set(ctx.seg_slot)), dtype=torch.int64, device=self.model.device)
-        kept = {entry: state.index_select(0, slots) for entry, state in states.items()}
-        try:
-            return self.model.forward(ctx, self._view, rows_dev, n_logit_rows)
-        except BaseException:
-            for entry, state in states.items():
-                state.index_copy_(0, slots, kept[entry])
-            raise
+        return _pass_keeping_state(self.model, self.cache.states, ctx, self._view, rows_dev, n_logit_rows)
 
     # ------------------------------------------------------------------ captured steps of other shapes
     def _step_graph_for(self, seg_len, seg_pos0, n_logit_rows: int, every_row_wanted: bool):
@@ -310,10 +297,27 @@ class Runner:
                 del self._graphs[min(self._graphs, key=lambda k: self._graphs[k].last_used)]
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()
-            g = self._graphs[(batch, bracket)] = _DecodeGraph(self.model, self._view, bracket, batch, self._graph_pool)
+            g = self._graphs[(batch, bracket)] = _DecodeGraph(self.model, self._view, bracket, batch, self._graph_pool, self.cache.states)
         g.last_used = self.steps_run
         self.steps_replayed += 1 if g.calls >= 1 else 0
         return g.run(meta, seg_slot, seg_pos0, tokens_on_device)
+
+
+def _pass_keeping_state(model: DecoderModel, states, ctx: StepContext, view, rows_dev, n_logit_rows: int):
+    """The pass, launched kernel by kernel.  Fixed-size state is committed only by a pass that succeeds: parts write their
+    state slots as they go, so the slots of the step's requests are kept aside first and put back if the pass raises (the
+    requests' lengths have not moved yet, and pages reserved for the step stay with their requests for the next try).  A
+    pass that is being captured changes nothing if it raises, and a replay runs no code of the parts."""
+    if not states:
+        return model.forward(ctx, view, rows_dev, n_logit_rows)
+    slots = torch.tensor(sorted(set(ctx.seg_slot)), dtype=torch.int64, device=model.device)
+    kept = {entry: state.index_select(0, slots) for entry, state in states.items()}
+    try:
+        return model.forward(ctx, view, rows_dev, n_logit_rows)
+    except BaseException:
+        for entry, state in states.items():
+            state.index_copy_(0, slots, kept[entry])
+        raise
 
 
 def _context_bracket(longest: int, most: int) -> int:
@@ -407,9 +411,9 @@ class _DecodeGraph:
     its graphs must not form a reference cycle, or they would be freed by the cycle collector at a moment of its
     choosing, possibly while another graph is being captured, which the HIP runtime answers by aborting."""
 
-    def __init__(self, model: DecoderModel, view, longest_context: int, batch: int, pool=None):
+    def __init__(self, model: DecoderModel, view, longest_context: int, batch: int, pool=None, states=None):
         from ..kernels.ops import AttentionPlan
-        self.model, self.view, self.batch, self.pool, self.last_used = model, view, batch, pool, 0
+        self.model, self.view, self.batch, self.pool, self.last_used, self.states = model, view, batch, pool, 0, states
         dev = model.device
         self.meta = torch.zeros((3, batch), dtype=torch.int32, device=dev)
         self.logit_rows = torch.arange(batch, dtype=torch.int32, device=dev)
@@ -434,7 +438,7 @@ class _DecodeGraph:
         self.calls += 1
         if self.graph is None:
             if self.calls < 2:          # the first step of a batch size runs as it is; a size that comes again is captured
-                return self.model.forward(self._context(seg_slot, seg_pos0), self.view, self.logit_rows, self.batch)
+                return _pass_keeping_state(self.model, self.states, self._context(seg_slot, seg_pos0), self.view, self.logit_rows, self.batch)
             # Capturing records the launches without running them, so this step runs once more below, by replay.
             # No garbage collection meanwhile: freeing device memory or another graph inside a capture aborts.
             torch.cuda.synchronize()

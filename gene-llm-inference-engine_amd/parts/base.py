@@ -81,10 +81,13 @@ class Part:
     """Common construction: `spec`, `tensors` (by name, on the device), compute dtype, device.
 
     `graph_safe` says that everything in the part's work that changes from step to step is read on
-    the device (from the context's tensors, the page tables and the cache), never from the
-    context's host-side lists: only then may a decode step be captured once and replayed.  It is
-    False unless a part says otherwise, and one part that is not makes the runner launch every
-    step anew."""
+    the device (from the context's tensors, the page tables, the cache and the state slots), never from
+    the context's host-side lists, and that no shape depends on the data: only then may a step be
+    captured once and replayed.  What a captured pass may take from the host is its shape, which every
+    replay shares: the number of rows, where each request's rows begin and how many they are
+    (`seg_start`, `seg_len`); not the requests' slots or positions (`seg_slot`, `seg_pos0`: on the
+    device they are `row_slot` and `row_pos`).  It is False unless a part says otherwise, and one
+    part that is not makes the runner launch every step anew."""
     graph_safe = False
 
     def __init__(self, spec, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device):

@@ -268,7 +268,33 @@ def test_toy_architecture_under_every_cut(toy_model, dtype, mode):
     else:
         rounded = {rid: toy.plain_logits(cfg, weights, toks, store=lambda t: t.to(torch.bfloat16).double()) for rid, toks in requests.items()}
         assert_within_bfloat16_noise(got, lambda k: exact[k[0]][k[1]], lambda k: rounded[k[0]][k[1]], mode)
-    assert runner.use_graphs is False                                 # the toy mixer reads host-side step data: no step of this model is captured
+    # Every toy part reads what changes from step to step on the device (the decay mixer its state's slot, too), so the
+    # steps of this model are captured like Llama's: the decode steps of a request's tail, and shapes that come again.
+    assert runner.use_graphs is True
+    if mode == "tail_singly":
+        assert runner._graphs and all(g.graph is not None for g in runner._graphs.values()) and runner.steps_replayed >= 100
+
+
+def test_a_part_whose_shapes_follow_the_data_switches_capturing_off(toy_model, monkeypatch):
+    """The routed feed-forward that takes each expert's rows out (shapes that depend on the routing) says graph_safe = False:
+    the runner then launches every step anew, and the logits are the same."""
+    from geneinfer_amd.engine import Runner, StepEntry, load_model
+    cfg, folder, weights, requests = toy_model
+    monkeypatch.setattr(toy.RoutedFeedForward, "gathered", True)
+    model = load_model(folder, "float32", DEV)
+    assert model.graph_safe is False
+    runner = Runner(model, page_size=4, max_tokens=256, max_requests=2)
+    assert runner.use_graphs is False
+    toks = requests["t3"]
+    runner.open("a")
+    runner.step([StepEntry("a", toks[:-4], ())])
+    exact = toy.plain_logits(cfg, weights, toks)
+    for i in range(len(toks) - 4, len(toks)):
+        got = runner.step([StepEntry("a", [toks[i]], (0,))])[0].cpu()
+        assert relative_error(got, exact[i]) < 2e-5
+    assert not runner._graphs and runner.steps_replayed == 0
+    runner.close("a")
+    runner.cache.check_consistency()
 
 
 def test_a_pass_that_raises_leaves_state_and_lengths_as_they_were(toy_model):

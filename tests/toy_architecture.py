@@ -44,7 +44,12 @@ class DecaySpec:
 
 class DecayMixer(Mixer):
     """State per request: s [hidden] in 32-bit.  Rows of a request are taken in order; the state is
-    read at the start of the request's rows and written back after them."""
+    read at the start of the request's rows and written back after them.
+
+    Which slot a request's state lies in is read on the device (the slot of the request's first row), and only the
+    cut of the step into requests (where each begins, how many rows it has) comes from the host's lists: that cut is
+    part of a captured pass's shape, the slots are not, so the mixer may be captured and replayed."""
+    graph_safe = True
 
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
@@ -60,12 +65,13 @@ class DecayMixer(Mixer):
         return StateNeed((spec.hidden_size,), torch.float32)
 
     def forward(self, h, residual, ctx, cache):
-        for slot, start, n in zip(ctx.seg_slot, ctx.seg_start, ctx.seg_len):
-            s = cache.state[slot].clone()
+        for start, n in zip(ctx.seg_start, ctx.seg_len):
+            slot = ctx.row_slot[start:start + 1].long()
+            s = cache.state.index_select(0, slot)[0]
             for i in range(start, start + n):
                 s = self.spec.decay * s + h[i].float()
                 residual[i] += self.w @ s
-            cache.state[slot] = s
+            cache.state.index_copy_(0, slot, s[None])
 
 
 @dataclass(frozen=True)
@@ -78,6 +84,7 @@ class CenteredNormSpec:
 
 class CenteredNorm(Norm):
     """w * (x - mean(x)) / sqrt(var(x) + eps), in 32-bit; the result is stored as the consumer asks."""
+    graph_safe = True
 
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
@@ -96,7 +103,10 @@ class CenteredNorm(Norm):
 class ParallelBlock:
     """x += mixer(norm(x)) + feed_forward(norm(x)): one norm, read by both halves.  What the model asks of a block:
     `tensor_needs(layer_spec)`, `cache_need(layer_spec)`, `forward(x, ctx, cache)`, `graph_safe`."""
-    graph_safe = False
+
+    @property
+    def graph_safe(self):
+        return all(getattr(p, "graph_safe", False) for p in (self.mixer_norm, self.mixer, self.feed_forward))
 
     def __init__(self, spec, tensors, dtype, device):
         self.spec = spec
@@ -193,7 +203,14 @@ class RoutedSpec:
 
 class RoutedFeedForward(FeedForward):
     """Per row: the expert with the largest router logit (the lowest index among equals), scaled by its softmax
-    probability.  Everything in 32-bit."""
+    probability.  Everything in 32-bit.  Every expert is worked out for every row and the chosen one's result kept, so
+    that no shape depends on the routing and the pass can be captured; `gathered=True` takes each expert's rows out
+    instead (what a real one would do; its shapes follow the data, so such a part says graph_safe = False)."""
+    gathered = False
+
+    @property
+    def graph_safe(self):
+        return not self.gathered
 
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
@@ -216,10 +233,14 @@ class RoutedFeedForward(FeedForward):
         chosen = torch.argmax(logits, dim=-1)                 # the first of equal maxima
         share = torch.softmax(logits, dim=-1).gather(1, chosen[:, None])
         for i, (gate, up, down) in enumerate(self.experts):
-            rows = torch.nonzero(chosen == i).flatten()
-            if rows.numel():
-                x = h[rows]
-                residual[rows] += share[rows] * ((torch.nn.functional.silu(x @ gate.T) * (x @ up.T)) @ down.T)
+            if self.gathered:
+                rows = torch.nonzero(chosen == i).flatten()
+                if rows.numel():
+                    x = h[rows]
+                    residual[rows] += share[rows] * ((torch.nn.functional.silu(x @ gate.T) * (x @ up.T)) @ down.T)
+            else:
+                result = (torch.nn.functional.silu(h @ gate.T) * (h @ up.T)) @ down.T
+                residual += torch.where((chosen == i)[:, None], share * result, torch.zeros_like(result))
 
 
 @dataclass(frozen=True)
