@@ -43,6 +43,12 @@ __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_ex
 // tiles[i] = {first row in the step, number of rows, position of the first row, request slot};
 // workgroup w takes tiles[PAIR * w .. PAIR * w + PAIR), of one request (a tile of 0 rows fills a pair).
 constexpr int KV_TILE = 64;
+// The running maximum a row's exponentials are taken against need not be the true one: any m gives the same O / l as long as
+// nothing overflows.  So m follows the scores only when one of a wave's rows has risen above it by more than this (in units of
+// log2 e: e^(s - m) then stays under 2^8, nothing for 32-bit sums, and bfloat16 keeps its relative precision at every size),
+// and the rescaling of everything gathered so far, a third of a tile's vector instructions, leaves the common path: with the
+// true maximum some row of 32 has a new one in most tiles.  The first keys a row sees always set it (-inf + slack = -inf).
+constexpr float MAX_SLACK = 8.0f;
 
 template <int HD, int NW, int PAIR>
 __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
@@ -236,21 +242,21 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
             }
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale2;             // scale2 > 0: the maximum of the scaled scores
             const float m_new = fmaxf(m, mx);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;      // a row that has seen nothing yet
-            float sum = 0.f;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                s[v] = exp2_fast(fmaf(s[v], scale2, -m_use));
-                sum += s[v];
-            }
-            if (__any(m_new != m)) {                                      // some row's maximum rose: rescale what was gathered so far
-                const float corr = exp2_fast(m - m_use);
+            if (__any(m_new > m + MAX_SLACK)) {                           // some row's maximum rose by much: rescale what was gathered so far
+                const float corr = exp2_fast(m - ((m_new == -INFINITY) ? 0.f : m_new));
                 l *= corr;
 #pragma unroll
                 for (int i = 0; i < DT; ++i)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) o[i][v] *= corr;
                 m = m_new;
+            }
+            const float m_use = (m == -INFINITY) ? 0.f : m;              // a row that has seen nothing yet
+            float sum = 0.f;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                s[v] = exp2_fast(fmaf(s[v], scale2, -m_use));
+                sum += s[v];
             }
             l += sum;
 #pragma unroll
@@ -505,7 +511,16 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
                 for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[h][v]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64)) * scale2;
             const float m_new = fmaxf(m, mx);
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            if (__any(m_new > m + MAX_SLACK)) {
+                const float corr = exp2_fast(m - ((m_new == -INFINITY) ? 0.f : m_new));
+                l *= corr;
+#pragma unroll
+                for (int i = 0; i < DT; ++i)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) o[i][v] *= corr;
+                m = m_new;
+            }
+            const float m_use = (m == -INFINITY) ? 0.f : m;
             float sum = 0.f;
 #pragma unroll
             for (int h = 0; h < 2; ++h)
@@ -514,15 +529,6 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
                     s[h][v] = exp2_fast(fmaf(s[h][v], scale2, -m_use));
                     sum += s[h][v];
                 }
-            if (__any(m_new != m)) {
-                const float corr = exp2_fast(m - m_use);
-                l *= corr;
-#pragma unroll
-                for (int i = 0; i < DT; ++i)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) o[i][v] *= corr;
-                m = m_new;
-            }
             l += sum;
 #pragma unroll
             for (int t = 0; t < 4; ++t) {                     // four groups of 16 keys: slot e of this lane is key 16 t + 8 hf + e

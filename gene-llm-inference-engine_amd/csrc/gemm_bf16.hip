@@ -1296,7 +1296,9 @@ static int launch_slim(const void* A, const void* W, void* C, int epi, int M, in
 // 17 to 32 rows, a narrow output and a short k: one launch of the slim kernel with two tiles of activation rows.  Measured at
 // N = 3072 and 2048, K = 2048 against the skinny kernel's partial sums and their second kernel: 9 against 13 us at 17 and 32 rows,
 // 11 against 13 at 48, 13 against 13 at 64; at K = 8192 (every workgroup reads all the activations: 1 MB at 64 rows) 21 to 43 us
-// against 16 to 19, so longer k and more rows stay with the skinny kernel.
+// against 16 to 19, so longer k and more rows stay with the skinny kernel.  Rows beyond 32 given to further workgroups of two tiles (a
+// second grid dimension: 256 workgroups at 64 rows and N = 2048, each with 64 KB of weights and its own 128 KB of A) measured
+// equal at 33 to 64 rows and 3 % slower in the whole step from 65 rows on: not kept.
 static bool takes_slim_tiles(int M, int N, int K, int epi) {
     return !takes_slim(M, N, K) && M <= 32 && K <= 2048 && epi != EPI_GATED_BF16 && gi_gemm_bf16_skinny_splits(N, K) > 0;
 }

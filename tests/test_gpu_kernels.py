@@ -414,7 +414,7 @@ def test_rows_of_every_kind_of_sampler_in_one_call():
 
 
 # ------------------------------------------------------------------------------------- attention
-def build_paged(requests, n_kv, hd, page_size, dtype, seed, scale_one=None, gone_before=None):
+def build_paged(requests, n_kv, hd, page_size, dtype, seed, scale_one=None, gone_before=None, shape_keys=None):
     """Dense keys/values per request, written into a paged cache with scrambled pages and a rim of
     NaN pages that nothing may touch.  requests: list of context lengths.  gone_before: per request index, a position;
     pages that lie wholly before it have been given back (a window has passed them): their table entries are -1 and
@@ -432,6 +432,8 @@ def build_paged(requests, n_kv, hd, page_size, dtype, seed, scale_one=None, gone
         v = torch.randn(n, n_kv, hd, generator=g).to(dtype)
         if scale_one is not None and n > scale_one[0]:
             k[scale_one[0]] *= scale_one[1]                    # one far key that must stand out
+        if shape_keys is not None:
+            k = shape_keys(slot, k.float()).to(dtype)
         dense.append((k, v))
         for i in range(-(-n // page_size)):
             if gone_before is not None and (i + 1) * page_size <= gone_before.get(slot, 0):
@@ -567,6 +569,51 @@ def test_many_prompt_tiles_of_many_heads(window):
     ops().attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window)
     want = plain_attention_rows(q, dense, rows, n_heads, n_kv, hd, window)
     assert rel(out, want) < 8e-3, rel(out, want)
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd", [(4, 2, 64), (4, 2, 128), (64, 16, 64)])
+def test_prompt_attention_with_scores_that_climb_along_the_context(n_heads, n_kv, hd):
+    """Every query points along one direction and the keys' share of that direction climbs with their position, by 2 to 12
+    units of log2 e from one tile of 64 keys to the next, and falls again behind position 800: the running maximum of a
+    row moves in every tile, by less and by more than what the kernels let it lag behind.  Scores reach 60 and more, so a
+    maximum applied wrongly once is a factor and not a rounding error.  A whole prompt of several tiles, a portion on a
+    cached context and a single row (in the last case: more workgroups than compute units, the other prompt kernel)."""
+    from geneinfer_amd.parts import StepContext
+    ps = 16
+    contexts = [1200, 900, 50]
+    segs = [(0, 0, 1200), (1, 700, 200), (2, 49, 1)]
+    g = torch.Generator().manual_seed(11)
+    direction = torch.nn.functional.normalize(torch.randn(n_kv, hd, generator=g), dim=-1)
+    pos_all = torch.arange(1200, dtype=torch.float32)
+    # slope per position in nats of the final score: gentle, then steep, then falling
+    slope = torch.where(pos_all < 300, 0.02, torch.where(pos_all < 800, 0.13, -0.09))
+    height = torch.cumsum(slope, 0)                                        # the score a unit query gives the key at a position
+    q_gain = 3.0
+
+    def shape_keys(slot, k):
+        n = k.shape[0]
+        return 0.3 * k + (height[:n] * math.sqrt(hd) / q_gain)[:, None, None] * direction[None]
+
+    cache, table, dense = build_paged(contexts, n_kv, hd, ps, torch.bfloat16, seed=hd + 2, shape_keys=shape_keys)
+    rows, seg_start, seg_len, seg_pos0, seg_slot = [], [], [], [], []
+    for slot, pos0, n in segs:
+        seg_start.append(len(rows)); seg_len.append(n); seg_pos0.append(pos0); seg_slot.append(slot + 1)
+        rows += [(slot, pos0 + i) for i in range(n)]
+    T = len(rows)
+    q = (q_gain * direction.repeat_interleave(n_heads // n_kv, 0).reshape(1, n_heads * hd) + 0.3 * torch.randn(T, n_heads * hd, generator=g)).to(torch.bfloat16).to(DEV)
+    pos = torch.tensor([p for _, p in rows], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([s_ + 1 for s_, _ in rows], dtype=torch.int32, device=DEV)
+    ctx = StepContext(n_rows=T, dtype=torch.bfloat16, device=torch.device(DEV), tokens=pos, row_pos=pos, row_slot=slots, seg_slot=seg_slot,
+                      seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0)
+    out = torch.full((T, n_heads * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops().attention(q, cache, out, ctx, table, n_heads, n_kv, hd, None)
+    k0 = dense[0][0]
+    top = float((k0[:, 0].double() @ q[0].double().cpu().view(n_heads, hd)[0]).max() / math.sqrt(hd))
+    assert top > 40, top                                                   # the scores do climb as meant
+    want = plain_attention_rows(q, dense, rows, n_heads, n_kv, hd, None)
+    assert rel(out, want) < 8e-3, rel(out, want)
+    worst_row = float(((out.double().cpu() - want).norm(dim=1) / want.norm(dim=1)).max())
+    assert worst_row < 3e-2, worst_row                                     # no row is off by a factor
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
