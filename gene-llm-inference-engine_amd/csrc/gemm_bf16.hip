@@ -987,31 +987,38 @@ __global__ __launch_bounds__(256) void skinny_reduce_rope_store_kernel(const flo
 // two blocks ahead of the products.  The slices' sums meet in LDS and are added in slice order.
 // ROWS = 8 leaves half of each product idle and doubles the number of workgroups for narrow outputs.
 // HAND: with the two halves of a norm handed from product to product (`NormIn`, `NormOut` above).
-template <int STRIPS, int ROWS, int EPI, bool HAND>
+// FOLD (ROWS = 8 and at most 8 rows of A): the product's rows 8..15, idle otherwise on both sides, take the same 8 weight rows and
+// the same rows of A at the next 32 of k, so that a block is 256 wide, every lane loads, and a row's eight lanes read 128
+// contiguous bytes; of the 16 x 16 result the two 8 x 8 blocks on the diagonal are the two halves' sums (the other two mix the
+// halves and are dropped).
+template <int STRIPS, int ROWS, int EPI, bool HAND, bool FOLD = false>
 __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
                                                             int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in, NormOut norm_out) {
-    constexpr int SLICES = 8 / STRIPS, STEP = SLICES * SK, DEPTH = 3;
+    static_assert(!FOLD || ROWS == 8, "folding k into the idle rows needs strips of 8 weight rows");
+    constexpr int BLOCK = FOLD ? 2 * SK : SK, SPAN = BLOCK / 4;       // k of a block, and of one of its four products
+    constexpr int SLICES = 8 / STRIPS, STEP = SLICES * BLOCK, DEPTH = 3;
     __shared__ float red[8][64][4];
     __shared__ float row_scale[16];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int strip = wave % STRIPS, slice = wave / STRIPS;
-    const int r = lane & 15, q = lane >> 4;
+    const int r = FOLD ? lane & 7 : lane & 15, q = lane >> 4;
+    const int k_lane = 8 * q + (FOLD ? 32 * ((lane >> 3) & 1) : 0);   // where in a product's span of k this lane reads
     const int n = (blockIdx.x * STRIPS + strip) * ROWS + r;
     const bool w_ok = r < ROWS && n < N, x_ok = r < M;
-    const bf16_t* wrow = W + (size_t)(w_ok ? n : 0) * ldw + 8 * q;
-    const bf16_t* xrow = A + (size_t)(x_ok ? r : 0) * lda + 8 * q;
+    const bf16_t* wrow = W + (size_t)(w_ok ? n : 0) * ldw + k_lane;
+    const bf16_t* xrow = A + (size_t)(x_ok ? r : 0) * lda + k_lane;
 
     floatx4 acc = floatx4{};
     uint4 w_buf[DEPTH][4], x_buf[DEPTH][4];
     auto fetch = [&](int k0, uint4* w, uint4* x) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const bool in = k0 + 32 * j + 8 * q < K;
-            w[j] = (in && w_ok) ? load16(wrow + k0 + 32 * j) : uint4{0, 0, 0, 0};
-            x[j] = (in && x_ok) ? load16(xrow + k0 + 32 * j) : uint4{0, 0, 0, 0};
+            const bool in = k0 + SPAN * j + k_lane < K;
+            w[j] = (in && w_ok) ? load16(wrow + k0 + SPAN * j) : uint4{0, 0, 0, 0};
+            x[j] = (in && x_ok) ? load16(xrow + k0 + SPAN * j) : uint4{0, 0, 0, 0};
         }
     };
-    const int k_first = slice * SK;
+    const int k_first = slice * BLOCK;
 #pragma unroll
     for (int d = 0; d < DEPTH - 1; ++d) fetch(k_first + d * STEP, w_buf[d], x_buf[d]);      // beyond K: zeros, no loads
     // The pieces of the rows' sums of squares, 32 or 64 threads a row: asked for behind the first weights, they have come when
@@ -1071,6 +1078,10 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
                 float sum = 0.f;
 #pragma unroll
                 for (int s = 0; s < SLICES; ++s) sum += red[s * STRIPS + st][src_lane][v];
+                if constexpr (FOLD) {                           // the other half of k: row m + 8, column c + 8 of the product
+#pragma unroll
+                    for (int s = 0; s < SLICES; ++s) sum += red[s * STRIPS + st][src_lane + 40][v];
+                }
                 if constexpr (HAND) sum *= r;
                 const int col = (blockIdx.x * STRIPS + st) * ROWS + c;
                 if (col < N) {
@@ -1286,7 +1297,17 @@ static int launch_slim(const void* A, const void* W, void* C, int epi, int M, in
         if (epi == EPI_STORE_F32) SLIM(1, 16, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 16, EPI_ADD_F32); else SLIM(1, 16, EPI_STORE_BF16);
     } else {                                   // a narrow output: strips of 8 rows, twice the workgroups
         dim3 grid((N + 7) / 8);
-        if (epi == EPI_STORE_F32) SLIM(1, 8, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 8, EPI_ADD_F32); else SLIM(1, 8, EPI_STORE_BF16);
+#define SLIM_FOLD(EPI_)                                                                                                                                \
+    do {                                                                                                                                               \
+        if (hand) gemm_bf16_slim_kernel<1, 8, EPI_, true, true><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out); \
+        else gemm_bf16_slim_kernel<1, 8, EPI_, false, true><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out);     \
+    } while (0)
+        if (M <= 8) {                          // ... and up to 8 rows of A: both idle halves of the products take a further 32 of k
+            if (epi == EPI_STORE_F32) SLIM_FOLD(EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM_FOLD(EPI_ADD_F32); else SLIM_FOLD(EPI_STORE_BF16);
+        } else {
+            if (epi == EPI_STORE_F32) SLIM(1, 8, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 8, EPI_ADD_F32); else SLIM(1, 8, EPI_STORE_BF16);
+        }
+#undef SLIM_FOLD
     }
 #undef SLIM
     GI_CHECK_LAUNCH("gemm_bf16 (slim)");
