@@ -987,35 +987,46 @@ __global__ __launch_bounds__(256) void skinny_reduce_rope_store_kernel(const flo
 // two blocks ahead of the products.  The slices' sums meet in LDS and are added in slice order.
 // ROWS = 8 leaves half of each product idle and doubles the number of workgroups for narrow outputs.
 // HAND: with the two halves of a norm handed from product to product (`NormIn`, `NormOut` above).
-// FOLD (ROWS = 8 and at most 8 rows of A): the product's rows 8..15, idle otherwise on both sides, take the same 8 weight rows and
-// the same rows of A at the next 32 of k, so that a block is 256 wide, every lane loads, and a row's eight lanes read 128
-// contiguous bytes; of the 16 x 16 result the two 8 x 8 blocks on the diagonal are the two halves' sums (the other two mix the
-// halves and are dropped).
-template <int STRIPS, int ROWS, int EPI, bool HAND, bool FOLD = false>
+// FOLD (ROWS = 8): the product's rows 8..15, idle otherwise on the weights' side, take the same 8 weight rows at the next 32 of k, and
+// the other operand 8 rows of A at both places likewise, so that a block is 256 wide, every lane loads weights, and a row's eight
+// lanes read 128 contiguous bytes; of the 16 x 16 result the two 8 x 8 blocks on the diagonal are the two halves' sums (the other
+// two mix the halves and are dropped).  FOLD = 1: at most 8 rows of A, one product per weight fragment; FOLD = 2: up to 16, in two
+// groups of 8 rows that share the weight fragment.
+template <int STRIPS, int ROWS, int EPI, bool HAND, int FOLD = 0>
 __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
                                                             int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in, NormOut norm_out) {
-    static_assert(!FOLD || ROWS == 8, "folding k into the idle rows needs strips of 8 weight rows");
+    static_assert(FOLD == 0 || ROWS == 8, "folding k into the idle rows needs strips of 8 weight rows");
     constexpr int BLOCK = FOLD ? 2 * SK : SK, SPAN = BLOCK / 4;       // k of a block, and of one of its four products
-    constexpr int SLICES = 8 / STRIPS, STEP = SLICES * BLOCK, DEPTH = 3;
-    __shared__ float red[8][64][4];
+    constexpr int XT = FOLD == 2 ? 2 : 1;                             // groups of rows of A
+    constexpr int SLICES = 8 / STRIPS, STEP = SLICES * BLOCK, DEPTH = FOLD == 2 ? 2 : 3;
+    __shared__ float red[8][XT][64][4];
     __shared__ float row_scale[16];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int strip = wave % STRIPS, slice = wave / STRIPS;
     const int r = FOLD ? lane & 7 : lane & 15, q = lane >> 4;
     const int k_lane = 8 * q + (FOLD ? 32 * ((lane >> 3) & 1) : 0);   // where in a product's span of k this lane reads
     const int n = (blockIdx.x * STRIPS + strip) * ROWS + r;
-    const bool w_ok = r < ROWS && n < N, x_ok = r < M;
+    const bool w_ok = r < ROWS && n < N;
     const bf16_t* wrow = W + (size_t)(w_ok ? n : 0) * ldw + k_lane;
-    const bf16_t* xrow = A + (size_t)(x_ok ? r : 0) * lda + k_lane;
+    const bf16_t* xrow[XT];
+    bool x_ok[XT];
+#pragma unroll
+    for (int t = 0; t < XT; ++t) {
+        x_ok[t] = 8 * t + r < M;
+        xrow[t] = A + (size_t)(x_ok[t] ? 8 * t + r : 0) * lda + k_lane;
+    }
 
-    floatx4 acc = floatx4{};
-    uint4 w_buf[DEPTH][4], x_buf[DEPTH][4];
-    auto fetch = [&](int k0, uint4* w, uint4* x) {
+    floatx4 acc[XT];
+#pragma unroll
+    for (int t = 0; t < XT; ++t) acc[t] = floatx4{};
+    uint4 w_buf[DEPTH][4], x_buf[DEPTH][XT][4];
+    auto fetch = [&](int k0, uint4* w, uint4 (*x)[4]) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const bool in = k0 + SPAN * j + k_lane < K;
             w[j] = (in && w_ok) ? load16(wrow + k0 + SPAN * j) : uint4{0, 0, 0, 0};
-            x[j] = (in && x_ok) ? load16(xrow + k0 + SPAN * j) : uint4{0, 0, 0, 0};
+#pragma unroll
+            for (int t = 0; t < XT; ++t) x[t][j] = (in && x_ok[t]) ? load16(xrow[t] + k0 + SPAN * j) : uint4{0, 0, 0, 0};
         }
     };
     const int k_first = slice * BLOCK;
@@ -1040,11 +1051,15 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
             fetch(k0 + (d + DEPTH - 1) * STEP, w_buf[(d + DEPTH - 1) % DEPTH], x_buf[(d + DEPTH - 1) % DEPTH]);
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x_buf[d][j]), as_bf16x8(w_buf[d][j]), acc, 0, 0, 0);
+#pragma unroll
+                for (int t = 0; t < XT; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x_buf[d][t][j]), as_bf16x8(w_buf[d][j]), acc[t], 0, 0, 0);
         }
     }
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave][lane][v] = acc[v];
+    for (int t = 0; t < XT; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][t][lane][v] = acc[t][v];
     if constexpr (HAND) {
         if (norm_in.squares != nullptr) {
             float sum = 0.f;
@@ -1057,30 +1072,32 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
         }
     }
     __syncthreads();
-    // Element v of a lane's result: activation row 4*q + v, weight row r of the strip.
+    // Element v of a lane's result: activation row 4*q + v, weight row r of the strip (folded: of the group's 8 rows, and the
+    // second half of k at row + 8, weight row + 8).
     if (tid < 256 * (EPI == EPI_GATED_BF16 ? 1 : STRIPS)) {
         const int st = tid >> 8, e = tid & 255, m = e >> 4, c = e & 15;
-        const int src_lane = c + 16 * (m >> 2), v = m & 3;
+        const int group = FOLD ? m >> 3 : 0, m_in = FOLD ? m & 7 : m;
+        const int src_lane = c + 16 * (m_in >> 2), v = m_in & 3;
         float r = 1.0f;
         if constexpr (HAND) r = norm_in.squares != nullptr ? row_scale[m] : 1.0f;
         float square = 0.f;
-        if (m < M && c < ROWS) {
+        if (m < M && c < ROWS && group < XT) {
             if constexpr (EPI == EPI_GATED_BF16) {
                 float gate = 0.f, up = 0.f;
 #pragma unroll
                 for (int s = 0; s < SLICES; ++s) {
-                    gate += red[s * STRIPS + 0][src_lane][v];
-                    up += red[s * STRIPS + 1][src_lane][v];
+                    gate += red[s * STRIPS + 0][0][src_lane][v];
+                    up += red[s * STRIPS + 1][0][src_lane][v];
                 }
                 if constexpr (HAND) { gate *= r; up *= r; }
                 ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 16 + c] = f32_to_bf16(silu_gate(gate, up));
             } else {
                 float sum = 0.f;
 #pragma unroll
-                for (int s = 0; s < SLICES; ++s) sum += red[s * STRIPS + st][src_lane][v];
-                if constexpr (FOLD) {                           // the other half of k: row m + 8, column c + 8 of the product
+                for (int s = 0; s < SLICES; ++s) sum += red[s * STRIPS + st][group][src_lane][v];
+                if constexpr (FOLD != 0) {                      // the other half of k: row + 8, column + 8 of the product
 #pragma unroll
-                    for (int s = 0; s < SLICES; ++s) sum += red[s * STRIPS + st][src_lane + 40][v];
+                    for (int s = 0; s < SLICES; ++s) sum += red[s * STRIPS + st][group][src_lane + 40][v];
                 }
                 if constexpr (HAND) sum *= r;
                 const int col = (blockIdx.x * STRIPS + st) * ROWS + c;
@@ -1297,15 +1314,16 @@ static int launch_slim(const void* A, const void* W, void* C, int epi, int M, in
         if (epi == EPI_STORE_F32) SLIM(1, 16, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 16, EPI_ADD_F32); else SLIM(1, 16, EPI_STORE_BF16);
     } else {                                   // a narrow output: strips of 8 rows, twice the workgroups
         dim3 grid((N + 7) / 8);
-#define SLIM_FOLD(EPI_)                                                                                                                                \
+#define SLIM_FOLD(EPI_, FOLD_)                                                                                                                         \
     do {                                                                                                                                               \
-        if (hand) gemm_bf16_slim_kernel<1, 8, EPI_, true, true><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out); \
-        else gemm_bf16_slim_kernel<1, 8, EPI_, false, true><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out);     \
+        if (hand) gemm_bf16_slim_kernel<1, 8, EPI_, true, FOLD_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out); \
+        else gemm_bf16_slim_kernel<1, 8, EPI_, false, FOLD_><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out);     \
     } while (0)
-        if (M <= 8) {                          // ... and up to 8 rows of A: both idle halves of the products take a further 32 of k
-            if (epi == EPI_STORE_F32) SLIM_FOLD(EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM_FOLD(EPI_ADD_F32); else SLIM_FOLD(EPI_STORE_BF16);
+        // the idle halves of the products take a further 32 of k: for up to 8 rows of A on both sides, for more on the weights' side
+        if (M <= 8) {
+            if (epi == EPI_STORE_F32) SLIM_FOLD(EPI_STORE_F32, 1); else if (epi == EPI_ADD_F32) SLIM_FOLD(EPI_ADD_F32, 1); else SLIM_FOLD(EPI_STORE_BF16, 1);
         } else {
-            if (epi == EPI_STORE_F32) SLIM(1, 8, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 8, EPI_ADD_F32); else SLIM(1, 8, EPI_STORE_BF16);
+            if (epi == EPI_STORE_F32) SLIM_FOLD(EPI_STORE_F32, 2); else if (epi == EPI_ADD_F32) SLIM_FOLD(EPI_ADD_F32, 2); else SLIM_FOLD(EPI_STORE_BF16, 2);
         }
 #undef SLIM_FOLD
     }
