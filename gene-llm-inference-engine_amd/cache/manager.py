@@ -211,17 +211,18 @@ class CacheManager:
         self.evicted_pages = 0                       # pages taken back from the prefix index so far
 
     def enable_prefix_sharing(self) -> bool:
-        """Lets requests share the pages of equal prompt prefixes (`self.prefix`).  Possible when one group of
-        pages without a window holds all of a request's past: with a window, pages of a prefix are given back
-        while it is still shared; with fixed-size state, the state after the prefix would have to be kept too."""
-        if self.prefix is None and len(self.groups) == 1 and self.groups[0].need.window is None and not self._state_needed:
-            self.prefix = PrefixIndex(self.groups[0].pool, self.page_size)
+        """Lets requests share the pages of equal prompt prefixes (`self.prefix`).  Possible when pages without a
+        window hold all of a request's past, in one group or in several: with a window, pages of a prefix are given
+        back while it is still shared; with fixed-size state, the state after the prefix would have to be kept too."""
+        if self.prefix is None and self.groups and all(g.need.window is None for g in self.groups) and not self._state_needed:
+            self.prefix = PrefixIndex(self.groups[0].pool, self.page_size, [g.pool for g in self.groups[1:]])
         return self.prefix is not None
 
     # ------------------------------------------------------------------------------ requests
     def open(self, request: Hashable, shared_pages: Sequence[int] = ()) -> int:
-        """shared_pages: full pages of an equal prompt prefix, retained for this request by `self.prefix.match`;
-        the request starts with their positions in place."""
+        """shared_pages: full pages of an equal prompt prefix, retained for this request by `self.prefix.match`
+        (the first group's; the index knows the other groups' pages for the same positions); the request starts with
+        their positions in place."""
         if request in self._slot:
             raise CacheError(f"request {request!r} is already open")
         if not self._free_slots:
@@ -237,6 +238,9 @@ class CacheManager:
             s[slot].zero_()
         if shared_pages:
             self.groups[0].adopt(slot, shared_pages)
+            others = [self.prefix.companions(int(p)) for p in shared_pages] if len(self.groups) > 1 else []
+            for gi, g in enumerate(self.groups[1:]):
+                g.adopt(slot, [pages[gi] for pages in others])
         return slot
 
     def pages_of(self, request: Hashable) -> List[int]:
@@ -247,6 +251,13 @@ class CacheManager:
         """The same as an array (a view of the table's row: read it now, do not keep it)."""
         g, slot = self.groups[0], self.slot(request)
         return g.table_host[slot, int(g.first_live[slot]):int(g.n_held[slot])]
+
+    def index_prefix(self, request: Hashable, tokens: Sequence[int], n_tokens: int, after=None) -> int:
+        """Names the request's full pages under its first `n_tokens` positions in the prefix index (`PrefixIndex.insert`, which
+        says what `after` is): the pages of every group."""
+        slot = self.slot(request)
+        others = [g.table_host[slot, int(g.first_live[slot]):int(g.n_held[slot])] for g in self.groups[1:]]
+        return self.prefix.insert(tokens, n_tokens, self.page_row(request), after=after, companions=others)
 
     def evictable_pages(self) -> int:
         return self.prefix.evictable() if self.prefix is not None else 0
@@ -262,15 +273,16 @@ class CacheManager:
         when it needs them.  Whoever reserves (a scheduler's step, a lone `generate`, a replay) gets them, whether or
         not it was the one that filled the index."""
         out = self.free_pages()
-        if self.prefix is not None:
-            out[0] += self.prefix.evictable()
+        if self.prefix is not None:                # (a page the index gives back is one page of every group)
+            out = [n + self.prefix.evictable() for n in out]
         return out
 
     def _make_room(self, need: Sequence[int]) -> bool:
         """True if every group has `need[g]` free pages, after index-only pages were taken back where that helps."""
-        if self.prefix is not None and need[0] > self.groups[0].pool.free_count and need[0] <= self.groups[0].pool.free_count + self.prefix.evictable():
-            if all(n <= g.pool.free_count for n, g in zip(need[1:], self.groups[1:])):
-                self.evict(need[0] - self.groups[0].pool.free_count)
+        if self.prefix is not None:
+            short = max(n - g.pool.free_count for n, g in zip(need, self.groups))
+            if 0 < short <= self.prefix.evictable():
+                self.evict(short)
         return all(n <= g.pool.free_count for n, g in zip(need, self.groups))
 
     def close(self, request: Hashable) -> None:
@@ -433,9 +445,13 @@ class CacheManager:
                     if p < 0:
                         raise CacheError(f"group {gi}: request {request!r} holds no page at a live place")
                     holders.setdefault(p, []).append(request)
-                    if len(holders[p]) > 1 and (self.prefix is None or gi != 0):
+                    if len(holders[p]) > 1 and self.prefix is None:
                         raise CacheError(f"group {gi}: page {p} is held by {holders[p][0]!r} and {request!r}")
-            indexed = set(self.prefix.pages()) if self.prefix is not None and gi == 0 else set()
+            indexed = set()
+            if self.prefix is not None:
+                indexed = set(self.prefix.pages()) if gi == 0 else {self.prefix.companions(p)[gi - 1] for p in self.prefix.pages()}
+                if len(indexed) != len(self.prefix):
+                    raise CacheError(f"group {gi}: the prefix index names a page twice")
             in_use = set(holders) | indexed
             free = set(g.pool._free)
             if len(free) != len(g.pool._free):

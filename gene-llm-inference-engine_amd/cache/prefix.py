@@ -16,6 +16,13 @@ they are recognised as stale when popped (the node's stamp has moved on).
 
 What it does is what the reference's prefix cache does (src/model/prefix_cache.h:1-11): full pages
 only, one reference per named page, `match` retains for the caller, leaves nobody uses go first.
+
+A model whose layers keep their keys in several groups of pages (other head counts or sizes, each
+group with a pool of its own) has one page per group for the same positions.  The index then names
+the first group's page and keeps the other groups' pages beside it (`companions`): whoever holds one
+of them holds all (requests take and give back their pages of all groups together), so the first
+pool's reference counts speak for the others, and what is retained, released or given back is the
+whole set.
 """
 from __future__ import annotations
 
@@ -26,18 +33,18 @@ from .pages import PagePool
 
 
 class _Node:
-    __slots__ = ("page", "tokens", "parent", "children", "stamp", "only_mine")
+    __slots__ = ("page", "tokens", "parent", "children", "stamp", "only_mine", "companions")
 
-    def __init__(self, page: int, tokens: Tuple[int, ...], parent: Optional["_Node"], stamp: int):
-        self.page, self.tokens, self.parent = page, tokens, parent
+    def __init__(self, page: int, tokens: Tuple[int, ...], parent: Optional["_Node"], stamp: int, companions: Tuple[int, ...] = ()):
+        self.page, self.tokens, self.parent, self.companions = page, tokens, parent, companions
         self.children: Dict[Tuple[int, ...], "_Node"] = {}
         self.stamp = stamp                  # time of last use; also tells a fresh heap entry from a stale one
         self.only_mine = False              # the index's reference is the page's only one
 
 
 class PrefixIndex:
-    def __init__(self, pool: PagePool, page_size: int):
-        self.pool, self.page_size = pool, int(page_size)
+    def __init__(self, pool: PagePool, page_size: int, other_pools: Sequence[PagePool] = ()):
+        self.pool, self.page_size, self.other_pools = pool, int(page_size), tuple(other_pools)
         self._first: Dict[Tuple[int, ...], _Node] = {}       # the root's children
         self._by_page: Dict[int, _Node] = {}
         self._only_mine = 0                                   # named pages whose reference count is 1
@@ -90,19 +97,28 @@ class PrefixIndex:
             if nxt is None:
                 break
             self.pool.retain(nxt.page)
+            for pool, page in zip(self.other_pools, nxt.companions):
+                pool.retain(page)
             self._touch(nxt)
             found.append(nxt.page)
             node = nxt
         return found
 
-    def insert(self, tokens: Sequence[int], n_tokens: int, pages: Sequence[int], after=None) -> int:
+    def companions(self, page: int) -> Tuple[int, ...]:
+        """The other groups' pages for the positions of a named page of the first group, in the order of `other_pools`."""
+        return self._by_page[page].companions
+
+    def insert(self, tokens: Sequence[int], n_tokens: int, pages: Sequence[int], after=None, companions: Sequence[Sequence[int]] = ()) -> int:
         """The first n_tokens positions of a request hold `tokens` in `pages` (its page table): its full pages
         are named, each under the page before it, unless that place is taken already (then the page that has
         it is followed, whatever the request's own copy).  Returns how many pages were newly named.
 
         `after`: what `last_walk` was after an earlier insert of the same request (its tokens up to there unchanged):
         the walk then starts behind the pages that one passed, unless the index has forgotten the last of them
-        meanwhile (then it starts at the root as without it)."""
+        meanwhile (then it starts at the root as without it).  `companions`: the request's page tables in the other
+        groups, one per pool of `other_pools`."""
+        if len(companions) != len(self.other_pools):
+            raise ValueError(f"the index names pages of {1 + len(self.other_pools)} groups, {1 + len(companions)} page tables were given")
         ps, node, added, first = self.page_size, None, 0, 0
         if after is not None and self._by_page.get(after[0].page) is after[0]:
             node, first = after
@@ -119,10 +135,12 @@ class PrefixIndex:
             if page in self._by_page:       # a page has one place in the tree
                 break
             self._clock += 1
-            new = _Node(page, key, node, self._clock)
+            new = _Node(page, key, node, self._clock, tuple(int(table[i]) for table in companions))
             self._by_page[page] = new
             self._children_of(node)[key] = new
             self.pool.retain(page)          # (the hook sees a named page with at least two holders: nothing to count)
+            for pool, other in zip(self.other_pools, new.companions):
+                pool.retain(other)
             node = new
             added += 1
             self.last_walk = (new, i + 1)
@@ -139,6 +157,8 @@ class PrefixIndex:
         if node.only_mine:
             self._only_mine -= 1
         self.pool.release(node.page)
+        for pool, other in zip(self.other_pools, node.companions):
+            pool.release(other)
         if node.parent is not None:
             self._offer(node.parent)        # it may have become a leaf nobody uses
 
@@ -185,10 +205,12 @@ class PrefixIndex:
 
     def clear(self) -> None:
         """Forgets everything (pages that requests use stay with them)."""
-        pages = list(self._by_page)
+        nodes = list(self._by_page.values())
         self._by_page.clear()
         self._first.clear()
         self._idle_leaves.clear()
         self._only_mine = 0
-        for page in pages:
-            self.pool.release(page)
+        for node in nodes:
+            self.pool.release(node.page)
+            for pool, other in zip(self.other_pools, node.companions):
+                pool.release(other)

@@ -277,7 +277,7 @@ class Engine:
         job.fed += n
         if self.prefix is not None and job.fed // self.prefix.page_size > job.indexed_upto // self.prefix.page_size:
             # the pages that became full; the walk goes on where this job's last one ended, not from the first page
-            self.prefix.insert(job.tokens, job.fed, self.runner.cache.page_row(job.key), after=job.indexed_after)
+            self.runner.cache.index_prefix(job.key, job.tokens, job.fed, after=job.indexed_after)
             job.indexed_upto, job.indexed_after = job.fed, self.prefix.last_walk
         if nxt is not None:
             st.logits_rows += 1

@@ -353,7 +353,88 @@ def test_requests_open_on_shared_pages():
         m2.open("x", [0])
 
 
-def test_prefix_sharing_needs_one_group_without_window_or_state():
+def test_requests_open_on_shared_pages_of_every_group():
+    """Two groups of pages without a window (other head counts): the index names the first group's pages and keeps the other
+    group's beside them; a request that opens on a match holds both, and a page given back is one of each group."""
+    other = PagedKvNeed(1, 32)
+    m = manager([FULL, other, FULL], n_pages=8, page_size=4, max_requests=3, max_positions=32)
+    assert len(m.groups) == 2 and m.enable_prefix_sharing()
+    m.groups[1].pool._free.reverse()                                              # (so that the two groups hand out other page numbers)
+    m.open("a")
+    m.reserve([("a", 10)]); m.advance("a", 10)
+    tokens = list(range(10))
+    a0, a1 = [g.held_pages(m.slot("a")) for g in m.groups]
+    assert a0 != a1
+    assert m.index_prefix("a", tokens, 10) == 2
+    m.open("b", m.prefix.match(tokens + [77], 10))
+    assert m.length("b") == 8 and [g.held_pages(m.slot("b")) for g in m.groups] == [a0[:2], a1[:2]]
+    m.check_consistency()
+    m.reserve([("b", 3)]); m.advance("b", 3)
+    m.close("a")
+    m.check_consistency()
+    assert m.free_pages() == [5, 5] and m.evictable_pages() == 0
+    m.close("b")
+    assert m.free_pages() == [6, 6] and m.available_pages() == [8, 8] and m.evictable_pages() == 2
+    m.open("c")
+    m.reserve([("c", 30)])                                                          # needs all 8 pages of both groups: the index gives its two back
+    assert m.free_pages() == [0, 0] and len(m.prefix) == 0
+    m.close("c")
+    m.check_consistency()
+    assert m.free_pages() == [8, 8]
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_shared_prefixes_over_two_groups_keep_the_books_under_random_use(seed):
+    """Requests over a small alphabet open on matched pages of two groups, grow, name their pages, are cut back and end, in
+    random order, on a pool so small that the index has to give pages back: after every action no page of either group is
+    lost, held twice without the index knowing, or counted wrongly, and both groups hold the same number of pages."""
+    import random
+    rng = random.Random(seed)
+    m = manager([FULL, PagedKvNeed(1, 32)], n_pages=14, page_size=2, max_requests=4, max_positions=24)
+    assert m.enable_prefix_sharing()
+    m.groups[1].pool._free.reverse()
+    live, walks = {}, {}
+    for turn in range(500):
+        roll = rng.random()
+        if roll < 0.35 and len(live) < 4:
+            tokens = [rng.randrange(2) for _ in range(rng.choice([3, 4, 6, 9, 12]))]
+            shared = m.prefix.match(tokens, len(tokens) - 1)
+            m.open(turn, shared)
+            live[turn], walks[turn] = tokens, None
+        elif roll < 0.7 and live:
+            r = rng.choice(list(live))
+            n = min(rng.randint(1, 4), len(live[r]) - m.length(r))
+            if n > 0:
+                try:
+                    m.reserve([(r, n)])
+                except OutOfPages:
+                    continue
+                m.advance(r, n)
+                m.index_prefix(r, live[r], m.length(r), after=walks[r])
+                walks[r] = m.prefix.last_walk
+        elif roll < 0.8 and live:
+            r = rng.choice(list(live))
+            if m.length(r) > 0:
+                try:
+                    m.truncate(r, rng.randrange(m.length(r)))
+                except OutOfPages:
+                    pass
+                walks[r] = None
+        elif live:
+            r = rng.choice(list(live))
+            m.close(r)
+            del live[r], walks[r]
+        m.check_consistency()
+        free = m.free_pages()
+        assert free[0] == free[1] and m.available_pages() == [free[0] + m.evictable_pages()] * 2
+    for r in list(live):
+        m.close(r)
+    m.prefix.clear()
+    m.check_consistency()
+    assert m.free_pages() == [14, 14]
+
+
+def test_prefix_sharing_needs_pages_without_window_or_state():
     assert not manager([FULL, WINDOW], n_pages=8, page_size=4, max_requests=2, max_positions=32).enable_prefix_sharing()
     assert not manager([WINDOW], n_pages=8, page_size=4, max_requests=2, max_positions=32).enable_prefix_sharing()
     from geneinfer_amd.cache import StateNeed
