@@ -11,7 +11,7 @@ from ..config import ModelSpec, read_config
 from ..kernels import ops
 from ..parts import LayerCache, StepContext, block_class, linear, model_tensor_needs, norm_class, row_transform_class, weight_bytes
 from ..parts.linear import activation_dtype_for
-from ..parts.norm import HandedRows
+from ..parts.norm import HandedRows, norm_to_hand_on
 from ..weights import load_tensors, random_tensors
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
@@ -111,9 +111,8 @@ class DecoderModel:
         first = self.layers[self.run_order[0].layer] if self.run_order else None
         if (first is not None and not self.after_embedding and self.trace is None and self.dtype == torch.bfloat16
                 and getattr(first, "hands_norm_on", False) and ctx.max_seg_len == 1):         # (decode steps: the one norm kernel of a step that is all launches)
-            norm, reader = first.first_reader()
-            if (hasattr(norm, "handed_weight") and getattr(reader, "accepts_deferred_norm", False) and hasattr(reader, "takes_handed_norm")
-                    and reader.takes_handed_norm(ctx.n_rows)):
+            norm = norm_to_hand_on(first.first_reader(), ctx.n_rows)
+            if norm is not None:
                 scaled = torch.empty((ctx.n_rows, self.spec.hidden_size), dtype=torch.bfloat16, device=self.device)
                 squares = torch.empty((ctx.n_rows, 1), dtype=torch.float32, device=self.device)
                 ops.embed_handing(self.embedding, ctx.tokens, x, norm.handed_weight(), scaled, squares)

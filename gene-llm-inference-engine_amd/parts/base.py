@@ -124,6 +124,16 @@ class FeedForward(Part):
 #                                  `linear_onto(..., then)` and returns what that returns (the `HandedRows`, or None).
 
 
+# Optional, for a block (an arrangement of parts; of however many halves):
+#   hands_norm_on = True           the block plays the same game towards its neighbours in the run order: `first_reader()` returns the
+#                                  norm that reads the residual first in it and the part that reads the normed rows, and `forward`
+#                                  takes the keywords `handed` (that norm as whoever wrote the residual last left it, `HandedRows` or
+#                                  None) and `next_reader` (`first_reader()` of whatever reads the residual after the block, or None)
+#                                  and returns that reader's norm handed on, or None.  The model only carries these between the blocks
+#                                  (and plays the first writer and the last reader itself: the token rows, the final norm and the
+#                                  head); `norm_to_hand_on` in parts/norm.py is the one test of whether a reader can take it.
+
+
 class Norm(Part):
     def __call__(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
         raise NotImplementedError

@@ -6,6 +6,7 @@ The residual stream x is float32 [T, hidden] and is changed in place."""
 from __future__ import annotations
 
 from .base import feed_forward_class, mixer_class, norm_class, register_block
+from .norm import norm_to_hand_on
 
 
 class PreNormBlock:
@@ -49,12 +50,7 @@ class PreNormBlock:
 
     @staticmethod
     def _then(part, reader, n_rows):
-        norm, consumer = reader if reader is not None else (None, None)
-        if (norm is None or not getattr(part, "hands_norm_on", False) or not hasattr(norm, "handed_weight")
-                or not getattr(consumer, "accepts_deferred_norm", False) or not hasattr(consumer, "takes_handed_norm")
-                or not consumer.takes_handed_norm(n_rows)):
-            return None
-        return norm
+        return norm_to_hand_on(reader, n_rows) if getattr(part, "hands_norm_on", False) else None
 
     def forward(self, x, ctx, cache, handed=None, next_reader=None):
         """handed: this block's first norm as whoever wrote x last left it, or None.  next_reader: `first_reader()` of whatever

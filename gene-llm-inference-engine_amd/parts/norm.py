@@ -42,6 +42,17 @@ class HandedRows(NormedRows):
         self.scaled, self.squares, self.eps = scaled, squares, norm.eps
 
 
+def norm_to_hand_on(reader, n_rows: int):
+    """reader: (norm, part) as a block's `first_reader()` gives it, or None.  The norm, if whoever writes the rows it reads
+    next can apply it half way (`HandedRows`): it has weights to apply so (`handed_weight`) and the part's first product
+    finishes such a norm at this number of rows (`accepts_deferred_norm`, `takes_handed_norm`); None otherwise."""
+    norm, part = reader if reader is not None else (None, None)
+    if (norm is None or not hasattr(norm, "handed_weight") or not getattr(part, "accepts_deferred_norm", False)
+            or not hasattr(part, "takes_handed_norm") or not part.takes_handed_norm(n_rows)):
+        return None
+    return norm
+
+
 class RmsNorm(Norm):
     graph_safe = True
 
