@@ -63,12 +63,10 @@ class PageGroup:
         return max(0, -(-new_length // self.page_size) - int(self.n_held[slot]))
 
     def grow(self, slot: int, new_length: int) -> None:
-        first = int(self.n_held[slot])
-        for _ in range(self.pages_for(slot, new_length)):
-            i = int(self.n_held[slot])
-            self.table_host[slot, i] = self.pool.allocate()
-            self.n_held[slot] = i + 1
-        if int(self.n_held[slot]) > first:
+        first, count = int(self.n_held[slot]), self.pages_for(slot, new_length)
+        if count > 0:
+            self.table_host[slot, first:first + count] = self.pool.allocate_many(count)
+            self.n_held[slot] = first + count
             self._changed(slot, first)
 
     def adopt(self, slot: int, pages: Sequence[int]) -> None:

@@ -45,6 +45,19 @@ class PagePool:
         self._refs[page] = 1
         return page
 
+    def allocate_many(self, count: int) -> List[int]:
+        """`count` pages in the order in which `allocate` would hand them out, or `OutOfPages` with nothing changed."""
+        if count > len(self._free):
+            raise OutOfPages(f"{count} pages wanted, {len(self._free)} free")
+        if count <= 0:
+            return []
+        pages = self._free[-count:][::-1]
+        del self._free[-count:]
+        refs = self._refs
+        for page in pages:
+            refs[page] = 1
+        return pages
+
     def retain(self, page: int) -> None:
         self._check(page)
         if self._refs[page] == 0:

@@ -166,7 +166,6 @@ class Runner:
         n_rows, token_arrays = self._validate(entries)
         self.cache.reserve([(e.request, len(e.tokens)) for e in entries])       # OutOfPages: nothing changed
         self._uploads.begin_step()
-        self.cache.sync(self._uploads.put)
 
         meta = np.empty((3, n_rows), dtype=np.int32)                            # tokens, positions, slots
         seg_slot, seg_start, seg_len, seg_pos0, logit_rows = [], [], [], [], []
@@ -184,15 +183,19 @@ class Runner:
         every_row_wanted = logit_rows == list(range(n_rows))
         graph = self._step_graph_for(seg_len, seg_pos0, len(logit_rows), every_row_wanted)
         if graph is not None and graph.calls >= 1:           # a shape that has come before: captured now, replayed from then on
+            self.cache.sync(self._uploads.put)
             logits = graph.run(self._uploads, meta, logit_rows, seg_start, seg_len, seg_pos0, seg_slot)
             self.steps_replayed += 1
         else:
             if graph is not None:
                 graph.calls += 1
+            # the step's numbers and the page tables' changed columns go over in one copy: the first is only laid down, the second sends both
             if logit_rows:
-                meta_dev, rows_dev = self._uploads.put(meta, np.asarray(logit_rows, dtype=np.int32))
+                meta_dev, rows_dev = self._uploads.put(meta, np.asarray(logit_rows, dtype=np.int32), send=False)
             else:
-                meta_dev, rows_dev = self._uploads.put(meta), None
+                meta_dev, rows_dev = self._uploads.put(meta, send=False), None
+            self.cache.sync(self._uploads.put)
+            self._uploads.flush()
             meta_dev = meta_dev.view(3, n_rows)
             ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
                               row_slot=meta_dev[2], seg_slot=seg_slot, seg_start=seg_start, seg_len=seg_len, seg_pos0=seg_pos0,
@@ -351,17 +354,18 @@ class _StepUploads:
         self.host = [torch.empty(capacity, dtype=torch.int32, pin_memory=on_gpu) for _ in range(self.DEPTH)]
         self.dev = [torch.empty(capacity, dtype=torch.int32, device=device) for _ in range(self.DEPTH)]
         self.done = [None] * self.DEPTH
-        self.turn, self.used = 0, 0
+        self.turn, self.used, self.sent = 0, 0, 0
 
     def begin_step(self) -> None:
         self.turn = (self.turn + 1) % self.DEPTH
-        self.used = 0
+        self.used, self.sent = 0, 0
         if self.done[self.turn] is not None:
             self.done[self.turn].synchronize()
 
-    def put(self, *arrays):
+    def put(self, *arrays, send: bool = True):
         """The arrays on the device (int32, flattened): one tensor for one array, a tuple for several, which then
-        go over in one copy."""
+        go over in one copy.  send=False only lays them down in the pinned buffer: they go over with the next `put`
+        that sends, or with `flush`, and what is returned is valid from then on."""
         flats = [np.ascontiguousarray(values, dtype=np.int32).reshape(-1) for values in arrays]
         first, spans = self.used, []
         for flat in flats:
@@ -373,10 +377,16 @@ class _StepUploads:
             self.host[self.turn][a:a + flat.size] = torch.from_numpy(flat)
             spans.append((a, a + flat.size))
             self.used = (a + flat.size + 3) & ~3                # pieces start at multiples of 16 bytes
-        last = spans[-1][1]
-        self.dev[self.turn][first:last].copy_(self.host[self.turn][first:last], non_blocking=True)
+        if send:
+            self.flush()
         pieces = tuple(self.dev[self.turn][a:b] for a, b in spans)
         return pieces[0] if len(pieces) == 1 else pieces
+
+    def flush(self) -> None:
+        """Sends what has been laid down since the last copy."""
+        if self.used > self.sent:
+            self.dev[self.turn][self.sent:self.used].copy_(self.host[self.turn][self.sent:self.used], non_blocking=True)
+            self.sent = self.used
 
     def stage(self, values: np.ndarray) -> torch.Tensor:
         """The values in this step's pinned buffer only (for a copy the caller makes itself, into its own device memory)."""
@@ -386,6 +396,8 @@ class _StepUploads:
             return torch.from_numpy(flat.copy())
         a, b = self.used, self.used + n
         self.used = (b + 3) & ~3
+        if self.sent == a:                                      # (not the ring's to send)
+            self.sent = self.used
         self.host[self.turn][a:b] = torch.from_numpy(flat)
         return self.host[self.turn][a:b]
 
@@ -396,6 +408,8 @@ class _StepUploads:
             return torch.empty(n, dtype=torch.int32, pin_memory=torch.device(self.device).type == "cuda")
         a = self.used
         self.used = (a + n + 3) & ~3
+        if self.sent == a:
+            self.sent = self.used
         return self.host[self.turn][a:a + n]
 
     def end_step(self) -> None:

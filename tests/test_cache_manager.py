@@ -19,6 +19,19 @@ def test_pool_hands_out_page_0_first_and_the_last_freed_next():          # src/m
     assert pool.free_count == 0
 
 
+def test_pool_hands_out_many_pages_in_the_order_of_single_ones():
+    a, b = PagePool(9), PagePool(9)
+    for pool in (a, b):
+        held = [pool.allocate() for _ in range(5)]
+        for p in (held[1], held[3], held[0]):
+            pool.release(p)
+    assert a.allocate_many(4) == [b.allocate() for _ in range(4)] and a.free_count == b.free_count == 3
+    assert all(a.ref_count(p) == b.ref_count(p) for p in range(9))
+    with pytest.raises(OutOfPages):
+        a.allocate_many(4)
+    assert a.free_count == 3 and a.allocate_many(0) == [] and len(a.allocate_many(3)) == 3 and a.free_count == 0
+
+
 def test_pool_misuse_raises():
     pool = PagePool(2)
     p = pool.allocate()
