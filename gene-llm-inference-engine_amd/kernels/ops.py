@@ -529,19 +529,25 @@ def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096,
     measured slower than either neighbour), the context is cut into as many pieces as fit in one round instead, in workgroups
     of 8, 4, 3 or 2 waves, with as few splits as that allows: 65 rows 73 -> 57 us a layer, 96 rows 90 -> 74, 40 rows 46 -> 38,
     56 rows 2.10 -> 1.92 ms a step (heads of 64 channels); 65 rows 127 -> 111 us (heads of 128).  The small batches whose kernel
-    also rotates and stores the new key keep the plain rule: their workgroups are short, and 8 and 16 rows measured 5 and 3 %
-    slower with one round."""
+    also rotates and stores the new key keep the plain rule at heads of 64 channels: their workgroups are short, and 8 and 16 rows
+    measured 5 and 3 % slower with one round.  At 128 channels that kernel's registers leave room for 8 waves a compute unit, and
+    there one round is the faster cut whenever the plain rule needs more (8 rows: 30 -> 27 us a layer at a context of 2,100, 35 ->
+    29 at 3,000; the step of the 8B shape 4.82 -> 4.79 ms at 8 rows, 5.47 -> 5.31 at 16)."""
     group = n_heads // n_kv
     groups = n_decode * n_kv * ((group + 15) // 16)
     max_waves = min(8, lib().gi_attention_decode_max_waves(hd))
     base = _decode_plain_shape(groups, span, max_waves, target_waves)
-    if target_waves != 4096 or fused:
+    if target_waves != 4096 or (fused and hd < 128):
         return base
     gh = min(group, 16)
     rounds = groups * base[0] / _decode_places(hd, fused, base[1], gh)
-    short_last_round = rounds > 1 and 0 < rounds - int(rounds) < (0.5 if base[0] > 1 else 0.3)
-    if not (short_last_round or 5 <= base[1] <= 7):
-        return base
+    if fused:                        # (heads of 128 channels: 8 waves a compute unit, and a second round costs what it brings)
+        if rounds <= 1:
+            return base
+    else:
+        short_last_round = rounds > 1 and 0 < rounds - int(rounds) < (0.5 if base[0] > 1 else 0.3)
+        if not (short_last_round or 5 <= base[1] <= 7):
+            return base
     best = None
     for n_waves in (8, 4, 3, 2):
         if n_waves > max_waves:
