@@ -592,33 +592,44 @@ struct DecodeShape {                                      // waves a workgroup m
     static constexpr int MAX_WAVES = HD <= 128 ? 8 : 4;
 };
 
-// Channels c .. c+7 of a head and what their rotation needs, as loaded (`src` points at the head's
-// channel 0): the loads are issued early and the rotation is taken when the values are needed.
-struct Unrotated8 {
-    float4 a[2], b[2], cs[2], sn[2];
+// Channels c .. c+7 of a head and their partners in the other half, as loaded (`src` points at the head's channel 0), and the
+// cosines and sines of their angles, which the row's queries and its key share: the loads are issued early and the rotation is
+// taken when the values are needed.
+struct Pairs8 {
+    float4 a[2], b[2];
+};
+struct Angles8 {
+    float4 cs[2], sn[2];
     bool low;
 };
-__device__ __forceinline__ Unrotated8 load_unrotated8(const float* __restrict__ src, const float* __restrict__ cos_row,
-                                                      const float* __restrict__ sin_row, int c, int half) {
-    Unrotated8 u;
+__device__ __forceinline__ Angles8 load_angles8(const float* __restrict__ cos_row, const float* __restrict__ sin_row, int c, int half) {
+    Angles8 u;
     u.low = c < half;
     const int cl = u.low ? c : c - half;
 #pragma unroll
     for (int h4 = 0; h4 < 2; ++h4) {
-        u.a[h4] = *reinterpret_cast<const float4*>(src + cl + 4 * h4);
-        u.b[h4] = *reinterpret_cast<const float4*>(src + cl + half + 4 * h4);
         u.cs[h4] = cos_row ? *reinterpret_cast<const float4*>(cos_row + cl + 4 * h4) : float4{1.f, 1.f, 1.f, 1.f};
         u.sn[h4] = sin_row ? *reinterpret_cast<const float4*>(sin_row + cl + 4 * h4) : float4{0.f, 0.f, 0.f, 0.f};
     }
     return u;
 }
+__device__ __forceinline__ Pairs8 load_pairs8(const float* __restrict__ src, int c, int half) {
+    Pairs8 u;
+    const int cl = c < half ? c : c - half;
+#pragma unroll
+    for (int h4 = 0; h4 < 2; ++h4) {
+        u.a[h4] = *reinterpret_cast<const float4*>(src + cl + 4 * h4);
+        u.b[h4] = *reinterpret_cast<const float4*>(src + cl + half + 4 * h4);
+    }
+    return u;
+}
 __device__ __forceinline__ float rotate1(bool low, float a, float b, float c, float s) { return low ? a * c - b * s : a * s + b * c; }
-__device__ __forceinline__ uint4 rotated8(const Unrotated8& u) {
+__device__ __forceinline__ uint4 rotated8(const Pairs8& p, const Angles8& u) {
     uint32_t w[4];
 #pragma unroll
     for (int h4 = 0; h4 < 2; ++h4) {
-        w[2 * h4] = pack2(rotate1(u.low, u.a[h4].x, u.b[h4].x, u.cs[h4].x, u.sn[h4].x), rotate1(u.low, u.a[h4].y, u.b[h4].y, u.cs[h4].y, u.sn[h4].y));
-        w[2 * h4 + 1] = pack2(rotate1(u.low, u.a[h4].z, u.b[h4].z, u.cs[h4].z, u.sn[h4].z), rotate1(u.low, u.a[h4].w, u.b[h4].w, u.cs[h4].w, u.sn[h4].w));
+        w[2 * h4] = pack2(rotate1(u.low, p.a[h4].x, p.b[h4].x, u.cs[h4].x, u.sn[h4].x), rotate1(u.low, p.a[h4].y, p.b[h4].y, u.cs[h4].y, u.sn[h4].y));
+        w[2 * h4 + 1] = pack2(rotate1(u.low, p.a[h4].z, p.b[h4].z, u.cs[h4].z, u.sn[h4].z), rotate1(u.low, p.a[h4].w, p.b[h4].w, u.cs[h4].w, u.sn[h4].w));
     }
     return uint4{w[0], w[1], w[2], w[3]};
 }
@@ -641,15 +652,16 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
     const int head = g * group + head_in_group;
     // The unrotated queries depend on the row alone: their loads go out first, ahead of the chain
     // position -> page table -> keys.
-    [[maybe_unused]] Unrotated8 q_raw[KSTEPS];
-    [[maybe_unused]] const float* cos_row = nullptr;
-    [[maybe_unused]] const float* sin_row = nullptr;
+    [[maybe_unused]] Pairs8 q_raw[KSTEPS];
+    [[maybe_unused]] Angles8 angles[KSTEPS];
     if constexpr (FUSED) {
-        cos_row = cos_t ? cos_t + (size_t)row * (HD / 2) : nullptr;
-        sin_row = sin_t ? sin_t + (size_t)row * (HD / 2) : nullptr;
+        const float* cos_row = cos_t ? cos_t + (size_t)row * (HD / 2) : nullptr;
+        const float* sin_row = sin_t ? sin_t + (size_t)row * (HD / 2) : nullptr;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) angles[s] = load_angles8(cos_row, sin_row, 32 * s + 8 * q4, HD / 2);
         if (head_ok) {
 #pragma unroll
-            for (int s = 0; s < KSTEPS; ++s) q_raw[s] = load_unrotated8(qf + (size_t)row * ldq + (size_t)head * HD, cos_row, sin_row, 32 * s + 8 * q4, HD / 2);
+            for (int s = 0; s < KSTEPS; ++s) q_raw[s] = load_pairs8(qf + (size_t)row * ldq + (size_t)head * HD, 32 * s + 8 * q4, HD / 2);
         }
     }
     const int my_pos = pos[row];
@@ -668,18 +680,7 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
     const bf16_t* kbase = cache + (long)g * page_size * HD;
     const bf16_t* vbase = cache + v_plane + (long)g * HD * page_size;
 
-    // the row's own key and value, likewise before the page table is read
     const bool has_own = FUSED && kf != nullptr && begin < end && end == my_pos + 1;     // this wave's piece holds the row's own position
-    [[maybe_unused]] Unrotated8 k_raw[KSTEPS];
-    [[maybe_unused]] float v_raw[DT];
-    if constexpr (FUSED) {
-        if (has_own) {
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) k_raw[ks] = load_unrotated8(kf + (size_t)row * ldk + (size_t)g * HD, cos_row, sin_row, 32 * ks + 8 * q4, HD / 2);
-#pragma unroll
-            for (int i = 0; i < DT; ++i) v_raw[i] = vf[(size_t)row * ldv + (size_t)g * HD + 16 * i + r];
-        }
-    }
 
     // Loads run ahead of the products: the keys of the next 32 positions and the values of these 32
     // are requested before the scores of these 32 are taken.  An address beyond the row's own range
@@ -700,14 +701,25 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
     uint4 own_key[KSTEPS];
     bf16_t own_value[DT];
     if constexpr (FUSED) {
+        // The row's own key and value (for the one wave whose piece ends at the row's position) are asked for when the first keys
+        // are on their way and rotated behind the queries: at heads of 128 channels queries, key and angles at once are 200
+        // registers a lane, which halves the waves a compute unit holds.
+        [[maybe_unused]] Pairs8 k_raw[KSTEPS];
+        [[maybe_unused]] float v_raw[DT];
+        if (has_own) {
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) qreg[s] = as_bf16x8(head_ok ? rotated8(q_raw[s]) : uint4{0, 0, 0, 0});
+            for (int ks = 0; ks < KSTEPS; ++ks) k_raw[ks] = load_pairs8(kf + (size_t)row * ldk + (size_t)g * HD, 32 * ks + 8 * q4, HD / 2);
+#pragma unroll
+            for (int i = 0; i < DT; ++i) v_raw[i] = vf[(size_t)row * ldv + (size_t)g * HD + 16 * i + r];
+        }
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) qreg[s] = as_bf16x8(head_ok ? rotated8(q_raw[s], angles[s]) : uint4{0, 0, 0, 0});
         if (has_own) {
             bf16_t* page = cache + (long)tab[page_index(my_pos)] * page_stride;
             const int place = place_of(my_pos);
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) {
-                own_key[ks] = rotated8(k_raw[ks]);
+                own_key[ks] = rotated8(k_raw[ks], angles[ks]);
                 if (r == 0 && hg == 0)
                     *reinterpret_cast<uint4*>(page + (long)g * page_size * HD + (long)place * HD + 32 * ks + 8 * q4) = own_key[ks];
             }
