@@ -673,6 +673,10 @@ constexpr int KB = 2 * SK, X_STRIDE = KB + 8;         // k per block of the work
 // The kernel for at most 16 rows: a thread keeps 8 pieces while the products run (more would cost the kernel its second
 // workgroup per compute unit); 64 threads share a row where there are at most 8 rows, 32 otherwise.
 constexpr int SLIM_PIECES = 8;
+// Outputs of fewer than so many strips of 16 weight rows take strips of 8, twice the workgroups; with up to 8 rows of A, where a
+// strip of 8 leaves no lane idle (FOLD = 1 below), of fewer than twice as many (measured at N = 4096 to 6144: 1 to 2 % of the
+// decode step at 1 to 8 rows, and 7 % the other way at 12 and 16 rows).
+constexpr int SLIM_NARROW_STRIPS = 256;
 __host__ __device__ constexpr int slim_max_parts(int M) { return SLIM_PIECES * (M <= 8 ? 64 : 32); }
 // The kernels for 17 to 128 rows: the kernel that adds the partial sums onto x writes one piece per 1024 columns.
 constexpr int REDUCE_COLUMNS = 1024, REDUCE_MAX_PARTS = 8;
@@ -1296,7 +1300,8 @@ static bool takes_slim(int M, int N, int K) {
 }
 
 // Workgroups of the slim kernel for an output of N columns that is not gated: the pieces a row's sum of squares comes in.
-static int slim_parts(int N) { return (N + 15) / 16 >= 256 ? (N + 15) / 16 : (N + 7) / 8; }
+static bool slim_wide_strips(int M, int N) { return (N + 15) / 16 > (M <= 8 ? 2 * SLIM_NARROW_STRIPS : SLIM_NARROW_STRIPS) - 1; }
+static int slim_parts(int M, int N) { return slim_wide_strips(M, N) ? (N + 15) / 16 : (N + 7) / 8; }
 
 static int launch_slim(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in,
                        NormOut norm_out, hipStream_t stream) {
@@ -1309,7 +1314,7 @@ static int launch_slim(const void* A, const void* W, void* C, int epi, int M, in
     if (epi == EPI_GATED_BF16) {
         dim3 grid(N / 32);
         SLIM(2, 16, EPI_GATED_BF16);
-    } else if ((N + 15) / 16 >= 256) {
+    } else if (slim_wide_strips(M, N)) {
         dim3 grid((N + 15) / 16);
         if (epi == EPI_STORE_F32) SLIM(1, 16, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 16, EPI_ADD_F32); else SLIM(1, 16, EPI_STORE_BF16);
     } else {                                   // a narrow output: strips of 8 rows, twice the workgroups
@@ -1479,7 +1484,7 @@ static int launch_large(const void* A, const void* W, void* C, int epi, int M, i
 // onto the rows.
 GI_API int gi_gemm_bf16_norm_parts(int M, int N, int K) {
     if (takes_slim(M, N, K)) {
-        const int parts = slim_parts(N);
+        const int parts = slim_parts(M, N);
         return parts <= slim_max_parts(M) ? parts : 0;
     }
     if (takes_slim_tiles(M, N, K, EPI_ADD_F32)) return (N + 15) / 16 <= TILES_MAX_PARTS ? (N + 15) / 16 : 0;
