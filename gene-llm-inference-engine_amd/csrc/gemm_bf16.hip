@@ -310,7 +310,7 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int EPI>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
                                                              int M, int N, int K, long lda, long ldw, long ldc, int k_per_split,
-                                                             long split_stride, NormIn norm_in, RopeStore rope) {
+                                                             long split_stride, NormIn norm_in, RopeStore rope, NormOut norm_out) {
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int ROWS = BM + BN, STAGE_BYTES = ROWS * 128, LOADS = ROWS / 8 / (WAVES_M * WAVES_N);      // loads per wave and stage
     static_assert(ROWS % (8 * WAVES_M * WAVES_N) == 0, "the rows of a stage must divide among the waves' loads");
@@ -407,6 +407,44 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
         __syncthreads();
         qkv_tile_rope_store<64 * WAVES_M * WAVES_N>(tile, places, m0, n0, M, N, rope);
         return;
+    }
+    if constexpr (EPI == EPI_ADD_F32 && BM == 128 && BN == 128 && STAGES * STAGE_BYTES >= 128 * 128 * 4) {
+        if (norm_out.scaled != nullptr) {
+            // The sums go onto 32-bit rows whose next reader is a norm: the tile is laid into LDS (the ring is free once everyone
+            // has read the last block) and leaves row by row, 32 threads a row with four columns each: the rows' new values, the
+            // same times the norm's weights in bfloat16, and the tile's piece of every row's sum of squares (N is a multiple of 128).
+            constexpr int NT = 64 * WAVES_M * WAVES_N;
+            __syncthreads();
+            float* tile = reinterpret_cast<float*>(ring);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        tile[(wm + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3)) * 128 + wn + j * 32 + (lane & 31)] = acc[i][j][v];
+            __syncthreads();
+            const int c4 = (tid & 31) * 4;
+            const float4 g = *reinterpret_cast<const float4*>(norm_out.g + n0 + c4);
+            for (int row = tid >> 5; row < 128; row += NT / 32) {
+                const int m = m0 + row;
+                float square = 0.f;
+                if (m < M) {
+                    const float4 t = *reinterpret_cast<const float4*>(tile + row * 128 + c4);
+                    float4* at = reinterpret_cast<float4*>((float*)C + (size_t)m * ldc + n0 + c4);
+                    float4 x = *at;
+                    x.x += t.x; x.y += t.y; x.z += t.z; x.w += t.w;
+                    *at = x;
+                    *reinterpret_cast<uint2*>(norm_out.scaled + (size_t)m * norm_out.ld + n0 + c4) =
+                        uint2{f32x2_to_bf16x2(g.x * x.x, g.y * x.y), f32x2_to_bf16x2(g.z * x.z, g.w * x.w)};
+                    square = x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+                }
+#pragma unroll
+                for (int off = 16; off > 0; off >>= 1) square += __shfl_xor(square, off, 64);
+                if ((tid & 31) == 0 && m < M) norm_out.squares[(size_t)m * gridDim.x + blockIdx.x] = square;
+            }
+            return;
+        }
     }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -1407,10 +1445,19 @@ static int launch_skinny(const void* A, const void* W, void* C, int epi, int M, 
 
 static const RopeStore NO_ROPE = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, nullptr, nullptr, 0, 0, 0, 0, 0};
 
+// The pieces per row that a product of more than 128 rows writes when it hands a norm on, 0 if it cannot: one per tile of 128 columns
+// from the epilogue of the kernel with tiles of 128 x 128, one per 1024 columns where k is shared out and a second kernel adds the
+// shares; not from the ping-pong kernel.
+static int large_norm_parts(int M, int N, int K) {
+    if (K % PK != 0 || N < 128 || takes_pingpong(M, N)) return 0;
+    if (gi_gemm_bf16_piped_splits(M, N, K) > 1) return N % REDUCE_COLUMNS == 0 && N / REDUCE_COLUMNS <= REDUCE_MAX_PARTS ? N / REDUCE_COLUMNS : 0;
+    return N % 128 == 0 && N / 128 <= PIPED_MAX_PARTS ? N / 128 : 0;
+}
+
 // More than 128 rows, K a multiple of 64, 128 columns or more: the kernels that load their operands straight into LDS.
 // `rope` != null: the sums are those of an attention layer's q/k/v product and go where it says (`epi` is then not looked at).
 static int launch_large(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, float* scratch,
-                        long scratch_floats, NormIn norm_in, const RopeStore* rope, hipStream_t stream) {
+                        long scratch_floats, NormIn norm_in, const RopeStore* rope, hipStream_t stream, NormOut norm_out = NO_NORM_OUT) {
 #define PIPED(BM_, BN_, WM_, WN_, ST_, EPI_, OUT_, LDC_, SPLITS_, KPS_, SLAB_, NORM_, ROPE_)                                            \
     do {                                                                                                                                \
         constexpr int bytes = ST_ * (BM_ + BN_) * 128;                                                                                  \
@@ -1422,7 +1469,7 @@ static int launch_large(const void* A, const void* W, void* C, int epi, int M, i
         }                                                                                                                               \
         dim3 grid((N + BN_ - 1) / BN_, (M + BM_ - 1) / BM_, SPLITS_);                                                                   \
         gemm_bf16_piped_kernel<BM_, BN_, WM_, WN_, ST_, EPI_><<<grid, 64 * WM_ * WN_, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, OUT_, M, N, K, lda, \
-                                                                                                        ldw, LDC_, KPS_, SLAB_, NORM_, ROPE_); \
+                                                                                                        ldw, LDC_, KPS_, SLAB_, NORM_, ROPE_, norm_out); \
     } while (0)
 #define PIPED_EPI(BM_, BN_, WM_, WN_, ST_)                                                                                              \
     do {                                                                                                                                \
@@ -1444,12 +1491,13 @@ static int launch_large(const void* A, const void* W, void* C, int epi, int M, i
             GI_CHECK_LAUNCH("gemm_bf16 (reduce, rotate, store)");
             return 0;
         }
-        return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream, norm_in);
+        return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream, norm_in, norm_out);
     }
     // Measured at 2,048 rows (K = 2048 and 8192): where 256 x 256 tiles give every compute unit one or more, they halve
     // the traffic into LDS and run the two groups of waves out of step (the ping-pong kernel); otherwise 128 x 128, two
     // workgroups per unit with two stages each when there are enough tiles, else one workgroup of eight waves with four stages.
     const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    GI_REQUIRE(norm_out.scaled == nullptr || (!takes_pingpong(M, N) && large_norm_parts(M, N, K) > 0), "gemm_bf16: a product of M %d, N %d, K %d hands no norm on", M, N, K);
     if (takes_pingpong(M, N) && rope == nullptr) {     // a 256 x 256 tile or more for every compute unit: the ping-pong kernel
 #define PINGPONG(EPI_)                                                                                                                  \
     do {                                                                                                                                \
@@ -1488,7 +1536,8 @@ GI_API int gi_gemm_bf16_norm_parts(int M, int N, int K) {
         return parts <= slim_max_parts(M) ? parts : 0;
     }
     if (takes_slim_tiles(M, N, K, EPI_ADD_F32)) return (N + 15) / 16 <= TILES_MAX_PARTS ? (N + 15) / 16 : 0;
-    if (M <= 16 || M > SKINNY_MAX_ROWS || gi_gemm_bf16_skinny_splits(N, K) == 0) return 0;
+    if (M > SKINNY_MAX_ROWS) return large_norm_parts(M, N, K);
+    if (M <= 16 || gi_gemm_bf16_skinny_splits(N, K) == 0) return 0;
     return N % REDUCE_COLUMNS == 0 && N / REDUCE_COLUMNS <= REDUCE_MAX_PARTS ? N / REDUCE_COLUMNS : 0;
 }
 
@@ -1534,7 +1583,12 @@ GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dty
         GI_REQUIRE(squares_in == nullptr || parts_in <= consumer_max_parts(M), "gemm_bf16: %d pieces of a sum of squares, at most %d", parts_in, consumer_max_parts(M));
         return launch_slim_tiles(A, W, C, epi, M, N, K, lda, ldw, ldc, norm_in, norm_out, stream);
     }
-    GI_REQUIRE(M <= SKINNY_MAX_ROWS, "gemm_bf16: no norm is handed on by or to a product of %d rows", M);
+    if (M > SKINNY_MAX_ROWS) {                   // the rows of prompts: a norm is handed on (to a q/k/v product that takes it), none is taken
+        GI_REQUIRE(squares_in == nullptr && scaled_out != nullptr, "gemm_bf16: a product of %d rows takes no norm handed on", M);
+        GI_REQUIRE(ldc % 4 == 0 && ld_scaled % 4 == 0 && ((uintptr_t)C & 15) == 0 && ((uintptr_t)scaled_out & 7) == 0 && ((uintptr_t)g & 15) == 0,
+                   "gemm_bf16: handing a norm on from %d rows needs aligned operands", M);
+        return launch_large(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, NO_NORM_IN, nullptr, stream, norm_out);
+    }
     return launch_skinny(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, norm_in, norm_out, stream);
 }
 

@@ -16,8 +16,9 @@ import torch
 from ..cache.needs import PagedKvNeed
 from ..kernels import ops
 from ..weights.loader import TensorNeed
-from .base import Mixer, position_class, register_mixer
-from .linear import activation_dtype_for, linear, linear_onto, rows_for_product
+from .base import Mixer, PositionEncoding, position_class, register_mixer
+from .linear import activation_dtype_for, linear, linear_onto
+from .norm import HandedRows, NormedRows
 
 
 def qkv_rotate_store_attend(h, w_qkv, ctx, cache, *, n_heads, n_kv_heads, head_dim, position=None, window=None, in_dtype=None,
@@ -43,9 +44,12 @@ def qkv_rotate_store_attend(h, w_qkv, ctx, cache, *, n_heads, n_kv_heads, head_d
             and cache.kv.dtype == torch.bfloat16 and in_dtype == torch.bfloat16
             and ops.gemm_bf16_qkv_rope_store_takes(T, w_qkv.shape[0], w_qkv.shape[1], head_dim)):
         # the product's own last step (the kernel that adds up the shares of k, or the epilogue over a tile) rotates and writes the pages
-        rows, norm_in = rows_for_product(h, w_qkv)
-        if norm_in is not None and norm_in[0].shape[1] > ops.gemm_bf16_qkv_rope_store_max_parts(T, w_qkv.shape[0], w_qkv.shape[1]):
-            rows, norm_in = h.materialize(), None
+        # (this product finishes a norm handed on at every number of rows it is taken at, if the pieces are few enough)
+        if (isinstance(h, HandedRows) and h.scaled.stride(0) % 8 == 0 and h.scaled.data_ptr() % 16 == 0
+                and h.squares.shape[1] <= ops.gemm_bf16_qkv_rope_store_max_parts(T, w_qkv.shape[0], w_qkv.shape[1])):
+            rows, norm_in = h.scaled, (h.squares, h.eps)
+        else:
+            rows, norm_in = (h.materialize() if isinstance(h, NormedRows) else h), None
         if ops.gemm_bf16_supports(rows, w_qkv, att):
             q_rot = torch.empty((T, a_dim), dtype=torch.bfloat16, device=ctx.device)
             ops.gemm_bf16_qkv_rope_store(rows, w_qkv, cos, sin, ctx.row_pos, ctx.row_slot, cache.table, q_rot, cache.kv, n_heads, n_kv_heads,
@@ -102,7 +106,13 @@ class Attention(Mixer):
         return PagedKvNeed(spec.n_kv_heads, spec.head_dim, spec.window)
 
     def takes_handed_norm(self, n_rows: int) -> bool:
-        return self.in_dtype == torch.bfloat16 and ops.gemm_bf16_takes_norm(n_rows, self.w_qkv.shape[0], self.w_qkv.shape[1])
+        if self.in_dtype != torch.bfloat16:
+            return False
+        if ops.gemm_bf16_takes_norm(n_rows, self.w_qkv.shape[0], self.w_qkv.shape[1]):
+            return True
+        # the rows of prompts: the q/k/v product that rotates and fills the pages itself finishes the norm, where it serves
+        half_split = self.position is None or getattr(type(self.position), "half_split_tables", None) is not PositionEncoding.half_split_tables
+        return half_split and ops.gemm_bf16_qkv_rope_store_takes(n_rows, self.w_qkv.shape[0], self.w_qkv.shape[1], self.spec.head_dim)
 
     def forward(self, h, residual, ctx, cache, then=None):
         s = self.spec

@@ -32,18 +32,6 @@ def linear(a, weight: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
     return ops.gemm_exact(a, weight, out, accumulate)
 
 
-def rows_for_product(a, weight: torch.Tensor, gated: bool = False):
-    """What a product with `weight` reads for `a`: the rows, and `norm_in` for `ops.gemm_bf16` if they are a norm half applied
-    that this product can finish (None otherwise: the rows are then whole)."""
-    if isinstance(a, HandedRows):
-        if (weight.dtype == torch.bfloat16 and a.scaled.stride(0) % 8 == 0 and a.scaled.data_ptr() % 16 == 0
-                and ops.gemm_bf16_takes_norm(a.scaled.shape[0], weight.shape[0], weight.shape[1], gated)):
-            return a.scaled, (a.squares, a.eps)
-    if isinstance(a, NormedRows):
-        a = a.materialize()
-    return a, None
-
-
 def linear_onto(a: torch.Tensor, weight: torch.Tensor, residual: torch.Tensor, then=None):
     """residual += a @ weight.T.  `then`: the norm that reads `residual` next, if it and its reader can take it half applied
     (see `HandedRows`); the product then also does the norm's share and the `HandedRows` are returned, None otherwise."""

@@ -236,6 +236,34 @@ def test_norm_handed_from_one_product_to_the_next(m, d, k1, n2, gated):
     assert err_handed < 1.5 * err_usual + 1e-6, (err_handed, err_usual)
 
 
+@pytest.mark.parametrize("m,d,k1", [(2048, 2048, 8192), (1100, 2048, 2048), (300, 2048, 2048), (2048, 3072, 8192), (700, 1024, 512), (130, 256, 192),
+                                    (4100, 3072, 256)])
+def test_norm_handed_on_by_a_product_of_many_rows(m, d, k1):
+    """The rows of prompts: the product that adds onto the residual writes g * x and the pieces of the rows' sums of squares from
+    its tiles' epilogues (one piece per 128 columns), or from the kernel that adds the shares of k (one per 1024).  The rows are
+    what the plain product leaves, bit for bit; sizes at which the kernels do not do it are refused."""
+    o = ops()
+    a = randn(m, k1, dtype=torch.bfloat16, seed=1)
+    w1 = randn(d, k1, dtype=torch.bfloat16, seed=2, scale=0.05)
+    g = (1 + 0.1 * randn(d, seed=4)).float()
+    x0 = randn(m, d, seed=5)
+    parts = o.gemm_bf16_norm_parts(m, d, k1)
+    assert parts in (d // 128, d // 1024), parts
+    plain_x = x0.clone()
+    o.gemm_bf16(a, w1, plain_x, accumulate=True)
+    x, scaled, squares = x0.clone(), torch.full((m, d), float("nan"), dtype=torch.bfloat16, device=DEV), torch.full((m, parts), float("nan"), device=DEV)
+    o.gemm_bf16(a, w1, x, accumulate=True, norm_out=(g, scaled, squares))
+    assert torch.equal(x, plain_x)
+    assert torch.equal(scaled, (g * x).to(torch.bfloat16))
+    assert rel(squares.double().sum(1), (x.double() ** 2).sum(1)) < 1e-6
+    width = d // parts
+    assert rel(squares.double(), (x.double() ** 2).view(m, parts, width).sum(2)) < 1e-6            # every piece is its columns' sum
+    assert o.gemm_bf16_norm_parts(8192, 8192, 512) == 0 and o.gemm_bf16_norm_parts(300, 200, 512) == 0        # the ping-pong kernel; a ragged width
+    with pytest.raises(o.KernelError):
+        o.gemm_bf16(randn(8192, 512, dtype=torch.bfloat16, seed=1), randn(8192, 512, dtype=torch.bfloat16, seed=2), torch.zeros(8192, 8192, device=DEV),
+                    accumulate=True, norm_out=((1 + 0 * randn(8192, seed=4)).float(), torch.empty(8192, 8192, dtype=torch.bfloat16, device=DEV), torch.empty(8192, 64, device=DEV)))
+
+
 @pytest.mark.parametrize("m,hidden,n_heads,n_kv,hd,page_size,rotate,handed", [(64, 2048, 32, 8, 64, 16, True, True), (40, 2048, 32, 8, 64, 16, True, False),
                                                                               (128, 3072, 24, 8, 128, 16, True, True), (33, 512, 6, 1, 32, 8, False, False),
                                                                               (17, 4096, 32, 8, 128, 32, True, False), (100, 1024, 2, 1, 256, 16, True, True),
