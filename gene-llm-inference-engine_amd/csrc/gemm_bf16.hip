@@ -105,6 +105,13 @@ __device__ __forceinline__ void tile_row_scales(float* scales, const NormIn& n, 
     }
 }
 
+// The factor of one row: rsqrt(mean square + eps) from the pieces of its sum of squares, read and added one by one.
+__device__ __forceinline__ float row_scale_of(const NormIn& n, int row) {      // a few pieces: read and added one by one
+    float sum = 0.f;
+    for (int p = 0; p < n.parts; ++p) sum += n.squares[(size_t)row * n.parts + p];
+    return 1.0f / sqrtf(sum / (float)n.dim + n.eps);
+}
+
 // Where the rows of a tile of 128 go in the cache: per row the page's offset and the place in the page, and per group of
 // eight rows whether they are eight consecutive positions of one request that begin at a multiple of eight (rows of a prompt).
 struct TilePlaces {
@@ -484,7 +491,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
 // 23 clocks when nothing else runs and 70 to 140 here, wherever in the two phases it is put.
 template <int BN, int EPI>
 __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
-                                                                int M, int N, int K, long lda, long ldw, long ldc) {
+                                                                int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in) {
     static_assert(BN == 256, "the sharing of the loads below is written for 256 x 256 tiles");
     constexpr int BM = 256, WAVES = 8, WM = 64, WN = BN / 2, TM = WM / 32, TN = WN / 32;
     constexpr int ROWS = BM + BN, STAGE_BYTES = ROWS * 128, LOADS = ROWS / 8 / WAVES;      // a wave-wide load fills 8 rows of 128 bytes
@@ -548,6 +555,28 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const bf16_t* _
     if (n_k > 1) {
 #pragma unroll
         for (int i = 0; i < 2; ++i) load_rows(source((wave * 2 + i) * 8 + (lane >> 3)), (wave * 2 + i) * 8, 1);
+    }
+    // With a norm handed on (the gated product: the rows of A are g * x, and the results lack the rows' rsqrt(mean square + eps)),
+    // the tile's 256 rows' factors are worked out once, a thread a row (16-byte reads of the row's pieces where they allow it: a lane
+    // that asked for its rows' pieces one by one cost the kernel 18 us at 16 pieces), and wait in LDS for the epilogue (asked for behind the first block's loads; the
+    // barriers of the loop lie between this write and the epilogue's reads).
+    __shared__ float row_scale[EPI == EPI_GATED_BF16 ? BM : 1];
+    if constexpr (EPI == EPI_GATED_BF16) {
+        if (norm_in.squares != nullptr) {
+            if (tid < BM) {
+                const float* pieces = norm_in.squares + (size_t)min(m0 + tid, M - 1) * norm_in.parts;
+                float sum = 0.f;
+                if ((norm_in.parts & 3) == 0 && ((uintptr_t)norm_in.squares & 15) == 0) {
+                    for (int p = 0; p < norm_in.parts; p += 4) {
+                        const float4 v = *reinterpret_cast<const float4*>(pieces + p);
+                        sum += v.x; sum += v.y; sum += v.z; sum += v.w;
+                    }
+                } else {
+                    for (int p = 0; p < norm_in.parts; ++p) sum += pieces[p];
+                }
+                row_scale[tid] = 1.0f / sqrtf(sum / (float)norm_in.dim + norm_in.eps);
+            }
+        }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     phase_barrier();
@@ -615,8 +644,9 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const bf16_t* _
                     const int j = 4 * part + jj;
 #pragma unroll
                     for (int q = 0; q < 2; ++q) {
-                        const uint2 packed = {f32x2_to_bf16x2(silu_gate_fast(acc[i][j][4 * q], acc[i][j][4 * q + 8]), silu_gate_fast(acc[i][j][4 * q + 1], acc[i][j][4 * q + 9])),
-                                              f32x2_to_bf16x2(silu_gate_fast(acc[i][j][4 * q + 2], acc[i][j][4 * q + 10]), silu_gate_fast(acc[i][j][4 * q + 3], acc[i][j][4 * q + 11]))};
+                        const float rs = norm_in.squares != nullptr ? row_scale[wm + i * 32 + (lane & 31)] : 1.0f;
+                        const uint2 packed = {f32x2_to_bf16x2(silu_gate_fast(acc[i][j][4 * q] * rs, acc[i][j][4 * q + 8] * rs), silu_gate_fast(acc[i][j][4 * q + 1] * rs, acc[i][j][4 * q + 9] * rs)),
+                                              f32x2_to_bf16x2(silu_gate_fast(acc[i][j][4 * q + 2] * rs, acc[i][j][4 * q + 10] * rs), silu_gate_fast(acc[i][j][4 * q + 3] * rs, acc[i][j][4 * q + 11] * rs))};
                         *reinterpret_cast<uint2*>(mine + (i * 32 + (lane & 31)) * STAGE_ROW + (jj * 16 + 8 * q + 4 * (lane >> 5)) * 2) = packed;
                     }
                 }
@@ -719,11 +749,6 @@ __host__ __device__ constexpr int slim_max_parts(int M) { return SLIM_PIECES * (
 // The kernels for 17 to 128 rows: the kernel that adds the partial sums onto x writes one piece per 1024 columns.
 constexpr int REDUCE_COLUMNS = 1024, REDUCE_MAX_PARTS = 8;
 
-__device__ __forceinline__ float row_scale_of(const NormIn& n, int row) {      // a few pieces: read and added one by one
-    float sum = 0.f;
-    for (int p = 0; p < n.parts; ++p) sum += n.squares[(size_t)row * n.parts + p];
-    return 1.0f / sqrtf(sum / (float)n.dim + n.eps);
-}
 
 // The same for all M rows into `scales` (LDS, at least 32 floats or M), by a workgroup of 512 threads; the caller puts a barrier
 // before the use.  With many pieces (the writer was a kernel for at most 32 rows with a piece per workgroup: at most
@@ -1498,6 +1523,8 @@ static int launch_large(const void* A, const void* W, void* C, int epi, int M, i
     // workgroups per unit with two stages each when there are enough tiles, else one workgroup of eight waves with four stages.
     const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     GI_REQUIRE(norm_out.scaled == nullptr || (!takes_pingpong(M, N) && large_norm_parts(M, N, K) > 0), "gemm_bf16: a product of M %d, N %d, K %d hands no norm on", M, N, K);
+    GI_REQUIRE(norm_in.squares == nullptr || rope != nullptr || (epi == EPI_GATED_BF16 && takes_pingpong(M, N) && norm_in.parts <= PIPED_MAX_PARTS),
+               "gemm_bf16: a product of M %d, N %d, K %d takes no norm handed on in %d pieces", M, N, K, norm_in.parts);
     if (takes_pingpong(M, N) && rope == nullptr) {     // a 256 x 256 tile or more for every compute unit: the ping-pong kernel
 #define PINGPONG(EPI_)                                                                                                                  \
     do {                                                                                                                                \
@@ -1509,7 +1536,7 @@ static int launch_large(const void* A, const void* W, void* C, int epi, int M, i
             raised = true;                                                                                                              \
         }                                                                                                                               \
         dim3 grid((N + 255) / 256, (M + 255) / 256);                                                                                    \
-        gemm_bf16_pingpong_kernel<256, EPI_><<<grid, 512, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc); \
+        gemm_bf16_pingpong_kernel<256, EPI_><<<grid, 512, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in); \
     } while (0)
         GI_REQUIRE(lda < (1L << 22) && ldw < (1L << 22), "gemm_bf16: row strides %ld, %ld are too large for the tile-relative addressing", lda, ldw);
         if (epi == EPI_STORE_F32) PINGPONG(EPI_STORE_F32); else if (epi == EPI_ADD_F32) PINGPONG(EPI_ADD_F32);
@@ -1545,7 +1572,8 @@ GI_API int gi_gemm_bf16_norm_parts(int M, int N, int K) {
 // of as many rows.
 GI_API int gi_gemm_bf16_takes_norm(int M, int N, int K, int gated) {
     if (takes_slim(M, N, K) || takes_slim_tiles(M, N, K, gated ? EPI_GATED_BF16 : EPI_STORE_F32)) return 1;
-    if (M > SKINNY_MAX_ROWS) return 0;
+    if (M > SKINNY_MAX_ROWS)                      // the rows of prompts: the gated product on the ping-pong kernel scales in its epilogue
+        return gated && K % PK == 0 && N >= 128 && takes_pingpong(M, N) ? 1 : 0;
     if (gi_gemm_bf16_skinny_splits(N, K) == 0) return 1;      // the weight-streaming kernel finishes its columns and scales them
     return M > 32 && !gated ? 1 : 0;                          // the kernel that adds the shares of k scales: with a few pieces only
 }
@@ -1584,10 +1612,9 @@ GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dty
         return launch_slim_tiles(A, W, C, epi, M, N, K, lda, ldw, ldc, norm_in, norm_out, stream);
     }
     if (M > SKINNY_MAX_ROWS) {                   // the rows of prompts: a norm is handed on (to a q/k/v product that takes it), none is taken
-        GI_REQUIRE(squares_in == nullptr && scaled_out != nullptr, "gemm_bf16: a product of %d rows takes no norm handed on", M);
-        GI_REQUIRE(ldc % 4 == 0 && ld_scaled % 4 == 0 && ((uintptr_t)C & 15) == 0 && ((uintptr_t)scaled_out & 7) == 0 && ((uintptr_t)g & 15) == 0,
+        GI_REQUIRE(scaled_out == nullptr || (ldc % 4 == 0 && ld_scaled % 4 == 0 && ((uintptr_t)C & 15) == 0 && ((uintptr_t)scaled_out & 7) == 0 && ((uintptr_t)g & 15) == 0),
                    "gemm_bf16: handing a norm on from %d rows needs aligned operands", M);
-        return launch_large(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, NO_NORM_IN, nullptr, stream, norm_out);
+        return launch_large(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, norm_in, nullptr, stream, norm_out);
     }
     return launch_skinny(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, norm_in, norm_out, stream);
 }

@@ -198,7 +198,11 @@ def test_rope_cos_sin_uses_64_bit_angles():
                                             (64, 2048, 8192, 16384, True), (64, 2048, 2048, 3072, False), (40, 2048, 8192, 3072, False), (17, 2048, 8192, 16384, True),
                                             (100, 4096, 14336, 6144, False), (128, 3072, 8192, 16384, True), (33, 1024, 512, 12288, False),
                                             (24, 2048, 2048, 16384, True), (24, 2048, 8192, 3072, False), (14, 2048, 2048, 16384, True), (32, 2048, 2048, 2048, False),
-                                            (17, 264, 136, 12288, False), (13, 4096, 4096, 28672, True)])
+                                            (17, 264, 136, 12288, False), (13, 4096, 4096, 28672, True),
+                                            # the rows of prompts: from the tiles of 128 x 128 (or the kernel that adds the shares of k) to the gated
+                                            # product on the kernel with tiles of 256 x 256
+                                            (2048, 2048, 2048, 16384, True), (2048, 2048, 8192, 16384, True), (1024, 2048, 2048, 16384, True),
+                                            (1500, 3072, 1024, 16384, True)])
 def test_norm_handed_from_one_product_to_the_next(m, d, k1, n2, gated):
     """A product that adds onto rows x also writes g * x and the pieces of the rows' sums of squares; the next product reads
     g * x and multiplies its results by rsqrt(mean(x^2) + eps).  The rows x are what the plain product leaves, bit for bit; the
@@ -211,7 +215,7 @@ def test_norm_handed_from_one_product_to_the_next(m, d, k1, n2, gated):
     g = (1 + 0.1 * randn(d, seed=4)).float()
     x0 = randn(m, d, seed=5)
     parts = o.gemm_bf16_norm_parts(m, d, k1)
-    assert parts and o.gemm_bf16_takes_norm(m, n2, d), "every case here is one the kernels take"
+    assert parts and o.gemm_bf16_takes_norm(m, n2, d, gated), "every case here is one the kernels take"
     plain_x = x0.clone()
     o.gemm_bf16(a, w1, plain_x, accumulate=True)
     x, scaled, squares = x0.clone(), torch.full((m, d), float("nan"), dtype=torch.bfloat16, device=DEV), torch.full((m, parts), float("nan"), device=DEV)
