@@ -143,10 +143,12 @@ class PageGroup:
             self.table_host[slot, i] = new
         self._changed(slot, min(keep, length // self.page_size))
 
-    def sync(self, upload=None) -> None:
+    def sync(self, upload=None, stage=None) -> None:
         """Brings the device's copy of the changed rows up to date.  Only the columns that changed go over: from the
         first changed entry of any dirty row to the last entry that a dirty row holds or held on the device (a request
-        that crosses into a new page sends one column, not its whole row of max_positions / page_size entries)."""
+        that crosses into a new page sends one column, not its whole row of max_positions / page_size entries).
+        `upload(arrays...)`: int32 arrays -> device tensors without waiting for the device; `stage(array)`: the array in
+        pinned memory, for a copy made here (one changed row, a prompt's usually, goes straight into its place so)."""
         if self.table_dev is None or not self.dirty:
             self.dirty.clear()
             return
@@ -156,6 +158,9 @@ class PageGroup:
         hi = int(max(self.n_held[rows].max(), self.on_device[rows].max()))
         self.on_device[rows] = self.n_held[rows]
         if hi <= lo:
+            return
+        if stage is not None and len(rows) == 1:
+            self.table_dev[rows[0], lo:hi].copy_(stage(self.table_host[rows[0], lo:hi]), non_blocking=True)
             return
         block = self.table_host[rows, lo:hi]
         if upload is not None:                 # int32 array -> device tensor without waiting for the device
@@ -417,11 +422,12 @@ class CacheManager:
             g.rewind(slot, length)
         self._length[request] = length
 
-    def sync(self, upload=None) -> None:
+    def sync(self, upload=None, stage=None) -> None:
         """Brings the device copies of changed page tables up to date.  `upload(int32 arrays...) -> device tensors`
-        is the caller's way of copying without waiting for the device (it must take a snapshot at once)."""
+        is the caller's way of copying without waiting for the device (it must take a snapshot at once); `stage(array)
+        -> the same in pinned memory`, if it has one, lets a single changed row go straight to its place."""
         for g in self.groups:
-            g.sync(upload)
+            g.sync(upload, stage)
 
     # --------------------------------------------------------------------------------- views
     def kv(self, entry: int):

@@ -180,10 +180,10 @@ class Runner:
             row += n
 
         dev = self.model.device
-        every_row_wanted = logit_rows == list(range(n_rows))
+        every_row_wanted = len(logit_rows) == n_rows and logit_rows == list(range(n_rows))
         graph = self._step_graph_for(seg_len, seg_pos0, len(logit_rows), every_row_wanted)
         if graph is not None and graph.calls >= 1:           # a shape that has come before: captured now, replayed from then on
-            self.cache.sync(self._uploads.put)
+            self.cache.sync(self._uploads.put, self._uploads.stage)
             logits = graph.run(self._uploads, meta, logit_rows, seg_start, seg_len, seg_pos0, seg_slot)
             self.steps_replayed += 1
         else:
@@ -194,7 +194,7 @@ class Runner:
                 meta_dev, rows_dev = self._uploads.put(meta, np.asarray(logit_rows, dtype=np.int32), send=False)
             else:
                 meta_dev, rows_dev = self._uploads.put(meta, send=False), None
-            self.cache.sync(self._uploads.put)
+            self.cache.sync(self._uploads.put, self._uploads.stage)
             self._uploads.flush()
             meta_dev = meta_dev.view(3, n_rows)
             ctx = StepContext(n_rows=n_rows, dtype=self.model.dtype, device=dev, tokens=meta_dev[0], row_pos=meta_dev[1],
@@ -272,7 +272,7 @@ class Runner:
             raise StepError(f"the step holds {n} rows, more than max_rows = {self.max_rows}")
         cache.reserve_one_each(requests, slots, lengths)                        # OutOfPages: nothing changed
         self._uploads.begin_step()
-        cache.sync(self._uploads.put)
+        cache.sync(self._uploads.put, self._uploads.stage)
         # Captured steps exist for some batch sizes only: rows of the spare slot, at position 0, fill the step up to the next of them.
         fill = captured_batch_size(n, self.max_rows) - n
         if fill:
@@ -352,6 +352,7 @@ class _StepUploads:
         self.device, self.capacity = device, capacity
         on_gpu = torch.device(device).type == "cuda"
         self.host = [torch.empty(capacity, dtype=torch.int32, pin_memory=on_gpu) for _ in range(self.DEPTH)]
+        self.host_np = [h.numpy() for h in self.host]            # the same memory, for numpy to write into
         self.dev = [torch.empty(capacity, dtype=torch.int32, device=device) for _ in range(self.DEPTH)]
         self.done = [None] * self.DEPTH
         self.turn, self.used, self.sent = 0, 0, 0
@@ -374,7 +375,7 @@ class _StepUploads:
                 self.used = first
                 pieces = tuple(torch.from_numpy(f.copy()).to(self.device) for f in flats)
                 return pieces[0] if len(pieces) == 1 else pieces
-            self.host[self.turn][a:a + flat.size] = torch.from_numpy(flat)
+            self.host_np[self.turn][a:a + flat.size] = flat
             spans.append((a, a + flat.size))
             self.used = (a + flat.size + 3) & ~3                # pieces start at multiples of 16 bytes
         if send:
@@ -398,7 +399,7 @@ class _StepUploads:
         self.used = (b + 3) & ~3
         if self.sent == a:                                      # (not the ring's to send)
             self.sent = self.used
-        self.host[self.turn][a:b] = torch.from_numpy(flat)
+        self.host_np[self.turn][a:b] = flat
         return self.host[self.turn][a:b]
 
     def region(self, n: int) -> torch.Tensor:
