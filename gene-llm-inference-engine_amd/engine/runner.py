@@ -9,6 +9,7 @@ keeps the same promises, src/model/model.h:63-76, src/model/transformer.cpp:483-
 """
 from __future__ import annotations
 
+import array
 import gc
 
 from dataclasses import dataclass, field
@@ -130,8 +131,11 @@ class Runner:
                 raise StepError(f"request {e.request!r} is not open")
             if len(e.tokens) == 0:
                 raise StepError(f"request {e.request!r} brings no tokens")
-            try:
-                tokens = np.asarray(e.tokens, dtype=np.int64)              # (checked as a whole: a prompt portion has thousands)
+            try:                                                            # (checked as a whole: a prompt portion has thousands)
+                if type(e.tokens) is list:                                  # (the quickest way from a list of Python numbers to an array)
+                    tokens = np.frombuffer(array.array("q", e.tokens), dtype=np.int64)
+                else:
+                    tokens = np.asarray(e.tokens, dtype=np.int64)
             except (TypeError, ValueError, OverflowError):
                 raise StepError(f"the tokens of request {e.request!r} are not integers") from None
             if tokens.ndim != 1 or int(tokens.min()) < 0 or int(tokens.max()) >= vocab:
