@@ -507,12 +507,14 @@ def _decode_places(hd, fused, n_waves, gh):
     return lib().gi_compute_units() * (per_unit if per_unit > 0 else max(1, 16 // n_waves))
 
 
-def _decode_plain_shape(groups, span, max_waves, target_waves=4096):
-    """About `target_waves` waves in all, pieces of at least 64 positions; one split when a workgroup's waves cover them."""
-    pieces = max(1, min(-(-target_waves // groups), -(-span // 64)))
+def _decode_plain_shape(groups, span, max_waves, target_waves=4096, small=False):
+    """About `target_waves` waves in all, pieces of at least 64 positions; one split when a workgroup's waves cover them.
+    small (a few rows, heads of up to 64 channels, the kernel with rotation inside): pieces down to 32 positions, and workgroups
+    of 8 waves while there are few of them (up to 64 groups of heads: half the partial results for the second kernel to merge)."""
+    pieces = max(1, min(-(-target_waves // groups), -(-span // (32 if small else 64))))
     if pieces <= max_waves:
         return (1, pieces)
-    n_waves = min(4, max_waves)
+    n_waves = min(8 if small and groups <= 64 else 4, max_waves)
     return (min(-(-pieces // n_waves), 256), n_waves)
 
 
@@ -530,13 +532,15 @@ def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096,
     of 8, 4, 3 or 2 waves, with as few splits as that allows: 65 rows 73 -> 57 us a layer, 96 rows 90 -> 74, 40 rows 46 -> 38,
     56 rows 2.10 -> 1.92 ms a step (heads of 64 channels); 65 rows 127 -> 111 us (heads of 128).  The small batches whose kernel
     also rotates and stores the new key keep the plain rule at heads of 64 channels: their workgroups are short, and 8 and 16 rows
-    measured 5 and 3 % slower with one round.  At 128 channels that kernel's registers leave room for 8 waves a compute unit, and
+    measured 5 and 3 % slower with one round.  What helps them is more and shorter pieces in fewer, larger workgroups (`small` in
+    `_decode_plain_shape`; attention and combine kernel together, context 2,100: 1 row 11.4 -> 9.9 us a layer, 4 rows 13.8 -> 12.2,
+    6 rows 15.8 -> 14.8, 8 rows 17.5 -> 17.0; context 1,100: 8 rows 12.9 -> 11.8).  At 128 channels that kernel's registers leave room for 8 waves a compute unit, and
     there one round is the faster cut whenever the plain rule needs more (8 rows: 30 -> 27 us a layer at a context of 2,100, 35 ->
     29 at 3,000; the step of the 8B shape 4.82 -> 4.79 ms at 8 rows, 5.47 -> 5.31 at 16)."""
     group = n_heads // n_kv
     groups = n_decode * n_kv * ((group + 15) // 16)
     max_waves = min(8, lib().gi_attention_decode_max_waves(hd))
-    base = _decode_plain_shape(groups, span, max_waves, target_waves)
+    base = _decode_plain_shape(groups, span, max_waves, target_waves, small=fused and hd <= 64)
     if target_waves != 4096 or (fused and hd < 128):
         return base
     gh = min(group, 16)

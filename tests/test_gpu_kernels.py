@@ -747,7 +747,8 @@ def test_decode_attention_shape_leaves_no_nearly_empty_round(hd):
     for rows in range(1, 17):                              # the kernel that also rotates and stores: the plain rule at 64 channels, one round at 128
         splits, n_waves = o.decode_attention_shape(rows, n_heads, n_kv, hd, span, fused=True)
         if hd == 64:
-            assert (splits, n_waves) == o._decode_plain_shape(rows * n_kv, span, 8)
+            assert (splits, n_waves) == o._decode_plain_shape(rows * n_kv, span, 8, small=True)
+            assert o._decode_piece(span, splits * n_waves) >= 32 and (n_waves == 8) == (rows * n_kv <= 64 or splits == 1)
         else:
             assert rows * n_kv * splits <= o._decode_places(hd, True, n_waves, 4) or (splits, n_waves) == o._decode_plain_shape(rows * n_kv, span, 8)
             assert o._decode_piece(span, splits * n_waves) >= 64
