@@ -529,7 +529,7 @@ def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096,
     against 50 at 64).  So where the plain rule leaves a last round less than half full (less than a third where it has one
     split: there is no combine kernel to save then, and fewer pieces mean longer waves), or workgroups of 5 to 7 waves (which
     measured slower than either neighbour), the context is cut into as many pieces as fit in one round instead, in workgroups
-    of 8, 4, 3 or 2 waves, with as few splits as that allows: 65 rows 73 -> 57 us a layer, 96 rows 90 -> 74, 40 rows 46 -> 38,
+    of 8 or 4 waves (of 3 or 2 where those leave fewer than 6 pieces), with as few splits as that allows: 65 rows 73 -> 57 us a layer, 96 rows 90 -> 74, 40 rows 46 -> 38,
     56 rows 2.10 -> 1.92 ms a step (heads of 64 channels); 65 rows 127 -> 111 us (heads of 128).  The small batches whose kernel
     also rotates and stores the new key keep the plain rule at heads of 64 channels: their workgroups are short, and 8 and 16 rows
     measured 5 and 3 % slower with one round.  What helps them is more and shorter pieces in fewer, larger workgroups (`small` in
@@ -552,15 +552,20 @@ def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096,
         short_last_round = rounds > 1 and 0 < rounds - int(rounds) < (0.5 if base[0] > 1 else 0.3)
         if not (short_last_round or 5 <= base[1] <= 7):
             return base
-    best = None
-    for n_waves in (8, 4, 3, 2):
-        if n_waves > max_waves:
-            continue
-        splits = min(_decode_places(hd, fused, n_waves, gh) // groups, 256)         # as many as still fit in one round
-        while splits > 1 and _decode_piece(span, splits * n_waves) < 64:
-            splits -= 1
-        if splits >= 1 and (best is None or splits * n_waves > best[0] * best[1] or (splits * n_waves == best[0] * best[1] and splits < best[0])):
-            best = (splits, n_waves)
+    def most_pieces(widths):
+        best = None
+        for n_waves in widths:
+            if n_waves > max_waves:
+                continue
+            splits = min(_decode_places(hd, fused, n_waves, gh) // groups, 256)         # as many as still fit in one round
+            while splits > 1 and _decode_piece(span, splits * n_waves) < 64:
+                splits -= 1
+            if splits >= 1 and (best is None or splits * n_waves > best[0] * best[1] or (splits * n_waves == best[0] * best[1] and splits < best[0])):
+                best = (splits, n_waves)
+        return best
+    best = most_pieces((8, 4))
+    if best is None or best[0] * best[1] < 6:        # narrow workgroups only where wide ones leave few pieces: many small ones run slower than the same pieces in wide ones
+        best = most_pieces((8, 4, 3, 2))
     return best or base
 
 
