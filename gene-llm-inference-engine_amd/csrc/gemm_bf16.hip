@@ -731,6 +731,12 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const bf16_t* _
 // block, lane (r = lane%16, q = lane/16) holds k0 + 128*half + 32j + 8q .. +8 of weight row r, so
 // the four lanes of a row read 64 contiguous bytes per load.  The activations of a block go
 // through LDS (they are shared by the strips) and are fetched into registers one block ahead.
+// Cycle stamps of a workgroup's blocks (64 rows, gate/up: 5,300 clocks a block) showed a wait for every load in flight where the
+// block's activations are stored into LDS (the weights asked for one block earlier included: the compiler counts loads exactly
+// only if none of them is skipped by a lane or a block) and the products waiting for one LDS read each (1,250 clocks for 16
+// products); with every load issued by everyone, barriers that wait for LDS only and the reads one product ahead: 850 clocks for
+// the products, gate/up 21.4 -> 18.8 us at 17 rows, 25.5 -> 23.1 at 64, the decode step 2 to 3 % shorter at 17 to 128 rows.
+// (Up to four tiles of rows the kernel stays within 128 registers, two workgroups a compute unit.)
 // The halves' sums meet in LDS.  PARTIAL: the sums of the k range go to P[split][M][N] and a
 // second kernel adds the splits in order; otherwise the workgroup saw all of k and writes the
 // result with its epilogue itself.
@@ -777,7 +783,7 @@ __device__ __forceinline__ void row_scales_into(float* scales, const NormIn& n, 
 }
 
 template <int MT, int EPI, bool PARTIAL>
-__global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
+__global__ __launch_bounds__(512, MT == 2 ? 4 : 2) void gemm_bf16_skinny_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
                                                               float* __restrict__ P, int M, int N, int K, long lda, long ldw, long ldc,
                                                               int k_per_split, NormIn norm_in) {
     __shared__ __attribute__((aligned(16))) bf16_t Xs[MT * 16 * X_STRIDE];
@@ -795,47 +801,66 @@ __global__ __launch_bounds__(512) void gemm_bf16_skinny_kernel(const bf16_t* __r
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = floatx4{};
 
+    // Every load of the loop is issued by every lane in every block (addresses beyond the range are clamped into it) and the
+    // barriers wait for LDS only, so the compiler counts the loads in flight exactly: a block waits for its own activations and
+    // weights and leaves the two blocks of weights and the block of activations behind them on their way (with a load that some
+    // lanes or blocks skip it waits for all of them at the first use).  What a clamped load brings is finite and meets a zero or
+    // is dropped: weights of k beyond the range are replaced by zeros where the range's last block is ragged, and results of rows
+    // beyond M are never written.
     uint4 w_buf[3][4], x_reg[MT];
-    auto fetch_w = [&](int k0, uint4* w) {
+    const int w_last = K - 8 - (SK * half + 8 * q);           // the last 16 bytes of a weight row, from `wrow`
+    auto fetch_w = [&](int k0, uint4 (&w)[4]) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) w[j] = (k0 + SK * half + 32 * j + 8 * q < k_end) ? load16(wrow + k0 + 32 * j) : uint4{0, 0, 0, 0};
+        for (int j = 0; j < 4; ++j) w[j] = load16(wrow + min(k0 + 32 * j, w_last));
     };
-    auto fetch_x = [&](int k0) {                      // rows beyond M and k beyond the range are zero
+    const int x_row = tid / (KB / 8), x_k = (tid % (KB / 8)) * 8;             // of this thread's first 16 bytes of a block; its others lie 16 rows further each
+    auto fetch_x = [&](int k0) {
 #pragma unroll
-        for (int c = 0; c < MT; ++c) {
-            const int e = tid + 512 * c, row = e / (KB / 8), k = k0 + (e % (KB / 8)) * 8;
-            x_reg[c] = (row < M && k < k_end) ? load16(A + (size_t)row * lda + k) : uint4{0, 0, 0, 0};
-        }
+        for (int c = 0; c < MT; ++c) x_reg[c] = load16(A + (size_t)min(x_row + 16 * c, M - 1) * lda + min(k0 + x_k, K - 8));
     };
     fetch_x(k_begin);
     fetch_w(k_begin, w_buf[0]);
     fetch_w(k_begin + KB, w_buf[1]);
     if (scaled_rows) row_scales_into(row_scale, norm_in, M);                   // (the loop's barriers lie before its use)
-    for (int k0 = k_begin; k0 < k_end; k0 += 3 * KB) {
+    // One block of 256 k: `w_use` holds its weights, `w_fill` takes those of the block after the next.  The activations of the
+    // products' next 32 k are read from LDS while those of these 32 are multiplied.
+    auto block = [&](int kk, const uint4 (&w_use)[4], uint4 (&w_fill)[4]) __attribute__((always_inline)) {
+        barrier_lds();                                // everyone has finished reading the previous block
 #pragma unroll
-        for (int d = 0; d < 3; ++d) {                 // buffer d holds the weights of block k0 + d*KB
-            const int kk = k0 + d * KB;
-            if (kk < k_end) {                         // the same for every thread of the workgroup
-                __syncthreads();                      // everyone has finished reading the previous block
-#pragma unroll
-                for (int c = 0; c < MT; ++c) {
-                    const int e = tid + 512 * c;
-                    *reinterpret_cast<uint4*>(&Xs[(e / (KB / 8)) * X_STRIDE + (e % (KB / 8)) * 8]) = x_reg[c];
-                }
-                __syncthreads();
-                fetch_x(kk + KB);
-                fetch_w(kk + 2 * KB, w_buf[(d + 2) % 3]);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const bf16x8 b = as_bf16x8(w_buf[d][j]);
-#pragma unroll
-                    for (int t = 0; t < MT; ++t) {
-                        const bf16x8 a = as_bf16x8(*reinterpret_cast<const uint4*>(&Xs[(t * 16 + r) * X_STRIDE + SK * half + 32 * j + 8 * q]));
-                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t], 0, 0, 0);
-                    }
-                }
-            }
+        for (int c = 0; c < MT; ++c) {
+            const int e = tid + 512 * c;
+            *reinterpret_cast<uint4*>(&Xs[(e / (KB / 8)) * X_STRIDE + (e % (KB / 8)) * 8]) = x_reg[c];
         }
+        barrier_lds();
+        fetch_x(kk + KB);
+        fetch_w(kk + 2 * KB, w_fill);
+        const bool ragged = kk + KB > k_end;          // the same for the whole workgroup
+        const bf16_t* x_rows = &Xs[r * X_STRIDE + SK * half + 8 * q];
+        bf16x8 a[2][MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) a[0][t] = as_bf16x8(*reinterpret_cast<const uint4*>(x_rows + t * 16 * X_STRIDE));
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (j + 1 < 4) {
+#pragma unroll
+                for (int t = 0; t < MT; ++t) a[(j + 1) & 1][t] = as_bf16x8(*reinterpret_cast<const uint4*>(x_rows + t * 16 * X_STRIDE + 32 * (j + 1)));
+            }
+            uint4 w = w_use[j];
+            if (ragged && kk + SK * half + 32 * j + 8 * q >= k_end) w = uint4{0, 0, 0, 0};
+            const bf16x8 b = as_bf16x8(w);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j & 1][t], b, acc[t], 0, 0, 0);
+        }
+    };
+    int kk = k_begin;
+    for (; kk + 2 * KB < k_end; kk += 3 * KB) {       // three blocks a trip (the last may be ragged): the buffers' roles come round
+        block(kk, w_buf[0], w_buf[2]);
+        block(kk + KB, w_buf[1], w_buf[0]);
+        block(kk + 2 * KB, w_buf[2], w_buf[1]);
+    }
+    if (kk < k_end) {
+        block(kk, w_buf[0], w_buf[2]);
+        if (kk + KB < k_end) block(kk + KB, w_buf[1], w_buf[0]);
     }
     // the second half's sums join the first's
     if (half == 1) {
