@@ -1085,7 +1085,7 @@ __global__ __launch_bounds__(256) void skinny_reduce_rope_store_kernel(const flo
 // two mix the halves and are dropped).  FOLD = 1: at most 8 rows of A, one product per weight fragment; FOLD = 2: up to 16, in two
 // groups of 8 rows that share the weight fragment.
 template <int STRIPS, int ROWS, int EPI, bool HAND, int FOLD = 0>
-__global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
+__global__ __launch_bounds__(512, 4) void gemm_bf16_slim_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
                                                             int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in, NormOut norm_out) {
     static_assert(FOLD == 0 || ROWS == 8, "folding k into the idle rows needs strips of 8 weight rows");
     constexpr int BLOCK = FOLD ? 2 * SK : SK, SPAN = BLOCK / 4;       // k of a block, and of one of its four products
@@ -1098,15 +1098,14 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
     const int r = FOLD ? lane & 7 : lane & 15, q = lane >> 4;
     const int k_lane = 8 * q + (FOLD ? 32 * ((lane >> 3) & 1) : 0);   // where in a product's span of k this lane reads
     const int n = (blockIdx.x * STRIPS + strip) * ROWS + r;
-    const bool w_ok = r < ROWS && n < N;
-    const bf16_t* wrow = W + (size_t)(w_ok ? n : 0) * ldw + k_lane;
+    // Every lane issues every load of a block (a row beyond the operand is clamped into it and lands in results that are never
+    // written; in a row's last, ragged block k is clamped too and the activations beyond K become zeros), and what a wave skips it
+    // skips as a whole: the compiler then counts the loads in flight, and a block's products wait for that block alone.
+    const bf16_t* wrow = W + (size_t)min(n, N - 1) * ldw + k_lane;
     const bf16_t* xrow[XT];
-    bool x_ok[XT];
 #pragma unroll
-    for (int t = 0; t < XT; ++t) {
-        x_ok[t] = 8 * t + r < M;
-        xrow[t] = A + (size_t)(x_ok[t] ? 8 * t + r : 0) * lda + k_lane;
-    }
+    for (int t = 0; t < XT; ++t) xrow[t] = A + (size_t)min(8 * t + r, M - 1) * lda + k_lane;
+    const int k_last = K - 8 - k_lane;                        // the last 16 bytes of a row, from `wrow` and `xrow`
 
     floatx4 acc[XT];
 #pragma unroll
@@ -1115,37 +1114,65 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
     auto fetch = [&](int k0, uint4* w, uint4 (*x)[4]) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const bool in = k0 + SPAN * j + k_lane < K;
-            w[j] = (in && w_ok) ? load16(wrow + k0 + SPAN * j) : uint4{0, 0, 0, 0};
+            const int at = min(k0 + SPAN * j, k_last);
+            w[j] = load16(wrow + at);
 #pragma unroll
-            for (int t = 0; t < XT; ++t) x[t][j] = (in && x_ok[t]) ? load16(xrow[t] + k0 + SPAN * j) : uint4{0, 0, 0, 0};
+            for (int t = 0; t < XT; ++t) x[t][j] = load16(xrow[t] + at);
         }
     };
-    const int k_first = slice * BLOCK;
-#pragma unroll
-    for (int d = 0; d < DEPTH - 1; ++d) fetch(k_first + d * STEP, w_buf[d], x_buf[d]);      // beyond K: zeros, no loads
-    // The pieces of the rows' sums of squares, 32 or 64 threads a row: asked for behind the first weights, they have come when
-    // the products are done.
+    // The pieces of the rows' sums of squares, 32 or 64 threads a row: asked for ahead of the first weights (loads come back in
+    // the order they were issued) and added up behind the requests for those, so that one register waits for the epilogue, not eight.
     float piece[HAND ? SLIM_PIECES : 1];
+    [[maybe_unused]] float pieces_sum = 0.f;
     const int sharing = M <= 8 ? 64 : 32, piece_row = M <= 8 ? tid >> 6 : tid >> 5;
     if constexpr (HAND) {
         if (norm_in.squares != nullptr) {
+            const float* row_pieces = norm_in.squares + (size_t)min(piece_row, M - 1) * norm_in.parts;
 #pragma unroll
-            for (int i = 0; i < SLIM_PIECES; ++i) {
-                const int p = (tid & (sharing - 1)) + sharing * i;
-                piece[i] = (piece_row < M && p < norm_in.parts) ? norm_in.squares[(size_t)piece_row * norm_in.parts + p] : 0.f;
-            }
+            for (int i = 0; i < SLIM_PIECES; ++i) piece[i] = row_pieces[min((tid & (sharing - 1)) + sharing * i, norm_in.parts - 1)];
         }
     }
-    for (int k0 = k_first; k0 < K; k0 += DEPTH * STEP) {
+    const int k_first = slice * BLOCK;
+    const int n_blocks = k_first < K ? (K - k_first + STEP - 1) / STEP : 0;       // of this wave
 #pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {                     // buffer d holds block k0 + d*STEP
-            fetch(k0 + (d + DEPTH - 1) * STEP, w_buf[(d + DEPTH - 1) % DEPTH], x_buf[(d + DEPTH - 1) % DEPTH]);
+    for (int d = 0; d < DEPTH - 1; ++d)
+        if (d < n_blocks) fetch(k_first + d * STEP, w_buf[d], x_buf[d]);
+    if constexpr (HAND) {
+        if (norm_in.squares != nullptr) {
+#pragma unroll
+            for (int i = 0; i < SLIM_PIECES; ++i)
+                if (piece_row < M && (tid & (sharing - 1)) + sharing * i < norm_in.parts) pieces_sum += piece[i];
+        }
+    }
+    // Block b of the wave lies in buffer b % DEPTH; its products are behind the request for block b + DEPTH - 1.
+    auto products = [&](int b, uint4* w, uint4 (*x)[4]) __attribute__((always_inline)) {
+        const int kb = k_first + b * STEP;
+        if (kb + BLOCK > K) {                                 // the row's end lies in this block
 #pragma unroll
             for (int j = 0; j < 4; ++j)
+                if (kb + SPAN * j + k_lane >= K) {
 #pragma unroll
-                for (int t = 0; t < XT; ++t)
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x_buf[d][t][j]), as_bf16x8(w_buf[d][j]), acc[t], 0, 0, 0);
+                    for (int t = 0; t < XT; ++t) x[t][j] = uint4{0, 0, 0, 0};
+                }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int t = 0; t < XT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x[t][j]), as_bf16x8(w[j]), acc[t], 0, 0, 0);
+    };
+    int b = 0;
+    for (; b + 2 * DEPTH - 1 <= n_blocks; b += DEPTH) {      // trips in which nothing is skipped: exact waits
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            fetch(k_first + (b + d + DEPTH - 1) * STEP, w_buf[(d + DEPTH - 1) % DEPTH], x_buf[(d + DEPTH - 1) % DEPTH]);
+            products(b + d, w_buf[d], x_buf[d]);
+        }
+    }
+    for (; b < n_blocks; b += DEPTH) {                        // the end of the wave's blocks
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            if (b + d + DEPTH - 1 < n_blocks) fetch(k_first + (b + d + DEPTH - 1) * STEP, w_buf[(d + DEPTH - 1) % DEPTH], x_buf[(d + DEPTH - 1) % DEPTH]);
+            if (b + d < n_blocks) products(b + d, w_buf[d], x_buf[d]);
         }
     }
 #pragma unroll
@@ -1154,9 +1181,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_kernel(const bf16_t* __res
         for (int v = 0; v < 4; ++v) red[wave][t][lane][v] = acc[t][v];
     if constexpr (HAND) {
         if (norm_in.squares != nullptr) {
-            float sum = 0.f;
-#pragma unroll
-            for (int i = 0; i < SLIM_PIECES; ++i) sum += piece[i];
+            float sum = pieces_sum;
             if (sharing == 64) sum += __shfl_xor(sum, 32, 64);
 #pragma unroll
             for (int off = 16; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
@@ -1236,15 +1261,11 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_tiles_kernel(const bf16_t*
     const int tid = threadIdx.x, lane = tid & 63, slice = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
     const int n = blockIdx.x * 16 + r;
-    const bool w_ok = n < N;
-    const bf16_t* wrow = W + (size_t)(w_ok ? n : 0) * ldw + 8 * q;
+    const bf16_t* wrow = W + (size_t)min(n, N - 1) * ldw + 8 * q;         // (every lane issues every load of a block, as in the kernel above)
     const bf16_t* xrow[MT];
-    bool x_ok[MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        x_ok[t] = t * 16 + r < M;
-        xrow[t] = A + (size_t)(x_ok[t] ? t * 16 + r : 0) * lda + 8 * q;
-    }
+    for (int t = 0; t < MT; ++t) xrow[t] = A + (size_t)min(t * 16 + r, M - 1) * lda + 8 * q;
+    const int k_last = K - 8 - 8 * q;
     floatx4 acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = floatx4{};
@@ -1252,24 +1273,41 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_tiles_kernel(const bf16_t*
     auto fetch = [&](int k0, uint4* w, uint4 (*x)[4]) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const bool in = k0 + 32 * j + 8 * q < K;
-            w[j] = (in && w_ok) ? load16(wrow + k0 + 32 * j) : uint4{0, 0, 0, 0};
+            const int at = min(k0 + 32 * j, k_last);
+            w[j] = load16(wrow + at);
 #pragma unroll
-            for (int t = 0; t < MT; ++t) x[t][j] = (in && x_ok[t]) ? load16(xrow[t] + k0 + 32 * j) : uint4{0, 0, 0, 0};
+            for (int t = 0; t < MT; ++t) x[t][j] = load16(xrow[t] + at);
         }
     };
     const int k_first = slice * SK;
-    fetch(k_first, w_buf[0], x_buf[0]);
+    const int n_blocks = k_first < K ? (K - k_first + STEP - 1) / STEP : 0;       // of this wave
+    if (n_blocks > 0) fetch(k_first, w_buf[0], x_buf[0]);
     if (norm_in.squares != nullptr) row_scales_into(row_scale, norm_in, M);      // (the barrier behind the products lies before its use)
-    for (int k0 = k_first; k0 < K; k0 += DEPTH * STEP) {
-#pragma unroll
-        for (int d = 0; d < DEPTH; ++d) {                     // buffer d holds block k0 + d*STEP
-            fetch(k0 + (d + 1) * STEP, w_buf[(d + 1) % DEPTH], x_buf[(d + 1) % DEPTH]);
+    auto products = [&](int b, uint4* w, uint4 (*x)[4]) __attribute__((always_inline)) {
+        const int kb = k_first + b * STEP;
+        if (kb + SK > K) {                                    // the row's end lies in this block: weights of k beyond it become zeros
 #pragma unroll
             for (int j = 0; j < 4; ++j)
+                if (kb + 32 * j + 8 * q >= K) w[j] = uint4{0, 0, 0, 0};
+        }
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x_buf[d][t][j]), as_bf16x8(w_buf[d][j]), acc[t], 0, 0, 0);
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(x[t][j]), as_bf16x8(w[j]), acc[t], 0, 0, 0);
+    };
+    int b = 0;
+    for (; b + 2 * DEPTH - 1 <= n_blocks; b += DEPTH) {      // trips in which nothing is skipped
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            fetch(k_first + (b + d + 1) * STEP, w_buf[(d + 1) % DEPTH], x_buf[(d + 1) % DEPTH]);
+            products(b + d, w_buf[d], x_buf[d]);
+        }
+    }
+    for (; b < n_blocks; b += DEPTH) {                        // the end of the wave's blocks
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            if (b + d + 1 < n_blocks) fetch(k_first + (b + d + 1) * STEP, w_buf[(d + 1) % DEPTH], x_buf[(d + 1) % DEPTH]);
+            if (b + d < n_blocks) products(b + d, w_buf[d], x_buf[d]);
         }
     }
 #pragma unroll
