@@ -10,6 +10,7 @@
 // long as both operands assign k to lanes in the same way: probabilities stay in the registers
 // in which the score product left them, and the value operand is loaded to match.
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -645,7 +646,7 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
     extern __shared__ float merged[];                        // [wave][gh][HD + 2]
     const int group = n_heads / n_kv, hg_per_kv = (group + 15) / 16;
     const int row = rows ? rows[blockIdx.x] : blockIdx.x, g = blockIdx.y / hg_per_kv, hg = blockIdx.y % hg_per_kv, split = blockIdx.z;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), n_waves = blockDim.x >> 6;
     const int r = lane & 15, q4 = lane >> 4;
     const int head_in_group = hg * 16 + r;
     const bool head_ok = head_in_group < group;
@@ -666,7 +667,7 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
     }
     const int my_pos = pos[row];
     const int lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
-    const int* tab = table + (size_t)slots[row] * table_stride;
+    const int* tab = table + (size_t)__builtin_amdgcn_readfirstlane(slots[row]) * table_stride;
     // every row cuts its own range into pieces (multiples of 32), one per wave of every split; short rows leave later pieces empty
     const int n_pieces = n_splits * n_waves, piece = split * n_waves + wave;
     const int span = my_pos + 1 - (lo & ~31);
@@ -685,17 +686,31 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
     // Loads run ahead of the products: the keys of the next 32 positions and the values of these 32
     // are requested before the scores of these 32 are taken.  An address beyond the row's own range
     // is clamped into it; what it brings is masked below.
-    uint4 k_cur[2][KSTEPS], k_nxt[2][KSTEPS];
-    auto load_keys = [&](int kv0, uint4 (&dst)[2][KSTEPS]) {
+    // A tile's 32 positions are two blocks of 16, each within one page (pages hold a multiple of 16 positions), so the two page
+    // numbers of a tile are the same for the whole wave: they come through the scalar unit, a tile ahead of the keys that need them
+    // (a page number fetched per lane is a vector load like the keys and values, and those come back in the order they were asked
+    // for: waiting for it meant waiting for every key and value requested before it, several round trips to memory per tile).
+    const int first_page = page_index(lo), last_page = page_index(my_pos);
+    auto pages_of = [&](int kv0, int (&pg)[2]) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) pg[t] = tab[__builtin_amdgcn_readfirstlane(min(max(page_index(kv0 + 16 * t), first_page), last_page))];
+    };
+    uint4 k_a[2][KSTEPS], k_b[2][KSTEPS];
+    auto load_keys = [&](int kv0, const int (&pg)[2], uint4 (&dst)[2][KSTEPS]) {
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int kv = min(max(kv0 + 16 * t + r, lo), my_pos);
-            const bf16_t* krow = kbase + (long)tab[page_index(kv)] * page_stride + (long)place_of(kv) * HD + 8 * q4;
+            const bf16_t* krow = kbase + (long)pg[t] * page_stride + (long)place_of(kv) * HD + 8 * q4;
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ++ks) dst[t][ks] = load16(krow + 32 * ks);
         }
     };
-    if (begin < end) load_keys(begin, k_cur);
+    int pg_cur[2] = {0, 0}, pg_nxt[2] = {0, 0};
+    if (begin < end) {
+        pages_of(begin, pg_cur);
+        pages_of(begin + 32, pg_nxt);
+        load_keys(begin, pg_cur, k_a);
+    }
 
     bf16x8 qreg[KSTEPS];
     uint4 own_key[KSTEPS];
@@ -742,26 +757,33 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
 #pragma unroll
     for (int i = 0; i < DT; ++i) o[i] = floatx4{};
     float m = -INFINITY, l = 0.f;
-    for (int kv0 = begin; kv0 < end; kv0 += 32) {
+    // One tile of 32 positions: its keys lie in `k_use`; with a tile behind it (NEXT), that tile's keys are requested into `k_fill`
+    // and the page numbers of the tile after that through the scalar unit.  No load of a tile is skipped by a lane or by a
+    // condition inside it, so the compiler counts the loads in flight: the scores wait for this tile's keys alone, the output's
+    // products for its values alone.
+    auto tile = [&](int kv0, auto next, uint4 (&k_use)[2][KSTEPS], uint4 (&k_fill)[2][KSTEPS]) __attribute__((always_inline)) {
+        constexpr bool NEXT = decltype(next)::value;
+        int pg_far[2] = {0, 0};
+        if constexpr (NEXT) pages_of(kv0 + 64, pg_far);
         // slot e of this lane in the value product is key position kv0 + 16*(e/4) + 4*q4 + e%4
         const int kva = min(max(kv0 + 4 * q4, lo & ~3), my_pos & ~3), kvb = min(max(kv0 + 16 + 4 * q4, lo & ~3), my_pos & ~3);
-        const bf16_t* va = vbase + (long)tab[page_index(kva)] * page_stride + place_of(kva) + (long)r * page_size;
-        const bf16_t* vb = vbase + (long)tab[page_index(kvb)] * page_stride + place_of(kvb) + (long)r * page_size;
+        const bf16_t* va = vbase + (long)pg_cur[0] * page_stride + place_of(kva) + (long)r * page_size;
+        const bf16_t* vb = vbase + (long)pg_cur[1] * page_stride + place_of(kvb) + (long)r * page_size;
         uint2 vx[DT], vy[DT];
 #pragma unroll
         for (int i = 0; i < DT; ++i) {
             vx[i] = load8(va + (long)(16 * i) * page_size);
             vy[i] = load8(vb + (long)(16 * i) * page_size);
         }
-        if (kv0 + 32 < end) load_keys(kv0 + 32, k_nxt);
-        if constexpr (FUSED) {
-            if (has_own && kv0 + 32 >= end) {             // the last block of the piece: the row's own key and value go in
+        if constexpr (NEXT) load_keys(kv0 + 32, pg_nxt, k_fill);
+        if constexpr (FUSED && !NEXT) {
+            if (has_own) {                                // the last tile of the piece: the row's own key and value go in
                 const int off = my_pos - kv0;             // 0 .. 31
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
                     if ((off >> 4) == t && (off & 15) == r) {
 #pragma unroll
-                        for (int ks = 0; ks < KSTEPS; ++ks) k_cur[t][ks] = own_key[ks];
+                        for (int ks = 0; ks < KSTEPS; ++ks) k_use[t][ks] = own_key[ks];
                     }
                 if (((off & 15) >> 2) == q4) {
                     const int e = off & 3;
@@ -784,7 +806,7 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
         for (int t = 0; t < 2; ++t) {
             s[t] = floatx4{};
 #pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(k_cur[t][ks]), qreg[ks], s[t], 0, 0, 0);
+            for (int ks = 0; ks < KSTEPS; ++ks) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(k_use[t][ks]), qreg[ks], s[t], 0, 0, 0);
         }
         // element v of s[t]: key position kv0 + 16*t + 4*q4 + v, query head r
         float mx = -INFINITY;
@@ -820,10 +842,25 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
             for (int v = 0; v < 4; ++v) o[i][v] *= corr;
             o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(uint4{vx[i].x, vx[i].y, vy[i].x, vy[i].y}), as_bf16x8(pb), o[i], 0, 0, 0);
         }
+        if constexpr (NEXT) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) k_cur[t][ks] = k_nxt[t][ks];
+            for (int t = 0; t < 2; ++t) {
+                pg_cur[t] = pg_nxt[t];
+                pg_nxt[t] = pg_far[t];
+            }
+        }
+    };
+    // The two key buffers take turns; the piece's last tile has nothing behind it.
+    int kv0 = begin;
+    for (; kv0 + 64 < end; kv0 += 64) {
+        tile(kv0, std::true_type{}, k_a, k_b);
+        tile(kv0 + 32, std::true_type{}, k_b, k_a);
+    }
+    if (kv0 + 32 < end) {
+        tile(kv0, std::true_type{}, k_a, k_b);
+        tile(kv0 + 32, std::false_type{}, k_b, k_a);
+    } else if (kv0 < end) {
+        tile(kv0, std::false_type{}, k_a, k_b);
     }
 
     // The waves' results meet in LDS: element v of o[i] is channel 16*i + 4*q4 + v of query head r.
@@ -987,12 +1024,21 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
 // Waves a workgroup of the decode kernel may have for this head size.
 GI_API int gi_attention_decode_max_waves(int hd) { return hd <= 128 ? 8 : 4; }
 
+// LDS a workgroup of the decode kernel asks for: what its waves' results need, and at least so much that a compute unit holds no
+// more than 16 of the kernel's waves (of 160 KB: with 20 waves a unit, which the registers allow at heads of 64 channels, contexts
+// cut over several workgroups took 2 to 4 % longer a step at 40 to 72 rows).
+static size_t decode_lds_bytes(int hd, int n_waves, int gh) {
+    const size_t need = (size_t)n_waves * gh * (hd + 2) * sizeof(float);
+    const size_t floor_ = (size_t)(160.0 * 1024.0 / (16.0 / n_waves + 0.5));
+    return need > floor_ ? need : (floor_ < 64 * 1024 ? floor_ : 64 * 1024);
+}
+
 // Workgroups of `n_waves` waves of the decode kernel that a compute unit holds at once (by the kernel's registers and its LDS for
 // `gh` query heads per key/value head, at most 16), as the runtime works it out; 0 if it cannot say.  The cut of the context
 // over workgroups is chosen by it: workgroups beyond what the chip holds run as a second round.
 GI_API int gi_attention_decode_workgroups_per_unit(int hd, int fused, int n_waves, int gh) {
     if (n_waves < 1 || n_waves > gi_attention_decode_max_waves(hd) || gh < 1 || gh > 16) return 0;
-    const size_t lds = (size_t)n_waves * gh * (hd + 2) * sizeof(float);
+    const size_t lds = decode_lds_bytes(hd, n_waves, gh);
     int n = 0;
     hipError_t e = hipErrorInvalidValue;
 #define ASK2(HD, FUSED_) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)attention_decode_kernel<HD, FUSED_>, 64 * n_waves, lds)
@@ -1043,6 +1089,7 @@ GI_API int gi_attention_decode_bf16(const void* q, const float* qf, const float*
         lds = (size_t)n_waves * gh * (hd + 2) * sizeof(float);
     }
     GI_REQUIRE(lds <= 64 * 1024, "attention_decode: %d heads of size %d per key/value head do not fit", gh, hd);
+    lds = decode_lds_bytes(hd, n_waves, gh);
     dim3 grid(n_rows, n_kv * hg, n_splits);
 #define GO2(HD, FUSED_)                                                                                                                    \
     attention_decode_kernel<HD, FUSED_><<<grid, 64 * n_waves, lds, stream>>>((const bf16_t*)q, qf, kf, vf, ldq, ldk, ldv, cos_t, sin_t,   \

@@ -511,11 +511,35 @@ def _decode_plain_shape(groups, span, max_waves, target_waves=4096, small=False)
     """About `target_waves` waves in all, pieces of at least 64 positions; one split when a workgroup's waves cover them.
     small (a few rows, heads of up to 64 channels, the kernel with rotation inside): pieces down to 32 positions, and workgroups
     of 8 waves while there are few of them (up to 64 groups of heads: half the partial results for the second kernel to merge)."""
+    if small:
+        target_waves //= 2          # (its waves ask for the next keys while they multiply: half as many, twice as long, measured faster at 4 to 12 rows)
     pieces = max(1, min(-(-target_waves // groups), -(-span // (32 if small else 64))))
     if pieces <= max_waves:
         return (1, pieces)
     n_waves = min(8 if small and groups <= 64 else 4, max_waves)
     return (min(-(-pieces // n_waves), 256), n_waves)
+
+
+# What the decode kernel's workgroups reach (measured at heads of 64 and 128 channels, 17 to 128 rows, contexts of 1,100 to
+# 16,384): a compute unit pulls about 31 GB/s for one workgroup and 27 GB/s for several, however many waves they have (from
+# four up), the chip 5.9 TB/s, and a second kernel that merges splits costs about 6 us with the partial results it reads.
+_DECODE_UNIT_MB_PER_S, _DECODE_SHARED_UNIT_MB_PER_S, _DECODE_CHIP_MB_PER_S, _DECODE_MERGE_US = 31e3, 27e3, 5.9e6, 6.0
+
+
+def _decode_single_split(groups, span, hd, max_waves):
+    """(1, waves) if one workgroup per (row, group of heads) over the whole context, which needs no second kernel, is expected
+    to be no slower than a context cut over several; else None.  Without splits the compute unit with the most workgroups sets
+    the time (`groups` over the units, rounded up, each pulling its share of the bytes at a unit's rate); with them the chip's
+    rate does, plus the merge.  Of a bracket of contexts three quarters are taken as read.  Four waves where a wave's share
+    stays under 200 KB and there is a workgroup for every unit, else eight."""
+    units = lib().gi_compute_units()
+    mbytes = groups * 0.75 * span * hd * 4 / 1e6
+    most = -(-groups // units)                       # workgroups of the busiest compute unit
+    single_us = max(most * (mbytes / groups) / (_DECODE_UNIT_MB_PER_S if most == 1 else _DECODE_SHARED_UNIT_MB_PER_S), mbytes / _DECODE_CHIP_MB_PER_S) * 1e6
+    if groups < units // 2 or single_us > mbytes / _DECODE_CHIP_MB_PER_S * 1e6 + _DECODE_MERGE_US:
+        return None
+    n_waves = 8 if groups < units or 0.75 * span / 4 * hd * 4 > 200e3 else 4
+    return (1, min(n_waves, max_waves))
 
 
 @lru_cache(maxsize=None)
@@ -536,13 +560,23 @@ def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096,
     `_decode_plain_shape`; attention and combine kernel together, context 2,100: 1 row 11.4 -> 9.9 us a layer, 4 rows 13.8 -> 12.2,
     6 rows 15.8 -> 14.8, 8 rows 17.5 -> 17.0; context 1,100: 8 rows 12.9 -> 11.8).  At 128 channels that kernel's registers leave room for 8 waves a compute unit, and
     there one round is the faster cut whenever the plain rule needs more (8 rows: 30 -> 27 us a layer at a context of 2,100, 35 ->
-    29 at 3,000; the step of the 8B shape 4.82 -> 4.79 ms at 8 rows, 5.47 -> 5.31 at 16)."""
+    29 at 3,000; the step of the 8B shape 4.82 -> 4.79 ms at 8 rows, 5.47 -> 5.31 at 16).
+
+    Since the kernel's waves ask for the next keys while they multiply (page numbers through the scalar unit, no wait for loads
+    that are not needed yet), a wave is cheap to run for long, and from 17 rows on a context that is not cut at all is often the
+    faster one: no partial results, no second kernel (`_decode_single_split` says when: 24 rows 27 -> 21 us a layer at a context
+    of 2,100, 32 rows 31 -> 25, 64 rows 50 -> 47 with four waves instead of eight, 96 rows 76 -> 69; 24 rows at heads of 128
+    channels 48 -> 38).  The rules above decide the rest."""
     group = n_heads // n_kv
     groups = n_decode * n_kv * ((group + 15) // 16)
     max_waves = min(8, lib().gi_attention_decode_max_waves(hd))
     base = _decode_plain_shape(groups, span, max_waves, target_waves, small=fused and hd <= 64)
     if target_waves != 4096 or (fused and hd < 128):
         return base
+    if not fused:
+        single = _decode_single_split(groups, span, hd, max_waves)
+        if single is not None:
+            return single
     gh = min(group, 16)
     rounds = groups * base[0] / _decode_places(hd, fused, base[1], gh)
     if fused:                        # (heads of 128 channels: 8 waves a compute unit, and a second round costs what it brings)

@@ -730,13 +730,21 @@ def test_decode_attention_from_unrotated_products(n_heads, n_kv, hd, ps, window,
 
 @pytest.mark.parametrize("hd", [64, 128])
 def test_decode_attention_shape_leaves_no_nearly_empty_round(hd):
-    """The cut of the context over workgroups: whatever the number of rows, the workgroups either fit the chip at once, or their
-    last round is not a small remainder; pieces never fall under 64 positions and the waves cover the span."""
+    """The cut of the context over workgroups: whatever the number of rows, the context is either not cut at all (a workgroup of 4
+    or 8 waves per row and group of heads, where the busiest compute unit is expected to be done no later than the chip's memory
+    plus a merging kernel), or the workgroups fit the chip at once, or their last round is not a small remainder; pieces never
+    fall under 64 positions and the waves cover the span."""
     o = ops()
     n_heads, n_kv, span = 32, 8, 4096
+    uncut = 0
     for rows in list(range(17, 130)) + [192, 256, 500]:
         splits, n_waves = o.decode_attention_shape(rows, n_heads, n_kv, hd, span)
         assert 1 <= n_waves <= 8 and splits >= 1 and not 5 <= n_waves <= 7
+        single = o._decode_single_split(rows * n_kv, span, hd, 8)
+        if single is not None:
+            assert (splits, n_waves) == single and splits == 1 and n_waves in (4, 8)
+            uncut += 1
+            continue
         assert splits * n_waves == 1 or o._decode_piece(span, splits * n_waves) >= 64
         rounds = rows * n_kv * splits / o._decode_places(hd, False, n_waves, 4)
         plain = o._decode_plain_shape(rows * n_kv, span, 8)
@@ -744,6 +752,9 @@ def test_decode_attention_shape_leaves_no_nearly_empty_round(hd):
             assert rounds <= 1, (rows, splits, n_waves, rounds)
         else:
             assert rounds <= 1 or rounds - int(rounds) == 0 or rounds - int(rounds) >= 0.3, (rows, splits, n_waves, rounds)
+    assert 30 <= uncut <= 100                              # (a workgroup for every compute unit, or a whole number of them: 32, 64, 96, 128 rows; not 40 or 65)
+    assert o._decode_single_split(64 * n_kv, span, hd, 8) is not None and o._decode_single_split(65 * n_kv, span, hd, 8) is None
+    assert o._decode_single_split(8 * n_kv, span, hd, 8) is None
     for rows in range(1, 17):                              # the kernel that also rotates and stores: the plain rule at 64 channels, one round at 128
         splits, n_waves = o.decode_attention_shape(rows, n_heads, n_kv, hd, span, fused=True)
         if hd == 64:
