@@ -912,15 +912,27 @@ constexpr int MAX_SPLITS = 256;
 __global__ __launch_bounds__(64) void attention_decode_combine_kernel(const float* __restrict__ part, bf16_t* __restrict__ out,
                                                                      const int* __restrict__ rows, int n_heads, int hd, int n_splits) {
     __shared__ float weight[MAX_SPLITS], weighted_l[MAX_SPLITS];
+    constexpr int EARLY = 8;                                 // splits whose channels are asked for together with the splits' {m, l}
     const int idx = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const float* src = part + ((size_t)idx * n_heads + head) * n_splits * (hd + 2);
+    // Every lane issues every load (a split or channel beyond the end is clamped into the range and not used), and the first
+    // channels do not wait for the weights: one round trip to memory for up to EARLY splits, not two.
     float mine_m[MAX_SPLITS / 64], mine_l[MAX_SPLITS / 64];
+#pragma unroll
+    for (int i = 0; i < MAX_SPLITS / 64; ++i) {
+        const int s = min(lane + 64 * i, n_splits - 1);
+        mine_m[i] = src[(size_t)s * (hd + 2)];
+        mine_l[i] = src[(size_t)s * (hd + 2) + 1];
+    }
+    float early[2][EARLY];                                   // channels lane and lane + 64 (heads of up to 128 channels)
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int s = 0; s < EARLY; ++s) early[c][s] = src[(size_t)min(s, n_splits - 1) * (hd + 2) + 2 + min(lane + 64 * c, hd - 1)];
     float big = -INFINITY;
 #pragma unroll
     for (int i = 0; i < MAX_SPLITS / 64; ++i) {
-        const int s = lane + 64 * i;
-        mine_m[i] = s < n_splits ? src[(size_t)s * (hd + 2)] : -INFINITY;
-        mine_l[i] = s < n_splits ? src[(size_t)s * (hd + 2) + 1] : 0.f;
+        if (lane + 64 * i >= n_splits) { mine_m[i] = -INFINITY; mine_l[i] = 0.f; }
         big = fmaxf(big, mine_m[i]);
     }
     big = wave_max(big);
@@ -937,10 +949,16 @@ __global__ __launch_bounds__(64) void attention_decode_combine_kernel(const floa
     float denom = 0.f;
     for (int s = 0; s < n_splits; ++s) denom += weighted_l[s];
     const float inv = 1.0f / denom;
-    for (int d = lane; d < hd; d += 64) {
+    const int n_early = min(n_splits, EARLY);
+    for (int d = lane, c = 0; d < hd; d += 64, ++c) {
         float acc = 0.f;
+        if (c < 2) {
+#pragma unroll
+            for (int s = 0; s < EARLY; ++s)
+                if (s < n_early) acc = fmaf(weight[s], c == 0 ? early[0][s] : early[1][s], acc);
+        }
 #pragma unroll 8
-        for (int s = 0; s < n_splits; ++s) acc = fmaf(weight[s], src[(size_t)s * (hd + 2) + 2 + d], acc);
+        for (int s = c < 2 ? n_early : 0; s < n_splits; ++s) acc = fmaf(weight[s], src[(size_t)s * (hd + 2) + 2 + d], acc);
         out[((size_t)(rows ? rows[idx] : idx) * n_heads + head) * hd + d] = f32_to_bf16(acc * inv);
     }
 }
