@@ -656,14 +656,17 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
     [[maybe_unused]] Pairs8 q_raw[KSTEPS];
     [[maybe_unused]] Angles8 angles[KSTEPS];
     if constexpr (FUSED) {
-        const float* cos_row = cos_t ? cos_t + (size_t)row * (HD / 2) : nullptr;
-        const float* sin_row = sin_t ? sin_t + (size_t)row * (HD / 2) : nullptr;
+        // (every lane asks for its queries, a lane without a head for the group's first head's: what it brings is dropped; with a
+        // load that some lanes skip the compiler waits for all loads in flight at the first use of any)
+        if (cos_t != nullptr && sin_t != nullptr) {
 #pragma unroll
-        for (int s = 0; s < KSTEPS; ++s) angles[s] = load_angles8(cos_row, sin_row, 32 * s + 8 * q4, HD / 2);
-        if (head_ok) {
+            for (int s = 0; s < KSTEPS; ++s) angles[s] = load_angles8(cos_t + (size_t)row * (HD / 2), sin_t + (size_t)row * (HD / 2), 32 * s + 8 * q4, HD / 2);
+        } else {
 #pragma unroll
-            for (int s = 0; s < KSTEPS; ++s) q_raw[s] = load_pairs8(qf + (size_t)row * ldq + (size_t)head * HD, 32 * s + 8 * q4, HD / 2);
+            for (int s = 0; s < KSTEPS; ++s) angles[s] = load_angles8(nullptr, nullptr, 32 * s + 8 * q4, HD / 2);
         }
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) q_raw[s] = load_pairs8(qf + (size_t)row * ldq + (size_t)(head_ok ? head : g * group) * HD, 32 * s + 8 * q4, HD / 2);
     }
     const int my_pos = pos[row];
     const int lo = (window > 0 && my_pos - window + 1 > 0) ? my_pos - window + 1 : 0;
@@ -705,11 +708,25 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
             for (int ks = 0; ks < KSTEPS; ++ks) dst[t][ks] = load16(krow + 32 * ks);
         }
     };
+    // The values of a tile are asked for behind the products of the tile before it (the first tile's behind its keys), into the
+    // registers those products have just read.  Slot e of a lane in the value product is key position kv0 + 16*(e/4) + 4*q4 + e%4.
+    uint2 vx[DT], vy[DT];
+    auto load_values = [&](int kv0, const int (&pg)[2]) {
+        const int kva = min(max(kv0 + 4 * q4, lo & ~3), my_pos & ~3), kvb = min(max(kv0 + 16 + 4 * q4, lo & ~3), my_pos & ~3);
+        const bf16_t* va = vbase + (long)pg[0] * page_stride + place_of(kva) + (long)r * page_size;
+        const bf16_t* vb = vbase + (long)pg[1] * page_stride + place_of(kvb) + (long)r * page_size;
+#pragma unroll
+        for (int i = 0; i < DT; ++i) {
+            vx[i] = load8(va + (long)(16 * i) * page_size);
+            vy[i] = load8(vb + (long)(16 * i) * page_size);
+        }
+    };
     int pg_cur[2] = {0, 0}, pg_nxt[2] = {0, 0};
     if (begin < end) {
         pages_of(begin, pg_cur);
         pages_of(begin + 32, pg_nxt);
         load_keys(begin, pg_cur, k_a);
+        load_values(begin, pg_cur);
     }
 
     bf16x8 qreg[KSTEPS];
@@ -758,23 +775,13 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
     for (int i = 0; i < DT; ++i) o[i] = floatx4{};
     float m = -INFINITY, l = 0.f;
     // One tile of 32 positions: its keys lie in `k_use`; with a tile behind it (NEXT), that tile's keys are requested into `k_fill`
-    // and the page numbers of the tile after that through the scalar unit.  No load of a tile is skipped by a lane or by a
-    // condition inside it, so the compiler counts the loads in flight: the scores wait for this tile's keys alone, the output's
-    // products for its values alone.
+    // and the page numbers of the tile after that through the scalar unit; behind its products that tile's values.  No load of
+    // a tile is skipped by a lane or by a condition inside it, so the compiler counts the loads in flight: the scores wait for
+    // this tile's keys alone, the output's products for its values alone.
     auto tile = [&](int kv0, auto next, uint4 (&k_use)[2][KSTEPS], uint4 (&k_fill)[2][KSTEPS]) __attribute__((always_inline)) {
         constexpr bool NEXT = decltype(next)::value;
         int pg_far[2] = {0, 0};
         if constexpr (NEXT) pages_of(kv0 + 64, pg_far);
-        // slot e of this lane in the value product is key position kv0 + 16*(e/4) + 4*q4 + e%4
-        const int kva = min(max(kv0 + 4 * q4, lo & ~3), my_pos & ~3), kvb = min(max(kv0 + 16 + 4 * q4, lo & ~3), my_pos & ~3);
-        const bf16_t* va = vbase + (long)pg_cur[0] * page_stride + place_of(kva) + (long)r * page_size;
-        const bf16_t* vb = vbase + (long)pg_cur[1] * page_stride + place_of(kvb) + (long)r * page_size;
-        uint2 vx[DT], vy[DT];
-#pragma unroll
-        for (int i = 0; i < DT; ++i) {
-            vx[i] = load8(va + (long)(16 * i) * page_size);
-            vy[i] = load8(vb + (long)(16 * i) * page_size);
-        }
         if constexpr (NEXT) load_keys(kv0 + 32, pg_nxt, k_fill);
         if constexpr (FUSED && !NEXT) {
             if (has_own) {                                // the last tile of the piece: the row's own key and value go in
@@ -843,6 +850,7 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
             o[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(uint4{vx[i].x, vx[i].y, vy[i].x, vy[i].y}), as_bf16x8(pb), o[i], 0, 0, 0);
         }
         if constexpr (NEXT) {
+            load_values(kv0 + 32, pg_nxt);
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 pg_cur[t] = pg_nxt[t];
