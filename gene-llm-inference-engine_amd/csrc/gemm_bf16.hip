@@ -105,12 +105,28 @@ __device__ __forceinline__ void tile_row_scales(float* scales, const NormIn& n, 
     }
 }
 
-// The factor of one row: rsqrt(mean square + eps) from the pieces of its sum of squares, read and added one by one.
-__device__ __forceinline__ float row_scale_of(const NormIn& n, int row) {      // a few pieces: read and added one by one
+// The factor of one row: rsqrt(mean square + eps) from the pieces of its sum of squares, added in their order.  The first eight
+// pieces are asked for at once, by every lane (an index beyond the pieces is clamped and what it brings not added): a caller can
+// ask early (`row_pieces`) and finish where the factor is needed (`row_scale_from`), with its other loads in flight in between.
+struct RowPieces {
+    float v[8];
+};
+__device__ __forceinline__ RowPieces row_pieces(const NormIn& n, int row) {
+    RowPieces r;
+    const float* pieces = n.squares + (size_t)row * n.parts;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) r.v[u] = pieces[min(u, n.parts - 1)];
+    return r;
+}
+__device__ __forceinline__ float row_scale_from(const NormIn& n, int row, const RowPieces& r) {
     float sum = 0.f;
-    for (int p = 0; p < n.parts; ++p) sum += n.squares[(size_t)row * n.parts + p];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        if (u < n.parts) sum += r.v[u];
+    for (int p = 8; p < n.parts; ++p) sum += n.squares[(size_t)row * n.parts + p];
     return 1.0f / sqrtf(sum / (float)n.dim + n.eps);
 }
+__device__ __forceinline__ float row_scale_of(const NormIn& n, int row) { return row_scale_from(n, row, row_pieces(n, row)); }
 
 // Where the rows of a tile of 128 go in the cache: per row the page's offset and the place in the page, and per group of
 // eight rows whether they are eight consecutive positions of one request that begin at a multiple of eight (rows of a prompt).
@@ -920,6 +936,16 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
                                                             NormIn norm_in, NormOut norm_out) {
     const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VEC, slab = (size_t)M * N;
     if (i >= slab) return;
+    const size_t row = i / N, col = i % N, o = row * ldc + col;      // (VEC divides N: the VEC columns lie in one row)
+    // Everything the result needs besides the partial sums (the row's pieces of the norm before, the old values and the gains of
+    // the norm behind) is asked for ahead of them: one round trip to memory for all of it, not one after the other.
+    [[maybe_unused]] RowPieces pieces;
+    if (norm_in.squares != nullptr) pieces = row_pieces(norm_in, (int)row);
+    [[maybe_unused]] float4 old4 = {0.f, 0.f, 0.f, 0.f}, gain4 = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (VEC == 4 && EPI == EPI_ADD_F32) {
+        old4 = *reinterpret_cast<const float4*>((const float*)C + o);
+        if (norm_out.scaled != nullptr) gain4 = *reinterpret_cast<const float4*>(norm_out.g + col);
+    }
     float s[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) s[v] = 0.f;
@@ -942,9 +968,8 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
                 for (int v = 0; v < VEC; ++v) s[v] += part[u][v];
             }
     }
-    const size_t row = i / N, col = i % N, o = row * ldc + col;      // (VEC divides N: the VEC columns lie in one row)
     if (norm_in.squares != nullptr) {
-        const float rs = row_scale_of(norm_in, (int)row);
+        const float rs = row_scale_from(norm_in, (int)row, pieces);
 #pragma unroll
         for (int v = 0; v < VEC; ++v) s[v] *= rs;
     }
@@ -956,13 +981,13 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
             *reinterpret_cast<uint2*>((bf16_t*)C + o) = packed;
         } else {
             float4* dst = reinterpret_cast<float4*>((float*)C + o);
-            float4 x = EPI == EPI_ADD_F32 ? *dst : float4{0.f, 0.f, 0.f, 0.f};
+            float4 x = old4;
             x.x += s[0]; x.y += s[1]; x.z += s[2]; x.w += s[3];
             *dst = x;
             if constexpr (EPI == EPI_ADD_F32) {
                 if (norm_out.scaled != nullptr) {                    // (the same for every thread of the kernel)
                     __shared__ float wave_squares[4];
-                    const float4 g = *reinterpret_cast<const float4*>(norm_out.g + col);
+                    const float4 g = gain4;
                     uint2 packed;
                     packed.x = (unsigned)f32_to_bf16(g.x * x.x) | ((unsigned)f32_to_bf16(g.y * x.y) << 16);
                     packed.y = (unsigned)f32_to_bf16(g.z * x.z) | ((unsigned)f32_to_bf16(g.w * x.w) << 16);
@@ -1009,17 +1034,34 @@ __global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* 
 // multiple of 256 columns, so that a wave lies in one row and holds whole heads).
 __global__ __launch_bounds__(256) void skinny_reduce_rope_store_kernel(const float* __restrict__ P, int M, int N, int splits, NormIn norm_in, RopeStore rs) {
     const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4, slab = (size_t)M * N;
-    const bool live = i < slab;                              // (whole waves are live or not: 256 divides N)
-    const size_t row = live ? i / N : 0;
-    const int col = live ? (int)(i % N) : 0;
-    int p = 0, slot = 0;
-    if (live) {
-        p = rs.pos[row];
-        slot = rs.slot[row];
+    if (i >= slab) return;                                   // (whole waves: 256 divides N, so the exchange below has all its lanes)
+    const size_t row = i / N;
+    const int col = (int)(i % N);
+    const int a_dim = rs.n_heads * rs.hd, kv_dim = rs.n_kv * rs.hd, half = rs.hd / 2;
+    const int which = col < a_dim ? 0 : col < a_dim + kv_dim ? 1 : 2;                        // queries, keys, values
+    const int c = which == 0 ? col : which == 1 ? col - a_dim : col - a_dim - kv_dim;        // the column among them
+    const int h = c / rs.hd, kk = c % rs.hd;
+    // Everything is asked for at once, by every lane: position and slot first (the page number, which needs them, then waits for
+    // them alone), the row's pieces of the norm, the angles (a lane with values asks too and drops them), the first eight splits.
+    const int p = rs.pos[row], slot = rs.slot[row];
+    [[maybe_unused]] RowPieces pieces;
+    if (norm_in.squares != nullptr) pieces = row_pieces(norm_in, (int)row);
+    float4 cc = {1.f, 1.f, 1.f, 1.f}, ss = {0.f, 0.f, 0.f, 0.f};
+    if (rs.cos_t != nullptr) {
+        cc = *reinterpret_cast<const float4*>(rs.cos_t + row * half + kk % half);
+        ss = *reinterpret_cast<const float4*>(rs.sin_t + row * half + kk % half);
     }
+    float4 part[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) part[u] = *reinterpret_cast<const float4*>(P + (size_t)min(u, splits - 1) * slab + i);
+    const long page = rs.table[(size_t)slot * rs.table_stride + p / rs.page_size];
     float s[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int sp0 = 0; live && sp0 < splits; sp0 += 8) {
-        float4 part[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+        if (u < splits) {
+            s[0] += part[u].x; s[1] += part[u].y; s[2] += part[u].z; s[3] += part[u].w;
+        }
+    for (int sp0 = 8; sp0 < splits; sp0 += 8) {
 #pragma unroll
         for (int u = 0; u < 8; ++u) part[u] = *reinterpret_cast<const float4*>(P + (size_t)min(sp0 + u, splits - 1) * slab + i);
 #pragma unroll
@@ -1028,29 +1070,22 @@ __global__ __launch_bounds__(256) void skinny_reduce_rope_store_kernel(const flo
                 s[0] += part[u].x; s[1] += part[u].y; s[2] += part[u].z; s[3] += part[u].w;
             }
     }
-    if (live && norm_in.squares != nullptr) {
-        const float scale = row_scale_of(norm_in, (int)row);
+    if (norm_in.squares != nullptr) {
+        const float scale = row_scale_from(norm_in, (int)row, pieces);
 #pragma unroll
         for (int v = 0; v < 4; ++v) s[v] *= scale;
     }
-    const int a_dim = rs.n_heads * rs.hd, kv_dim = rs.n_kv * rs.hd, half = rs.hd / 2;
-    const int which = col < a_dim ? 0 : col < a_dim + kv_dim ? 1 : 2;                        // queries, keys, values
-    const int c = which == 0 ? col : which == 1 ? col - a_dim : col - a_dim - kv_dim;        // the column among them
-    const int h = c / rs.hd, kk = c % rs.hd;
     float out[4] = {s[0], s[1], s[2], s[3]};
     if (rs.cos_t != nullptr) {                               // (every lane takes part in the exchange, whatever it holds)
         float other[4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) other[v] = __shfl_xor(s[v], half / 4, 64);
-        if (live && which != 2) {
-            const float4 cc = *reinterpret_cast<const float4*>(rs.cos_t + row * half + kk % half);
-            const float4 ss = *reinterpret_cast<const float4*>(rs.sin_t + row * half + kk % half);
+        if (which != 2) {
             const float cs[4] = {cc.x, cc.y, cc.z, cc.w}, sn[4] = {ss.x, ss.y, ss.z, ss.w};
 #pragma unroll
             for (int v = 0; v < 4; ++v) out[v] = kk < half ? s[v] * cs[v] - other[v] * sn[v] : other[v] * sn[v] + s[v] * cs[v];
         }
     }
-    if (!live) return;
     uint2 packed;
     packed.x = (unsigned)f32_to_bf16(out[0]) | ((unsigned)f32_to_bf16(out[1]) << 16);
     packed.y = (unsigned)f32_to_bf16(out[2]) | ((unsigned)f32_to_bf16(out[3]) << 16);
@@ -1058,7 +1093,6 @@ __global__ __launch_bounds__(256) void skinny_reduce_rope_store_kernel(const flo
         *reinterpret_cast<uint2*>(rs.q_out + row * a_dim + c) = packed;
         return;
     }
-    const long page = rs.table[(size_t)slot * rs.table_stride + p / rs.page_size];
     const int place = p % rs.page_size;
     bf16_t* keys = rs.cache + page * rs.page_stride;
     bf16_t* values = keys + (size_t)rs.n_kv * rs.page_size * rs.hd;
@@ -1120,6 +1154,16 @@ __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_kernel(const bf16_t* __
             for (int t = 0; t < XT; ++t) x[t][j] = load16(xrow[t] + at);
         }
     };
+    // What the epilogue adds onto (the thread's element of the 32-bit rows, and the next norm's gain for its column) is asked for
+    // before anything else: it comes from the memory-side cache while the weights stream, not behind them as one more round trip.
+    [[maybe_unused]] float old_value = 0.f, gain = 0.f;
+    if constexpr (EPI == EPI_ADD_F32) {
+        const int e_m = (tid & 255) >> 4, e_col = (blockIdx.x * STRIPS + (tid >> 8) % STRIPS) * ROWS + (tid & 15);
+        old_value = ((const float*)C)[(size_t)min(e_m, M - 1) * ldc + min(e_col, N - 1)];
+        if constexpr (HAND) {
+            if (norm_out.scaled != nullptr) gain = norm_out.g[min(e_col, N - 1)];
+        }
+    }
     // The pieces of the rows' sums of squares, 32 or 64 threads a row: asked for ahead of the first weights (loads come back in
     // the order they were issued) and added up behind the requests for those, so that one register waits for the epilogue, not eight.
     float piece[HAND ? SLIM_PIECES : 1];
@@ -1219,15 +1263,14 @@ __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_kernel(const bf16_t* __
                 if constexpr (HAND) sum *= r;
                 const int col = (blockIdx.x * STRIPS + st) * ROWS + c;
                 if (col < N) {
-                    if constexpr (HAND && EPI == EPI_ADD_F32) {
-                        if (norm_out.scaled != nullptr) {
-                            float* at = (float*)C + (size_t)m * ldc + col;
-                            const float x = *at + sum;
-                            *at = x;
-                            norm_out.scaled[(size_t)m * norm_out.ld + col] = f32_to_bf16(norm_out.g[col] * x);
-                            square = x * x;
-                        } else {
-                            write_out<EPI>(C, (size_t)m * ldc + col, sum);
+                    if constexpr (EPI == EPI_ADD_F32) {
+                        const float x = old_value + sum;
+                        ((float*)C)[(size_t)m * ldc + col] = x;
+                        if constexpr (HAND) {
+                            if (norm_out.scaled != nullptr) {
+                                norm_out.scaled[(size_t)m * norm_out.ld + col] = f32_to_bf16(gain * x);
+                                square = x * x;
+                            }
                         }
                     } else {
                         write_out<EPI>(C, (size_t)m * ldc + col, sum);
@@ -1252,7 +1295,7 @@ __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_kernel(const bf16_t* __
 // One launch does the product and its epilogue; the alternative, k shared out over workgroups with partial sums in memory and a
 // second kernel to add them, costs that kernel's launch and as many bytes of partial sums as the output projection has weights.
 template <int MT, int EPI>
-__global__ __launch_bounds__(512) void gemm_bf16_slim_tiles_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
+__global__ __launch_bounds__(512, 4) void gemm_bf16_slim_tiles_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
                                                                   int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in, NormOut norm_out) {
     constexpr int SLICES = 8, STEP = SLICES * SK, DEPTH = 2;
     __shared__ float red[SLICES][MT][64][4];
@@ -1279,6 +1322,13 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_tiles_kernel(const bf16_t*
             for (int t = 0; t < MT; ++t) x[t][j] = load16(xrow[t] + at);
         }
     };
+    // (what the epilogue adds onto is asked for first, as in the kernel above: every thread has one result, e = tid below)
+    [[maybe_unused]] float old_value = 0.f, gain = 0.f;
+    if constexpr (EPI == EPI_ADD_F32) {
+        const int e_row = 16 * (tid >> 8) + ((tid >> 4) & 15), e_col = blockIdx.x * 16 + (tid & 15);
+        old_value = ((const float*)C)[(size_t)min(e_row, M - 1) * ldc + min(e_col, N - 1)];
+        if (norm_out.scaled != nullptr) gain = norm_out.g[min(e_col, N - 1)];
+    }
     const int k_first = slice * SK;
     const int n_blocks = k_first < K ? (K - k_first + STEP - 1) / STEP : 0;       // of this wave
     if (n_blocks > 0) fetch(k_first, w_buf[0], x_buf[0]);
@@ -1327,10 +1377,9 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_tiles_kernel(const bf16_t*
             if (norm_out.scaled != nullptr) {                   // (every thread comes here once: MT * 256 results, 512 threads)
                 float square = 0.f;
                 if (row < M && col < N) {
-                    float* at = (float*)C + (size_t)row * ldc + col;
-                    const float x = *at + sum;
-                    *at = x;
-                    norm_out.scaled[(size_t)row * norm_out.ld + col] = f32_to_bf16(norm_out.g[col] * x);
+                    const float x = old_value + sum;
+                    ((float*)C)[(size_t)row * ldc + col] = x;
+                    norm_out.scaled[(size_t)row * norm_out.ld + col] = f32_to_bf16(gain * x);
                     square = x * x;
                 }
 #pragma unroll
@@ -1338,6 +1387,8 @@ __global__ __launch_bounds__(512) void gemm_bf16_slim_tiles_kernel(const bf16_t*
                 if (c == 0 && row < M) norm_out.squares[(size_t)row * gridDim.x + blockIdx.x] = square;
                 continue;
             }
+            if (row < M && col < N) ((float*)C)[(size_t)row * ldc + col] = old_value + sum;
+            continue;
         }
         if (row < M && col < N) write_out<EPI>(C, (size_t)row * ldc + col, sum);
     }
