@@ -19,6 +19,14 @@ constexpr int NT = 1024;
 // wins at every comparison, so the result is the lowest index of the maximum.
 constexpr int CHUNK = 4096;
 
+// A thread's values of a run of CHUNK logits (i = begin + thread + 256 u), asked for at once by every thread (an index beyond
+// the run is clamped and what it brings not used): a loop that reads and compares one by one is sixteen round trips to memory.
+constexpr int PER_THREAD = CHUNK / 256;
+__device__ __forceinline__ void load_run(const float* __restrict__ row, int begin, int end, float (&v)[PER_THREAD]) {
+#pragma unroll
+    for (int u = 0; u < PER_THREAD; ++u) v[u] = row[min(begin + (int)threadIdx.x + 256 * u, end - 1)];
+}
+
 __device__ __forceinline__ void better(float& bv, int& bi, float ov, int oi) {
     if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
 }
@@ -31,9 +39,12 @@ __global__ __launch_bounds__(256) void argmax_chunks_kernel(const float* __restr
     const int begin = blockIdx.x * CHUNK, end = min(vocab, begin + CHUNK);
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = begin + threadIdx.x; i < end; i += 256) {
-        const float v = row[i];
-        if (v > bv || bi == 0x7fffffff) { bv = v; bi = i; }      // ascending i: strict > keeps the lowest index
+    float v[PER_THREAD];
+    load_run(row, begin, end, v);
+#pragma unroll
+    for (int u = 0; u < PER_THREAD; ++u) {
+        const int i = begin + threadIdx.x + 256 * u;
+        if (i < end && (v[u] > bv || bi == 0x7fffffff)) { bv = v[u]; bi = i; }      // ascending i: strict > keeps the lowest index
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) better(bv, bi, __shfl_xor(bv, off, 64), __shfl_xor(bi, off, 64));
@@ -71,8 +82,11 @@ __global__ __launch_bounds__(256) void chunk_max_kernel(const float* __restrict_
     }
     const float* row = logits + (size_t)blockIdx.y * stride;
     const int begin = blockIdx.x * CHUNK, end = min(vocab, begin + CHUNK);
-    float mx = -INFINITY;
-    for (int i = begin + threadIdx.x; i < end; i += 256) mx = fmaxf(mx, row[i]);
+    float mx = -INFINITY, v[PER_THREAD];
+    load_run(row, begin, end, v);
+#pragma unroll
+    for (int u = 0; u < PER_THREAD; ++u)
+        if (begin + (int)threadIdx.x + 256 * u < end) mx = fmaxf(mx, v[u]);
     mx = wave_max(mx);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
     __syncthreads();
@@ -100,10 +114,16 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(const float* __restrict_
     const float temp = temperature[blockIdx.y], mx = row_max(part_m + (size_t)blockIdx.y * n_chunks, n_chunks);
     const int begin = blockIdx.x * CHUNK, end = min(vocab, begin + CHUNK);
     double sum = 0.0;
-    for (int i = begin + threadIdx.x; i < end; i += 256) {
-        const float e = expf((row[i] - mx) / temp);
-        if (kept != nullptr) kept[(size_t)blockIdx.y * vocab + i] = e;
-        sum += (double)e;
+    float v[PER_THREAD];
+    load_run(row, begin, end, v);
+#pragma unroll
+    for (int u = 0; u < PER_THREAD; ++u) {
+        const int i = begin + threadIdx.x + 256 * u;
+        if (i < end) {
+            const float e = expf((v[u] - mx) / temp);
+            if (kept != nullptr) kept[(size_t)blockIdx.y * vocab + i] = e;
+            sum += (double)e;
+        }
     }
     sum = wave_sum_f64(sum);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = sum;
