@@ -99,9 +99,16 @@ __device__ __forceinline__ double wave_sum_f64(double v) {
     return v;
 }
 
-__device__ __forceinline__ float row_max(const float* __restrict__ part_m, int n_chunks) {       // the same value in every thread
+// The row's maximum from its runs' maxima, the same value in every thread of a workgroup of 256: the threads read the runs'
+// maxima side by side and meet in LDS (`red`: 4 floats; a barrier inside, so every thread of the workgroup must come here).
+__device__ __forceinline__ float row_max(const float* __restrict__ part_m, int n_chunks, float* red) {
     float mx = -INFINITY;
-    for (int c = 0; c < n_chunks; ++c) mx = fmaxf(mx, part_m[c]);
+    for (int c = threadIdx.x; c < n_chunks; c += 256) mx = fmaxf(mx, part_m[c]);
+    mx = wave_max(mx);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
     return mx;
 }
 
@@ -110,12 +117,13 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(const float* __restrict_
                                                         const float* __restrict__ part_m, double* __restrict__ part_s, float* __restrict__ kept,
                                                         int vocab, long stride, int n_chunks) {
     __shared__ double red[4];
+    __shared__ float red_max[4];
     const float* row = logits + (size_t)blockIdx.y * stride;
-    const float temp = temperature[blockIdx.y], mx = row_max(part_m + (size_t)blockIdx.y * n_chunks, n_chunks);
     const int begin = blockIdx.x * CHUNK, end = min(vocab, begin + CHUNK);
-    double sum = 0.0;
     float v[PER_THREAD];
     load_run(row, begin, end, v);
+    const float temp = temperature[blockIdx.y], mx = row_max(part_m + (size_t)blockIdx.y * n_chunks, n_chunks, red_max);
+    double sum = 0.0;
 #pragma unroll
     for (int u = 0; u < PER_THREAD; ++u) {
         const int i = begin + threadIdx.x + 256 * u;
@@ -132,6 +140,7 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(const float* __restrict_
 }
 
 constexpr int RUN = CHUNK / 256;            // tokens a thread of the last stage owns
+constexpr int MAX_RUNS = 1024;              // runs of a row that the last stage holds in LDS (a vocabulary of 4 M tokens)
 
 __global__ __launch_bounds__(256) void sample_pick_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
                                                           const float* __restrict__ uniform, const float* __restrict__ part_m,
@@ -139,26 +148,47 @@ __global__ __launch_bounds__(256) void sample_pick_kernel(const float* __restric
                                                           int n_chunks) {
     __shared__ double wave_total[4];
     __shared__ int winner;
+    __shared__ float red_max[4];
+    __shared__ double run_sums[MAX_RUNS];
+    __shared__ double before_run;
+    __shared__ int the_run;
     const float* row = logits + (size_t)blockIdx.x * stride;
-    const float temp = temperature[blockIdx.x], mx = row_max(part_m + (size_t)blockIdx.x * n_chunks, n_chunks);
     const double* sums = part_s + (size_t)blockIdx.x * n_chunks;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int c = tid; c < n_chunks; c += 256) run_sums[c] = sums[c];           // side by side; added up in index order below
+    const float temp = temperature[blockIdx.x], mx = row_max(part_m + (size_t)blockIdx.x * n_chunks, n_chunks, red_max);     // (its barriers stand behind the writes above)
     // The reference normalises p by a 32-bit 1/sum before it draws; the draw compares u * sum(p) with
     // cumulative p, which is the same comparison scaled by a constant, so it is made on the
     // unnormalised values here.
-    double total = 0.0;
-    for (int c = 0; c < n_chunks; ++c) total += sums[c];
-    const double r = (double)uniform[blockIdx.x] * total;
-    int chunk = n_chunks - 1;                // the run that holds r (the last one if rounding lets none hold it)
-    double before = 0.0;
-    for (int c = 0; c < n_chunks - 1; ++c) {
-        if (r < before + sums[c]) { chunk = c; break; }
-        before += sums[c];
+    if (tid == 0) {
+        double total = 0.0;
+        for (int c = 0; c < n_chunks; ++c) total += run_sums[c];
+        const double r0 = (double)uniform[blockIdx.x] * total;
+        int chunk = n_chunks - 1;            // the run that holds r (the last one if rounding lets none hold it)
+        double before = 0.0;
+        for (int c = 0; c < n_chunks - 1; ++c) {
+            if (r0 < before + run_sums[c]) { chunk = c; break; }
+            before += run_sums[c];
+        }
+        the_run = chunk;
+        before_run = before;
+        run_sums[0] = r0;                    // (the sums have served)
     }
+    __syncthreads();
+    const int chunk = the_run;
+    double before = before_run;
+    const double r = run_sums[0];
     const int begin = chunk * CHUNK, end = min(vocab, begin + CHUNK);
     const int lo = min(end, begin + tid * RUN), hi = min(end, lo + RUN);
+    float mine_p[RUN];                       // the thread's tokens' p, asked for at once
+#pragma unroll
+    for (int u = 0; u < RUN; ++u) mine_p[u] = row[min(lo + u, vocab - 1)];
     double mine = 0.0;
-    for (int i = lo; i < hi; ++i) mine += (double)expf((row[i] - mx) / temp);
+#pragma unroll
+    for (int u = 0; u < RUN; ++u) {
+        mine_p[u] = expf((mine_p[u] - mx) / temp);
+        if (lo + u < hi) mine += (double)mine_p[u];
+    }
     double c = mine;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {                  // inclusive prefix sum over the lanes of a wave
@@ -173,9 +203,13 @@ __global__ __launch_bounds__(256) void sample_pick_kernel(const float* __restric
     if (lo < hi && r >= run_start && r < run_stop) {          // at most one thread
         double walk = run_start;
         int pick = min(hi, vocab - 1);
-        for (int i = lo; i < hi; ++i) {
-            walk += (double)expf((row[i] - mx) / temp);
-            if (r < walk) { pick = i; break; }
+        bool found = false;
+#pragma unroll
+        for (int u = 0; u < RUN; ++u) {
+            if (!found && lo + u < hi) {
+                walk += (double)mine_p[u];
+                if (r < walk) { pick = lo + u; found = true; }
+            }
         }
         winner = pick;
     }
@@ -554,6 +588,7 @@ GI_API int gi_sample_temperature(const float* logits, const float* temperature, 
     GI_REQUIRE(n_rows > 0 && n_rows <= 65535 && vocab > 0 && stride >= vocab, "sample_temperature: bad sizes (rows %d, vocab %d, stride %ld)", n_rows, vocab, stride);
     GI_REQUIRE(part_m != nullptr && part_s != nullptr, "sample_temperature: scratch is missing");
     const int n_chunks = gi_argmax_chunks(vocab);
+    GI_REQUIRE(n_chunks <= MAX_RUNS, "sample_temperature: a vocabulary of %d tokens is more than %d runs of %d", vocab, MAX_RUNS, CHUNK);
     chunk_max_kernel<<<dim3(n_chunks, n_rows), 256, 0, stream>>>(logits, part_m, vocab, stride, n_chunks, nullptr, 0);
     GI_CHECK_LAUNCH("sample_temperature (maxima)");
     chunk_sum_kernel<<<dim3(n_chunks, n_rows), 256, 0, stream>>>(logits, temperature, part_m, part_s, nullptr, vocab, stride, n_chunks);
