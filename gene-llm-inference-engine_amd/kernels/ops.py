@@ -571,12 +571,14 @@ def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096,
     groups = n_decode * n_kv * ((group + 15) // 16)
     max_waves = min(8, lib().gi_attention_decode_max_waves(hd))
     base = _decode_plain_shape(groups, span, max_waves, target_waves, small=fused and hd <= 64)
-    if target_waves != 4096 or (fused and hd < 128):
+    if target_waves != 4096:
         return base
-    if not fused:
+    if not fused or n_decode > 16:                   # (more than 16 rows: whichever kernel serves them)
         single = _decode_single_split(groups, span, hd, max_waves)
         if single is not None:
             return single
+    if fused and hd < 128:
+        return base
     gh = min(group, 16)
     units = lib().gi_compute_units()
     places = lambda n_waves: min(_decode_places(hd, fused, n_waves, gh), units) if fused else _decode_places(hd, fused, n_waves, gh)
@@ -679,9 +681,10 @@ def attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window=None):
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window)
 
 
-# With many rows the chip is full of waves and the fused kernel's extra registers cost more than the
-# rotation kernel's launch (measured at the Llama-3.2-1B shape: +2..3 % at 1 and 8 rows, -10 % at 64).
-FUSED_DECODE_MAX_ROWS = 16
+# Up to so many rows the decode kernel rotates and writes the pages itself.  It saves the rotation kernel's launch wherever the
+# q/k/v product does not rotate and store in its own epilogue (which it does from 33 rows on, and for long k from 17): +2..3 % a
+# step at 1 and 8 rows, and at 17 to 32 rows of the Llama-3.2-1B shape (24 rows 1.323 -> 1.290 ms).
+FUSED_DECODE_MAX_ROWS = 32
 
 
 def attention_from_products(q, k, v, cos, sin, cache, out, ctx, table, n_heads, n_kv, hd, window=None) -> bool:
