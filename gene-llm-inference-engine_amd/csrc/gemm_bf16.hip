@@ -436,7 +436,15 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
             // The sums go onto 32-bit rows whose next reader is a norm: the tile is laid into LDS (the ring is free once everyone
             // has read the last block) and leaves row by row, 32 threads a row with four columns each: the rows' new values, the
             // same times the norm's weights in bfloat16, and the tile's piece of every row's sum of squares (N is a multiple of 128).
-            constexpr int NT = 64 * WAVES_M * WAVES_N;
+            constexpr int NT = 64 * WAVES_M * WAVES_N, PASSES = 128 / (NT / 32);
+            // What the sums are added onto is asked for first, all of a thread's rows at once (a row beyond M is clamped and not
+            // written): read row by row behind the tile, it was a round trip to memory a row, eight in a row at the end of the kernel.
+            const int c4 = (tid & 31) * 4;
+            const float4 g = *reinterpret_cast<const float4*>(norm_out.g + n0 + c4);
+            float4 old[PASSES];
+#pragma unroll
+            for (int it = 0; it < PASSES; ++it)
+                old[it] = *reinterpret_cast<const float4*>((const float*)C + (size_t)min(m0 + (tid >> 5) + it * (NT / 32), M - 1) * ldc + n0 + c4);
             __syncthreads();
             float* tile = reinterpret_cast<float*>(ring);
 #pragma unroll
@@ -447,15 +455,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
                     for (int v = 0; v < 16; ++v)
                         tile[(wm + i * 32 + 8 * (v / 4) + 4 * (lane >> 5) + (v & 3)) * 128 + wn + j * 32 + (lane & 31)] = acc[i][j][v];
             __syncthreads();
-            const int c4 = (tid & 31) * 4;
-            const float4 g = *reinterpret_cast<const float4*>(norm_out.g + n0 + c4);
-            for (int row = tid >> 5; row < 128; row += NT / 32) {
-                const int m = m0 + row;
+#pragma unroll
+            for (int it = 0; it < PASSES; ++it) {
+                const int row = (tid >> 5) + it * (NT / 32), m = m0 + row;
                 float square = 0.f;
                 if (m < M) {
                     const float4 t = *reinterpret_cast<const float4*>(tile + row * 128 + c4);
                     float4* at = reinterpret_cast<float4*>((float*)C + (size_t)m * ldc + n0 + c4);
-                    float4 x = *at;
+                    float4 x = old[it];
                     x.x += t.x; x.y += t.y; x.z += t.z; x.w += t.w;
                     *at = x;
                     *reinterpret_cast<uint2*>(norm_out.scaled + (size_t)m * norm_out.ld + n0 + c4) =
