@@ -196,10 +196,13 @@ __global__ __launch_bounds__(256) void sample_pick_kernel(const float* __restric
         if (lane >= off) c += below;
     }
     if (lane == 63) wave_total[wave] = c;
+    const double c_below = __shfl_up(c, 1, 64);
     if (tid == 0) winner = min(end, vocab - 1);              // if rounding leaves r beyond the run: the next token in index order
     __syncthreads();
     for (int w = 0; w < wave; ++w) before += wave_total[w];
-    const double run_stop = before + c, run_start = run_stop - mine;
+    // A thread's tokens start where the thread before it stops, as the same sum: taken as `run_stop - mine` the start would fall
+    // back onto an earlier thread's tokens wherever those weigh less than the last bit of this thread's (u = 0 before a heavy token).
+    const double run_start = lane ? before + c_below : before, run_stop = before + c;
     if (lo < hi && r >= run_start && r < run_stop) {          // at most one thread
         double walk = run_start;
         int pick = min(hi, vocab - 1);

@@ -357,6 +357,21 @@ def test_sample_temperature_matches_the_inverse_distribution():
                 assert abs(got - want) == 1 and float((cum - float(us[i])).abs().min()) < 1e-6, (vocab, i, got, want)
 
 
+@pytest.mark.parametrize("vocab,light,heavy", [(100, 5, 40), (3000, 100, 1000), (3000, 17, 2999), (9000, 4000, 4095), (9000, 70, 5000)])
+def test_a_draw_of_zero_takes_the_first_token_that_has_any_probability(vocab, light, heavy):
+    """u = 0 stops at the first token whose probability is not zero (src/sampler/sampler.cpp:119-128), however little it weighs
+    beside a later one: 1e-35 before a token of probability 1 is below the last bit of the running sum in 64-bit, so a thread that
+    found where its tokens start by taking its own sum off the running one would start at 0 too and claim the draw."""
+    from plain_sampler import sample
+    logits = torch.full((3, vocab), -30.0)
+    logits[:, heavy] = 0.0
+    logits[0, light], logits[1, light], logits[2, light] = -0.8, -1.0, -1.04          # p = 1.8e-35, 3.8e-44 (subnormal), 0 at T = 0.01
+    out = torch.empty(3, dtype=torch.int32, device=DEV)
+    ops().sample_temperature(logits.to(DEV), torch.full((3,), 0.01, device=DEV), torch.zeros(3, device=DEV), out)
+    assert [sample(row.numpy(), 0.01, 0, 1.0, 0.0) for row in logits] == [light, light, heavy]
+    assert out.tolist() == [light, light, heavy]
+
+
 def on_an_edge(logits, temperature, top_k, top_p, u, got, want):
     """Whether the plain sampler could give `got` for `want` by rounding alone: two tokens whose probabilities differ in the
     last bits change places in the order, or u, or top_p times the kept mass, falls within 2e-6 of a boundary."""
