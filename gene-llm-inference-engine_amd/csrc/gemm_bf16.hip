@@ -3,7 +3,7 @@
 // Both operands are row-major with k contiguous, so each lane's operand of a matrix instruction is
 // one 16-byte load of 8 consecutive k.  Five kernels:
 //
-//   pingpong  large prompt-sized products (a 256 x 256 tile for every compute unit): operands loaded
+//   pingpong  large prompt-sized products (256 x 256 tiles for most of the compute units): operands loaded
 //           from global memory straight into two LDS stages; the workgroup's eight waves form two
 //           groups that take turns at reading LDS and at the matrix instructions.
 //   piped   the other products of 128 rows or more (K a multiple of 64): tiles of 128 x 128,
@@ -1443,8 +1443,14 @@ GI_API long gi_gemm_bf16_scratch_floats(int M, int N, int K) {
 // The most pieces a reader of M rows takes: what a writer of as many rows makes.
 static int consumer_max_parts(int M) { return M <= 16 ? slim_max_parts(M) : M <= 32 ? TILES_MAX_PARTS : REDUCE_MAX_PARTS; }
 
-// Whether a product of more than 128 rows takes the ping-pong kernel: a 256 x 256 tile or more for every compute unit.
-static bool takes_pingpong(int M, int N) { return (long)((M + 255) / 256) * ((N + 255) / 256) >= gi_compute_units(); }
+// Whether a product of more than 128 rows takes the ping-pong kernel: 256 x 256 tiles for three quarters of the compute units or
+// more.  (Measured on whole prompts, gate/up being the one product wide enough: with 192 tiles on 256 units 640 and 768 rows of
+// the Llama-3.2-1B shape take 2.94 and 3.51 ms against 3.27 and 3.81 with tiles of 128 x 128, the 3B shape 7.4 and 7.6 against 8.1
+// and 8.3, 320 to 512 rows of the 8B shape, 224 tiles, 10.7 to 11.0 against 12.1 to 12.5; with 128 tiles, half of the units, 512
+// rows take 2.82 ms against 2.73.  Long prompts whose narrower products reach that many tiles gain as much although this kernel
+// hands no norm on and the norm's own kernel runs again: 4,096 rows of the 3B shape 28.3 against 31.0 ms, 3,072 of the 8B shape
+// 47.4 against 52.8.)
+static bool takes_pingpong(int M, int N) { return (long)((M + 255) / 256) * ((N + 255) / 256) >= gi_compute_units() * 3 / 4; }
 
 static const NormIn NO_NORM_IN = {nullptr, 0, 0.f, 1};
 static const NormOut NO_NORM_OUT = {nullptr, nullptr, 0, nullptr};
@@ -1639,14 +1645,14 @@ static int launch_large(const void* A, const void* W, void* C, int epi, int M, i
         }
         return reduce_partials(scratch, C, epi, M, N, splits, ldc, stream, norm_in, norm_out);
     }
-    // Measured at 2,048 rows (K = 2048 and 8192): where 256 x 256 tiles give every compute unit one or more, they halve
+    // Measured at 2,048 rows (K = 2048 and 8192): where 256 x 256 tiles give three quarters of the compute units one or more, they halve
     // the traffic into LDS and run the two groups of waves out of step (the ping-pong kernel); otherwise 128 x 128, two
     // workgroups per unit with two stages each when there are enough tiles, else one workgroup of eight waves with four stages.
     const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
     GI_REQUIRE(norm_out.scaled == nullptr || (!takes_pingpong(M, N) && large_norm_parts(M, N, K) > 0), "gemm_bf16: a product of M %d, N %d, K %d hands no norm on", M, N, K);
     GI_REQUIRE(norm_in.squares == nullptr || rope != nullptr || (epi == EPI_GATED_BF16 && takes_pingpong(M, N) && norm_in.parts <= PIPED_MAX_PARTS),
                "gemm_bf16: a product of M %d, N %d, K %d takes no norm handed on in %d pieces", M, N, K, norm_in.parts);
-    if (takes_pingpong(M, N) && rope == nullptr) {     // a 256 x 256 tile or more for every compute unit: the ping-pong kernel
+    if (takes_pingpong(M, N) && rope == nullptr) {     // 256 x 256 tiles for most of the compute units: the ping-pong kernel
 #define PINGPONG(EPI_)                                                                                                                  \
     do {                                                                                                                                \
         constexpr int bytes = 2 * 512 * 128;                                                                                            \

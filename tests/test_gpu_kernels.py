@@ -63,8 +63,10 @@ def test_gemm_exact_rows_alone_have_the_same_bits(w_dtype, k):
                                    (513, 384, 1024), (2048, 96, 160),
                                    # the LDS-ring kernel: one block of k, edge tiles, each of its three tile choices
                                    (256, 160, 64), (130, 129, 192), (2100, 2200, 192), (4000, 8200, 128),
-                                   # the ping-pong kernel (a 256 x 256 tile or more for every compute unit): one block of k, an odd number of them, edges
+                                   # the ping-pong kernel (256 x 256 tiles for every compute unit or more): one block of k, an odd number of them, edges
                                    (4100, 4104, 64), (4096, 4100, 320),
+                                   # ... with tiles for three quarters of the compute units only (3 x 64, and 3 x 65 with an edge on both sides)
+                                   (768, 16384, 64), (520, 16400, 192),
                                    # ... and with k shared out over workgroups because the tiles are few
                                    (200, 256, 1024), (300, 2048, 2048), (129, 130, 512),
                                    # 65 to 128 rows: the skinny kernel with six or eight tiles of rows, narrow outputs (k shared out) and wide ones
@@ -92,7 +94,7 @@ def test_gemm_bf16(m, n, k, out_dtype, accumulate):
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 8), (5, 48, 136), (16, 160, 96), (17, 176, 64), (64, 32, 264), (70, 192, 128), (300, 8192 // 16, 2048 // 8),
                                        (72, 8192, 2048), (128, 6144, 264), (100, 288, 136),
                                        (40, 6144, 264), (13, 6160, 72), (64, 8192, 512), (2048, 1024, 192), (600, 288, 64), (200, 512, 1024),
-                                       (4100, 2064, 128)])
+                                       (4100, 2064, 128), (640, 8192, 128), (530, 8208, 192)])
 def test_gemm_bf16_gated(m, inter, k):
     a = randn(m, k, dtype=torch.bfloat16, seed=15)
     gate, up = randn(inter, k, dtype=torch.bfloat16, seed=16, scale=0.3), randn(inter, k, dtype=torch.bfloat16, seed=17, scale=0.3)
@@ -202,7 +204,9 @@ def test_rope_cos_sin_uses_64_bit_angles():
                                             # the rows of prompts: from the tiles of 128 x 128 (or the kernel that adds the shares of k) to the gated
                                             # product on the kernel with tiles of 256 x 256
                                             (2048, 2048, 2048, 16384, True), (2048, 2048, 8192, 16384, True), (1024, 2048, 2048, 16384, True),
-                                            (1500, 3072, 1024, 16384, True)])
+                                            (1500, 3072, 1024, 16384, True),
+                                            # ... with tiles of 256 x 256 for three quarters of the compute units
+                                            (640, 2048, 2048, 16384, True), (530, 2048, 8192, 16384, True)])
 def test_norm_handed_from_one_product_to_the_next(m, d, k1, n2, gated):
     """A product that adds onto rows x also writes g * x and the pieces of the rows' sums of squares; the next product reads
     g * x and multiplies its results by rsqrt(mean(x^2) + eps).  The rows x are what the plain product leaves, bit for bit; the
@@ -241,7 +245,7 @@ def test_norm_handed_from_one_product_to_the_next(m, d, k1, n2, gated):
 
 
 @pytest.mark.parametrize("m,d,k1", [(2048, 2048, 8192), (1100, 2048, 2048), (300, 2048, 2048), (2048, 3072, 8192), (700, 1024, 512), (130, 256, 192),
-                                    (4100, 3072, 256)])
+                                    (3000, 3072, 256), (4100, 2048, 256)])
 def test_norm_handed_on_by_a_product_of_many_rows(m, d, k1):
     """The rows of prompts: the product that adds onto the residual writes g * x and the pieces of the rows' sums of squares from
     its tiles' epilogues (one piece per 128 columns), or from the kernel that adds the shares of k (one per 1024).  The rows are
