@@ -772,7 +772,9 @@ constexpr int KB = 2 * SK, X_STRIDE = KB + 8;         // k per block of the work
 constexpr int SLIM_PIECES = 8;
 // Outputs of fewer than so many strips of 16 weight rows take strips of 8, twice the workgroups; with up to 8 rows of A, where a
 // strip of 8 leaves no lane idle (FOLD = 1 below), of fewer than twice as many (measured at N = 4096 to 6144: 1 to 2 % of the
-// decode step at 1 to 8 rows, and 7 % the other way at 12 and 16 rows).
+// decode step at 1 to 8 rows, and 7 % the other way at 12 and 16 rows); a product that adds onto rows and hands a norm on does
+// so up to 3 rows only (N = 4096, K = 4096 and 14336 at 8 rows: 18.5 us with strips of 16 against 20.5, the step of the 8B shape
+// 4.47 -> 4.3 ms; equal at 4 rows, 0.5 % the other way at 1 and 2).
 constexpr int SLIM_NARROW_STRIPS = 256;
 __host__ __device__ constexpr int slim_max_parts(int M) { return SLIM_PIECES * (M <= 8 ? 64 : 32); }
 // The kernels for 17 to 128 rows: the kernel that adds the partial sums onto x writes one piece per 1024 columns.
@@ -1490,8 +1492,15 @@ static bool takes_slim(int M, int N, int K) {
 }
 
 // Workgroups of the slim kernel for an output of N columns that is not gated: the pieces a row's sum of squares comes in.
-static bool slim_wide_strips(int M, int N) { return (N + 15) / 16 > (M <= 8 ? 2 * SLIM_NARROW_STRIPS : SLIM_NARROW_STRIPS) - 1; }
-static int slim_parts(int M, int N) { return slim_wide_strips(M, N) ? (N + 15) / 16 : (N + 7) / 8; }
+// (A product that adds onto rows may hand a norm on, with one piece of the rows' sums of squares per workgroup: it takes strips
+// of 8 only where the reader takes that many pieces.  N = 3072 at 9 to 16 rows: 384 strips of 8 would be more than the 256 pieces
+// a reader of so many rows takes, and the norm's own kernel would run twice a layer; 192 strips of 16 hand it on.)
+static bool slim_wide_strips(int M, int N, int epi) {
+    const bool doubled = M <= 8 && (epi != EPI_ADD_F32 || M <= 3);
+    const bool few = (N + 15) / 16 <= (doubled ? 2 * SLIM_NARROW_STRIPS : SLIM_NARROW_STRIPS) - 1;
+    return !(few && (epi != EPI_ADD_F32 || (N + 7) / 8 <= slim_max_parts(M)));
+}
+static int slim_parts(int M, int N) { return slim_wide_strips(M, N, EPI_ADD_F32) ? (N + 15) / 16 : (N + 7) / 8; }
 
 static int launch_slim(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in,
                        NormOut norm_out, hipStream_t stream) {
@@ -1504,7 +1513,7 @@ static int launch_slim(const void* A, const void* W, void* C, int epi, int M, in
     if (epi == EPI_GATED_BF16) {
         dim3 grid(N / 32);
         SLIM(2, 16, EPI_GATED_BF16);
-    } else if (slim_wide_strips(M, N)) {
+    } else if (slim_wide_strips(M, N, epi)) {
         dim3 grid((N + 15) / 16);
         if (epi == EPI_STORE_F32) SLIM(1, 16, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 16, EPI_ADD_F32); else SLIM(1, 16, EPI_STORE_BF16);
     } else {                                   // a narrow output: strips of 8 rows, twice the workgroups

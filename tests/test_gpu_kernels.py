@@ -201,6 +201,9 @@ def test_rope_cos_sin_uses_64_bit_angles():
                                             (100, 4096, 14336, 6144, False), (128, 3072, 8192, 16384, True), (33, 1024, 512, 12288, False),
                                             (24, 2048, 2048, 16384, True), (24, 2048, 8192, 3072, False), (14, 2048, 2048, 16384, True), (32, 2048, 2048, 2048, False),
                                             (17, 264, 136, 12288, False), (13, 4096, 4096, 28672, True),
+                                            # strips of 16 weight rows where strips of 8 would make more pieces than the reader takes (9 to 16 rows), and
+                                            # from 4 rows on for the product that hands on with 256 strips or more
+                                            (12, 3072, 8192, 5120, False), (16, 3072, 3072, 16384, True), (8, 4096, 14336, 6144, False), (4, 4096, 4096, 28672, True),
                                             # the rows of prompts: from the tiles of 128 x 128 (or the kernel that adds the shares of k) to the gated
                                             # product on the kernel with tiles of 256 x 256
                                             (2048, 2048, 2048, 16384, True), (2048, 2048, 8192, 16384, True), (1024, 2048, 2048, 16384, True),
