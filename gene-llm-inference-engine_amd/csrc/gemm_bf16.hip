@@ -1484,10 +1484,15 @@ static int reduce_partials(const float* scratch, void* C, int epi, int M, int N,
 
 // Up to 16 rows the slim kernel (no LDS staging, one launch) is the faster one, except for wide outputs with more
 // than a few rows, where its per-workgroup reading of the activations costs more than the skinny kernel's staging
-// (measured crossovers at K = 2048: 12 rows for 256 strips of 64 columns, 5 rows for 2004 strips).
+// (measured crossovers, whole decode steps: 12 rows for 256 strips of 64 columns at K = 2048, 8 to 9 rows for 256 strips at
+// K = 3072, 3 rows for 448 strips at K = 4096, where the 8B shape's step lost 3 to 5 % at 6 to 10 rows with the crossover at 12;
+// 5 rows for the 2004 strips of the vocabulary at K = 2048): the longer the rows and the more strips, the sooner, as
+// 12 * (2048 / K) * (256 / strips), between 3 and 12.
 static bool takes_slim(int M, int N, int K) {
     const int strips64 = (N + 63) / 64;
-    const bool wide_skinny = gi_gemm_bf16_skinny_splits(N, K) == 0 && (M >= 12 || (M >= 5 && strips64 >= 1024));
+    const double fitted = 12.0 * (2048.0 / K) * (256.0 / strips64);
+    const int wide_rows = strips64 >= 1024 ? 5 : fitted < 3 ? 3 : fitted > 12 ? 12 : (int)(fitted + 0.5);
+    const bool wide_skinny = gi_gemm_bf16_skinny_splits(N, K) == 0 && M >= wide_rows;
     return M <= 16 && !wide_skinny;
 }
 
