@@ -1140,7 +1140,7 @@ __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_kernel(const bf16_t* __
     const int strip = wave % STRIPS, slice = wave / STRIPS;
     const int r = FOLD ? lane & 7 : lane & 15, q = lane >> 4;
     const int k_lane = 8 * q + (FOLD ? 32 * ((lane >> 3) & 1) : 0);   // where in a product's span of k this lane reads
-    const int n = (blockIdx.x * STRIPS + strip) * ROWS + r;
+    const int n = (blockIdx.x * STRIPS + strip) * ROWS + (r < ROWS ? r : ROWS - 1);      // (lanes beyond a strip of 10 or 12 rows ask for its last row again)
     // Every lane issues every load of a block (a row beyond the operand is clamped into it and lands in results that are never
     // written; in a row's last, ragged block k is clamped too and the activations beyond K become zeros), and what a wave skips it
     // skips as a whole: the compiler then counts the loads in flight, and a block's products wait for that block alone.
@@ -1508,16 +1508,17 @@ static bool slim_wide_strips(int M, int N, int epi) {
 // Weight rows per workgroup of the slim kernel for an output that is not gated: 16 or 8 by the rules above, unless that many
 // workgroups fill the compute units unevenly (384 strips of 8 or 192 of 16 on 256 units: a quarter of the chip waits for the
 // rest) and strips of 12 or 10 rows fill them evenly (3,072 columns: 256 strips of 12) with no more pieces than a reader takes.
-// Measured on the decode step: 8 to 16 rows of the 1B shape (q/k/v of 3,072 columns) 1 to 2 % faster, 8 rows of the 3B shape
-// (rows of 3,072: 11.7 against 12.9 us a product) 1.4 %; 1 to 4 rows 0.5 to 4 % slower, where a strip of 8 folds k into its idle
-// lanes, and 640 strips of 8 (5,120 columns, five sixths even) are faster than 512 of 10 (11.9 against 12.9 us).
+// A product's 16 weight rows beyond such a strip repeat its last row (the same cache line, no further traffic) and their results
+// are dropped.  Measured on the decode step: the 1B shape (q/k/v of 3,072 columns) 1 to 2 % faster at 1 to 16 rows, the 3B shape
+// (rows of 3,072: 11.7 against 12.9 us a product at 8 rows) 3 to 5 %.  640 strips of 8 (5,120 columns, five sixths even) are
+// faster than 512 of 10 (11.9 against 12.9 us): the even strips are taken where the usual ones are less than four fifths even.
 static int slim_strip_rows(int M, int N, int epi) {
     const int usual = slim_wide_strips(M, N, epi) ? 16 : 8, units = gi_compute_units();
     auto evenness = [&](int rows) {
         const int groups = (N + rows - 1) / rows;
         return (double)groups / ((groups + units - 1) / units * units);
     };
-    if (M < 8 || evenness(usual) >= 0.8) return usual;      // (few rows: the folded strips of 8 are worth more than even filling)
+    if (evenness(usual) >= 0.8) return usual;
     for (int rows : {12, 10})
         if (evenness(rows) >= 0.95 && (epi != EPI_ADD_F32 || (N + rows - 1) / rows <= slim_max_parts(M))) return rows;
     return usual;
@@ -1541,7 +1542,7 @@ static int launch_slim(const void* A, const void* W, void* C, int epi, int M, in
     } else if (slim_strip_rows(M, N, epi) == 16) {
         dim3 grid((N + 15) / 16);
         if (epi == EPI_STORE_F32) SLIM(1, 16, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 16, EPI_ADD_F32); else SLIM(1, 16, EPI_STORE_BF16);
-    } else if (slim_strip_rows(M, N, epi) == 12) {     // (of the 16 weight rows a workgroup loads, the last 4 are the next strip's and their results are dropped)
+    } else if (slim_strip_rows(M, N, epi) == 12) {     // (the last 4 of a product's 16 weight rows are the strip's last row again; their results are dropped)
         dim3 grid((N + 11) / 12);
         if (epi == EPI_STORE_F32) SLIM(1, 12, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 12, EPI_ADD_F32); else SLIM(1, 12, EPI_STORE_BF16);
     } else if (slim_strip_rows(M, N, epi) == 10) {
