@@ -1305,14 +1305,17 @@ __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_kernel(const bf16_t* __
 // second kernel to add them, costs that kernel's launch and as many bytes of partial sums as the output projection has weights.
 template <int MT, int EPI>
 __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_tiles_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
-                                                                  int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in, NormOut norm_out) {
+                                                                  int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in, NormOut norm_out,
+                                                                  int strip_rows) {
     constexpr int SLICES = 8, STEP = SLICES * SK, DEPTH = 2;
     __shared__ float red[SLICES][MT][64][4];
     __shared__ float row_scale[MT * 16 < 32 ? 32 : MT * 16];
     static_assert(MT == 2, "the epilogue's sums of squares take every thread's one result to lie in one row of 16 threads");
     const int tid = threadIdx.x, lane = tid & 63, slice = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
-    const int n = blockIdx.x * 16 + r;
+    // strip_rows (8, 12 or 16) of the product's 16 weight rows are the workgroup's own; lanes beyond them ask for its last row again
+    // (the same cache line) and their results are dropped
+    const int n = blockIdx.x * strip_rows + min(r, strip_rows - 1);
     const bf16_t* wrow = W + (size_t)min(n, N - 1) * ldw + 8 * q;         // (every lane issues every load of a block, as in the kernel above)
     const bf16_t* xrow[MT];
 #pragma unroll
@@ -1334,7 +1337,7 @@ __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_tiles_kernel(const bf16
     // (what the epilogue adds onto is asked for first, as in the kernel above: every thread has one result, e = tid below)
     [[maybe_unused]] float old_value = 0.f, gain = 0.f;
     if constexpr (EPI == EPI_ADD_F32) {
-        const int e_row = 16 * (tid >> 8) + ((tid >> 4) & 15), e_col = blockIdx.x * 16 + (tid & 15);
+        const int e_row = 16 * (tid >> 8) + ((tid >> 4) & 15), e_col = blockIdx.x * strip_rows + (tid & 15);
         old_value = ((const float*)C)[(size_t)min(e_row, M - 1) * ldc + min(e_col, N - 1)];
         if (norm_out.scaled != nullptr) gain = norm_out.g[min(e_col, N - 1)];
     }
@@ -1377,7 +1380,7 @@ __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_tiles_kernel(const bf16
     // Element v of a lane's result for tile t: activation row 16*t + 4*q + v, weight row r of the strip.
     for (int e = tid; e < MT * 256; e += 512) {
         const int t = e >> 8, m = (e >> 4) & 15, c = e & 15;
-        const int src_lane = c + 16 * (m >> 2), v = m & 3, row = 16 * t + m, col = blockIdx.x * 16 + c;
+        const int src_lane = c + 16 * (m >> 2), v = m & 3, row = 16 * t + m, col = c < strip_rows ? blockIdx.x * strip_rows + c : N;
         float sum = 0.f;
 #pragma unroll
         for (int s = 0; s < SLICES; ++s) sum += red[s][t][src_lane][v];
@@ -1578,14 +1581,30 @@ static bool takes_slim_tiles(int M, int N, int K, int epi) {
     return !takes_slim(M, N, K) && M <= 32 && K <= 2048 && epi != EPI_GATED_BF16 && gi_gemm_bf16_skinny_splits(N, K) > 0;
 }
 
+// Weight rows per workgroup of that kernel: 16, or 12 or 8 where strips of 16 fill the compute units unevenly and those fill
+// them evenly (2,048 columns: 256 strips of 8, not 128 of 16; 3,072: 256 of 12, not 192 of 16: the decode step of the 1B shape at 17 to 32
+// rows 1 to 1.5 % faster), never more strips than a reader takes pieces.
+static int tiles_strip_rows(int N) {
+    const int units = gi_compute_units();
+    auto evenness = [&](int rows) {
+        const int groups = (N + rows - 1) / rows;
+        return (double)groups / ((groups + units - 1) / units * units);
+    };
+    if (evenness(16) >= 0.8) return 16;
+    for (int rows : {12, 8})
+        if (evenness(rows) >= 0.95 && (N + rows - 1) / rows <= TILES_MAX_PARTS) return rows;
+    return 16;
+}
+
 static int launch_slim_tiles(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, NormIn norm_in,
                              NormOut norm_out, hipStream_t stream) {
-    dim3 grid((N + 15) / 16);
+    const int strip_rows = tiles_strip_rows(N);
+    dim3 grid((N + strip_rows - 1) / strip_rows);
 #define SLIM_TILES(MT_)                                                                                                                             \
     do {                                                                                                                                            \
-        if (epi == EPI_STORE_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out); \
-        else if (epi == EPI_ADD_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_ADD_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out); \
-        else gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_BF16><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out); \
+        if (epi == EPI_STORE_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out, strip_rows); \
+        else if (epi == EPI_ADD_F32) gemm_bf16_slim_tiles_kernel<MT_, EPI_ADD_F32><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out, strip_rows); \
+        else gemm_bf16_slim_tiles_kernel<MT_, EPI_STORE_BF16><<<grid, 512, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, norm_in, norm_out, strip_rows); \
     } while (0)
     SLIM_TILES(2);
 #undef SLIM_TILES
@@ -1730,7 +1749,10 @@ GI_API int gi_gemm_bf16_norm_parts(int M, int N, int K) {
         const int parts = slim_parts(M, N);
         return parts <= slim_max_parts(M) ? parts : 0;
     }
-    if (takes_slim_tiles(M, N, K, EPI_ADD_F32)) return (N + 15) / 16 <= TILES_MAX_PARTS ? (N + 15) / 16 : 0;
+    if (takes_slim_tiles(M, N, K, EPI_ADD_F32)) {
+        const int parts = (N + tiles_strip_rows(N) - 1) / tiles_strip_rows(N);
+        return parts <= TILES_MAX_PARTS ? parts : 0;
+    }
     if (M > SKINNY_MAX_ROWS) return large_norm_parts(M, N, K);
     if (M <= 16 || gi_gemm_bf16_skinny_splits(N, K) == 0) return 0;
     return N % REDUCE_COLUMNS == 0 && N / REDUCE_COLUMNS <= REDUCE_MAX_PARTS ? N / REDUCE_COLUMNS : 0;
