@@ -78,7 +78,9 @@ def test_gemm_exact_rows_alone_have_the_same_bits(w_dtype, k):
                                    # up to 8 rows and a narrow output: the idle halves of the matrix instructions take a further 32 of k (blocks of 256, cut anywhere)
                                    (8, 2048, 8192), (4, 3072, 2048), (2, 3072, 264), (6, 1000, 1000), (7, 60, 8200), (8, 8, 32), (5, 24, 40),
                                    # ... and 9 to 16 rows, in two groups of 8 that share the weights
-                                   (12, 2048, 8192), (9, 100, 136), (16, 3072, 2048), (13, 1000, 1000), (16, 8, 32)])
+                                   (12, 2048, 8192), (9, 100, 136), (16, 3072, 2048), (13, 1000, 1000), (16, 8, 32),
+                                   # strips of 12 or 8 weight rows that fill the compute units evenly, the last strip ragged (up to 16 rows, and 17 to 32)
+                                   (13, 3000, 264), (8, 3071, 264), (3, 3072, 2048), (20, 2000, 264), (32, 2920, 2048)])
 @pytest.mark.parametrize("out_dtype,accumulate", [(torch.float32, False), (torch.float32, True), (torch.bfloat16, False)])
 def test_gemm_bf16(m, n, k, out_dtype, accumulate):
     a, w = randn(m, k, dtype=torch.bfloat16, seed=5), randn(n, k, dtype=torch.bfloat16, seed=6)
